@@ -1,0 +1,232 @@
+"""TEST INFRASTRUCTURE ONLY: numpy-facing wrappers over ``oracle/liboracle.so``.
+
+``liboracle.so`` is this repo's CPU restatement (``oracle/oracle.cpp``) of the
+TenniS reference hot path.  It is the parity checker for the HIP kernels; only
+tests, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py``
+may import this module.  The product path never does.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_PATH = os.path.join(_HERE, "liboracle.so")
+_lib = None
+
+_vp = ctypes.c_void_p
+_i = ctypes.c_int
+_i64 = ctypes.c_int64
+_f = ctypes.c_float
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_PATH):
+            raise RuntimeError("oracle not built: run `make -C oracle oracle`")
+        L = ctypes.CDLL(_PATH)
+        L.orc_set_threads.argtypes = [_i]
+        L.orc_get_max_threads.restype = _i
+        L.orc_quantize_f32.argtypes = [_vp, _i64, _vp, _i, _vp]
+        L.orc_im2col_i8.argtypes = [_vp] + [_i] * 13 + [_vp, ctypes.c_int8]
+        L.orc_im2col_f32.argtypes = [_vp] + [_i] * 13 + [_vp, _f]
+        L.orc_gemm_i8.argtypes = [_i, _i, _i, _vp, _vp, _vp, _i]
+        L.orc_conv2d_quantized.argtypes = [_vp, _i, _i, _i, _i, _vp] + [_i] * 11 + [_f, _vp, _vp, _vp, _i]
+        L.orc_add_bias_f32.argtypes = [_vp, _i64, _i, _i64, _vp, _vp]
+        L.orc_relu_f32.argtypes = [_vp, _i64, _vp]
+        L.orc_leaky_relu_f32.argtypes = [_vp, _i64, _f, _vp]
+        L.orc_epilogue.argtypes = [_vp, _i64, _i, _i64, _vp, _vp, _vp, _i, _f, _vp, _vp, _i, _vp]
+        L.orc_conv2d_i8_fused.argtypes = ([_vp, _i, _i, _i, _i, _vp] + [_i] * 11 +
+                                          [_f, _vp, _vp, _i, _f, _vp, _vp, _i, _vp])
+        L.orc_gemm_i8_dequant.argtypes = [_i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]
+        L.orc_gemm_f32.argtypes = [_i, _i, _i, _vp, _vp, _vp]
+        L.orc_conv2d_f32.argtypes = [_vp, _i, _i, _i, _i, _vp] + [_i] * 11 + [_f, _vp]
+        L.orc_inner_prod_f32.argtypes = [_vp, _i, _i, _vp, _i, _i, _vp]
+        L.orc_winograd_f63.argtypes = [_vp, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _f, _vp]
+        _lib = L
+    return _lib
+
+
+def set_threads(n):
+    lib().orc_set_threads(int(n))
+
+
+def max_threads():
+    return lib().orc_get_max_threads()
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(_vp)
+
+
+def _c(a, dt):
+    return None if a is None else np.ascontiguousarray(a, dt)
+
+
+def out_hw(h, w, kh, kw, pads, strides, dilations):
+    """include/backend/common_function.h:30-40."""
+    ho = (h + pads[0] + pads[1] - (dilations[0] * (kh - 1) + 1)) // strides[0] + 1
+    wo = (w + pads[2] + pads[3] - (dilations[1] * (kw - 1) + 1)) // strides[1] + 1
+    return ho, wo
+
+
+def quantize(x, scales):
+    x = _c(x, np.float32)
+    s = _c(np.atleast_1d(scales), np.float32)
+    out = np.empty(x.shape, np.int8)
+    lib().orc_quantize_f32(_p(x), x.size, _p(s), s.size, _p(out))
+    return out
+
+
+def im2col(x, kh, kw, pads, strides, dilations, padding_value=0):
+    c, h, w = x.shape
+    ho, wo = out_hw(h, w, kh, kw, pads, strides, dilations)
+    out = np.empty((c * kh * kw, ho * wo), x.dtype)
+    x = np.ascontiguousarray(x)
+    fn = lib().orc_im2col_i8 if x.dtype == np.int8 else lib().orc_im2col_f32
+    fn(_p(x), c, h, w, kh, kw, *pads, *strides, *dilations, _p(out), padding_value)
+    return out
+
+
+def gemm_i8(a, b, faithful=False):
+    a = _c(a, np.int8)
+    b = _c(b, np.int8)
+    m, k = a.shape
+    n = b.shape[1]
+    c = np.empty((m, n), np.int32)
+    lib().orc_gemm_i8(m, n, k, _p(a), _p(b), _p(c), int(faithful))
+    return c
+
+
+def conv2d_quantized(x, w, dq, pads=(0, 0, 0, 0), strides=(1, 1), dilations=(1, 1), padding_value=0.0,
+                     return_acc=False, faithful=False):
+    x = _c(x, np.int8)
+    w = _c(w, np.int8)
+    dq = _c(dq, np.float32)
+    n, c, h, wd = x.shape
+    cout, _, kh, kw = w.shape
+    ho, wo = out_hw(h, wd, kh, kw, pads, strides, dilations)
+    out = np.empty((n, cout, ho, wo), np.float32)
+    acc = np.empty((n, cout, ho, wo), np.int32) if return_acc else None
+    lib().orc_conv2d_quantized(_p(x), n, c, h, wd, _p(w), cout, kh, kw, *pads, *strides, *dilations,
+                               padding_value, _p(dq), _p(out), _p(acc), int(faithful))
+    return (out, acc) if return_acc else out
+
+
+def add_bias(x, bias, dim=1):
+    x = _c(x, np.float32)
+    bias = _c(bias, np.float32)
+    pre = int(np.prod(x.shape[:dim], dtype=np.int64))
+    inner = int(np.prod(x.shape[dim + 1:], dtype=np.int64))
+    out = np.empty_like(x)
+    lib().orc_add_bias_f32(_p(x), pre, x.shape[dim], inner, _p(bias), _p(out))
+    return out
+
+
+def relu(x):
+    x = _c(x, np.float32)
+    out = np.empty_like(x)
+    lib().orc_relu_f32(_p(x), x.size, _p(out))
+    return out
+
+
+def leaky_relu(x, scale):
+    x = _c(x, np.float32)
+    out = np.empty_like(x)
+    lib().orc_leaky_relu_f32(_p(x), x.size, scale, _p(out))
+    return out
+
+
+ACT = {None: 0, "none": 0, "relu": 1, "leaky_relu": 2}
+
+
+def epilogue(acc, dq, bias=None, act=None, slope=0.0, q_scales=None, row_scale=None, want_f32=True):
+    """acc is [pre, channels, *inner] int32."""
+    acc = _c(acc, np.int32)
+    pre, ch = acc.shape[0], acc.shape[1]
+    inner = int(np.prod(acc.shape[2:], dtype=np.int64))
+    dq = _c(dq, np.float32)
+    bias = _c(bias, np.float32)
+    row_scale = _c(row_scale, np.float32)
+    out = np.empty(acc.shape, np.float32) if want_f32 else None
+    qs = _c(None if q_scales is None else np.atleast_1d(q_scales), np.float32)
+    q = np.empty(acc.shape, np.int8) if qs is not None else None
+    lib().orc_epilogue(_p(acc), pre, ch, inner, _p(dq), _p(row_scale), _p(bias), ACT[act], slope, _p(out),
+                       _p(qs), 0 if qs is None else qs.size, _p(q))
+    return out, q
+
+
+def conv2d_i8_fused(x, w, dq, bias=None, act=None, slope=0.0, q_scales=None, pads=(0, 0, 0, 0), strides=(1, 1),
+                    dilations=(1, 1), padding_value=0.0):
+    x = _c(x, np.int8)
+    w = _c(w, np.int8)
+    dq = _c(dq, np.float32)
+    bias = _c(bias, np.float32)
+    n, c, h, wd = x.shape
+    cout, _, kh, kw = w.shape
+    ho, wo = out_hw(h, wd, kh, kw, pads, strides, dilations)
+    out = np.empty((n, cout, ho, wo), np.float32)
+    qs = _c(None if q_scales is None else np.atleast_1d(q_scales), np.float32)
+    q = np.empty((n, cout, ho, wo), np.int8) if qs is not None else None
+    lib().orc_conv2d_i8_fused(_p(x), n, c, h, wd, _p(w), cout, kh, kw, *pads, *strides, *dilations, padding_value,
+                              _p(dq), _p(bias), ACT[act], slope, _p(out), _p(qs), 0 if qs is None else qs.size,
+                              _p(q))
+    return out, q
+
+
+def gemm_i8_dequant(a, b, dq_w, dq_a=None, bias=None, return_acc=False):
+    a = _c(a, np.int8)
+    b = _c(b, np.int8)
+    m, k = a.shape
+    n = b.shape[1]
+    dq_w = _c(dq_w, np.float32)
+    dq_a = _c(dq_a, np.float32)
+    bias = _c(bias, np.float32)
+    out = np.empty((m, n), np.float32)
+    acc = np.empty((m, n), np.int32) if return_acc else None
+    lib().orc_gemm_i8_dequant(m, n, k, _p(a), _p(b), _p(dq_w), _p(dq_a), _p(bias), _p(out), _p(acc))
+    return (out, acc) if return_acc else out
+
+
+def gemm_f32(a, b):
+    a = _c(a, np.float32)
+    b = _c(b, np.float32)
+    m, k = a.shape
+    n = b.shape[1]
+    c = np.empty((m, n), np.float32)
+    lib().orc_gemm_f32(m, n, k, _p(a), _p(b), _p(c))
+    return c
+
+
+def conv2d_f32(x, w, pads=(0, 0, 0, 0), strides=(1, 1), dilations=(1, 1), padding_value=0.0):
+    x = _c(x, np.float32)
+    w = _c(w, np.float32)
+    n, c, h, wd = x.shape
+    cout, _, kh, kw = w.shape
+    ho, wo = out_hw(h, wd, kh, kw, pads, strides, dilations)
+    out = np.empty((n, cout, ho, wo), np.float32)
+    lib().orc_conv2d_f32(_p(x), n, c, h, wd, _p(w), cout, kh, kw, *pads, *strides, *dilations, padding_value,
+                         _p(out))
+    return out
+
+
+def inner_prod_f32(lhs, rhs, transpose=False):
+    lhs = _c(lhs, np.float32)
+    rhs = _c(rhs, np.float32)
+    m, k = lhs.shape
+    n = rhs.shape[0] if transpose else rhs.shape[1]
+    out = np.empty((m, n), np.float32)
+    lib().orc_inner_prod_f32(_p(lhs), m, k, _p(rhs), n, int(transpose), _p(out))
+    return out
+
+
+def winograd_f63(x, w, pads, padding_value=0.0):
+    x = _c(x, np.float32)
+    w = _c(w, np.float32)
+    n, c, h, wd = x.shape
+    cout = w.shape[0]
+    ho, wo = out_hw(h, wd, 3, 3, pads, (1, 1), (1, 1))
+    out = np.empty((n, cout, ho, wo), np.float32)
+    lib().orc_winograd_f63(_p(x), n, c, h, wd, _p(w), cout, *pads, padding_value, _p(out))
+    return out
