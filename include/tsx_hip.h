@@ -1,0 +1,125 @@
+/*
+ * tsx_hip.h -- the C ABI of the MI355X (gfx950) convolution hot path for TenniS.
+ *
+ * This is the drop-in boundary: plain pointers and sizes, no C++ or torch types.
+ * The "hip" device operator classes (tennis_amd/backend) call these launchers from
+ * the core methods TenniS declares per device; each entry point cites the reference
+ * interface it stands in for (paths relative to the TenniS tree).
+ *
+ * Conventions
+ *   - every pointer named *_dev is device memory on the current HIP device; the
+ *     library never owns, allocates or frees caller memory;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); all
+ *     launches are asynchronous on it, nothing synchronises;
+ *   - return value 0 = success; > 0 = a hipError_t from the runtime; < 0 = a
+ *     TSX_E_* argument/shape error.  tsx_last_error() gives the message (thread-local);
+ *   - tensors are NCHW, dense, row-major, exactly as the reference's operators see them.
+ */
+#ifndef TSX_HIP_H
+#define TSX_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TSX_E_INVALID   (-1)  /* bad argument / unsupported shape */
+#define TSX_E_WORKSPACE (-2)  /* workspace too small */
+#define TSX_E_NODEVICE  (-3)  /* no usable gfx950 device */
+
+const char *tsx_last_error(void);
+/* Library/ABI version (major*100 + minor). */
+int tsx_version(void);
+/* Number of compute units of the current device (for launch heuristics and roofline peaks). */
+int tsx_device_cu_count(void);
+
+/* Geometry of one 2-D convolution, as base::Conv2D / base::Conv2DQuantized hand it to
+ * their core: x [n,c,h,w], w [cout,c,kh,kw], Padding2D{top,bottom,left,right},
+ * Stride2D, Dilation2D (include/backend/common_structure.h:10-62).  Output size follows
+ * conv2d_forward (include/backend/common_function.h:30-40). */
+typedef struct tsx_conv2d_geom {
+    int32_t n, c, h, w;
+    int32_t cout, kh, kw;
+    int32_t pad_top, pad_bottom, pad_left, pad_right;
+    int32_t stride_h, stride_w;
+    int32_t dilation_h, dilation_w;
+} tsx_conv2d_geom;
+
+int tsx_conv2d_out_size(const tsx_conv2d_geom *g, int32_t *out_h, int32_t *out_w);
+
+/* Activation kinds of the fused epilogue. */
+#define TSX_ACT_NONE       0
+#define TSX_ACT_RELU       1  /* cpu::ReLU      src/kernels/cpu/relu.cpp:30-52 */
+#define TSX_ACT_LEAKY_RELU 2  /* cpu::LeakyReLU src/kernels/cpu/leaky_relu.cpp:41-66 */
+
+/* Fused epilogue applied to the int32 accumulators.  It reproduces, rounding for
+ * rounding, the reference's chain of separate operators on the fp32 tensor:
+ *   y = float(acc) * dq[channel]            conv2d_quantized_core.cpp:81-106
+ *   y = y * row_scale[row]    if row_scale  (GEMM only: per-row activation dequant)
+ *   y = y + bias[channel]     if bias       add_bias.cpp:47-85
+ *   y = act(y)                              relu.cpp / leaky_relu.cpp (incl. their SIMD-body /
+ *                                           scalar-tail difference in signed zero and NaN)
+ *   q = quantize(y)           if out_i8     quantize.cpp:70-125 with q_scales[n_qscales]
+ * All pointers are device pointers; unused ones are NULL. */
+typedef struct tsx_epilogue {
+    const float *dq_dev;        /* [channels] dequantize_scales */
+    const float *row_scale_dev; /* [rows] or NULL */
+    const float *bias_dev;      /* [channels] or NULL */
+    int32_t act;                /* TSX_ACT_* */
+    float slope;                /* leaky_relu scale */
+    const float *q_scales_dev;  /* [n_qscales] quantize_scale of the consumer, or NULL */
+    int32_t n_qscales;          /* must equal n (or rows) when q_scales_dev != NULL, as
+                                   base_quantize.cpp:26 requires of the consumer */
+} tsx_epilogue;
+
+/* ---------------------------------------------------------------- quantize
+ * cpu::Quantize::quantize (src/kernels/cpu/quantize.cpp:70-125; declared
+ * include/backend/base/base_quantize.h:24):  q = clamp(round(x * scale_g), -128, 127).
+ * n_scales == 1: first 8*floor(count/8) elements round half to even, the rest half away
+ * from zero; n_scales > 1: scale g covers the next ceil(count/n_scales) elements, all half
+ * away.  NaN / out-of-int32-range products give -128 (x86 conversion semantics). */
+int tsx_quantize_f32_i8(const float *x_dev, int64_t count, const float *scales_dev, int32_t n_scales,
+                        int8_t *out_dev, void *stream);
+
+/* ---------------------------------------------------------------- int8 conv2d
+ * cpu::Conv2DQuantizedCore::conv2d (src/kernels/cpu/quantized/conv2d_quantized_core.cpp:128-147,
+ * interface include/backend/base/base_conv2d_quantized_core.h:14-16): im2col<int8> + int8 GEMM
+ * with int32 accumulation + dequant, done here as one implicit-GEMM on the i8 MFMA units.
+ *
+ * Weights are repacked once (operator init) from OIHW int8 into MFMA operand tiles. */
+size_t tsx_conv2d_i8_packed_weight_bytes(const tsx_conv2d_geom *g);
+int tsx_conv2d_i8_pack_weights(const tsx_conv2d_geom *g, const int8_t *w_oihw_dev, void *packed_dev, void *stream);
+/* Scratch the conv needs (channel-blocked padded copy of the activations). */
+size_t tsx_conv2d_i8_workspace_bytes(const tsx_conv2d_geom *g);
+/* padding_value is the reference's float parameter; it is cast to int8 as the reference
+ * does (conv2d_quantized_core.cpp:72).  Any of out_f32_dev / out_i8_dev / out_acc_dev may be
+ * NULL; out_acc_dev receives the raw int32 accumulators (the reference's INT32 scratch). */
+int tsx_conv2d_i8_nchw(const tsx_conv2d_geom *g, const int8_t *x_dev, const void *packed_w_dev,
+                       float padding_value, const tsx_epilogue *ep, float *out_f32_dev, int8_t *out_i8_dev,
+                       int32_t *out_acc_dev, void *workspace_dev, size_t workspace_bytes, void *stream);
+/* Same, but takes the fp32 activations and the consumer-side quantize parameters, fusing
+ * base::Quantize (a1) into the layout pass that precedes the MFMA kernel. */
+int tsx_quantize_conv2d_i8_nchw(const tsx_conv2d_geom *g, const float *x_f32_dev, const float *x_scales_dev,
+                                int32_t n_x_scales, const void *packed_w_dev, float padding_value,
+                                const tsx_epilogue *ep, float *out_f32_dev, int8_t *out_i8_dev,
+                                int32_t *out_acc_dev, void *workspace_dev, size_t workspace_bytes, void *stream);
+
+/* ---------------------------------------------------------------- int8 GEMM (quantized inner_prod)
+ * cpu::math<int8_t,int32_t>::gemm (src/kernels/cpu/math_cpu.cpp:238-244) followed by the
+ * epilogue above: out[m][n] = ((float(acc)*dq[n]) * row_scale[m]) + bias[n].
+ * a: [m][k] int8 row-major (activations); weights packed from [k][n] row-major (the rhs of
+ * base::InnerProd, include/backend/base/base_inner_prod.h:32-48) or [n][k] when transposed. */
+size_t tsx_gemm_i8_packed_weight_bytes(int32_t k, int32_t n);
+int tsx_gemm_i8_pack_weights(int32_t k, int32_t n, int32_t transposed, const int8_t *w_dev, void *packed_dev,
+                             void *stream);
+size_t tsx_gemm_i8_workspace_bytes(int32_t m, int32_t k);
+int tsx_gemm_i8(int32_t m, int32_t n, int32_t k, const int8_t *a_dev, const void *packed_w_dev,
+                const tsx_epilogue *ep, float *out_f32_dev, int8_t *out_i8_dev, int32_t *out_acc_dev,
+                void *workspace_dev, size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TSX_HIP_H */

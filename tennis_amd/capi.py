@@ -1,0 +1,223 @@
+"""ctypes binding of the C ABI declared in include/tsx_hip.h.
+
+PyTorch is used only for device memory and streams: every function takes CUDA (HIP)
+tensors, hands their raw pointers to libtsx_hip.so and returns tensors.  There is no CPU
+fallback -- if the library is missing or a launch fails this module raises.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libtsx_hip.so")
+
+_vp = ctypes.c_void_p
+_i32 = ctypes.c_int32
+_i64 = ctypes.c_int64
+_f32 = ctypes.c_float
+_sz = ctypes.c_size_t
+
+ACT_NONE, ACT_RELU, ACT_LEAKY_RELU = 0, 1, 2
+_ACT = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "leaky_relu": ACT_LEAKY_RELU}
+
+
+class ConvGeom(ctypes.Structure):
+    """tsx_conv2d_geom."""
+    _fields_ = [(k, _i32) for k in ("n", "c", "h", "w", "cout", "kh", "kw", "pad_top", "pad_bottom", "pad_left",
+                                    "pad_right", "stride_h", "stride_w", "dilation_h", "dilation_w")]
+
+
+class Epilogue(ctypes.Structure):
+    """tsx_epilogue."""
+    _fields_ = [("dq_dev", _vp), ("row_scale_dev", _vp), ("bias_dev", _vp), ("act", _i32), ("slope", _f32),
+                ("q_scales_dev", _vp), ("n_qscales", _i32)]
+
+
+class TsxError(RuntimeError):
+    pass
+
+
+_lib = None
+
+# name -> (restype, argtypes); every symbol include/tsx_hip.h declares.
+SIGNATURES = {
+    "tsx_last_error": (ctypes.c_char_p, []),
+    "tsx_version": (ctypes.c_int, []),
+    "tsx_device_cu_count": (ctypes.c_int, []),
+    "tsx_conv2d_out_size": (ctypes.c_int, [ctypes.POINTER(ConvGeom), ctypes.POINTER(_i32), ctypes.POINTER(_i32)]),
+    "tsx_quantize_f32_i8": (ctypes.c_int, [_vp, _i64, _vp, _i32, _vp, _vp]),
+    "tsx_conv2d_i8_packed_weight_bytes": (_sz, [ctypes.POINTER(ConvGeom)]),
+    "tsx_conv2d_i8_pack_weights": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, _vp]),
+    "tsx_conv2d_i8_workspace_bytes": (_sz, [ctypes.POINTER(ConvGeom)]),
+    "tsx_conv2d_i8_nchw": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, _f32, ctypes.POINTER(Epilogue), _vp, _vp,
+                                          _vp, _vp, _sz, _vp]),
+    "tsx_quantize_conv2d_i8_nchw": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, _i32, _vp, _f32,
+                                                   ctypes.POINTER(Epilogue), _vp, _vp, _vp, _vp, _sz, _vp]),
+    "tsx_gemm_i8_packed_weight_bytes": (_sz, [_i32, _i32]),
+    "tsx_gemm_i8_pack_weights": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, _vp]),
+    "tsx_gemm_i8_workspace_bytes": (_sz, [_i32, _i32]),
+    "tsx_gemm_i8": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, ctypes.POINTER(Epilogue), _vp, _vp, _vp, _vp, _sz, _vp]),
+}
+
+
+def lib():
+    """Load libtsx_hip.so (built in-tree by `python -m tennis_amd.build`); never falls back."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise TsxError("libtsx_hip.so is not built: run `python -m tennis_amd.build` (no CPU fallback exists)")
+        L = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise TsxError("tsx error %d: %s" % (rc, lib().tsx_last_error().decode(errors="replace")))
+
+
+def _ptr(t):
+    return None if t is None else _vp(t.data_ptr())
+
+
+def _stream():
+    return _vp(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev(t, dtype):
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise TsxError("expected a device tensor")
+    return t.to(dtype).contiguous() if (t.dtype != dtype or not t.is_contiguous()) else t
+
+
+def make_geom(x_shape, w_shape, pads=(0, 0, 0, 0), strides=(1, 1), dilations=(1, 1)):
+    n, c, h, w = x_shape
+    cout, cw, kh, kw = w_shape
+    if cw != c:
+        raise TsxError("weight channels %d != input channels %d" % (cw, c))
+    return ConvGeom(n, c, h, w, cout, kh, kw, pads[0], pads[1], pads[2], pads[3], strides[0], strides[1],
+                    dilations[0], dilations[1])
+
+
+def conv_out_size(geom):
+    ho, wo = _i32(), _i32()
+    check(lib().tsx_conv2d_out_size(ctypes.byref(geom), ctypes.byref(ho), ctypes.byref(wo)))
+    return ho.value, wo.value
+
+
+def quantize(x, scales):
+    """tsx_quantize_f32_i8: x fp32 device tensor, scales fp32 device tensor [x.shape[0]] (or [1])."""
+    x = _dev(x, torch.float32)
+    scales = _dev(scales, torch.float32)
+    out = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    check(lib().tsx_quantize_f32_i8(_ptr(x), x.numel(), _ptr(scales), scales.numel(), _ptr(out), _stream()))
+    return out
+
+
+class _EpilogueArgs:
+    """Keeps the device tensors of an epilogue alive next to the C struct."""
+
+    def __init__(self, dq, bias=None, act=None, slope=0.0, q_scales=None, row_scale=None):
+        self.dq = _dev(dq, torch.float32)
+        self.bias = _dev(bias, torch.float32)
+        self.q_scales = _dev(q_scales, torch.float32)
+        self.row_scale = _dev(row_scale, torch.float32)
+        self.c = Epilogue(_ptr(self.dq), _ptr(self.row_scale), _ptr(self.bias), _ACT[act], float(slope),
+                          _ptr(self.q_scales), 0 if self.q_scales is None else self.q_scales.numel())
+
+
+class Conv2dI8:
+    """int8 conv2d with packed weights: the state a `conv2d_quantized` operator instance keeps.
+
+    Mirrors base::Conv2DQuantized (src/backend/base/base_conv2d_quantized.cpp:13-219): the
+    geometry and dequantize scales are fixed at init, weights are packed on first use.
+    """
+
+    def __init__(self, w_i8, pads=(0, 0, 0, 0), strides=(1, 1), dilations=(1, 1), padding_value=0.0):
+        self.w = _dev(w_i8, torch.int8)
+        self.pads, self.strides, self.dilations = tuple(pads), tuple(strides), tuple(dilations)
+        self.padding_value = float(padding_value)
+        self._packed = {}
+        self._workspace = None
+
+    def _plan(self, x_shape):
+        geom = make_geom(x_shape, self.w.shape, self.pads, self.strides, self.dilations)
+        key = (x_shape[1],)
+        if key not in self._packed:
+            nbytes = lib().tsx_conv2d_i8_packed_weight_bytes(ctypes.byref(geom))
+            if nbytes == 0:
+                raise TsxError("bad geometry: " + lib().tsx_last_error().decode())
+            packed = torch.empty(nbytes, dtype=torch.uint8, device=self.w.device)
+            check(lib().tsx_conv2d_i8_pack_weights(ctypes.byref(geom), _ptr(self.w), _ptr(packed), _stream()))
+            self._packed[key] = packed
+        ws_bytes = lib().tsx_conv2d_i8_workspace_bytes(ctypes.byref(geom))
+        if self._workspace is None or self._workspace.numel() < ws_bytes:
+            self._workspace = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=self.w.device)
+        return geom, self._packed[key], ws_bytes
+
+    def __call__(self, x, dq=None, bias=None, act=None, slope=0.0, q_scales=None, x_scales=None,
+                 want_f32=True, want_acc=False):
+        """x: int8 NCHW device tensor, or fp32 NCHW with x_scales (fused quantize).
+
+        Returns (out_f32 or None, out_i8 or None, acc_i32 or None)."""
+        fused_quant = x_scales is not None
+        x = _dev(x, torch.float32 if fused_quant else torch.int8)
+        geom, packed, ws_bytes = self._plan(tuple(x.shape))
+        ho, wo = conv_out_size(geom)
+        shape = (x.shape[0], self.w.shape[0], ho, wo)
+        ep = _EpilogueArgs(dq, bias, act, slope, q_scales) if dq is not None else None
+        out_f32 = torch.empty(shape, dtype=torch.float32, device=x.device) if (want_f32 and ep) else None
+        out_i8 = torch.empty(shape, dtype=torch.int8, device=x.device) if (ep and q_scales is not None) else None
+        acc = torch.empty(shape, dtype=torch.int32, device=x.device) if want_acc else None
+        epp = ctypes.byref(ep.c) if ep else None
+        if fused_quant:
+            xs = _dev(x_scales, torch.float32)
+            check(lib().tsx_quantize_conv2d_i8_nchw(ctypes.byref(geom), _ptr(x), _ptr(xs), xs.numel(), _ptr(packed),
+                                                    self.padding_value, epp, _ptr(out_f32), _ptr(out_i8), _ptr(acc),
+                                                    _ptr(self._workspace), ws_bytes, _stream()))
+        else:
+            check(lib().tsx_conv2d_i8_nchw(ctypes.byref(geom), _ptr(x), _ptr(packed), self.padding_value, epp,
+                                           _ptr(out_f32), _ptr(out_i8), _ptr(acc), _ptr(self._workspace), ws_bytes,
+                                           _stream()))
+        return out_f32, out_i8, acc
+
+
+class GemmI8:
+    """int8 GEMM (quantized inner_prod) with packed weights; rhs is [k][n], or [n][k] if transpose."""
+
+    def __init__(self, w_i8, transpose=False):
+        self.w = _dev(w_i8, torch.int8)
+        self.transpose = bool(transpose)
+        self.n, self.k = (self.w.shape if self.transpose else self.w.shape[::-1])
+        nbytes = lib().tsx_gemm_i8_packed_weight_bytes(self.k, self.n)
+        self.packed = torch.empty(nbytes, dtype=torch.uint8, device=self.w.device)
+        check(lib().tsx_gemm_i8_pack_weights(self.k, self.n, int(self.transpose), _ptr(self.w), _ptr(self.packed),
+                                             _stream()))
+        self._workspace = None
+
+    def __call__(self, a, dq=None, row_scale=None, bias=None, act=None, slope=0.0, q_scales=None, want_f32=True,
+                 want_acc=False):
+        a = _dev(a, torch.int8)
+        m, k = a.shape
+        if k != self.k:
+            raise TsxError("lhs has %d columns, weights %d rows" % (k, self.k))
+        ws_bytes = lib().tsx_gemm_i8_workspace_bytes(m, k)
+        if a.data_ptr() % 16:
+            ws_bytes = m * ((k + 63) // 64 * 64)
+        if self._workspace is None or self._workspace.numel() < ws_bytes:
+            self._workspace = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=a.device)
+        ep = _EpilogueArgs(dq, bias, act, slope, q_scales, row_scale) if dq is not None else None
+        shape = (m, self.n)
+        out_f32 = torch.empty(shape, dtype=torch.float32, device=a.device) if (want_f32 and ep) else None
+        out_i8 = torch.empty(shape, dtype=torch.int8, device=a.device) if (ep and q_scales is not None) else None
+        acc = torch.empty(shape, dtype=torch.int32, device=a.device) if want_acc else None
+        check(lib().tsx_gemm_i8(m, self.n, k, _ptr(a), _ptr(self.packed), ctypes.byref(ep.c) if ep else None,
+                                _ptr(out_f32), _ptr(out_i8), _ptr(acc), _ptr(self._workspace), ws_bytes, _stream()))
+        return out_f32, out_i8, acc

@@ -1,0 +1,519 @@
+// int8 conv2d / GEMM on the gfx950 i8 MFMA units: implicit-im2col GEMM with int32
+// accumulation and a fused dequant + bias + activation (+ requantize) epilogue.
+//
+// Stands in for cpu::Conv2DQuantizedCore::conv2d
+// (src/kernels/cpu/quantized/conv2d_quantized_core.cpp:18-147): per-image im2col<int8>
+// (src/kernels/cpu/im2col.cpp:37-111) + math<int8,int32>::gemm (math_cpu.cpp:143-244) +
+// float(acc)*dq[c].  Integer accumulation is exact, so the contraction order is free:
+//
+//   * activations are first *staged* into a channel-blocked, spatially padded copy
+//     xs[n][hs][ws][cp] (cp = channels rounded up to 64, halo = int8(padding_value)); a
+//     (tap, 64-channel block) K-step of any output position is then 64 contiguous bytes;
+//   * weights are packed once into MFMA operand order, K ordered (kh, kw, c-block) to match;
+//   * one workgroup computes a BM(cout) x BN(positions) tile, positions flattened over
+//     (n, ho, wo); operands go HBM/L2 -> registers -> LDS (double buffered) -> MFMA
+//     v_mfma_i32_32x32x32_i8.  Which operand is "rows" is a template switch so the
+//     accumulator lanes run along the contiguous output dimension (positions for NCHW
+//     conv output, features for row-major GEMM output).
+//
+// MFMA operand layout used (v_mfma_i32_32x32x32_i8, 64 lanes): lane l supplies row/column
+// (l % 32) and 16 consecutive K bytes of K-group (l / 32); A and B use the same K mapping,
+// so any consistent K permutation gives the same exact integer result.  Accumulator register
+// r of lane l holds row 8*(r/4) + 4*(l/32) + (r%4), column l % 32.
+#include "tsx_common.hpp"
+
+#include <cmath>
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int KSTEP = 64;  // bytes of K per pipeline step (two MFMAs of K=32)
+
+// ------------------------------------------------------------------ staging kernels
+
+struct StageGeom {
+    int n, c, h, w;        // source NCHW
+    int hs, ws, cp;        // staged extent
+    int pad_top, pad_left;
+    int pad_value;         // int8 halo value
+};
+
+// One lane produces one 16-byte channel chunk of one staged pixel.  Adjacent lanes take
+// adjacent ws, so each of the 16 byte loads is coalesced along W of the NCHW source.
+// QUANT: the source is fp32 and is quantized on the fly with the semantics of
+// cpu::Quantize (quantize.cpp:70-125) evaluated at the element's NCHW linear index.
+template <bool QUANT>
+__global__ __launch_bounds__(256) void stage_nchw_kernel(const void *__restrict__ src, StageGeom g,
+                                                        const float *__restrict__ scales, int n_scales,
+                                                        int64_t group_len, int64_t bulk8,
+                                                        int8_t *__restrict__ xs) {
+    const int chunks = g.cp / 16;
+    const int64_t total = int64_t(g.n) * g.hs * chunks * g.ws;
+    const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id >= total) return;
+    const int wsi = int(id % g.ws);
+    int64_t rest = id / g.ws;
+    const int chunk = int(rest % chunks);
+    rest /= chunks;
+    const int hsi = int(rest % g.hs);
+    const int ni = int(rest / g.hs);
+    const int hi = hsi - g.pad_top, wi = wsi - g.pad_left;
+    const bool inside = hi >= 0 && hi < g.h && wi >= 0 && wi < g.w;
+    uint32_t words[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int ci = chunk * 16 + v * 4 + j;
+            int q = 0;  // channel padding: weights there are zero as well
+            if (ci < g.c) {
+                q = g.pad_value;
+                if (inside) {
+                    const int64_t idx = ((int64_t(ni) * g.c + ci) * g.h + hi) * g.w + wi;
+                    if (QUANT) {
+                        const float s = n_scales == 1 ? scales[0] : scales[idx / group_len];
+                        q = tsx::quantize_value(__fmul_rn(static_cast<const float *>(src)[idx], s),
+                                                n_scales == 1 && idx < bulk8);
+                    } else {
+                        q = static_cast<const int8_t *>(src)[idx];
+                    }
+                }
+            }
+            word |= uint32_t(q & 0xff) << (8 * j);
+        }
+        words[v] = word;
+    }
+    const int64_t o = ((int64_t(ni) * g.hs + hsi) * g.ws + wsi) * g.cp + chunk * 16;
+    *reinterpret_cast<uint4 *>(xs + o) = make_uint4(words[0], words[1], words[2], words[3]);
+}
+
+// ------------------------------------------------------------------ weight packing
+
+// packed[ks][frag][half][lane][16]: ks = tap * cblocks + cb (tap = kh*KW + kw),
+// frag = cout / 32, and lane l of (frag, half) holds, for cout = frag*32 + l%32, the 16
+// channels cb*64 + half*32 + (l/32)*16 + 0..15 of that tap.  Rows >= cout and channels >= c
+// are zero.  w is OIHW ([cout][c][kh][kw]); for GEMM weights kh = kw = 1 and the element
+// (k, n) sits at w[k * ldk + n * ldn].
+__global__ __launch_bounds__(256) void pack_weights_kernel(const int8_t *__restrict__ w, int cout, int c, int taps,
+                                                          int64_t ld_cout, int64_t ld_c, int64_t ld_tap,
+                                                          int coutp, int cblocks, int8_t *__restrict__ packed) {
+    const int frags = coutp / 32;
+    const int64_t total = int64_t(taps) * cblocks * frags * 2 * 64;
+    const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id >= total) return;
+    const int lane = int(id % 64);
+    int64_t rest = id / 64;
+    const int half = int(rest % 2);
+    rest /= 2;
+    const int frag = int(rest % frags);
+    const int ks = int(rest / frags);
+    const int tap = ks / cblocks, cb = ks % cblocks;
+    const int co = frag * 32 + lane % 32;
+    const int c0 = cb * 64 + half * 32 + (lane / 32) * 16;
+    uint32_t words[4] = {0, 0, 0, 0};
+    if (co < cout) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int ci = c0 + j;
+            const int v = ci < c ? w[co * ld_cout + ci * ld_c + tap * ld_tap] : 0;
+            words[j / 4] |= uint32_t(v & 0xff) << (8 * (j % 4));
+        }
+    }
+    *reinterpret_cast<uint4 *>(packed + id * 16) = make_uint4(words[0], words[1], words[2], words[3]);
+}
+
+// ------------------------------------------------------------------ implicit GEMM
+
+struct GemmParams {
+    const int8_t *xs;      // staged activations
+    const int8_t *wp;      // packed weights
+    int positions;         // N*Ho*Wo (GEMM: rows)
+    int howo, wo;          // Ho*Wo, Wo
+    int hs, ws, cp;        // staged extent
+    int stride_h, stride_w, dil_h, dil_w, kw;
+    int taps, cblocks;
+    int cout, coutp;
+    // epilogue
+    const float *dq, *row_scale, *bias, *q_scales;
+    int act;
+    float slope;
+    int n_qscales;
+    int64_t q_group_len, q_bulk8, act_body;
+    float *out_f32;
+    int8_t *out_i8;
+    int32_t *out_acc;
+};
+
+__device__ __forceinline__ void emit(const GemmParams &p, int acc, int co, int pos) {
+    if (co >= p.cout || pos >= p.positions) return;
+    const int n = pos / p.howo;
+    const int hw = pos - n * p.howo;
+    const int64_t idx = (int64_t(n) * p.cout + co) * p.howo + hw;
+    if (p.out_acc) p.out_acc[idx] = acc;
+    if (!p.out_f32 && !p.out_i8) return;
+    float v = __fmul_rn(float(acc), p.dq[co]);
+    if (p.row_scale) v = __fmul_rn(v, p.row_scale[n]);
+    if (p.bias) v = __fadd_rn(v, p.bias[co]);
+    v = tsx::apply_act(v, p.act, p.slope, idx < p.act_body);
+    if (p.out_f32) p.out_f32[idx] = v;
+    if (p.out_i8) {
+        const float s = p.n_qscales == 1 ? p.q_scales[0] : p.q_scales[idx / p.q_group_len];
+        p.out_i8[idx] = int8_t(tsx::quantize_value(__fmul_rn(v, s), p.n_qscales == 1 && idx < p.q_bulk8));
+    }
+}
+
+// BM x BN tile, WGM x WGN wavefronts.  SWAP=false: MFMA rows = cout, columns = positions
+// (lanes along positions: NCHW conv output).  SWAP=true: rows = positions, columns = cout
+// (lanes along cout: row-major GEMM output, howo == 1).
+template <int BM, int BN, int WGM, int WGN, bool SWAP>
+__global__ __launch_bounds__(WGM *WGN * 64) void igemm_i8_kernel(GemmParams p) {
+    constexpr int THREADS = WGM * WGN * 64;
+    constexpr int FM = BM / WGM / 32, FN = BN / WGN / 32;
+    constexpr int A_BYTES = BM * KSTEP, B_BYTES = BN * KSTEP;
+    constexpr int A_LOADS = A_BYTES / 16 / THREADS, B_LOADS = B_BYTES / 16 / THREADS;
+    static_assert(A_LOADS >= 1 && B_LOADS >= 1, "tile too small for the workgroup");
+    static_assert(A_BYTES % (16 * THREADS) == 0 && B_BYTES % (16 * THREADS) == 0, "tile/threads mismatch");
+
+    __shared__ __attribute__((aligned(16))) int8_t lds[2][A_BYTES + B_BYTES];
+
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+
+    // Per-thread source offsets of the B (activation) chunks this thread copies.
+    int64_t b_src[B_LOADS];
+    int b_dst[B_LOADS];
+#pragma unroll
+    for (int i = 0; i < B_LOADS; ++i) {
+        const int q = tid + i * THREADS;
+        const int row = q / 4, chunk = q % 4;
+        int pos = n0 + row;
+        if (pos >= p.positions) pos = 0;  // clamp: computed but never stored
+        const int n = pos / p.howo;
+        const int r = pos - n * p.howo;
+        const int ho = r / p.wo, wo = r - ho * p.wo;
+        b_src[i] = ((int64_t(n) * p.hs + ho * p.stride_h) * p.ws + wo * p.stride_w) * p.cp + chunk * 16;
+        b_dst[i] = A_BYTES + row * 64 + ((chunk ^ ((row >> 1) & 3)) * 16);
+    }
+    const int8_t *a_src = p.wp + (int64_t(m0 / 32) * 2 * 64 + tid) * 16;
+    const int64_t a_kstride = int64_t(p.coutp / 32) * 2 * 64 * 16;
+
+    v16i acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+    const int ksteps = p.taps * p.cblocks;
+    uint4 a_reg[A_LOADS], b_reg[B_LOADS];
+
+    auto load_global = [&](int ks) {
+        const int tap = ks / p.cblocks, cb = ks - tap * p.cblocks;
+        const int kr = tap / p.kw, kc = tap - kr * p.kw;
+        const int64_t tap_off = (int64_t(kr) * p.dil_h * p.ws + kc * p.dil_w) * p.cp + cb * 64;
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i)
+            a_reg[i] = *reinterpret_cast<const uint4 *>(a_src + ks * a_kstride + int64_t(i) * THREADS * 16);
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i) b_reg[i] = *reinterpret_cast<const uint4 *>(p.xs + b_src[i] + tap_off);
+    };
+    auto store_lds = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) *reinterpret_cast<uint4 *>(&lds[buf][(tid + i * THREADS) * 16]) = a_reg[i];
+#pragma unroll
+        for (int i = 0; i < B_LOADS; ++i) *reinterpret_cast<uint4 *>(&lds[buf][b_dst[i]]) = b_reg[i];
+    };
+
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+
+    for (int ks = 0; ks < ksteps; ++ks) {
+        const int buf = ks & 1;
+        if (ks + 1 < ksteps) load_global(ks + 1);
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            v4i a[FM], b[FN];
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+                a[i] = *reinterpret_cast<const v4i *>(&lds[buf][(((wm * FM + i) * 2 + half) * 64 + lane) * 16]);
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+                const int row = (wn * FN + j) * 32 + lane % 32;
+                const int chunk = half * 2 + lane / 32;
+                b[j] = *reinterpret_cast<const v4i *>(&lds[buf][A_BYTES + row * 64 + ((chunk ^ ((row >> 1) & 3)) * 16)]);
+            }
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(b[j], a[i], acc[i][j], 0, 0, 0)
+                                     : __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+        if (ks + 1 < ksteps) store_lds(buf ^ 1);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int rr = 8 * (r / 4) + 4 * (lane / 32) + (r % 4), cc = lane % 32;
+                const int co = m0 + (wm * FM + i) * 32 + (SWAP ? cc : rr);
+                const int pos = n0 + (wn * FN + j) * 32 + (SWAP ? rr : cc);
+                emit(p, acc[i][j][r], co, pos);
+            }
+}
+
+// ------------------------------------------------------------------ host side
+
+constexpr int BM = 128, BN = 128;
+
+struct Plan {
+    int ho, wo, hs, ws, cp, cblocks, taps, coutp;
+    int64_t positions;
+    size_t staged_bytes, packed_bytes;
+};
+
+int make_plan(const tsx_conv2d_geom *g, Plan *pl) {
+    TSX_REQUIRE(g, "null geometry");
+    TSX_REQUIRE(g->n > 0 && g->c > 0 && g->h > 0 && g->w > 0 && g->cout > 0 && g->kh > 0 && g->kw > 0,
+                "conv2d_i8: non-positive extent");
+    TSX_REQUIRE(g->stride_h > 0 && g->stride_w > 0 && g->dilation_h > 0 && g->dilation_w > 0,
+                "conv2d_i8: stride and dilation must be positive");
+    TSX_REQUIRE(g->pad_top >= 0 && g->pad_bottom >= 0 && g->pad_left >= 0 && g->pad_right >= 0,
+                "conv2d_i8: negative padding is not supported");
+    pl->ho = tsx::conv_out(g->h, g->pad_top, g->pad_bottom, g->kh, g->stride_h, g->dilation_h);
+    pl->wo = tsx::conv_out(g->w, g->pad_left, g->pad_right, g->kw, g->stride_w, g->dilation_w);
+    TSX_REQUIRE(pl->ho > 0 && pl->wo > 0, "conv2d_i8: empty output %dx%d", pl->ho, pl->wo);
+    // Rows/columns the kernel actually reads: up to (ho-1)*stride + (k-1)*dilation.
+    pl->hs = (pl->ho - 1) * g->stride_h + (g->kh - 1) * g->dilation_h + 1;
+    pl->ws = (pl->wo - 1) * g->stride_w + (g->kw - 1) * g->dilation_w + 1;
+    pl->cp = int(tsx::round_up(g->c, KSTEP));
+    pl->cblocks = pl->cp / KSTEP;
+    pl->taps = g->kh * g->kw;
+    pl->coutp = int(tsx::round_up(g->cout, BM));
+    pl->positions = int64_t(g->n) * pl->ho * pl->wo;
+    TSX_REQUIRE(pl->positions < (int64_t(1) << 31), "conv2d_i8: too many output positions");
+    pl->staged_bytes = size_t(g->n) * pl->hs * pl->ws * pl->cp;
+    pl->packed_bytes = size_t(pl->taps) * pl->cblocks * pl->coutp * KSTEP;
+    return 0;
+}
+
+int check_epilogue(const tsx_epilogue *ep, const float *out_f32, const int8_t *out_i8, const int32_t *out_acc,
+                   int64_t groups) {
+    TSX_REQUIRE(out_f32 || out_i8 || out_acc, "no output requested");
+    if (out_f32 || out_i8) {
+        TSX_REQUIRE(ep && ep->dq_dev, "epilogue with dequantize scales required for fp32/int8 output");
+        TSX_REQUIRE(ep->act >= TSX_ACT_NONE && ep->act <= TSX_ACT_LEAKY_RELU, "unknown activation %d", ep->act);
+    }
+    if (out_i8) {
+        TSX_REQUIRE(ep->q_scales_dev, "int8 output needs q_scales_dev");
+        // base_quantize.cpp:26: the consumer's scale count equals its input's first extent
+        TSX_REQUIRE(ep->n_qscales == groups, "n_qscales (%d) must equal the output's first extent (%lld)",
+                    ep->n_qscales, (long long)groups);
+    }
+    return 0;
+}
+
+void fill_epilogue(GemmParams &p, const tsx_epilogue *ep, int64_t count, float *out_f32, int8_t *out_i8,
+                   int32_t *out_acc) {
+    p.dq = ep ? ep->dq_dev : nullptr;
+    p.row_scale = ep ? ep->row_scale_dev : nullptr;
+    p.bias = ep ? ep->bias_dev : nullptr;
+    p.q_scales = ep ? ep->q_scales_dev : nullptr;
+    p.act = ep ? ep->act : 0;
+    p.slope = ep ? ep->slope : 0.f;
+    p.n_qscales = ep ? ep->n_qscales : 0;
+    p.q_group_len = p.n_qscales > 0 ? int64_t(std::ceil(static_cast<float>(count) / static_cast<float>(p.n_qscales))) : 1;
+    p.q_bulk8 = (count >> 3) << 3;
+    p.act_body = count / 4 * 4;
+    p.out_f32 = out_f32;
+    p.out_i8 = out_i8;
+    p.out_acc = out_acc;
+}
+
+template <bool SWAP>
+int launch_igemm(const GemmParams &p, hipStream_t stream) {
+    dim3 grid(unsigned(tsx::ceil_div(p.positions, BN)), unsigned(p.coutp / BM));
+    hipLaunchKernelGGL((igemm_i8_kernel<BM, BN, 2, 2, SWAP>), grid, dim3(256), 0, stream, p);
+    TSX_LAUNCH_CHECK("igemm_i8_kernel");
+    return 0;
+}
+
+int run_conv(const tsx_conv2d_geom *g, const void *x, bool x_is_f32, const float *x_scales, int n_x_scales,
+             const void *packed_w, float padding_value, const tsx_epilogue *ep, float *out_f32, int8_t *out_i8,
+             int32_t *out_acc, void *workspace, size_t workspace_bytes, void *stream_) {
+    Plan pl;
+    int rc = make_plan(g, &pl);
+    if (rc) return rc;
+    rc = check_epilogue(ep, out_f32, out_i8, out_acc, g->n);
+    if (rc) return rc;
+    TSX_REQUIRE(x && packed_w, "conv2d_i8: null input");
+    TSX_REQUIRE(!(ep && ep->row_scale_dev), "conv2d_i8: row_scale is a GEMM-only epilogue term");
+    if (!workspace || workspace_bytes < pl.staged_bytes)
+        return tsx::fail(TSX_E_WORKSPACE, "conv2d_i8: workspace %zu < %zu bytes", workspace_bytes, pl.staged_bytes);
+    TSX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0 && reinterpret_cast<uintptr_t>(packed_w) % 16 == 0,
+                "conv2d_i8: workspace and packed weights must be 16-byte aligned");
+    hipStream_t stream = tsx::as_stream(stream_);
+
+    StageGeom sg{g->n, g->c, g->h, g->w, pl.hs, pl.ws, pl.cp, g->pad_top, g->pad_left,
+                 int(int8_t(padding_value))};  // T(padding_value), conv2d_quantized_core.cpp:72
+    const int64_t stage_threads = int64_t(g->n) * pl.hs * pl.ws * (pl.cp / 16);
+    const unsigned stage_blocks = unsigned(tsx::ceil_div(stage_threads, 256));
+    if (x_is_f32) {
+        TSX_REQUIRE(x_scales && n_x_scales >= 1, "quantize_conv2d_i8: missing quantize scales");
+        // base_quantize.cpp:26
+        TSX_REQUIRE(n_x_scales == g->n, "quantize_conv2d_i8: n_x_scales (%d) must equal the batch (%d)", n_x_scales, g->n);
+        const int64_t count = int64_t(g->n) * g->c * g->h * g->w;
+        const int64_t group_len = int64_t(std::ceil(static_cast<float>(count) / static_cast<float>(n_x_scales)));
+        hipLaunchKernelGGL(stage_nchw_kernel<true>, dim3(stage_blocks), dim3(256), 0, stream, x, sg, x_scales,
+                           n_x_scales, group_len, (count >> 3) << 3, static_cast<int8_t *>(workspace));
+    } else {
+        hipLaunchKernelGGL(stage_nchw_kernel<false>, dim3(stage_blocks), dim3(256), 0, stream, x, sg,
+                           static_cast<const float *>(nullptr), 1, int64_t(1), int64_t(0),
+                           static_cast<int8_t *>(workspace));
+    }
+    TSX_LAUNCH_CHECK("stage_nchw_kernel");
+
+    GemmParams p{};
+    p.xs = static_cast<const int8_t *>(workspace);
+    p.wp = static_cast<const int8_t *>(packed_w);
+    p.positions = int(pl.positions);
+    p.howo = pl.ho * pl.wo;
+    p.wo = pl.wo;
+    p.hs = pl.hs;
+    p.ws = pl.ws;
+    p.cp = pl.cp;
+    p.stride_h = g->stride_h;
+    p.stride_w = g->stride_w;
+    p.dil_h = g->dilation_h;
+    p.dil_w = g->dilation_w;
+    p.kw = g->kw;
+    p.taps = pl.taps;
+    p.cblocks = pl.cblocks;
+    p.cout = g->cout;
+    p.coutp = pl.coutp;
+    fill_epilogue(p, ep, int64_t(g->n) * g->cout * pl.ho * pl.wo, out_f32, out_i8, out_acc);
+    return launch_igemm<false>(p, stream);
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t tsx_conv2d_i8_packed_weight_bytes(const tsx_conv2d_geom *g) {
+    Plan pl;
+    return make_plan(g, &pl) ? 0 : pl.packed_bytes;
+}
+
+size_t tsx_conv2d_i8_workspace_bytes(const tsx_conv2d_geom *g) {
+    Plan pl;
+    return make_plan(g, &pl) ? 0 : pl.staged_bytes;
+}
+
+int tsx_conv2d_i8_pack_weights(const tsx_conv2d_geom *g, const int8_t *w_oihw_dev, void *packed_dev, void *stream) {
+    Plan pl;
+    int rc = make_plan(g, &pl);
+    if (rc) return rc;
+    TSX_REQUIRE(w_oihw_dev && packed_dev, "pack_weights: null pointer");
+    TSX_REQUIRE(reinterpret_cast<uintptr_t>(packed_dev) % 16 == 0, "pack_weights: packed buffer must be 16-byte aligned");
+    const int64_t threads = int64_t(pl.packed_bytes / 16);
+    hipLaunchKernelGGL(pack_weights_kernel, dim3(unsigned(tsx::ceil_div(threads, 256))), dim3(256), 0,
+                       tsx::as_stream(stream), w_oihw_dev, g->cout, g->c, pl.taps, int64_t(g->c) * pl.taps,
+                       int64_t(pl.taps), int64_t(1), pl.coutp, pl.cblocks, static_cast<int8_t *>(packed_dev));
+    TSX_LAUNCH_CHECK("pack_weights_kernel");
+    return 0;
+}
+
+int tsx_conv2d_i8_nchw(const tsx_conv2d_geom *g, const int8_t *x_dev, const void *packed_w_dev, float padding_value,
+                       const tsx_epilogue *ep, float *out_f32_dev, int8_t *out_i8_dev, int32_t *out_acc_dev,
+                       void *workspace_dev, size_t workspace_bytes, void *stream) {
+    return run_conv(g, x_dev, false, nullptr, 0, packed_w_dev, padding_value, ep, out_f32_dev, out_i8_dev, out_acc_dev,
+                    workspace_dev, workspace_bytes, stream);
+}
+
+int tsx_quantize_conv2d_i8_nchw(const tsx_conv2d_geom *g, const float *x_f32_dev, const float *x_scales_dev,
+                                int32_t n_x_scales, const void *packed_w_dev, float padding_value,
+                                const tsx_epilogue *ep, float *out_f32_dev, int8_t *out_i8_dev, int32_t *out_acc_dev,
+                                void *workspace_dev, size_t workspace_bytes, void *stream) {
+    return run_conv(g, x_f32_dev, true, x_scales_dev, n_x_scales, packed_w_dev, padding_value, ep, out_f32_dev,
+                    out_i8_dev, out_acc_dev, workspace_dev, workspace_bytes, stream);
+}
+
+// ---- GEMM: a [m][k] is a batch of m "images" with k channels and 1x1 extent.
+
+size_t tsx_gemm_i8_packed_weight_bytes(int32_t k, int32_t n) {
+    if (k <= 0 || n <= 0) return 0;
+    return size_t(tsx::round_up(k, KSTEP)) * size_t(tsx::round_up(n, BM));
+}
+
+int tsx_gemm_i8_pack_weights(int32_t k, int32_t n, int32_t transposed, const int8_t *w_dev, void *packed_dev,
+                             void *stream) {
+    TSX_REQUIRE(k > 0 && n > 0 && w_dev && packed_dev, "gemm_i8_pack_weights: bad argument");
+    TSX_REQUIRE(reinterpret_cast<uintptr_t>(packed_dev) % 16 == 0, "gemm_i8_pack_weights: packed buffer must be 16-byte aligned");
+    const int cblocks = int(tsx::round_up(k, KSTEP) / KSTEP), coutp = int(tsx::round_up(n, BM));
+    const int64_t threads = int64_t(cblocks) * coutp * KSTEP / 16;
+    // element (k, n): [k][n] row-major -> k*n_ + n ; transposed [n][k] -> n*k_ + k
+    const int64_t ld_cout = transposed ? k : 1, ld_c = transposed ? 1 : n;
+    hipLaunchKernelGGL(pack_weights_kernel, dim3(unsigned(tsx::ceil_div(threads, 256))), dim3(256), 0,
+                       tsx::as_stream(stream), w_dev, n, k, 1, ld_cout, ld_c, int64_t(0), coutp, cblocks,
+                       static_cast<int8_t *>(packed_dev));
+    TSX_LAUNCH_CHECK("pack_weights_kernel");
+    return 0;
+}
+
+size_t tsx_gemm_i8_workspace_bytes(int32_t m, int32_t k) {
+    if (m <= 0 || k <= 0) return 0;
+    return k % KSTEP == 0 ? 0 : size_t(m) * size_t(tsx::round_up(k, KSTEP));
+}
+
+int tsx_gemm_i8(int32_t m, int32_t n, int32_t k, const int8_t *a_dev, const void *packed_w_dev,
+                const tsx_epilogue *ep, float *out_f32_dev, int8_t *out_i8_dev, int32_t *out_acc_dev,
+                void *workspace_dev, size_t workspace_bytes, void *stream_) {
+    TSX_REQUIRE(m > 0 && n > 0 && k > 0, "gemm_i8: non-positive extent");
+    TSX_REQUIRE(a_dev && packed_w_dev, "gemm_i8: null input");
+    int rc = check_epilogue(ep, out_f32_dev, out_i8_dev, out_acc_dev, m);
+    if (rc) return rc;
+    hipStream_t stream = tsx::as_stream(stream_);
+    const int kp = int(tsx::round_up(k, KSTEP));
+    const int8_t *xs = a_dev;
+    if (kp != k || reinterpret_cast<uintptr_t>(a_dev) % 16 != 0) {
+        const size_t need = size_t(m) * kp;
+        if (!workspace_dev || workspace_bytes < need)
+            return tsx::fail(TSX_E_WORKSPACE, "gemm_i8: workspace %zu < %zu bytes", workspace_bytes, need);
+        TSX_REQUIRE(reinterpret_cast<uintptr_t>(workspace_dev) % 16 == 0, "gemm_i8: workspace must be 16-byte aligned");
+        StageGeom sg{m, k, 1, 1, 1, 1, kp, 0, 0, 0};
+        const int64_t threads = int64_t(m) * (kp / 16);
+        hipLaunchKernelGGL(stage_nchw_kernel<false>, dim3(unsigned(tsx::ceil_div(threads, 256))), dim3(256), 0, stream,
+                           static_cast<const void *>(a_dev), sg, static_cast<const float *>(nullptr), 1, int64_t(1),
+                           int64_t(0), static_cast<int8_t *>(workspace_dev));
+        TSX_LAUNCH_CHECK("stage_nchw_kernel");
+        xs = static_cast<const int8_t *>(workspace_dev);
+    }
+    GemmParams p{};
+    p.xs = xs;
+    p.wp = static_cast<const int8_t *>(packed_w_dev);
+    p.positions = m;
+    p.howo = 1;
+    p.wo = 1;
+    p.hs = 1;
+    p.ws = 1;
+    p.cp = kp;
+    p.stride_h = p.stride_w = p.dil_h = p.dil_w = p.kw = 1;
+    p.taps = 1;
+    p.cblocks = kp / KSTEP;
+    p.cout = n;
+    p.coutp = int(tsx::round_up(n, BM));
+    fill_epilogue(p, ep, int64_t(m) * n, out_f32_dev, out_i8_dev, out_acc_dev);
+    return launch_igemm<true>(p, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,85 @@
+// Shared host/device helpers of the gfx950 kernels behind include/tsx_hip.h.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "tsx_hip.h"
+
+namespace tsx {
+
+// Thread-local message behind tsx_last_error().
+char *error_buffer();
+int fail(int code, const char *fmt, ...);
+
+inline int check_hip(hipError_t e, const char *what) {
+    if (e == hipSuccess) return 0;
+    return fail(int(e), "%s: %s", what, hipGetErrorString(e));
+}
+
+#define TSX_HIP(expr)                                        \
+    do {                                                     \
+        int _rc = ::tsx::check_hip((expr), #expr);           \
+        if (_rc) return _rc;                                 \
+    } while (0)
+
+#define TSX_REQUIRE(cond, ...)                               \
+    do {                                                     \
+        if (!(cond)) return ::tsx::fail(TSX_E_INVALID, __VA_ARGS__); \
+    } while (0)
+
+// Launch check: the reference checks the runtime right after every launch and ejects
+// (include/kernels/gpu/gpu_kernel.h:13-19); here the error code goes back over the C ABI.
+#define TSX_LAUNCH_CHECK(name) TSX_HIP(hipGetLastError())
+
+inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline int64_t round_up(int64_t a, int64_t b) { return ceil_div(a, b) * b; }
+
+// Output extent of a convolution (include/backend/common_function.h:30-40).
+inline int conv_out(int in, int pad_a, int pad_b, int k, int stride, int dilation) {
+    return (in + pad_a + pad_b - (dilation * (k - 1) + 1)) / stride + 1;
+}
+
+// ---------------------------------------------------------------------------
+// Device-side scalar semantics shared by the quantize kernel and fused epilogues.
+// ---------------------------------------------------------------------------
+#ifdef __HIPCC__
+
+// q = clamp(round(v), -128, 127) with the reference's x86 conversion behaviour:
+// NaN and |v| >= 2^31 convert to INT_MIN, i.e. -128 after the clamp
+// (src/kernels/cpu/quantize.cpp:15-29,83-96).
+__device__ __forceinline__ int quantize_value(float v, bool half_even) {
+    if (!(__builtin_fabsf(v) < 2147483648.0f)) return -128;
+    // rintf = round half to even (_mm256_cvtps_epi32); roundf = half away from zero (round()).
+    const float r = half_even ? __builtin_rintf(v) : __builtin_roundf(v);
+    int q = int(r);
+    q = q > 127 ? 127 : q;
+    q = q < -128 ? -128 : q;
+    return q;
+}
+
+// relu / leaky_relu of element `in_body` (= linear index < 4*floor(count/4) of the whole
+// tensor): SIMD body vs scalar tail of src/kernels/cpu/relu.cpp:30-52 and
+// leaky_relu.cpp:41-66.  Body: max(x,0) returns +0 for -0 and NaN; the leaky form is one
+// fused multiply-add in the reference's FMA build.  Tail: std::max / ternary.
+__device__ __forceinline__ float apply_act(float v, int act, float slope, bool in_body) {
+    if (act == TSX_ACT_RELU) {
+        return in_body ? (v > 0.f ? v : 0.f) : (v < 0.f ? 0.f : v);
+    }
+    if (act == TSX_ACT_LEAKY_RELU) {
+        if (in_body) {
+            const float mx = v > 0.f ? v : 0.f;
+            const float mn = v < 0.f ? v : 0.f;
+            return __builtin_fmaf(slope, mn, mx);
+        }
+        return v > 0.f ? v : __fmul_rn(v, slope);
+    }
+    return v;
+}
+
+#endif  // __HIPCC__
+
+}  // namespace tsx

@@ -1,0 +1,227 @@
+"""GPU parity of the int8 path through the C ABI (libtsx_hip.so) against the CPU oracle.
+
+Bar: bit-exact -- int32 accumulators, int8 (re)quantized values and the fp32 bit patterns of
+the dequant + bias + activation epilogue.
+"""
+import numpy as np
+import pytest
+
+from _util import bits, c2_like
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tsx():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from tennis_amd import capi
+    capi.lib()
+    return capi
+
+
+def _dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+# ---------------------------------------------------------------- quantize
+
+@pytest.mark.parametrize("shape,ns", [((1, 11), 1), ((2, 11), 2), ((1, 3, 7, 9), 1), ((5, 3, 7, 9), 5),
+                                      ((32, 77), 32), ((1, 4096), 1), ((7, 1000), 7), ((3, 64, 28, 28), 3)])
+def test_quantize(tsx, port, shape, ns):
+    rng = np.random.default_rng(100)
+    x = (rng.standard_normal(shape) * 50).astype(np.float32)
+    x.ravel()[::3] = np.round(x.ravel()[::3]) + 0.5          # exact ties
+    x.ravel()[:8] = [np.inf, -np.inf, np.nan, 3e9, -3e9, 127.5, -128.5, 1e20][:min(8, x.size)]
+    s = np.ones(ns, np.float32) if ns <= 2 else rng.uniform(0.25, 2, ns).astype(np.float32)
+    got = tsx.quantize(_dev(x), _dev(s)).cpu().numpy()
+    assert np.array_equal(got, port.quantize(x, s))
+
+
+def test_quantize_known_answers(tsx):
+    kat = np.array([.5, 1.5, 2.5, -.5, -1.5, 3.5, 4.5, 5.5, .5, 1.5, 2.5], np.float32)
+    one = tsx.quantize(_dev(kat.reshape(1, 11)), _dev(np.ones(1, np.float32))).cpu().numpy()
+    assert one.ravel().tolist() == [0, 2, 2, 0, -2, 4, 4, 6, 1, 2, 3]
+    two = tsx.quantize(_dev(np.stack([kat, kat])), _dev(np.ones(2, np.float32))).cpu().numpy()
+    assert two.tolist() == [[1, 2, 3, -1, -2, 4, 5, 6, 1, 2, 3]] * 2
+
+
+def test_quantize_unaligned_view(tsx, port):
+    import torch
+    rng = np.random.default_rng(101)
+    x = (rng.standard_normal(1003) * 30).astype(np.float32)
+    base = _dev(np.concatenate([[0.0], x]).astype(np.float32))
+    view = base[1:].view(1, 1003)                          # 4-byte aligned only
+    got = tsx.quantize(view, _dev(np.array([1.5], np.float32))).cpu().numpy()
+    assert np.array_equal(got, port.quantize(x.reshape(1, 1003), [1.5]))
+
+
+# ---------------------------------------------------------------- conv2d int8
+
+CONV_CASES = [
+    # n, c, h, w, cout, kh, kw, pads(t,b,l,r), strides, dilations
+    (2, 8, 6, 6, 4, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),
+    (1, 3, 9, 7, 5, 3, 3, (0, 0, 0, 0), (2, 2), (1, 1)),
+    (2, 16, 5, 5, 8, 1, 1, (0, 0, 0, 0), (1, 1), (1, 1)),
+    (1, 4, 8, 8, 3, 1, 1, (0, 0, 0, 0), (2, 2), (1, 1)),
+    (1, 5, 10, 9, 6, 3, 2, (2, 1, 0, 1), (1, 2), (2, 1)),
+    (3, 2, 7, 7, 7, 7, 7, (3, 3, 3, 3), (2, 2), (1, 1)),
+    (2, 64, 14, 14, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),
+    (1, 130, 9, 9, 200, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),     # ragged channels / cout > one tile
+    (5, 96, 7, 7, 129, 1, 1, (0, 0, 0, 0), (1, 1), (1, 1)),
+    (2, 256, 28, 28, 256, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),   # two images of BASELINE config 2
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv2d_i8_accumulators_and_dequant(tsx, port, case):
+    n, c, h, w, cout, kh, kw, pads, st, dl = case
+    rng = np.random.default_rng(200)
+    x = rng.integers(-128, 128, (n, c, h, w)).astype(np.int8)
+    wt = rng.integers(-128, 128, (cout, c, kh, kw)).astype(np.int8)
+    dq = rng.uniform(1e-4, 1e-2, cout).astype(np.float32)
+    conv = tsx.Conv2dI8(_dev(wt), pads, st, dl)
+    out, _, acc = conv(_dev(x), dq=_dev(dq), want_acc=True)
+    exp, exp_acc = port.conv2d_quantized(x, wt, dq, pads, st, dl, return_acc=True)
+    assert np.array_equal(acc.cpu().numpy(), exp_acc)
+    assert np.array_equal(bits(out.cpu().numpy()), bits(exp))
+
+
+def test_conv2d_i8_padding_value(tsx, port):
+    rng = np.random.default_rng(201)
+    x = rng.integers(-128, 128, (2, 5, 6, 7)).astype(np.int8)
+    wt = rng.integers(-128, 128, (9, 5, 3, 3)).astype(np.int8)
+    dq = np.ones(9, np.float32)
+    conv = tsx.Conv2dI8(_dev(wt), (1, 2, 2, 1), (1, 1), (1, 1), padding_value=-3.9)
+    _, _, acc = conv(_dev(x), dq=_dev(dq), want_acc=True)
+    _, exp = port.conv2d_quantized(x, wt, dq, (1, 2, 2, 1), padding_value=-3.9, return_acc=True)
+    assert np.array_equal(acc.cpu().numpy(), exp)
+
+
+def test_conv2d_i8_extreme_operands(tsx, port):
+    # -128 * -128 over K = 2304: the largest accumulator magnitude the layer can produce
+    x = np.full((1, 256, 3, 3), -128, np.int8)
+    wt = np.full((2, 256, 3, 3), -128, np.int8)
+    wt[1] = 127
+    dq = np.array([1.0, 0.5], np.float32)
+    conv = tsx.Conv2dI8(_dev(wt))
+    out, _, acc = conv(_dev(x), dq=_dev(dq), want_acc=True)
+    exp, exp_acc = port.conv2d_quantized(x, wt, dq, return_acc=True)
+    assert acc.cpu().numpy().ravel().tolist() == [128 * 128 * 2304, -128 * 127 * 2304]
+    assert np.array_equal(acc.cpu().numpy(), exp_acc)
+    assert np.array_equal(bits(out.cpu().numpy()), bits(exp))
+
+
+@pytest.mark.parametrize("act", [None, "relu", "leaky_relu"])
+@pytest.mark.parametrize("n", [1, 3])
+def test_conv2d_i8_fused_epilogue(tsx, port, act, n):
+    rng = np.random.default_rng(202)
+    x, x_scales, wq, dq, bias = c2_like(rng, n, 24, 9, 11, 40)
+    xq = port.quantize(x, x_scales)
+    qs = np.full(n, 9.0, np.float32)
+    bias[3] = -0.0
+    conv = tsx.Conv2dI8(_dev(wq), (1, 1, 1, 1))
+    out, q, _ = conv(_dev(xq), dq=_dev(dq), bias=_dev(bias), act=act, slope=0.1, q_scales=_dev(qs))
+    exp, exp_q = port.conv2d_i8_fused(xq, wq, dq, bias, act, 0.1, qs, pads=(1, 1, 1, 1))
+    assert np.array_equal(bits(out.cpu().numpy()), bits(exp))
+    assert np.array_equal(q.cpu().numpy(), exp_q)
+
+
+def test_conv2d_i8_epilogue_signed_zero_and_tail(tsx, port):
+    # all-zero accumulators with a negative dequant scale give -0.0; bias -0.0 keeps it; the
+    # reference's relu turns it into +0.0 in its SIMD body but not in its scalar tail.
+    x = np.zeros((1, 8, 3, 3), np.int8)
+    wt = np.ones((3, 8, 1, 1), np.int8)
+    dq = np.array([-1.0, 1.0, -2.0], np.float32)
+    bias = np.array([-0.0, -0.0, -0.0], np.float32)
+    conv = tsx.Conv2dI8(_dev(wt))
+    for act in ("relu", "leaky_relu"):
+        out, _, _ = conv(_dev(x), dq=_dev(dq), bias=_dev(bias), act=act, slope=0.1)
+        exp, _ = port.conv2d_i8_fused(x, wt, dq, bias, act, 0.1)
+        assert np.array_equal(bits(out.cpu().numpy()), bits(exp)), act
+    assert np.signbit(exp.ravel()[-1])        # 27 elements: the last three are the scalar tail
+
+
+def test_quantize_conv2d_fused_input(tsx, port):
+    rng = np.random.default_rng(203)
+    for n in (1, 4):
+        x, x_scales, wq, dq, bias = c2_like(rng, n, 70, 10, 9, 33)
+        x.ravel()[::5] = (np.round(x.ravel()[::5] * x_scales[0]) + 0.5) / x_scales[0]   # near-ties
+        conv = tsx.Conv2dI8(_dev(wq), (1, 1, 1, 1))
+        out, _, acc = conv(_dev(x), dq=_dev(dq), bias=_dev(bias), act="relu", x_scales=_dev(x_scales), want_acc=True)
+        xq = port.quantize(x, x_scales)
+        exp, _ = port.conv2d_i8_fused(xq, wq, dq, bias, "relu", pads=(1, 1, 1, 1))
+        assert np.array_equal(bits(out.cpu().numpy()), bits(exp))
+
+
+def test_conv2d_i8_baseline_config2_full(tsx, port):
+    """BASELINE config 2 at full size: 32x256x28x28, 256x256x3x3, s1 p1, dequant + bias + ReLU."""
+    rng = np.random.default_rng(1234)
+    x, x_scales, wq, dq, bias = c2_like(rng, 32, 256, 28, 28, 256)
+    conv = tsx.Conv2dI8(_dev(wq), (1, 1, 1, 1))
+    xq_dev = tsx.quantize(_dev(x), _dev(x_scales))
+    xq = port.quantize(x, x_scales)
+    assert np.array_equal(xq_dev.cpu().numpy(), xq)
+    out, _, acc = conv(xq_dev, dq=_dev(dq), bias=_dev(bias), act="relu", want_acc=True)
+    exp_acc = port.conv2d_quantized(xq, wq, dq, (1, 1, 1, 1), return_acc=True)[1]
+    assert np.array_equal(acc.cpu().numpy(), exp_acc)
+    exp, _ = port.epilogue(exp_acc, dq, bias, "relu")
+    assert np.array_equal(bits(out.cpu().numpy()), bits(exp))
+    # size-independent property: the convolution is linear in x, exactly, in integers
+    _, _, acc2 = conv(_dev((xq // 2).astype(np.int8)), want_acc=True)
+    _, _, acc3 = conv(_dev((xq - xq // 2).astype(np.int8)), want_acc=True)
+    assert np.array_equal((acc2 + acc3).cpu().numpy(), exp_acc)
+
+
+def test_conv2d_i8_rejects_bad_arguments(tsx):
+    import torch
+    wt = torch.zeros((4, 8, 3, 3), dtype=torch.int8, device="cuda")
+    conv = tsx.Conv2dI8(wt)
+    with pytest.raises(tsx.TsxError):
+        conv(torch.zeros((1, 8, 2, 2), dtype=torch.int8, device="cuda"), want_acc=True)   # empty output
+    with pytest.raises(tsx.TsxError):
+        conv(torch.zeros((1, 7, 5, 5), dtype=torch.int8, device="cuda"), want_acc=True)   # channel mismatch
+    with pytest.raises(tsx.TsxError):   # consumer scales must match the batch (base_quantize.cpp:26)
+        conv(torch.zeros((2, 8, 5, 5), dtype=torch.int8, device="cuda"), dq=torch.ones(4, device="cuda"),
+             q_scales=torch.ones(3, device="cuda"))
+
+
+# ---------------------------------------------------------------- int8 GEMM
+
+@pytest.mark.parametrize("m,k,n", [(1, 64, 32), (3, 70, 33), (32, 1024, 1024), (256, 1024, 1024), (130, 200, 260),
+                                   (1, 2048, 2048)])
+@pytest.mark.parametrize("transpose", [False, True])
+def test_gemm_i8(tsx, port, m, k, n, transpose):
+    rng = np.random.default_rng(300)
+    a = rng.integers(-128, 128, (m, k)).astype(np.int8)
+    b = rng.integers(-128, 128, (k, n)).astype(np.int8)
+    dqw = rng.uniform(1e-3, 1e-2, n).astype(np.float32)
+    dqa = rng.uniform(1e-3, 1e-2, m).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    g = tsx.GemmI8(_dev(b.T.copy() if transpose else b), transpose=transpose)
+    out, _, acc = g(_dev(a), dq=_dev(dqw), row_scale=_dev(dqa), bias=_dev(bias), want_acc=True)
+    exp, exp_acc = port.gemm_i8_dequant(a, b, dqw, dqa, bias, return_acc=True)
+    assert np.array_equal(acc.cpu().numpy(), exp_acc)
+    assert np.array_equal(bits(out.cpu().numpy()), bits(exp))
+
+
+def test_gemm_i8_largest_sweep_shape_by_rows(tsx, port):
+    """M=4096, K=N=4096 (largest shape of the GEMM sweep): rows are independent, so a random
+    subset of rows is checked against the oracle, all columns."""
+    rng = np.random.default_rng(301)
+    m = k = n = 4096
+    a = rng.integers(-128, 128, (m, k)).astype(np.int8)
+    b = rng.integers(-128, 128, (k, n)).astype(np.int8)
+    dqw = rng.uniform(1e-3, 1e-2, n).astype(np.float32)
+    dqa = rng.uniform(1e-3, 1e-2, m).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    g = tsx.GemmI8(_dev(b))
+    out, _, acc = g(_dev(a), dq=_dev(dqw), row_scale=_dev(dqa), bias=_dev(bias), want_acc=True)
+    rows = np.sort(rng.choice(m, 48, replace=False))
+    exp, exp_acc = port.gemm_i8_dequant(a[rows], b, dqw, dqa[rows], bias, return_acc=True)
+    assert np.array_equal(acc.cpu().numpy()[rows], exp_acc)
+    assert np.array_equal(bits(out.cpu().numpy()[rows]), bits(exp))
+    # checksum of checksums over the whole product: column sums of acc = (sum of rows of a) . b
+    colsum = acc.cpu().numpy().astype(np.int64).sum(axis=0)
+    assert np.array_equal(colsum, a.astype(np.int64).sum(axis=0) @ b.astype(np.int64))
