@@ -1,0 +1,194 @@
+#!/usr/bin/env python3
+"""Benchmark of the int8 conv2d hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Workload = BASELINE config 2: x fp32 32x256x28x28 ~ N(0,1) quantized per tensor
+(127/max|x|, one equal scale per image), weights 256x256x3x3 ~ N(0,0.05) int8 per output
+channel, stride 1, pad 1, int32 accumulation, fp32 dequant + bias + ReLU output.
+One "step" = one pass of the path over the batch: quantize+stage kernel, then the i8-MFMA
+implicit-GEMM kernel with the fused epilogue, inputs resident in HBM.
+
+Prints ONE JSON line.  `value` is the whole step's throughput in TOPS (2*MAC / step time);
+`roofline` is the MFMA kernel alone (HIP events around back-to-back launches) against the
+int8 dense MFMA peak; `cpu_baseline` times the same layer on the host cores with the
+compiled TenniS reference (kind "reference") or, where that is absent, the CPU oracle
+(kind "port").
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, 5.0 POP/s
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, 8 TB/s
+
+CFG = dict(n=32, c=256, h=28, w=28, cout=256, k=3, pad=1)
+
+
+def make_inputs(cfg, seed=1234):
+    rng = np.random.default_rng(seed)
+    n, c, h, w, cout, k = cfg["n"], cfg["c"], cfg["h"], cfg["w"], cfg["cout"], cfg["k"]
+    x = rng.standard_normal((n, c, h, w)).astype(np.float32)
+    wt = (rng.standard_normal((cout, c, k, k)) * 0.05).astype(np.float32)
+    bias = (rng.standard_normal(cout) * 0.1).astype(np.float32)
+    s_x = np.float32(127.0) / np.abs(x).max().astype(np.float32)
+    x_scales = np.full(n, s_x, np.float32)
+    wmax = np.abs(wt.reshape(cout, -1)).max(axis=1).astype(np.float32)
+    s_w = (np.float32(127.0) / wmax).astype(np.float32)
+    q = wt * s_w[:, None, None, None]
+    wq = np.clip(np.sign(q) * np.floor(np.abs(q) + 0.5), -127, 127).astype(np.int8)
+    dq = (np.float32(1.0) / (s_x * s_w)).astype(np.float32)
+    return x, x_scales, wq, dq, bias
+
+
+def cpu_baseline(x, x_scales, wq, dq, bias, pad, images):
+    """The reference's own operator chain on the host: quantize -> conv2d_quantized -> add_bias -> relu."""
+    xs = np.ascontiguousarray(x[:images])
+    sc = x_scales[:images]
+    pads = (pad, pad, pad, pad)
+    macs = images * wq.shape[0] * x.shape[2] * x.shape[3] * wq.shape[1] * wq.shape[2] * wq.shape[3]
+    try:
+        from oracle import ref
+        have_ref = ref.available()
+    except Exception:
+        have_ref = False
+    if have_ref:
+        t0 = time.perf_counter()
+        xq = ref.quantize(xs, sc, threads=1)
+        y = ref.conv2d_quantized(xq, wq, dq, pads=pads, threads=1)
+        y = ref.add_bias(y, bias, threads=1)
+        y = ref.relu(y, threads=1)
+        dt = time.perf_counter() - t0
+        kind, cores = "reference", 1
+        note = ("compiled TenniS CPU library (OpenMP+AVX2/FMA build), computing_thread_number=1: its int8 GEMM is "
+                "single-threaded scalar and its dequant loop is only correct at one thread")
+    else:
+        from oracle import port
+        port.set_threads(1)
+        t0 = time.perf_counter()
+        xq = port.quantize(xs, sc)
+        port.conv2d_i8_fused(xq, wq, dq, bias, "relu", pads=pads)
+        dt = time.perf_counter() - t0
+        kind, cores = "port", 1
+        note = "CPU oracle restatement, 1 thread"
+    return {"value": 2.0 * macs / dt / 1e12, "unit": "TOPS", "cores": cores, "kind": kind,
+            "sample": "%d of %d images of the same layer, %.2f s; %s" % (images, x.shape[0], dt, note),
+            "host_cpus": os.cpu_count()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--cpu-images", type=int, default=32, help="images of the batch timed on the CPU (0 = skip)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from tennis_amd import capi
+    import ctypes
+
+    if not torch.cuda.is_available():
+        print("bench.py needs the MI355X (no CPU fallback)", file=sys.stderr)
+        sys.exit(3)
+    L = capi.lib()
+    dev = torch.device("cuda:0")
+    cfg = CFG
+    x, x_scales, wq, dq, bias = make_inputs(cfg)
+    pad = cfg["pad"]
+
+    xd = torch.from_numpy(x).to(dev)
+    xsd = torch.from_numpy(x_scales).to(dev)
+    conv = capi.Conv2dI8(torch.from_numpy(wq).to(dev), (pad,) * 4)
+    ep = capi._EpilogueArgs(torch.from_numpy(dq).to(dev), torch.from_numpy(bias).to(dev), "relu")
+    geom, packed, ws_bytes = conv._plan(tuple(xd.shape))
+    ho, wo = capi.conv_out_size(geom)
+    out = torch.empty((cfg["n"], cfg["cout"], ho, wo), dtype=torch.float32, device=dev)
+    ws = conv._workspace
+    stream = capi._stream()
+    g = ctypes.byref(geom)
+    epp = ctypes.byref(ep.c)
+
+    def step():
+        capi.check(L.tsx_quantize_conv2d_i8_nchw(g, capi._ptr(xd), capi._ptr(xsd), xsd.numel(), capi._ptr(packed), 0.0,
+                                                 epp, capi._ptr(out), None, None, capi._ptr(ws), ws_bytes, stream))
+
+    def stage_only():
+        capi.check(L.tsx_conv2d_i8_stage(g, capi._ptr(xd), 1, capi._ptr(xsd), xsd.numel(), 0.0, capi._ptr(ws), ws_bytes,
+                                         stream))
+
+    def mfma_only():
+        capi.check(L.tsx_conv2d_i8_staged(g, capi._ptr(ws), capi._ptr(packed), epp, capi._ptr(out), None, None, stream))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+
+    def event_time(fn, reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        fn()
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps * 1e-3   # seconds per launch
+
+    reps = max(args.steps, 50)
+    t_mfma = event_time(mfma_only, reps)
+    t_stage = event_time(stage_only, reps)
+
+    macs = cfg["n"] * cfg["cout"] * ho * wo * cfg["c"] * cfg["k"] * cfg["k"]
+    ops = 2.0 * macs
+    tops = ops / (ms_per_step * 1e-3) / 1e12
+    kernel_tops = ops / t_mfma / 1e12
+    stage_bytes = 4.0 * x.size + float(ws_bytes)
+
+    result = {
+        "metric": "int8 conv2d TOPS & % MFMA peak; ResNet-50-shape img/s at bs=32, 1 MI355X",
+        "value": tops,
+        "unit": "TOPS",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8 x int8 -> int32 (fp32 epilogue)",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE config 2: int8 conv2d 32x256x28x28 * 256x256x3x3 s1 p1, fp32 dequant+bias+ReLU "
+                               "out; step = quantize+stage kernel + i8-MFMA implicit-GEMM kernel",
+                   "algorithmic_ops_per_step": ops, "pct_of_int8_mfma_peak_whole_step": 100.0 * tops / PEAK_INT8_TOPS},
+        "roofline": {"bound": "mfma", "kernel": "igemm_i8_kernel", "achieved": kernel_tops, "peak": PEAK_INT8_TOPS,
+                     "unit": "TFLOP/s", "frac": kernel_tops / PEAK_INT8_TOPS, "traffic": None,
+                     "note": "int8 multiply-accumulate ops (TOP/s); 2*N*Cout*Ho*Wo*Cin*9 = %.4g ops per launch, "
+                             "avg launch %.2f us over %d back-to-back launches" % (ops, t_mfma * 1e6, reps)},
+        "stage_kernel": {"bound": "hbm", "kernel": "stage_nchw_kernel<quantize>", "achieved": stage_bytes / t_stage / 1e9,
+                         "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": stage_bytes / t_stage / 1e9 / PEAK_HBM_GBS,
+                         "us": t_stage * 1e6, "bytes": stage_bytes},
+    }
+    if args.cpu_images > 0:
+        result["cpu_baseline"] = cpu_baseline(x, x_scales, wq, dq, bias, pad, min(args.cpu_images, cfg["n"]))
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

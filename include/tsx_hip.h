@@ -106,6 +106,17 @@ int tsx_quantize_conv2d_i8_nchw(const tsx_conv2d_geom *g, const float *x_f32_dev
                                 const tsx_epilogue *ep, float *out_f32_dev, int8_t *out_i8_dev,
                                 int32_t *out_acc_dev, void *workspace_dev, size_t workspace_bytes, void *stream);
 
+/* The two halves of the calls above, for callers that keep the staged activations around
+ * (several convolutions reading one tensor, or timing the MFMA kernel by itself):
+ *   stage  : NCHW int8 (x_is_f32 == 0) or NCHW fp32 + quantize (x_is_f32 != 0) -> channel-blocked
+ *            padded copy [n][hs][ws][round_up(c,64)], tsx_conv2d_i8_workspace_bytes() bytes;
+ *   staged : the implicit GEMM + epilogue on that copy. */
+int tsx_conv2d_i8_stage(const tsx_conv2d_geom *g, const void *x_dev, int32_t x_is_f32, const float *x_scales_dev,
+                        int32_t n_x_scales, float padding_value, void *staged_dev, size_t staged_bytes, void *stream);
+int tsx_conv2d_i8_staged(const tsx_conv2d_geom *g, const void *staged_dev, const void *packed_w_dev,
+                         const tsx_epilogue *ep, float *out_f32_dev, int8_t *out_i8_dev, int32_t *out_acc_dev,
+                         void *stream);
+
 /* ---------------------------------------------------------------- int8 GEMM (quantized inner_prod)
  * cpu::math<int8_t,int32_t>::gemm (src/kernels/cpu/math_cpu.cpp:238-244) followed by the
  * epilogue above: out[m][n] = ((float(acc)*dq[n]) * row_scale[m]) + bias[n].

@@ -24,7 +24,24 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
+    "-Rpass-analysis=kernel-resource-usage",
 ]
+
+
+def scratch_users(compiler_output):
+    """Kernels whose registers went to scratch memory, from hipcc's resource-usage remarks.
+
+    A private array that is demoted to scratch turns every use into a memory round trip, which
+    costs the MFMA kernels several-fold; the build refuses such an object file."""
+    bad, name = [], None
+    for line in compiler_output.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:")[1].split("[")[0].strip()
+        elif "ScratchSize [bytes/lane]:" in line:
+            size = int(line.split("ScratchSize [bytes/lane]:")[1].split("[")[0].strip())
+            if size and name:
+                bad.append((name, size))
+    return bad
 
 
 def sources():
@@ -49,8 +66,23 @@ def build(verbose=True, jobs=8):
     failed = False
     for src, p in procs:
         out, _ = p.communicate()
+        for name, size in scratch_users(out):
+            print("FAILED: kernel %s uses %d bytes/lane of scratch" % (name, size), file=sys.stderr)
+            failed = True
         # the host pass does not know the device-only feature flag; that note is harmless
-        out = "\n".join(l for l in out.splitlines() if "packed-fp32-ops" not in l)
+        keep, skip = [], 0
+        for l in out.splitlines():
+            if "packed-fp32-ops" in l:
+                continue
+            if "remark:" in l:
+                skip = 2      # the remark's source excerpt and caret line follow it
+                continue
+            if skip and (" | " in l or l.strip().startswith("|")):
+                skip -= 1
+                continue
+            skip = 0
+            keep.append(l)
+        out = "\n".join(keep)
         if out.strip() and verbose:
             print(out)
         if p.returncode != 0:

@@ -10,7 +10,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libtsx_hip.so")
+# TSX_HIP_LIBRARY overrides the in-tree library (e.g. a build kept elsewhere by the integrator).
+LIB_PATH = os.environ.get("TSX_HIP_LIBRARY") or os.path.join(_HERE, "lib", "libtsx_hip.so")
 
 _vp = ctypes.c_void_p
 _i32 = ctypes.c_int32
@@ -54,6 +55,9 @@ SIGNATURES = {
                                           _vp, _vp, _sz, _vp]),
     "tsx_quantize_conv2d_i8_nchw": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, _i32, _vp, _f32,
                                                    ctypes.POINTER(Epilogue), _vp, _vp, _vp, _vp, _sz, _vp]),
+    "tsx_conv2d_i8_stage": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _i32, _vp, _i32, _f32, _vp, _sz, _vp]),
+    "tsx_conv2d_i8_staged": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, ctypes.POINTER(Epilogue), _vp, _vp,
+                                            _vp, _vp]),
     "tsx_gemm_i8_packed_weight_bytes": (_sz, [_i32, _i32]),
     "tsx_gemm_i8_pack_weights": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, _vp]),
     "tsx_gemm_i8_workspace_bytes": (_sz, [_i32, _i32]),

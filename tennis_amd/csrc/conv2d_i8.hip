@@ -20,14 +20,14 @@
 // (l % 32) and 16 consecutive K bytes of K-group (l / 32); A and B use the same K mapping,
 // so any consistent K permutation gives the same exact integer result.  Accumulator register
 // r of lane l holds row 8*(r/4) + 4*(l/32) + (r%4), column l % 32.
-#include "tsx_common.hpp"
+#include "igemm_i8.hpp"
 
 #include <cmath>
 
 namespace {
 
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
+using tsx::v4i;
+using tsx::v16i;
 
 constexpr int KSTEP = 64;  // bytes of K per pipeline step (two MFMAs of K=32)
 
@@ -127,7 +127,7 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(const int8_t *__restr
 
 // ------------------------------------------------------------------ implicit GEMM
 
-struct GemmParams {
+struct GemmParams : tsx::EpiParams {
     const int8_t *xs;      // staged activations
     const int8_t *wp;      // packed weights
     int positions;         // N*Ho*Wo (GEMM: rows)
@@ -136,34 +136,9 @@ struct GemmParams {
     int stride_h, stride_w, dil_h, dil_w, kw;
     int taps, cblocks;
     int cout, coutp;
-    // epilogue
-    const float *dq, *row_scale, *bias, *q_scales;
-    int act;
-    float slope;
-    int n_qscales;
-    int64_t q_group_len, q_bulk8, act_body;
-    float *out_f32;
-    int8_t *out_i8;
-    int32_t *out_acc;
 };
 
-__device__ __forceinline__ void emit(const GemmParams &p, int acc, int co, int pos) {
-    if (co >= p.cout || pos >= p.positions) return;
-    const int n = pos / p.howo;
-    const int hw = pos - n * p.howo;
-    const int64_t idx = (int64_t(n) * p.cout + co) * p.howo + hw;
-    if (p.out_acc) p.out_acc[idx] = acc;
-    if (!p.out_f32 && !p.out_i8) return;
-    float v = __fmul_rn(float(acc), p.dq[co]);
-    if (p.row_scale) v = __fmul_rn(v, p.row_scale[n]);
-    if (p.bias) v = __fadd_rn(v, p.bias[co]);
-    v = tsx::apply_act(v, p.act, p.slope, idx < p.act_body);
-    if (p.out_f32) p.out_f32[idx] = v;
-    if (p.out_i8) {
-        const float s = p.n_qscales == 1 ? p.q_scales[0] : p.q_scales[idx / p.q_group_len];
-        p.out_i8[idx] = int8_t(tsx::quantize_value(__fmul_rn(v, s), p.n_qscales == 1 && idx < p.q_bulk8));
-    }
-}
+using tsx::emit;
 
 // BM x BN tile, WGM x WGN wavefronts.  SWAP=false: MFMA rows = cout, columns = positions
 // (lanes along positions: NCHW conv output).  SWAP=true: rows = positions, columns = cout
@@ -183,8 +158,8 @@ __global__ __launch_bounds__(WGM *WGN * 64) void igemm_i8_kernel(GemmParams p) {
     const int wm = wave / WGN, wn = wave % WGN;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
 
-    // Per-thread source offsets of the B (activation) chunks this thread copies.
-    int64_t b_src[B_LOADS];
+    // Source pointers of the 16-byte chunks this thread copies per K-step.
+    const int8_t *b_src[B_LOADS];
     int b_dst[B_LOADS];
 #pragma unroll
     for (int i = 0; i < B_LOADS; ++i) {
@@ -195,11 +170,25 @@ __global__ __launch_bounds__(WGM *WGN * 64) void igemm_i8_kernel(GemmParams p) {
         const int n = pos / p.howo;
         const int r = pos - n * p.howo;
         const int ho = r / p.wo, wo = r - ho * p.wo;
-        b_src[i] = ((int64_t(n) * p.hs + ho * p.stride_h) * p.ws + wo * p.stride_w) * p.cp + chunk * 16;
+        b_src[i] = p.xs + ((int64_t(n) * p.hs + ho * p.stride_h) * p.ws + wo * p.stride_w) * p.cp + chunk * 16;
         b_dst[i] = A_BYTES + row * 64 + ((chunk ^ ((row >> 1) & 3)) * 16);
     }
     const int8_t *a_src = p.wp + (int64_t(m0 / 32) * 2 * 64 + tid) * 16;
     const int64_t a_kstride = int64_t(p.coutp / 32) * 2 * 64 * 16;
+
+    // LDS read offsets of this lane's MFMA operands (per half: + 1024 for A, chunk swizzle for B)
+    int a_off[FM], b_off[FN][2];
+#pragma unroll
+    for (int i = 0; i < FM; ++i) a_off[i] = ((wm * FM + i) * 2 * 64 + lane) * 16;
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+        const int row = (wn * FN + j) * 32 + lane % 32;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int chunk = half * 2 + lane / 32;
+            b_off[j][half] = A_BYTES + row * 64 + ((chunk ^ ((row >> 1) & 3)) * 16);
+        }
+    }
 
     v16i acc[FM][FN];
 #pragma unroll
@@ -210,66 +199,116 @@ __global__ __launch_bounds__(WGM *WGN * 64) void igemm_i8_kernel(GemmParams p) {
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
     const int ksteps = p.taps * p.cblocks;
-    uint4 a_reg[A_LOADS], b_reg[B_LOADS];
+    v4i a_reg[A_LOADS], b_reg[B_LOADS];   // native vectors: arrays of HIP's uint4 struct can end up in scratch
 
-    auto load_global = [&](int ks) {
-        const int tap = ks / p.cblocks, cb = ks - tap * p.cblocks;
-        const int kr = tap / p.kw, kc = tap - kr * p.kw;
-        const int64_t tap_off = (int64_t(kr) * p.dil_h * p.ws + kc * p.dil_w) * p.cp + cb * 64;
-#pragma unroll
-        for (int i = 0; i < A_LOADS; ++i)
-            a_reg[i] = *reinterpret_cast<const uint4 *>(a_src + ks * a_kstride + int64_t(i) * THREADS * 16);
-#pragma unroll
-        for (int i = 0; i < B_LOADS; ++i) b_reg[i] = *reinterpret_cast<const uint4 *>(p.xs + b_src[i] + tap_off);
-    };
-    auto store_lds = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) *reinterpret_cast<uint4 *>(&lds[buf][(tid + i * THREADS) * 16]) = a_reg[i];
-#pragma unroll
-        for (int i = 0; i < B_LOADS; ++i) *reinterpret_cast<uint4 *>(&lds[buf][b_dst[i]]) = b_reg[i];
-    };
-
-    load_global(0);
-    store_lds(0);
-    __syncthreads();
-
-    for (int ks = 0; ks < ksteps; ++ks) {
-        const int buf = ks & 1;
-        if (ks + 1 < ksteps) load_global(ks + 1);
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            v4i a[FM], b[FN];
-#pragma unroll
-            for (int i = 0; i < FM; ++i)
-                a[i] = *reinterpret_cast<const v4i *>(&lds[buf][(((wm * FM + i) * 2 + half) * 64 + lane) * 16]);
-#pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                const int row = (wn * FN + j) * 32 + lane % 32;
-                const int chunk = half * 2 + lane / 32;
-                b[j] = *reinterpret_cast<const v4i *>(&lds[buf][A_BYTES + row * 64 + ((chunk ^ ((row >> 1) & 3)) * 16)]);
-            }
-#pragma unroll
-            for (int i = 0; i < FM; ++i)
-#pragma unroll
-                for (int j = 0; j < FN; ++j)
-                    acc[i][j] = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(b[j], a[i], acc[i][j], 0, 0, 0)
-                                     : __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], acc[i][j], 0, 0, 0);
-        }
-        if (ks + 1 < ksteps) store_lds(buf ^ 1);
-        __syncthreads();
+    // K-step ks = tap * cblocks + cb; (tap, cb) advance incrementally.
+    int tap = 0, cb = 0;
+    int64_t tap_off = 0;
+#define TSX_LOAD_GLOBAL()                                                                                       \
+    {                                                                                                           \
+        _Pragma("unroll") for (int i = 0; i < A_LOADS; ++i) a_reg[i] =  \
+            *reinterpret_cast<const v4i *>(a_src + int64_t(i) * THREADS * 16);                               \
+        _Pragma("unroll") for (int i = 0; i < B_LOADS; ++i) b_reg[i] =  \
+            *reinterpret_cast<const v4i *>(b_src[i] + tap_off);                                                \
+    }
+#define TSX_ADVANCE()                                                                                           \
+    {                                                                                                           \
+        a_src += a_kstride;                                                                                     \
+        if (++cb == p.cblocks) {                                                                                \
+            cb = 0;                                                                                             \
+            ++tap;                                                                                              \
+            const int kr = tap / p.kw, kc = tap - kr * p.kw;                                                    \
+            tap_off = (int64_t(kr) * p.dil_h * p.ws + kc * p.dil_w) * p.cp;                                     \
+        } else {                                                                                                \
+            tap_off += 64;                                                                                      \
+        }                                                                                                       \
+    }
+#define TSX_STORE_LDS(buf)                                                                                      \
+    {                                                                                                           \
+        _Pragma("unroll") for (int i = 0; i < A_LOADS; ++i)                                                     \
+            *reinterpret_cast<v4i *>(&lds[buf][(tid + i * THREADS) * 16]) = a_reg[i];                           \
+        _Pragma("unroll") for (int i = 0; i < B_LOADS; ++i)                                                     \
+            *reinterpret_cast<v4i *>(&lds[buf][b_dst[i]]) = b_reg[i];                                           \
+    }
+#define TSX_COMPUTE(buf)                                                                                        \
+    {                                                                                                           \
+        _Pragma("unroll") for (int half = 0; half < 2; ++half) {                                               \
+            v4i a[FM], b[FN];                                                                                   \
+            _Pragma("unroll") for (int i = 0; i < FM; ++i) a[i] =                                             \
+                *reinterpret_cast<const v4i *>(&lds[buf][a_off[i] + half * 1024]);                              \
+            _Pragma("unroll") for (int j = 0; j < FN; ++j) b[j] =                                             \
+                *reinterpret_cast<const v4i *>(&lds[buf][b_off[j][half]]);                                      \
+            _Pragma("unroll") for (int i = 0; i < FM; ++i) _Pragma("unroll") for (int j = 0; j < FN; ++j)     \
+                acc[i][j] = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(b[j], a[i], acc[i][j], 0, 0, 0)        \
+                                 : __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], acc[i][j], 0, 0, 0);       \
+        }                                                                                                       \
     }
 
+    TSX_LOAD_GLOBAL();
+    TSX_STORE_LDS(0);
+    __syncthreads();
+    int buf = 0;
+    for (int ks = 0; ks + 1 < ksteps; ++ks) {
+        TSX_ADVANCE();
+        TSX_LOAD_GLOBAL();      // K-step ks+1 -> registers, in flight during the MFMAs below
+        TSX_COMPUTE(buf);
+        TSX_STORE_LDS(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+    TSX_COMPUTE(buf);
+#undef TSX_LOAD_GLOBAL
+#undef TSX_ADVANCE
+#undef TSX_STORE_LDS
+#undef TSX_COMPUTE
+
+    // Accumulator register r of lane l: row 8*(r/4) + 4*(l/32) + r%4, column l%32.
+    if (!SWAP) {
+        // columns = positions (one per lane and j), rows = cout
+        int64_t base[FN];
+        bool ok[FN];
 #pragma unroll
-    for (int i = 0; i < FM; ++i)
+        for (int j = 0; j < FN; ++j) {
+            const int pos = n0 + (wn * FN + j) * 32 + lane % 32;
+            ok[j] = pos < p.positions;
+            const int n = pos / p.howo;
+            base[j] = int64_t(n) * p.cout * p.howo + (pos - n * p.howo);
+        }
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int co = m0 + (wm * FM + i) * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
+                if (co >= p.cout) continue;
+                const float dq = p.dq ? p.dq[co] : 0.f;
+                const float bias = p.bias ? p.bias[co] : 0.f;
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    if (ok[j]) emit(p, acc[i][j][r], base[j] + int64_t(co) * p.howo, dq, bias, 0.f);
+            }
+    } else {
+        // columns = cout (one per lane and i), rows = positions; output is [positions][cout]
+        float dq[FM], bias[FM];
+        int co[FM];
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+            co[i] = m0 + (wm * FM + i) * 32 + lane % 32;
+            const bool in = co[i] < p.cout;
+            dq[i] = (in && p.dq) ? p.dq[co[i]] : 0.f;
+            bias[i] = (in && p.bias) ? p.bias[co[i]] : 0.f;
+        }
 #pragma unroll
         for (int j = 0; j < FN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int rr = 8 * (r / 4) + 4 * (lane / 32) + (r % 4), cc = lane % 32;
-                const int co = m0 + (wm * FM + i) * 32 + (SWAP ? cc : rr);
-                const int pos = n0 + (wn * FN + j) * 32 + (SWAP ? rr : cc);
-                emit(p, acc[i][j][r], co, pos);
+                const int pos = n0 + (wn * FN + j) * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
+                if (pos >= p.positions) continue;
+                const float rs = p.row_scale ? p.row_scale[pos] : 0.f;
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+                    if (co[i] < p.cout) emit(p, acc[i][j][r], int64_t(pos) * p.cout + co[i], dq[i], bias[i], rs);
             }
+    }
 }
 
 // ------------------------------------------------------------------ host side
@@ -280,6 +319,10 @@ struct Plan {
     int ho, wo, hs, ws, cp, cblocks, taps, coutp;
     int64_t positions;
     size_t staged_bytes, packed_bytes;
+    // stride-1 layers whose tap window fits LDS take the window-stationary kernel
+    bool use_ws;
+    tsx::WsGeom wsg;
+    tsx::WsPlan wsp;
 };
 
 int make_plan(const tsx_conv2d_geom *g, Plan *pl) {
@@ -304,6 +347,16 @@ int make_plan(const tsx_conv2d_geom *g, Plan *pl) {
     TSX_REQUIRE(pl->positions < (int64_t(1) << 31), "conv2d_i8: too many output positions");
     pl->staged_bytes = size_t(g->n) * pl->hs * pl->ws * pl->cp;
     pl->packed_bytes = size_t(pl->taps) * pl->cblocks * pl->coutp * KSTEP;
+    pl->use_ws = false;
+    if (g->stride_h == 1 && g->stride_w == 1) {
+        pl->wsg = tsx::WsGeom{g->n, g->cout, pl->ho, pl->wo, pl->hs, pl->ws, pl->cp, pl->cblocks, g->kh, g->kw,
+                              g->dilation_h, g->dilation_w};
+        pl->wsp = tsx::ws_plan(pl->wsg);
+        if (pl->wsp.ok) {
+            pl->use_ws = true;
+            pl->packed_bytes = pl->wsp.packed_bytes;
+        }
+    }
     return 0;
 }
 
@@ -323,7 +376,7 @@ int check_epilogue(const tsx_epilogue *ep, const float *out_f32, const int8_t *o
     return 0;
 }
 
-void fill_epilogue(GemmParams &p, const tsx_epilogue *ep, int64_t count, float *out_f32, int8_t *out_i8,
+void fill_epilogue(tsx::EpiParams &p, const tsx_epilogue *ep, int64_t count, float *out_f32, int8_t *out_i8,
                    int32_t *out_acc) {
     p.dq = ep ? ep->dq_dev : nullptr;
     p.row_scale = ep ? ep->row_scale_dev : nullptr;
@@ -348,22 +401,12 @@ int launch_igemm(const GemmParams &p, hipStream_t stream) {
     return 0;
 }
 
-int run_conv(const tsx_conv2d_geom *g, const void *x, bool x_is_f32, const float *x_scales, int n_x_scales,
-             const void *packed_w, float padding_value, const tsx_epilogue *ep, float *out_f32, int8_t *out_i8,
-             int32_t *out_acc, void *workspace, size_t workspace_bytes, void *stream_) {
-    Plan pl;
-    int rc = make_plan(g, &pl);
-    if (rc) return rc;
-    rc = check_epilogue(ep, out_f32, out_i8, out_acc, g->n);
-    if (rc) return rc;
-    TSX_REQUIRE(x && packed_w, "conv2d_i8: null input");
-    TSX_REQUIRE(!(ep && ep->row_scale_dev), "conv2d_i8: row_scale is a GEMM-only epilogue term");
-    if (!workspace || workspace_bytes < pl.staged_bytes)
-        return tsx::fail(TSX_E_WORKSPACE, "conv2d_i8: workspace %zu < %zu bytes", workspace_bytes, pl.staged_bytes);
-    TSX_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0 && reinterpret_cast<uintptr_t>(packed_w) % 16 == 0,
-                "conv2d_i8: workspace and packed weights must be 16-byte aligned");
-    hipStream_t stream = tsx::as_stream(stream_);
-
+int run_stage(const tsx_conv2d_geom *g, const Plan &pl, const void *x, bool x_is_f32, const float *x_scales,
+              int n_x_scales, float padding_value, void *staged, size_t staged_bytes, hipStream_t stream) {
+    TSX_REQUIRE(x, "conv2d_i8: null input");
+    if (!staged || staged_bytes < pl.staged_bytes)
+        return tsx::fail(TSX_E_WORKSPACE, "conv2d_i8: workspace %zu < %zu bytes", staged_bytes, pl.staged_bytes);
+    TSX_REQUIRE(reinterpret_cast<uintptr_t>(staged) % 16 == 0, "conv2d_i8: workspace must be 16-byte aligned");
     StageGeom sg{g->n, g->c, g->h, g->w, pl.hs, pl.ws, pl.cp, g->pad_top, g->pad_left,
                  int(int8_t(padding_value))};  // T(padding_value), conv2d_quantized_core.cpp:72
     const int64_t stage_threads = int64_t(g->n) * pl.hs * pl.ws * (pl.cp / 16);
@@ -375,16 +418,26 @@ int run_conv(const tsx_conv2d_geom *g, const void *x, bool x_is_f32, const float
         const int64_t count = int64_t(g->n) * g->c * g->h * g->w;
         const int64_t group_len = int64_t(std::ceil(static_cast<float>(count) / static_cast<float>(n_x_scales)));
         hipLaunchKernelGGL(stage_nchw_kernel<true>, dim3(stage_blocks), dim3(256), 0, stream, x, sg, x_scales,
-                           n_x_scales, group_len, (count >> 3) << 3, static_cast<int8_t *>(workspace));
+                           n_x_scales, group_len, (count >> 3) << 3, static_cast<int8_t *>(staged));
     } else {
         hipLaunchKernelGGL(stage_nchw_kernel<false>, dim3(stage_blocks), dim3(256), 0, stream, x, sg,
                            static_cast<const float *>(nullptr), 1, int64_t(1), int64_t(0),
-                           static_cast<int8_t *>(workspace));
+                           static_cast<int8_t *>(staged));
     }
     TSX_LAUNCH_CHECK("stage_nchw_kernel");
+    return 0;
+}
 
+int run_staged(const tsx_conv2d_geom *g, const Plan &pl, const void *staged, const void *packed_w,
+               const tsx_epilogue *ep, float *out_f32, int8_t *out_i8, int32_t *out_acc, hipStream_t stream) {
+    int rc = check_epilogue(ep, out_f32, out_i8, out_acc, g->n);
+    if (rc) return rc;
+    TSX_REQUIRE(staged && packed_w, "conv2d_i8: null input");
+    TSX_REQUIRE(!(ep && ep->row_scale_dev), "conv2d_i8: row_scale is a GEMM-only epilogue term");
+    TSX_REQUIRE(reinterpret_cast<uintptr_t>(staged) % 16 == 0 && reinterpret_cast<uintptr_t>(packed_w) % 16 == 0,
+                "conv2d_i8: staged activations and packed weights must be 16-byte aligned");
     GemmParams p{};
-    p.xs = static_cast<const int8_t *>(workspace);
+    p.xs = static_cast<const int8_t *>(staged);
     p.wp = static_cast<const int8_t *>(packed_w);
     p.positions = int(pl.positions);
     p.howo = pl.ho * pl.wo;
@@ -402,7 +455,25 @@ int run_conv(const tsx_conv2d_geom *g, const void *x, bool x_is_f32, const float
     p.cout = g->cout;
     p.coutp = pl.coutp;
     fill_epilogue(p, ep, int64_t(g->n) * g->cout * pl.ho * pl.wo, out_f32, out_i8, out_acc);
+    if (pl.use_ws)
+        return tsx::ws_launch(pl.wsg, pl.wsp, p.xs, p.wp, static_cast<const tsx::EpiParams &>(p), stream);
     return launch_igemm<false>(p, stream);
+}
+
+int run_conv(const tsx_conv2d_geom *g, const void *x, bool x_is_f32, const float *x_scales, int n_x_scales,
+             const void *packed_w, float padding_value, const tsx_epilogue *ep, float *out_f32, int8_t *out_i8,
+             int32_t *out_acc, void *workspace, size_t workspace_bytes, void *stream_) {
+    Plan pl;
+    int rc = make_plan(g, &pl);
+    if (rc) return rc;
+    // validate the second half before launching the first
+    rc = check_epilogue(ep, out_f32, out_i8, out_acc, g->n);
+    if (rc) return rc;
+    TSX_REQUIRE(packed_w, "conv2d_i8: null packed weights");
+    hipStream_t stream = tsx::as_stream(stream_);
+    rc = run_stage(g, pl, x, x_is_f32, x_scales, n_x_scales, padding_value, workspace, workspace_bytes, stream);
+    if (rc) return rc;
+    return run_staged(g, pl, workspace, packed_w, ep, out_f32, out_i8, out_acc, stream);
 }
 
 }  // namespace
@@ -425,6 +496,9 @@ int tsx_conv2d_i8_pack_weights(const tsx_conv2d_geom *g, const int8_t *w_oihw_de
     if (rc) return rc;
     TSX_REQUIRE(w_oihw_dev && packed_dev, "pack_weights: null pointer");
     TSX_REQUIRE(reinterpret_cast<uintptr_t>(packed_dev) % 16 == 0, "pack_weights: packed buffer must be 16-byte aligned");
+    if (pl.use_ws)
+        return tsx::ws_pack_weights(pl.wsg, pl.wsp, w_oihw_dev, g->c, static_cast<int8_t *>(packed_dev),
+                                    tsx::as_stream(stream));
     const int64_t threads = int64_t(pl.packed_bytes / 16);
     hipLaunchKernelGGL(pack_weights_kernel, dim3(unsigned(tsx::ceil_div(threads, 256))), dim3(256), 0,
                        tsx::as_stream(stream), w_oihw_dev, g->cout, g->c, pl.taps, int64_t(g->c) * pl.taps,
@@ -446,6 +520,24 @@ int tsx_quantize_conv2d_i8_nchw(const tsx_conv2d_geom *g, const float *x_f32_dev
                                 void *workspace_dev, size_t workspace_bytes, void *stream) {
     return run_conv(g, x_f32_dev, true, x_scales_dev, n_x_scales, packed_w_dev, padding_value, ep, out_f32_dev,
                     out_i8_dev, out_acc_dev, workspace_dev, workspace_bytes, stream);
+}
+
+int tsx_conv2d_i8_stage(const tsx_conv2d_geom *g, const void *x_dev, int32_t x_is_f32, const float *x_scales_dev,
+                        int32_t n_x_scales, float padding_value, void *staged_dev, size_t staged_bytes, void *stream) {
+    Plan pl;
+    int rc = make_plan(g, &pl);
+    if (rc) return rc;
+    return run_stage(g, pl, x_dev, x_is_f32 != 0, x_scales_dev, n_x_scales, padding_value, staged_dev, staged_bytes,
+                     tsx::as_stream(stream));
+}
+
+int tsx_conv2d_i8_staged(const tsx_conv2d_geom *g, const void *staged_dev, const void *packed_w_dev,
+                         const tsx_epilogue *ep, float *out_f32_dev, int8_t *out_i8_dev, int32_t *out_acc_dev,
+                         void *stream) {
+    Plan pl;
+    int rc = make_plan(g, &pl);
+    if (rc) return rc;
+    return run_staged(g, pl, staged_dev, packed_w_dev, ep, out_f32_dev, out_i8_dev, out_acc_dev, tsx::as_stream(stream));
 }
 
 // ---- GEMM: a [m][k] is a batch of m "images" with k channels and 1x1 extent.

@@ -1,0 +1,344 @@
+// Window-stationary int8 convolution for stride-1 layers (the 3x3 body of ResNet-like nets
+// and BASELINE config 2) on v_mfma_i32_32x32x32_i8
+// (the 16x16x64 form runs at half the rate on this part).
+//
+// Same arithmetic as the generic implicit GEMM in conv2d_i8.hip (exact int32 sums of
+// cpu::Conv2DQuantizedCore, src/kernels/cpu/quantized/conv2d_quantized_core.cpp:18-147), but
+// a different data movement:
+//   * one workgroup (4 wavefronts) owns TH full output rows of one image x 256 output
+//     channels; wavefront w owns channels [64w, 64w+64) and all positions of the tile;
+//   * per 64-channel block the input *window* that all KH*KW taps of the tile read
+//     ((TH + (KH-1)*dil) rows x staged width) is copied once into LDS (double buffered,
+//     one block ahead, 80-byte pixel stride = bank-conflict-free 16-byte reads); every tap is
+//     then a shifted read of the same LDS data, so activations cross L2 -> CU once, not
+//     KH*KW times, and the K loop needs one barrier per channel block, not per K-step;
+//   * weights never touch LDS: each wavefront streams its own rows from the packed
+//     buffer (1 KiB contiguous per MFMA operand) into a 4-deep register ring, three
+//     K-steps ahead of use.
+// K order is (channel block, kh, kw); K-steps are padded with zero weights to a multiple
+// of the ring depth.
+//
+// MFMA operand layout (v_mfma_i32_32x32x32_i8): lane l supplies row/column l%32 and the 16
+// K bytes of group l/32 (two MFMAs, "halves", cover a 64-byte K-step); accumulator register r
+// of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32.  Rows = cout, columns = positions.
+#include "igemm_i8.hpp"
+
+namespace tsx {
+namespace {
+
+constexpr int RING = 4;         // A register ring depth (K-steps)
+constexpr int PIX = 80;         // LDS bytes per window pixel (64 + 16 pad)
+constexpr int WS_THREADS = 256;
+constexpr int WS_FM = 1;        // 32-cout fragments per wavefront
+constexpr int WS_BM = 4 * 32 * WS_FM;   // output channels per workgroup
+constexpr int MAX_FILL = 7;     // window chunks per thread per channel block
+constexpr int MAX_WP = MAX_FILL * WS_THREADS / 4;   // 448 window pixels
+
+struct WsParams : EpiParams {
+    const int8_t *xs;   // staged activations [n][hs][ws][cp]
+    const int8_t *wp;   // packed weights [ks_p][coutp/32][2 halves][64 lanes][16]
+    int cout, coutp, ho, wo, hs, ws, cp, cblocks, kh, kw, dil_h, dil_w;
+    int th, tiles_per_image, wr, wc, wpix, ksteps_p;
+};
+
+// packed[ks][frag][half][lane][16]: ks = cb*taps + tap; frag = cout/32; lane l: cout frag*32 + l%32,
+// channels cb*64 + half*32 + (l/32)*16 + 0..15.  K-steps >= cblocks*taps, rows >= cout, channels >= c: zero.
+__global__ __launch_bounds__(256) void ws_pack_kernel(const int8_t *__restrict__ w, int cout, int c, int taps,
+                                                     int cblocks, int ksteps_p, int coutp,
+                                                     int8_t *__restrict__ packed) {
+    const int frags = coutp / 32;
+    const int64_t total = int64_t(ksteps_p) * frags * 2 * 64;
+    const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id >= total) return;
+    const int lane = int(id % 64);
+    const int half = int((id / 64) % 2);
+    const int frag = int((id / 128) % frags);
+    const int ks = int(id / 128 / frags);
+    const int cb = ks / taps, tap = ks % taps;
+    const int co = frag * 32 + lane % 32;
+    const int c0 = cb * 64 + half * 32 + (lane / 32) * 16;
+    uint32_t words[4] = {0, 0, 0, 0};
+    if (co < cout && cb < cblocks) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int ci = c0 + j;
+            const int v = ci < c ? w[(int64_t(co) * c + ci) * taps + tap] : 0;
+            words[j / 4] |= uint32_t(v & 0xff) << (8 * (j % 4));
+        }
+    }
+    *reinterpret_cast<uint4 *>(packed + id * 16) = make_uint4(words[0], words[1], words[2], words[3]);
+}
+
+template <int NT, int FM>
+__global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p) {
+    extern __shared__ __attribute__((aligned(16))) int8_t lds[];   // 2 x wpix x PIX
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const int img = blockIdx.x / p.tiles_per_image;
+    const int th0 = (blockIdx.x - img * p.tiles_per_image) * p.th;   // first output row of the tile
+    const int m0 = (blockIdx.y * 4 + wave) * (32 * FM);             // first cout of this wavefront
+    const int taps = p.kh * p.kw;
+    const int win_bytes = p.wpix * PIX;
+
+    // ---- window fill bookkeeping: chunk q = tid + i*256 -> pixel q/4, 16-byte chunk q%4
+    const int8_t *fill_src[MAX_FILL];
+    int fill_dst[MAX_FILL];
+    static_for<0, MAX_FILL>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        const int q = tid + i * WS_THREADS;
+        int pix = q >> 2;
+        const int chunk = q & 3;
+        if (pix >= p.wpix) pix = p.wpix - 1;   // duplicates rewrite the same bytes
+        int wrow = pix / p.wc;
+        const int wcol = pix - wrow * p.wc;
+        int row = th0 + wrow;                  // stride 1: window row r is staged row th0 + r
+        if (row >= p.hs) row = p.hs - 1;       // partial last tile: rows never used by stored outputs
+        fill_src[i] = p.xs + ((int64_t(img) * p.hs + row) * p.ws + wcol) * p.cp + chunk * 16;
+        fill_dst[i] = pix * PIX + chunk * 16;
+    });
+    const int n_fill = (p.wpix * 4 + WS_THREADS - 1) / WS_THREADS;   // <= MAX_FILL, uniform
+    v4i wreg[MAX_FILL];   // native vectors: arrays of HIP's uint4 struct do not stay in registers
+
+    auto window_load = [&](int cb) __attribute__((always_inline)) {
+        static_for<0, MAX_FILL>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            if (i < n_fill) wreg[i] = *reinterpret_cast<const v4i *>(fill_src[i] + cb * 64);
+        });
+    };
+    auto window_store = [&](int buf) __attribute__((always_inline)) {
+        static_for<0, MAX_FILL>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            if (i < n_fill) *reinterpret_cast<v4i *>(&lds[buf * win_bytes + fill_dst[i]]) = wreg[i];
+        });
+    };
+
+    // ---- B operand addresses: fragment j, lane l -> tile position j*32 + l%32, K group l/32
+    int b_base[NT];
+    static_for<0, NT>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        int pos = j * 32 + lane % 32;
+        if (pos >= p.th * p.wo) pos = 0;       // padding positions: computed, never stored
+        const int oh = pos / p.wo, ow = pos - oh * p.wo;
+        b_base[j] = (oh * p.wc + ow) * PIX + (lane / 32) * 16;
+    });
+
+    // ---- A ring: the wavefront's FM fragments (32 cout each) x 2 halves of K-step ks, 1 KiB each
+    const int8_t *a_ptr = p.wp + (int64_t(m0 / 32) * 128 + lane) * 16;
+    const int64_t a_kstride = int64_t(p.coutp / 32) * 128 * 16;
+    v4i areg[RING][2 * FM];
+    auto a_load = [&](auto slot, int ks) __attribute__((always_inline)) {
+        constexpr int s = decltype(slot)::value;
+        if (ks >= p.ksteps_p) ks = p.ksteps_p - 1;
+        const int8_t *src = a_ptr + ks * a_kstride;
+        static_for<0, 2 * FM>([&](auto fc) {
+            constexpr int f = decltype(fc)::value;
+            areg[s][f] = *reinterpret_cast<const v4i *>(src + f * 1024);
+        });
+    };
+
+    v16i acc[FM][NT];
+    static_for<0, FM>([&](auto ic) {
+        static_for<0, NT>([&](auto jc) {
+            static_for<0, 16>([&](auto rc) { acc[decltype(ic)::value][decltype(jc)::value][decltype(rc)::value] = 0; });
+        });
+    });
+
+    // ---- prologue
+    window_load(0);
+    static_for<0, RING - 1>([&](auto sc) { a_load(sc, decltype(sc)::value); });
+    window_store(0);
+    __syncthreads();
+    int cb = 0, tap = 0, kr = 0, kc = 0, buf = 0;
+    window_load(p.cblocks > 1 ? 1 : 0);   // block cb+1, in flight during block cb's taps
+
+    // B fragments are read one half-step ahead of the MFMAs that use them (one wavefront per
+    // SIMD: nothing else hides the LDS latency).
+    v4i b0[NT], b1[NT];
+    auto b_read = [&](v4i(&dst)[NT], int off) __attribute__((always_inline)) {
+        static_for<0, NT>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            dst[j] = *reinterpret_cast<const v4i *>(&lds[b_base[j] + off]);
+        });
+    };
+    int toff = 0;   // buf * win_bytes + tap shift
+    b_read(b0, toff);
+
+    for (int ks0 = 0; ks0 < p.ksteps_p; ks0 += RING) {
+        static_for<0, RING>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            // prefetch weights of K-step ks0+u+RING-1 into the slot freed by the previous step
+            a_load(std::integral_constant<int, (u + RING - 1) % RING>{}, ks0 + u + RING - 1);
+            b_read(b1, toff + 32);                       // second half of this K-step
+            static_for<0, FM>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                static_for<0, NT>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value;
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[u][i * 2], b0[j], acc[i][j], 0, 0, 0);
+                });
+            });
+            // advance (cb, tap); on a channel-block boundary swap in the next window
+            ++tap;
+            if (++kc == p.kw) {
+                kc = 0;
+                ++kr;
+            }
+            if (tap == taps) {
+                tap = 0;
+                kr = 0;
+                kc = 0;
+                ++cb;
+                window_store(buf ^ 1);
+                __syncthreads();
+                buf ^= 1;
+                const int next = cb + 1 < p.cblocks ? cb + 1 : p.cblocks - 1;
+                window_load(next);
+            }
+            toff = buf * win_bytes + (kr * p.dil_h * p.wc + kc * p.dil_w) * PIX;
+            b_read(b0, toff);                            // first half of the next K-step
+            static_for<0, FM>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                static_for<0, NT>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value;
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[u][i * 2 + 1], b1[j], acc[i][j], 0, 0, 0);
+                });
+            });
+        });
+    }
+
+    // ---- epilogue: accumulator register r of lane l = cout 8*(r/4) + 4*(l/32) + r%4, position l%32
+    const int tile_pos = p.th * p.wo;
+    const int howo = p.ho * p.wo;
+    const int64_t count = int64_t(gridDim.x / p.tiles_per_image) * p.cout * howo;
+    // hot case: fp32 output only, every element inside the activation's SIMD-body range, and
+    // a tensor small enough for 32-bit lane offsets
+    const bool fast = p.out_f32 && !p.out_i8 && !p.out_acc && p.act_body == count && count < (int64_t(1) << 30);
+    static_for<0, FM>([&](auto fc) {
+        constexpr int f = decltype(fc)::value;
+        const int cf = m0 + f * 32;   // first cout of this fragment (uniform)
+        float dq[16], bias[16];
+        static_for<0, 16>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            const int co = cf + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
+            const bool in = co < p.cout;
+            dq[r] = (in && p.dq) ? p.dq[co] : 0.f;
+            bias[r] = (in && p.bias) ? p.bias[co] : 0.f;
+        });
+        static_for<0, NT>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const int pos = j * 32 + lane % 32;
+            const int oh = pos / p.wo, ow = pos - oh * p.wo;
+            const bool pos_ok = pos < tile_pos && th0 + oh < p.ho;
+            if (fast && cf + 32 <= p.cout) {
+                // uniform base in scalar registers + one 32-bit lane offset: no per-store address math
+                float *sbase = p.out_f32 + (int64_t(img) * p.cout + cf) * howo + int64_t(th0) * p.wo;
+                const unsigned lane_off = unsigned((4 * (lane / 32)) * howo + oh * p.wo + ow);
+                if (pos_ok) {
+                    static_for<0, 16>([&](auto rc) {
+                        constexpr int r = decltype(rc)::value;
+                        constexpr int dco = 8 * (r / 4) + (r % 4);
+                        float v = __fmul_rn(float(acc[f][j][r]), dq[r]);
+                        if (p.bias) v = __fadd_rn(v, bias[r]);
+                        (sbase + int64_t(dco) * howo)[lane_off] = apply_act(v, p.act, p.slope, true);
+                    });
+                }
+            } else {
+                const int co0 = cf + 4 * (lane / 32);
+                const int64_t base = (int64_t(img) * p.cout + co0) * howo + (th0 + oh) * p.wo + ow;
+                static_for<0, 16>([&](auto rc) {
+                    constexpr int r = decltype(rc)::value;
+                    constexpr int dco = 8 * (r / 4) + (r % 4);
+                    if (pos_ok && co0 + dco < p.cout)
+                        emit(p, acc[f][j][r], base + int64_t(dco) * howo, dq[r], bias[r], 0.f);
+                });
+            }
+        });
+    });
+}
+
+template <int NT>
+int launch_nt(const WsParams &p, dim3 grid, size_t lds_bytes, hipStream_t stream) {
+    // 32 cout per wavefront (128 per workgroup): two workgroups share a CU, so one
+    // wavefront's LDS/L2 waits are covered by the other on the same SIMD.
+    hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM>), grid, dim3(WS_THREADS), lds_bytes, stream, p);
+    TSX_LAUNCH_CHECK("conv_i8_ws_kernel");
+    return 0;
+}
+
+}  // namespace
+
+WsPlan ws_plan(const WsGeom &g) {
+    WsPlan pl{};
+    pl.ok = false;
+    // stride-1 only (the caller checks strides); positions of a tile must fit 8 fragments
+    if (g.wo > 128 || g.wo < 1) return pl;
+    int th = 128 / g.wo;
+    if (th > g.ho) th = g.ho;
+    // prefer the row count with the least padding per fragment group
+    int best = th, best_waste = 1 << 30;
+    for (int t = th; t >= 1 && t * 2 > th; --t) {
+        const int nt = (t * g.wo + 31) / 32;
+        const int tiles = (g.ho + t - 1) / t;
+        const int waste = tiles * nt * 32 - g.ho * g.wo;
+        if (waste < best_waste) {
+            best_waste = waste;
+            best = t;
+        }
+    }
+    pl.th = best;
+    pl.nt = (pl.th * g.wo + 31) / 32;
+    pl.tiles_per_image = (g.ho + pl.th - 1) / pl.th;
+    pl.wr = pl.th + (g.kh - 1) * g.dil_h;
+    pl.wc = g.ws;
+    pl.wp = pl.wr * pl.wc;
+    if (pl.wp > MAX_WP || size_t(2) * pl.wp * PIX > 65536) return pl;   // two windows must fit 64 KiB of LDS
+    const int ksteps = g.cblocks * g.kh * g.kw;
+    pl.ksteps_p = (ksteps + RING - 1) / RING * RING;
+    pl.coutp = (g.cout + WS_BM - 1) / WS_BM * WS_BM;
+    pl.packed_bytes = size_t(pl.ksteps_p) * pl.coutp * 64;
+    pl.ok = true;
+    return pl;
+}
+
+int ws_pack_weights(const WsGeom &g, const WsPlan &pl, const int8_t *w_oihw, int c, int8_t *packed, hipStream_t stream) {
+    const int64_t threads = int64_t(pl.packed_bytes / 16);
+    hipLaunchKernelGGL(ws_pack_kernel, dim3(unsigned(ceil_div(threads, 256))), dim3(256), 0, stream, w_oihw, g.cout, c,
+                       g.kh * g.kw, g.cblocks, pl.ksteps_p, pl.coutp, packed);
+    TSX_LAUNCH_CHECK("ws_pack_kernel");
+    return 0;
+}
+
+int ws_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t *packed, const EpiParams &ep,
+              hipStream_t stream) {
+    WsParams p{};
+    static_cast<EpiParams &>(p) = ep;
+    p.xs = xs;
+    p.wp = packed;
+    p.cout = g.cout;
+    p.coutp = pl.coutp;
+    p.ho = g.ho;
+    p.wo = g.wo;
+    p.hs = g.hs;
+    p.ws = g.ws;
+    p.cp = g.cp;
+    p.cblocks = g.cblocks;
+    p.kh = g.kh;
+    p.kw = g.kw;
+    p.dil_h = g.dil_h;
+    p.dil_w = g.dil_w;
+    p.th = pl.th;
+    p.tiles_per_image = pl.tiles_per_image;
+    p.wr = pl.wr;
+    p.wc = pl.wc;
+    p.wpix = pl.wp;
+    p.ksteps_p = pl.ksteps_p;
+    const dim3 grid(unsigned(g.n) * pl.tiles_per_image, unsigned(pl.coutp / WS_BM));
+    const size_t lds_bytes = size_t(2) * pl.wp * PIX;
+    switch (pl.nt) {
+        case 1: return launch_nt<1>(p, grid, lds_bytes, stream);
+        case 2: return launch_nt<2>(p, grid, lds_bytes, stream);
+        case 3: return launch_nt<3>(p, grid, lds_bytes, stream);
+        case 4: return launch_nt<4>(p, grid, lds_bytes, stream);
+    }
+    return fail(TSX_E_INVALID, "conv_i8_ws: unsupported fragment count %d", pl.nt);
+}
+
+}  // namespace tsx
