@@ -130,6 +130,40 @@ int tsx_gemm_i8(int32_t m, int32_t n, int32_t k, const int8_t *a_dev, const void
                 const tsx_epilogue *ep, float *out_f32_dev, int8_t *out_i8_dev, int32_t *out_acc_dev,
                 void *workspace_dev, size_t workspace_bytes, void *stream);
 
+/* ---------------------------------------------------------------- fp32 conv2d / inner_prod
+ * cpu::Conv2DCore::conv2d (src/kernels/cpu/conv2d_core.cpp:101-119, interface
+ * include/backend/base/base_conv2d_core.h:14-32): im2col + GEMM, here one implicit-GEMM kernel on
+ * the fp32 MFMA reading NCHW directly (weights are used as they are: no packing, no workspace).
+ * bias_dev (optional, [cout]) and act fuse the add_bias / relu operators that follow the conv in
+ * BASELINE config 1; pass NULL / TSX_ACT_NONE for the bare operator.  Parity bar for this
+ * floating-point path: 1e-4 relative / 1e-5 absolute against the reference CPU kernels. */
+int tsx_conv2d_f32_nchw(const tsx_conv2d_geom *g, const float *x_dev, const float *w_oihw_dev, float padding_value,
+                        const float *bias_dev, int32_t act, float slope, float *out_dev, void *stream);
+
+/* cpu::InnerProd::inner_prod (src/kernels/cpu/inner_prod.cpp:54-69, interface
+ * include/backend/base/base_inner_prod.h:32-48): out[m][n] = lhs[m][k] * rhs, rhs being [k][n], or
+ * [n][k] when transpose != 0. */
+int tsx_inner_prod_f32(int32_t m, int32_t n, int32_t k, const float *lhs_dev, const float *rhs_dev, int32_t transpose,
+                       float *out_dev, void *stream);
+
+/* ---------------------------------------------------------------- Winograd F(6x6, 3x3) fp32 conv2d
+ * Conv2dWinogradAlgorithm<float>::winograd_f63 (src/kernels/cpu/winograd_algorithm.cpp:846-947),
+ * reached in the reference through base::Conv2DWinograd's two core calls
+ * (include/backend/base/base_conv2d_winograd.h:24-27):
+ *   conv2d_tranform_kernel(mode, kernel, kernel_transformed)  -> tsx_winograd_f63_transform_kernel
+ *   conv2d_winograd(x, mode, padding, padding_value, w, ...)   -> tsx_conv2d_winograd_f63_nchw
+ * 3x3 kernels, stride 1, dilation 1 only.  The transformed kernel u_dev ([64][cout][cin] floats,
+ * tsx_winograd_f63_kernel_bytes) is this backend's own layout, produced and consumed only here.
+ * Transforms and accumulation order restate the reference's arithmetic exactly (including the
+ * fused multiply-adds of its AVX2/FMA build), so results match its F(6,3) to the bit; optional
+ * bias/activation are the add_bias / relu operators fused behind the output transform. */
+size_t tsx_winograd_f63_kernel_bytes(int32_t cout, int32_t cin);
+int tsx_winograd_f63_transform_kernel(int32_t cout, int32_t cin, const float *w_oihw_dev, float *u_dev, void *stream);
+size_t tsx_winograd_f63_workspace_bytes(const tsx_conv2d_geom *g);
+int tsx_conv2d_winograd_f63_nchw(const tsx_conv2d_geom *g, const float *x_dev, const float *u_dev, float padding_value,
+                                 const float *bias_dev, int32_t act, float slope, float *out_dev, void *workspace_dev,
+                                 size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -375,7 +375,12 @@ void orc_inner_prod_f32(const float *lhs, int m, int k, const float *rhs, int n,
 // padded bottom/right with padding_value to out_padded+2, result cut back).
 //   U = G g G^T (kernel, :504-566), V = B^T d B (input, :607-699), M_t = U_t V_t (64 GEMMs
 //   Cout x Cin x tiles through the fp32 GEMM above, :917-936), Y = A^T M A (:738-833).
-// The transform expressions keep the reference's factoring so rounding matches closely.
+// The reference writes the transforms as plain float expressions and is built with gcc -O3 -mfma,
+// whose default -ffp-contract=fast turns a*b+c patterns into fused multiply-adds; that choice
+// is part of the reference's numerics (F(6,3) amplifies single roundings to ~1e-5).  The fused
+// forms are written out explicitly here -- in `a*c1 - b*c2 [+ ...]` gcc fuses the FIRST product
+// and rounds the second -- and this file is compiled with -ffp-contract=off, so the result no
+// longer depends on the compiler.  Checked bit for bit against the compiled reference.
 // ---------------------------------------------------------------------------
 static void wino_f63_kernel(const float *g, float u[64]) {
     static const float G[8][3] = {{1.0f, 0.0f, 0.0f},
@@ -389,42 +394,41 @@ static void wino_f63_kernel(const float *g, float u[64]) {
     float tmp[3][8];
     for (int i = 0; i < 8; ++i)
         for (int r = 0; r < 3; ++r)
-            tmp[r][i] = g[r * 3 + 0] * G[i][0] + g[r * 3 + 1] * G[i][1] + g[r * 3 + 2] * G[i][2];
+            tmp[r][i] = std::fmaf(g[r * 3 + 2], G[i][2], std::fmaf(g[r * 3 + 0], G[i][0], g[r * 3 + 1] * G[i][1]));
     for (int i = 0; i < 8; ++i)
-        for (int j = 0; j < 8; ++j) u[i * 8 + j] = tmp[0][j] * G[i][0] + tmp[1][j] * G[i][1] + tmp[2][j] * G[i][2];
+        for (int j = 0; j < 8; ++j) u[i * 8 + j] = std::fmaf(tmp[2][j], G[i][2], std::fmaf(tmp[0][j], G[i][0], tmp[1][j] * G[i][1]));
 }
 
 static inline void wino_f63_bt(const float i0[8], float o[8]) {
-    o[0] = i0[0] - i0[6] + (i0[4] - i0[2]) * 5.25f;
-    o[7] = i0[7] - i0[1] + (i0[3] - i0[5]) * 5.25f;
-    float tmp12_a = (i0[2] + i0[6] - i0[4] * 4.25f);
-    float tmp12_b = (i0[1] + i0[5] - i0[3] * 4.25f);
+    o[0] = std::fmaf(i0[4] - i0[2], 5.25f, i0[0] - i0[6]);
+    o[7] = std::fmaf(i0[3] - i0[5], 5.25f, i0[7] - i0[1]);
+    float tmp12_a = std::fmaf(-i0[4], 4.25f, i0[2] + i0[6]);
+    float tmp12_b = std::fmaf(-i0[3], 4.25f, i0[1] + i0[5]);
     o[1] = tmp12_a + tmp12_b;
     o[2] = tmp12_a - tmp12_b;
-    float tmp34_a = (i0[6] + i0[2] * 0.25f - i0[4] * 1.25f);
-    float tmp34_b = (i0[1] * 0.5f - i0[3] * 2.5f + i0[5] * 2.f);
+    float tmp34_a = std::fmaf(-i0[4], 1.25f, std::fmaf(i0[2], 0.25f, i0[6]));
+    float tmp34_b = std::fmaf(i0[5], 2.f, std::fmaf(i0[1], 0.5f, -(i0[3] * 2.5f)));
     o[3] = tmp34_a + tmp34_b;
     o[4] = tmp34_a - tmp34_b;
-    float tmp56_a = (i0[6] + (i0[2] - i0[4] * 1.25f) * 4.f);
-    float tmp56_b = (i0[1] * 2.f - i0[3] * 2.5f + i0[5] * 0.5f);
+    float tmp56_a = std::fmaf(std::fmaf(-i0[4], 1.25f, i0[2]), 4.f, i0[6]);
+    float tmp56_b = std::fmaf(i0[5], 0.5f, std::fmaf(i0[1], 2.f, -(i0[3] * 2.5f)));
     o[5] = tmp56_a + tmp56_b;
     o[6] = tmp56_a - tmp56_b;
 }
 
 static inline void wino_f63_bt_col(const float d[8], float o[8]) {
-    // second pass (:668-692); note tmp12_b's operand order differs from the first pass
-    o[0] = d[0] - d[6] + (d[4] - d[2]) * 5.25f;
-    o[7] = d[7] - d[1] + (d[3] - d[5]) * 5.25f;
-    float tmp12_a = d[2] + d[6] - d[4] * 4.25f;
-    float tmp12_b = d[1] - d[3] * 4.25f + d[5];
+    o[0] = std::fmaf(d[4] - d[2], 5.25f, d[0] - d[6]);
+    o[7] = std::fmaf(d[3] - d[5], 5.25f, d[7] - d[1]);
+    float tmp12_a = std::fmaf(-d[4], 4.25f, d[2] + d[6]);
+    float tmp12_b = std::fmaf(-d[3], 4.25f, d[1]) + d[5];
     o[1] = tmp12_a + tmp12_b;
     o[2] = tmp12_a - tmp12_b;
-    float tmp34_a = d[6] + d[2] * 0.25f - d[4] * 1.25f;
-    float tmp34_b = d[1] * 0.5f - d[3] * 2.5f + d[5] * 2.f;
+    float tmp34_a = std::fmaf(-d[4], 1.25f, std::fmaf(d[2], 0.25f, d[6]));
+    float tmp34_b = std::fmaf(d[5], 2.f, std::fmaf(d[1], 0.5f, -(d[3] * 2.5f)));
     o[3] = tmp34_a + tmp34_b;
     o[4] = tmp34_a - tmp34_b;
-    float tmp56_a = d[6] + (d[2] - d[4] * 1.25f) * 4.f;
-    float tmp56_b = d[1] * 2.f - d[3] * 2.5f + d[5] * 0.5f;
+    float tmp56_a = std::fmaf(std::fmaf(-d[4], 1.25f, d[2]), 4.f, d[6]);
+    float tmp56_b = std::fmaf(d[5], 0.5f, std::fmaf(d[1], 2.f, -(d[3] * 2.5f)));
     o[5] = tmp56_a + tmp56_b;
     o[6] = tmp56_a - tmp56_b;
 }

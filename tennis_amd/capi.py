@@ -62,6 +62,13 @@ SIGNATURES = {
     "tsx_gemm_i8_pack_weights": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, _vp]),
     "tsx_gemm_i8_workspace_bytes": (_sz, [_i32, _i32]),
     "tsx_gemm_i8": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, ctypes.POINTER(Epilogue), _vp, _vp, _vp, _vp, _sz, _vp]),
+    "tsx_conv2d_f32_nchw": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, _f32, _vp, _i32, _f32, _vp, _vp]),
+    "tsx_inner_prod_f32": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp]),
+    "tsx_winograd_f63_kernel_bytes": (_sz, [_i32, _i32]),
+    "tsx_winograd_f63_transform_kernel": (ctypes.c_int, [_i32, _i32, _vp, _vp, _vp]),
+    "tsx_winograd_f63_workspace_bytes": (_sz, [ctypes.POINTER(ConvGeom)]),
+    "tsx_conv2d_winograd_f63_nchw": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, _f32, _vp, _i32, _f32, _vp, _vp,
+                                                    _sz, _vp]),
 }
 
 
@@ -225,3 +232,61 @@ class GemmI8:
         check(lib().tsx_gemm_i8(m, self.n, k, _ptr(a), _ptr(self.packed), ctypes.byref(ep.c) if ep else None,
                                 _ptr(out_f32), _ptr(out_i8), _ptr(acc), _ptr(self._workspace), ws_bytes, _stream()))
         return out_f32, out_i8, acc
+
+
+def conv2d_f32(x, w, pads=(0, 0, 0, 0), strides=(1, 1), dilations=(1, 1), padding_value=0.0, bias=None, act=None,
+               slope=0.0):
+    """tsx_conv2d_f32_nchw: fp32 implicit-GEMM conv2d (optionally + add_bias + activation)."""
+    x = _dev(x, torch.float32)
+    w = _dev(w, torch.float32)
+    bias = _dev(bias, torch.float32)
+    geom = make_geom(tuple(x.shape), tuple(w.shape), pads, strides, dilations)
+    ho, wo = conv_out_size(geom)
+    out = torch.empty((x.shape[0], w.shape[0], ho, wo), dtype=torch.float32, device=x.device)
+    check(lib().tsx_conv2d_f32_nchw(ctypes.byref(geom), _ptr(x), _ptr(w), float(padding_value), _ptr(bias), _ACT[act],
+                                    float(slope), _ptr(out), _stream()))
+    return out
+
+
+def inner_prod_f32(lhs, rhs, transpose=False):
+    """tsx_inner_prod_f32: out[m][n] = lhs[m][k] * rhs ([k][n], or [n][k] when transpose)."""
+    lhs = _dev(lhs, torch.float32)
+    rhs = _dev(rhs, torch.float32)
+    m, k = lhs.shape
+    n = rhs.shape[0] if transpose else rhs.shape[1]
+    if (rhs.shape[1] if transpose else rhs.shape[0]) != k:
+        raise TsxError("inner_prod: inner extents differ")
+    out = torch.empty((m, n), dtype=torch.float32, device=lhs.device)
+    check(lib().tsx_inner_prod_f32(m, n, k, _ptr(lhs), _ptr(rhs), int(bool(transpose)), _ptr(out), _stream()))
+    return out
+
+
+class WinogradF63:
+    """Winograd F(6,3) conv2d: the state of a `conv2d_winograd` operator instance (transformed kernel
+    cached at first use, base_conv2d_winograd.cpp:146-164)."""
+
+    def __init__(self, w, pads=(0, 0, 0, 0), padding_value=0.0):
+        self.w = _dev(w, torch.float32)
+        self.pads = tuple(pads)
+        self.padding_value = float(padding_value)
+        cout, cin = self.w.shape[0], self.w.shape[1]
+        self.u = torch.empty(lib().tsx_winograd_f63_kernel_bytes(cout, cin) // 4, dtype=torch.float32,
+                             device=self.w.device)
+        check(lib().tsx_winograd_f63_transform_kernel(cout, cin, _ptr(self.w), _ptr(self.u), _stream()))
+        self._workspace = None
+
+    def __call__(self, x, bias=None, act=None, slope=0.0):
+        x = _dev(x, torch.float32)
+        bias = _dev(bias, torch.float32)
+        geom = make_geom(tuple(x.shape), tuple(self.w.shape), self.pads)
+        ho, wo = conv_out_size(geom)
+        nbytes = lib().tsx_winograd_f63_workspace_bytes(ctypes.byref(geom))
+        if nbytes == 0:
+            raise TsxError("winograd: " + lib().tsx_last_error().decode())
+        if self._workspace is None or self._workspace.numel() < nbytes:
+            self._workspace = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+        out = torch.empty((x.shape[0], self.w.shape[0], ho, wo), dtype=torch.float32, device=x.device)
+        check(lib().tsx_conv2d_winograd_f63_nchw(ctypes.byref(geom), _ptr(x), _ptr(self.u), self.padding_value,
+                                                 _ptr(bias), _ACT[act], float(slope), _ptr(out), _ptr(self._workspace),
+                                                 nbytes, _stream()))
+        return out

@@ -3,22 +3,10 @@
 #pragma once
 #include "tsx_common.hpp"
 
-#include <type_traits>
-
 namespace tsx {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
-
-// Compile-time loop: register arrays are only ever indexed by constants, which keeps them
-// in VGPRs (runtime-indexed or loop-indexed arrays can end up in scratch memory).
-template <int I, int N, class F>
-__device__ __forceinline__ void static_for(F &&f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, N>(f);
-    }
-}
 
 struct EpiParams {
     const float *dq, *row_scale, *bias, *q_scales;

@@ -4,6 +4,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <type_traits>
 
 #include "tsx_hip.h"
 
@@ -47,6 +48,17 @@ inline int conv_out(int in, int pad_a, int pad_b, int k, int stride, int dilatio
 // Device-side scalar semantics shared by the quantize kernel and fused epilogues.
 // ---------------------------------------------------------------------------
 #ifdef __HIPCC__
+
+// Compile-time loop: register arrays are only ever indexed by constants, which keeps them
+// in VGPRs (loop-indexed arrays, and arrays of HIP's uint4/float4 structs, can end up in
+// scratch memory).
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
 
 // q = clamp(round(v), -128, 127) with the reference's x86 conversion behaviour:
 // NaN and |v| >= 2^31 convert to INT_MIN, i.e. -128 after the clamp

@@ -1,0 +1,326 @@
+// Winograd F(6x6, 3x3) fp32 convolution, restating
+// Conv2dWinogradAlgorithm<float>::winograd_f63 (src/kernels/cpu/winograd_algorithm.cpp:504-947)
+// with the padding rule of KernelCommonFunc::in_out_pad_and_fix_size
+// (src/kernels/common/function.cpp:14-78).
+//
+//   U = G g G^T      kernel transform, once per weight tensor          -> u[64][Cout][Cin]
+//   V = B^T d B      input transform of every 8x8 patch (stride 6)      -> v[N][64][Cin][tiles]
+//   M_t = U_t V_t    64 independent GEMMs (Cout x Cin x tiles) per image -> m[N][64][Cout][tiles]
+//   Y = A^T M A      output transform, cut to the true output size       -> out NCHW
+//
+// F(6,3) in fp32 amplifies single roundings to ~1e-5 of an O(1) output, the same size as the
+// parity tolerance, so this path reproduces the reference's arithmetic exactly instead of merely
+// approximating it:
+//   * every transform uses the reference's factoring AND its fused multiply-adds: the reference
+//     is built with gcc -O3 -mfma, whose default contraction fuses a*b+c patterns (in
+//     a*c1 - b*c2 it fuses the first product and rounds the second); those FMAs are written
+//     out explicitly here and the file is compiled with -ffp-contract=off;
+//   * the 64 small GEMMs accumulate like the reference's pack8/kernel_8x8 micro-kernel
+//     (src/kernels/cpu/math_cpu.cpp:386-700): one k-ascending FMA chain per output, and for
+//     columns beyond the last full block of 8 four interleaved chains combined as
+//     (s0+s1), (s2+s3), 0+s01, +s23.  They run on the vector ALUs -- the work is 4.4x smaller
+//     than the direct convolution and the fp32 MFMA would change the summation order.
+// All kernels here are memory/latency-bound elementwise or small-GEMM kernels.
+#include "tsx_common.hpp"
+
+namespace tsx {
+namespace {
+
+// ---------------------------------------------------------------- transforms (explicit FMAs)
+
+__device__ __forceinline__ void bt_row(const float *i0, float *o) {
+    // winograd_algorithm.cpp:640-663 (first pass over the rows of the patch)
+    o[0] = fmaf(i0[4] - i0[2], 5.25f, i0[0] - i0[6]);
+    o[7] = fmaf(i0[3] - i0[5], 5.25f, i0[7] - i0[1]);
+    const float tmp12_a = fmaf(-i0[4], 4.25f, i0[2] + i0[6]);
+    const float tmp12_b = fmaf(-i0[3], 4.25f, i0[1] + i0[5]);
+    o[1] = tmp12_a + tmp12_b;
+    o[2] = tmp12_a - tmp12_b;
+    const float tmp34_a = fmaf(-i0[4], 1.25f, fmaf(i0[2], 0.25f, i0[6]));
+    const float tmp34_b = fmaf(i0[5], 2.f, fmaf(i0[1], 0.5f, -(i0[3] * 2.5f)));
+    o[3] = tmp34_a + tmp34_b;
+    o[4] = tmp34_a - tmp34_b;
+    const float tmp56_a = fmaf(fmaf(-i0[4], 1.25f, i0[2]), 4.f, i0[6]);
+    const float tmp56_b = fmaf(i0[5], 0.5f, fmaf(i0[1], 2.f, -(i0[3] * 2.5f)));
+    o[5] = tmp56_a + tmp56_b;
+    o[6] = tmp56_a - tmp56_b;
+}
+
+__device__ __forceinline__ void bt_col(const float *d, float *o) {
+    // winograd_algorithm.cpp:668-692 (second pass; tmp12_b's operand order differs from the first)
+    o[0] = fmaf(d[4] - d[2], 5.25f, d[0] - d[6]);
+    o[7] = fmaf(d[3] - d[5], 5.25f, d[7] - d[1]);
+    const float tmp12_a = fmaf(-d[4], 4.25f, d[2] + d[6]);
+    const float tmp12_b = fmaf(-d[3], 4.25f, d[1]) + d[5];
+    o[1] = tmp12_a + tmp12_b;
+    o[2] = tmp12_a - tmp12_b;
+    const float tmp34_a = fmaf(-d[4], 1.25f, fmaf(d[2], 0.25f, d[6]));
+    const float tmp34_b = fmaf(d[5], 2.f, fmaf(d[1], 0.5f, -(d[3] * 2.5f)));
+    o[3] = tmp34_a + tmp34_b;
+    o[4] = tmp34_a - tmp34_b;
+    const float tmp56_a = fmaf(fmaf(-d[4], 1.25f, d[2]), 4.f, d[6]);
+    const float tmp56_b = fmaf(d[5], 0.5f, fmaf(d[1], 2.f, -(d[3] * 2.5f)));
+    o[5] = tmp56_a + tmp56_b;
+    o[6] = tmp56_a - tmp56_b;
+}
+
+__device__ __forceinline__ void at_pass(const float *t, float *o) {
+    // winograd_algorithm.cpp:775-795 / :808-830; every multiplier is a power of two, so fused
+    // and unfused forms round identically -- only the left-to-right order of the sums matters.
+    const float re0 = t[1] + t[2];
+    const float re1 = t[1] - t[2];
+    const float re2 = t[3] + t[4];
+    const float re3 = t[3] - t[4];
+    const float re4 = t[5] + t[6];
+    const float re5 = t[5] - t[6];
+    o[0] = t[0] + re0 + re2 + re4 * 32.f;
+    o[1] = re1 + re3 + re3 + re5 * 16.f;
+    o[2] = re0 + re2 * 4 + re4 * 8.f;
+    o[3] = re1 + re3 * 8 + re5 * 4.f;
+    o[4] = re0 + re2 * 16 + re4 + re4;
+    o[5] = re1 + re3 * 32 + re5 + t[7];
+}
+
+// U[t = i*8+j][cout][cin] = (G g G^T)[i][j]  (winograd_algorithm.cpp:504-566, before its pack8_A)
+__global__ __launch_bounds__(256) void wino_kernel_transform_kernel(const float *__restrict__ w, int cout, int cin,
+                                                                   float *__restrict__ u) {
+    const int id = blockIdx.x * blockDim.x + threadIdx.x;
+    if (id >= cout * cin) return;
+    const float G[8][3] = {{1.0f, 0.0f, 0.0f},
+                           {-2.f / 9, -2.f / 9, -2.f / 9},
+                           {-2.f / 9, 2.f / 9, -2.f / 9},
+                           {1.f / 90, 1.f / 45, 2.f / 45},
+                           {1.f / 90, -1.f / 45, 2.f / 45},
+                           {1.f / 45, 1.f / 90, 1.f / 180},
+                           {1.f / 45, -1.f / 90, 1.f / 180},
+                           {0.0f, 0.0f, 1.0f}};
+    float g[9];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) g[i] = w[int64_t(id) * 9 + i];
+    float tmp[3][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int r = 0; r < 3; ++r)
+            tmp[r][i] = fmaf(g[r * 3 + 2], G[i][2], fmaf(g[r * 3 + 0], G[i][0], g[r * 3 + 1] * G[i][1]));
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            u[int64_t(i * 8 + j) * cout * cin + id] =
+                fmaf(tmp[2][j], G[i][2], fmaf(tmp[0][j], G[i][0], tmp[1][j] * G[i][1]));
+}
+
+struct WinoGeom {
+    int n, c, h, w, cout, ho, wo, pad_top, pad_left, th, tw, tiles;
+    float padding_value;
+};
+
+// One thread per (image, channel, tile); adjacent lanes take adjacent tiles, so the 64 stores of a
+// lane (stride Cin*tiles) are coalesced across the wavefront.
+__global__ __launch_bounds__(256) void wino_input_transform_kernel(const float *__restrict__ x, WinoGeom g,
+                                                                  float *__restrict__ v) {
+    const int64_t total = int64_t(g.n) * g.c * g.tiles;
+    const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id >= total) return;
+    const int tile = int(id % g.tiles);
+    const int ch = int((id / g.tiles) % g.c);
+    const int img = int(id / g.tiles / g.c);
+    const int ty = tile / g.tw, tx = tile - ty * g.tw;
+    const float *src = x + (int64_t(img) * g.c + ch) * g.h * g.w;
+    float db[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        float row[8];
+        const int hh = ty * 6 + i - g.pad_top;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int ww = tx * 6 + j - g.pad_left;
+            // outside the tensor: the conv padding and the bottom/right fill both use padding_value
+            row[j] = (hh >= 0 && hh < g.h && ww >= 0 && ww < g.w) ? src[hh * g.w + ww] : g.padding_value;
+        }
+        bt_row(row, db[i]);
+    }
+    float *dst = v + (int64_t(img) * 64 * g.c + ch) * g.tiles + tile;
+    const int64_t stride = int64_t(g.c) * g.tiles;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        float col[8], o[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) col[r] = db[r][i];
+        bt_col(col, o);
+#pragma unroll
+        for (int r = 0; r < 8; ++r) dst[(r * 8 + i) * stride] = o[r];
+    }
+}
+
+// C[b][m][n] = A[b % 64][m][k] * B[b][k][n] in the reference's accumulation order
+// (math_cpu.cpp:386-700 as restated by the CPU oracle): m8/n8 = extents rounded down to 8.
+__global__ __launch_bounds__(256) void gemm_f32_seq_kernel(const float *__restrict__ a, const float *__restrict__ b,
+                                                          float *__restrict__ c, int m, int n, int k, int batches) {
+    const int64_t total = int64_t(batches) * m * n;
+    const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id >= total) return;
+    const int j = int(id % n);
+    const int i = int((id / n) % m);
+    const int bt = int(id / n / m);
+    const float *ar = a + (int64_t(bt % 64) * m + i) * k;
+    const float *bc = b + int64_t(bt) * k * n + j;
+    const int m8 = m / 8 * 8, n8 = n / 8 * 8, k4 = k / 4 * 4;
+    float r;
+    if (j < n8) {
+        float acc = 0.f;
+        for (int kk = 0; kk < k; ++kk) acc = fmaf(bc[int64_t(kk) * n], ar[kk], acc);
+        r = acc;
+    } else {
+        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+        for (int kk = 0; kk < k4; kk += 4) {
+            s0 = fmaf(ar[kk + 0], bc[int64_t(kk + 0) * n], s0);
+            s1 = fmaf(ar[kk + 1], bc[int64_t(kk + 1) * n], s1);
+            s2 = fmaf(ar[kk + 2], bc[int64_t(kk + 2) * n], s2);
+            s3 = fmaf(ar[kk + 3], bc[int64_t(kk + 3) * n], s3);
+        }
+        float acc;
+        if (i < m8) {
+            const float s01 = s0 + s1, s23 = s2 + s3;
+            acc = 0.f + s01;
+            acc = acc + s23;
+        } else {
+            acc = ((s0 + s1) + s2) + s3;
+        }
+        for (int kk = k4; kk < k; ++kk) acc = fmaf(ar[kk], bc[int64_t(kk) * n], acc);
+        r = acc;
+    }
+    c[id] = r;
+}
+
+// One thread per (image, cout, tile): Y = A^T M A, cut to the true output, then the optional
+// add_bias / activation that follow the convolution in the graph.
+__global__ __launch_bounds__(256) void wino_output_transform_kernel(const float *__restrict__ mm, WinoGeom g,
+                                                                   const float *__restrict__ bias, int act,
+                                                                   float slope, int64_t act_body,
+                                                                   float *__restrict__ out) {
+    const int64_t total = int64_t(g.n) * g.cout * g.tiles;
+    const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id >= total) return;
+    const int tile = int(id % g.tiles);
+    const int co = int((id / g.tiles) % g.cout);
+    const int img = int(id / g.tiles / g.cout);
+    const int ty = tile / g.tw, tx = tile - ty * g.tw;
+    const float *src = mm + (int64_t(img) * 64 * g.cout + co) * g.tiles + tile;
+    const int64_t stride = int64_t(g.cout) * g.tiles;
+    float tmpa[8][6];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        float t8[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) t8[j] = src[(i * 8 + j) * stride];
+        at_pass(t8, tmpa[i]);
+    }
+    const float bv = bias ? bias[co] : 0.f;
+    float *dst = out + (int64_t(img) * g.cout + co) * g.ho * g.wo;
+#pragma unroll
+    for (int i = 0; i < 6; ++i) {
+        float t8[8], o[6];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) t8[r] = tmpa[r][i];
+        at_pass(t8, o);
+        const int ww = tx * 6 + i;
+#pragma unroll
+        for (int r = 0; r < 6; ++r) {
+            const int hh = ty * 6 + r;
+            if (hh < g.ho && ww < g.wo) {
+                float val = o[r];
+                if (bias) val = __fadd_rn(val, bv);
+                const int64_t idx = (int64_t(img) * g.cout + co) * g.ho * g.wo + hh * g.wo + ww;
+                dst[hh * g.wo + ww] = apply_act(val, act, slope, idx < act_body);
+            }
+        }
+    }
+}
+
+int make_geom(const tsx_conv2d_geom *q, float padding_value, WinoGeom *g) {
+    TSX_REQUIRE(q, "winograd_f63: null geometry");
+    TSX_REQUIRE(q->kh == 3 && q->kw == 3 && q->stride_h == 1 && q->stride_w == 1 && q->dilation_h == 1 &&
+                    q->dilation_w == 1,
+                "winograd_f63: needs a 3x3 kernel with stride 1 and dilation 1");
+    TSX_REQUIRE(q->n > 0 && q->c > 0 && q->h > 0 && q->w > 0 && q->cout > 0, "winograd_f63: non-positive extent");
+    TSX_REQUIRE(q->pad_top >= 0 && q->pad_bottom >= 0 && q->pad_left >= 0 && q->pad_right >= 0,
+                "winograd_f63: negative padding is not supported");
+    g->n = q->n;
+    g->c = q->c;
+    g->h = q->h;
+    g->w = q->w;
+    g->cout = q->cout;
+    g->ho = q->h + q->pad_top + q->pad_bottom - 2;
+    g->wo = q->w + q->pad_left + q->pad_right - 2;
+    TSX_REQUIRE(g->ho > 0 && g->wo > 0, "winograd_f63: empty output %dx%d", g->ho, g->wo);
+    g->pad_top = q->pad_top;
+    g->pad_left = q->pad_left;
+    g->th = (g->ho + 5) / 6;
+    g->tw = (g->wo + 5) / 6;
+    g->tiles = g->th * g->tw;
+    g->padding_value = padding_value;
+    return 0;
+}
+
+}  // namespace
+}  // namespace tsx
+
+extern "C" {
+
+size_t tsx_winograd_f63_kernel_bytes(int32_t cout, int32_t cin) {
+    if (cout <= 0 || cin <= 0) return 0;
+    return size_t(64) * size_t(cout) * size_t(cin) * sizeof(float);
+}
+
+int tsx_winograd_f63_transform_kernel(int32_t cout, int32_t cin, const float *w_oihw_dev, float *u_dev, void *stream) {
+    TSX_REQUIRE(cout > 0 && cin > 0 && w_oihw_dev && u_dev, "winograd_f63_transform_kernel: bad argument");
+    const int total = cout * cin;
+    hipLaunchKernelGGL(tsx::wino_kernel_transform_kernel, dim3(unsigned(tsx::ceil_div(total, 256))), dim3(256), 0,
+                       tsx::as_stream(stream), w_oihw_dev, cout, cin, u_dev);
+    TSX_LAUNCH_CHECK("wino_kernel_transform_kernel");
+    return 0;
+}
+
+size_t tsx_winograd_f63_workspace_bytes(const tsx_conv2d_geom *q) {
+    tsx::WinoGeom g;
+    if (tsx::make_geom(q, 0.f, &g)) return 0;
+    return size_t(g.n) * 64 * g.tiles * (size_t(g.c) + size_t(g.cout)) * sizeof(float);
+}
+
+int tsx_conv2d_winograd_f63_nchw(const tsx_conv2d_geom *q, const float *x_dev, const float *u_dev, float padding_value,
+                                 const float *bias_dev, int32_t act, float slope, float *out_dev, void *workspace_dev,
+                                 size_t workspace_bytes, void *stream_) {
+    tsx::WinoGeom g;
+    int rc = tsx::make_geom(q, padding_value, &g);
+    if (rc) return rc;
+    TSX_REQUIRE(x_dev && u_dev && out_dev, "winograd_f63: null argument");
+    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_LEAKY_RELU, "winograd_f63: unknown activation %d", act);
+    const size_t need = tsx_winograd_f63_workspace_bytes(q);
+    if (!workspace_dev || workspace_bytes < need)
+        return tsx::fail(TSX_E_WORKSPACE, "winograd_f63: workspace %zu < %zu bytes", workspace_bytes, need);
+    hipStream_t stream = tsx::as_stream(stream_);
+    float *v = static_cast<float *>(workspace_dev);
+    float *mm = v + size_t(g.n) * 64 * g.c * g.tiles;
+
+    const int64_t in_threads = int64_t(g.n) * g.c * g.tiles;
+    hipLaunchKernelGGL(tsx::wino_input_transform_kernel, dim3(unsigned(tsx::ceil_div(in_threads, 256))), dim3(256), 0,
+                       stream, x_dev, g, v);
+    TSX_LAUNCH_CHECK("wino_input_transform_kernel");
+
+    const int batches = g.n * 64;
+    const int64_t gemm_threads = int64_t(batches) * g.cout * g.tiles;
+    hipLaunchKernelGGL(tsx::gemm_f32_seq_kernel, dim3(unsigned(tsx::ceil_div(gemm_threads, 256))), dim3(256), 0, stream,
+                       u_dev, v, mm, g.cout, g.tiles, g.c, batches);
+    TSX_LAUNCH_CHECK("gemm_f32_seq_kernel");
+
+    const int64_t out_threads = int64_t(g.n) * g.cout * g.tiles;
+    const int64_t count = int64_t(g.n) * g.cout * g.ho * g.wo;
+    hipLaunchKernelGGL(tsx::wino_output_transform_kernel, dim3(unsigned(tsx::ceil_div(out_threads, 256))), dim3(256), 0,
+                       stream, mm, g, bias_dev, act, slope, count / 4 * 4, out_dev);
+    TSX_LAUNCH_CHECK("wino_output_transform_kernel");
+    return 0;
+}
+
+}  // extern "C"

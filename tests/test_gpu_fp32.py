@@ -1,0 +1,133 @@
+"""GPU parity of the fp32 path (im2col-GEMM conv2d, inner_prod, Winograd F(6,3)) through the C ABI.
+
+Tolerance of the floating-point paths, from the path's contract: |gpu - ref| <= 1e-5 + 1e-4*|ref|
+(1e-4 relative / 1e-5 absolute).  Winograd additionally restates the reference's arithmetic
+operation for operation and is held to bit-exactness against the oracle."""
+import numpy as np
+import pytest
+
+from _util import bits
+
+pytestmark = pytest.mark.gpu
+
+REL, ABS = 1e-4, 1e-5
+
+
+def _close(a, b):
+    return np.all(np.abs(a.astype(np.float64) - b) <= ABS + REL * np.abs(b))
+
+
+@pytest.fixture(scope="module")
+def tsx():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from tennis_amd import capi
+    capi.lib()
+    return capi
+
+
+def _dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+CONV_CASES = [
+    # n, c, h, w, cout, kh, kw, pads(t,b,l,r), strides, dilations
+    (1, 8, 12, 12, 8, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),
+    (2, 5, 9, 7, 6, 3, 3, (0, 0, 0, 0), (2, 2), (1, 1)),
+    (2, 16, 8, 8, 8, 1, 1, (0, 0, 0, 0), (1, 1), (1, 1)),
+    (1, 3, 10, 11, 4, 3, 2, (2, 1, 0, 1), (1, 2), (2, 1)),
+    (3, 2, 7, 7, 7, 7, 7, (3, 3, 3, 3), (2, 2), (1, 1)),
+    (2, 70, 13, 9, 90, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),       # ragged in every GEMM dimension
+    (4, 128, 28, 28, 128, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),    # large enough for the 64x64 tiles
+    (1, 64, 56, 56, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),      # BASELINE config 1
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv2d_f32(tsx, port, case):
+    n, c, h, w, cout, kh, kw, pads, st, dl = case
+    rng = np.random.default_rng(400)
+    x = rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)
+    wt = (rng.standard_normal((cout, c, kh, kw)) * np.sqrt(2.0 / (c * kh * kw))).astype(np.float32)
+    got = tsx.conv2d_f32(_dev(x), _dev(wt), pads, st, dl).cpu().numpy()
+    exp = port.conv2d_f32(x, wt, pads, st, dl)
+    assert got.shape == exp.shape
+    assert _close(got, exp), np.abs(got - exp).max()
+
+
+def test_conv2d_f32_config1_bias_relu(tsx, port):
+    """BASELINE config 1: 1x64x56x56, 64x64x3x3 Kaiming-normal, bias N(0,0.01), s1 p1, then ReLU."""
+    rng = np.random.default_rng(1234)
+    x = rng.uniform(-1, 1, (1, 64, 56, 56)).astype(np.float32)
+    wt = (rng.standard_normal((64, 64, 3, 3)) * np.sqrt(2.0 / 576)).astype(np.float32)
+    bias = (rng.standard_normal(64) * 0.01).astype(np.float32)
+    got = tsx.conv2d_f32(_dev(x), _dev(wt), (1, 1, 1, 1), bias=_dev(bias), act="relu").cpu().numpy()
+    exp = port.relu(port.add_bias(port.conv2d_f32(x, wt, (1, 1, 1, 1)), bias))
+    assert _close(got, exp), np.abs(got - exp).max()
+    assert (got >= 0).all()
+
+
+def test_conv2d_f32_padding_value_and_exact_integers(tsx, port):
+    # small-integer data: every product and partial sum is exact in fp32, so any order gives equal bits
+    rng = np.random.default_rng(401)
+    x = rng.integers(-8, 9, (2, 6, 9, 10)).astype(np.float32)
+    wt = rng.integers(-4, 5, (5, 6, 3, 3)).astype(np.float32)
+    got = tsx.conv2d_f32(_dev(x), _dev(wt), (1, 2, 2, 1), (1, 1), (1, 1), padding_value=3.0).cpu().numpy()
+    exp = port.conv2d_f32(x, wt, (1, 2, 2, 1), padding_value=3.0)
+    assert np.array_equal(bits(got), bits(exp))
+
+
+@pytest.mark.parametrize("m,k,n", [(1, 64, 32), (3, 70, 33), (32, 1024, 1000), (130, 200, 260), (12, 2048, 1000)])
+@pytest.mark.parametrize("transpose", [False, True])
+def test_inner_prod_f32(tsx, port, m, k, n, transpose):
+    rng = np.random.default_rng(402)
+    lhs = rng.standard_normal((m, k)).astype(np.float32)
+    rhs = (rng.standard_normal((k, n)) * 0.05).astype(np.float32)
+    arg = np.ascontiguousarray(rhs.T) if transpose else rhs
+    got = tsx.inner_prod_f32(_dev(lhs), _dev(arg), transpose).cpu().numpy()
+    exp = port.inner_prod_f32(lhs, arg, transpose)
+    assert _close(got, exp), np.abs(got - exp).max()
+
+
+WINO_CASES = [
+    (1, 8, 12, 12, 8, (1, 1, 1, 1)),
+    (2, 16, 9, 11, 8, (1, 1, 1, 1)),
+    (1, 8, 10, 10, 16, (0, 0, 0, 0)),
+    (1, 5, 7, 7, 3, (2, 1, 1, 2)),
+    (2, 70, 20, 17, 36, (1, 1, 1, 1)),
+    (1, 64, 56, 56, 64, (1, 1, 1, 1)),      # BASELINE config 1 through F(6,3)
+]
+
+
+@pytest.mark.parametrize("case", WINO_CASES)
+def test_winograd_f63(tsx, port, case):
+    n, c, h, w, cout, pads = case
+    rng = np.random.default_rng(403)
+    x = rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)
+    wt = (rng.standard_normal((cout, c, 3, 3)) * np.sqrt(2.0 / (c * 9))).astype(np.float32)
+    op = tsx.WinogradF63(_dev(wt), pads)
+    got = op(_dev(x)).cpu().numpy()
+    exp = port.winograd_f63(x, wt, pads)
+    assert _close(got, exp), np.abs(got - exp).max()
+    # same operations in the same order as the reference's AVX2/FMA build: equal bits
+    assert np.array_equal(bits(got), bits(exp)), (bits(got) != bits(exp)).mean()
+
+
+def test_winograd_f63_padding_value_bias_relu(tsx, port):
+    rng = np.random.default_rng(404)
+    x = rng.uniform(-1, 1, (2, 8, 9, 9)).astype(np.float32)
+    wt = (rng.standard_normal((8, 8, 3, 3)) * 0.1).astype(np.float32)
+    bias = rng.standard_normal(8).astype(np.float32) * 0.1
+    op = tsx.WinogradF63(_dev(wt), (1, 1, 1, 1), padding_value=0.5)
+    got = op(_dev(x), bias=_dev(bias), act="relu").cpu().numpy()
+    exp = port.relu(port.add_bias(port.winograd_f63(x, wt, (1, 1, 1, 1), padding_value=0.5), bias))
+    assert np.array_equal(bits(got), bits(exp))
+
+
+def test_winograd_rejects_non_3x3(tsx):
+    import torch
+    with pytest.raises(tsx.TsxError):
+        op = tsx.WinogradF63(torch.zeros((4, 4, 3, 3), device="cuda"))
+        op.w = torch.zeros((4, 4, 5, 5), device="cuda")
+        op(torch.zeros((1, 4, 9, 9), device="cuda"))
