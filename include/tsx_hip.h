@@ -146,6 +146,17 @@ int tsx_conv2d_f32_nchw(const tsx_conv2d_geom *g, const float *x_dev, const floa
 int tsx_inner_prod_f32(int32_t m, int32_t n, int32_t k, const float *lhs_dev, const float *rhs_dev, int32_t transpose,
                        float *out_dev, void *stream);
 
+/* ---------------------------------------------------------------- stand-alone epilogue operators
+ * For graphs that keep them as separate nodes (HBM-bound: 4 B in + 4 B out per element).
+ *   tsx_add_bias_f32   cpu::AddBias   (src/kernels/cpu/add_bias.cpp:47-85): x is [pre][channels][inner]
+ *   tsx_relu_f32       cpu::ReLU      (src/kernels/cpu/relu.cpp:30-52)
+ *   tsx_leaky_relu_f32 cpu::LeakyReLU (src/kernels/cpu/leaky_relu.cpp:41-66)
+ * The activations reproduce the reference's SIMD-body / scalar-tail split (signed zero, NaN). */
+int tsx_add_bias_f32(const float *x_dev, int64_t pre, int32_t channels, int64_t inner, const float *bias_dev,
+                     float *out_dev, void *stream);
+int tsx_relu_f32(const float *x_dev, int64_t count, float *out_dev, void *stream);
+int tsx_leaky_relu_f32(const float *x_dev, int64_t count, float scale, float *out_dev, void *stream);
+
 /* ---------------------------------------------------------------- Winograd F(6x6, 3x3) fp32 conv2d
  * Conv2dWinogradAlgorithm<float>::winograd_f63 (src/kernels/cpu/winograd_algorithm.cpp:846-947),
  * reached in the reference through base::Conv2DWinograd's two core calls

@@ -1,0 +1,36 @@
+// The "hip" device of the backend: what TenniS's CUDA backend keeps in CUDAContextHandle
+// (include/kernels/gpu/cuda_context.h:13-43) minus the BLAS handle -- every kernel is hand-written.
+#pragma once
+#include "tsx_ts.h"
+
+namespace ts {
+namespace hip {
+
+static const char *const DEVICE = "hip";   // DeviceType holds at most 7 characters
+
+struct HipContextHandle {
+    void *stream = nullptr;   // hipStream_t of this DeviceContext
+    int device_id = 0;
+};
+
+// Stream of the DeviceContext bound to the calling thread (nullptr = default stream when an
+// operator is driven without a Workbench).
+void *current_stream();
+
+// Throws the reference's way (TS_LOG_ERROR << eject) when a C-ABI launcher reports an error
+// (include/kernels/gpu/gpu_kernel.h:13-19).
+void check(int tsx_rc, const char *what);
+
+template <typename OP>
+class OperatorOnHip : public OP {
+public:
+    MemoryDevice running_memory_device() override { return MemoryDevice(DEVICE, current_device_id()); }
+    static int current_device_id();
+};
+
+int context_device_id();
+template <typename OP>
+int OperatorOnHip<OP>::current_device_id() { return context_device_id(); }
+
+}  // namespace hip
+}  // namespace ts

@@ -1,0 +1,28 @@
+// Chooses the TenniS API the "hip" backend is compiled against: the real TenniS headers
+// (integration build, -DTSX_WITH_TENNIS with the TenniS include/ and src/ directories on the
+// include path) or this repository's self-contained restatement of the same interfaces.
+#pragma once
+#ifdef TSX_WITH_TENNIS
+#include <backend/base/base_add_bias.h>
+#include <backend/base/base_activation.h>
+#include <backend/base/base_conv2d.h>
+#include <backend/base/base_conv2d_quantized.h>
+#include <backend/base/base_conv2d_winograd.h>
+#include <backend/base/base_inner_prod.h>
+#include <backend/base/base_leaky_relu.h>
+#include <backend/base/base_quantize.h>
+#include <backend/name.h>
+#include <core/device_context.h>
+#include <core/tensor_builder.h>
+#include <global/hard_allocator.h>
+#include <global/hard_converter.h>
+#include <global/memory_device.h>
+#include <global/device_admin.h>
+#include <global/operator_factory.h>
+#include <runtime/stack.h>
+#include <utils/ctxmgr_lite.h>
+#include <utils/log.h>
+#else
+#include "../ts/base_ops.h"
+#include "../ts/ts_api.h"
+#endif

@@ -1,0 +1,402 @@
+// See base_ops.h.  Error conditions and messages follow the reference's skeletons so that a
+// graph which TenniS rejects at init()/infer() is rejected here for the same reason.
+#include "base_ops.h"
+
+namespace ts {
+namespace base {
+
+namespace {
+std::string list(const std::vector<int32_t> &a) {
+    std::ostringstream out;
+    out << "[";
+    for (size_t i = 0; i < a.size(); ++i) out << (i ? ", " : "") << a[i];
+    out << "]";
+    return out.str();
+}
+
+// RAII scratch frame: the core sees an empty stack and whatever it makes is dropped afterwards
+// (base_conv2d.cpp:195-204).
+struct ScratchFrame {
+    explicit ScratchFrame(Stack &s, int base) : stack(s) {
+        stack.push_base(base);
+        TS_AUTO_CHECK(stack.size() == 0);
+    }
+    ~ScratchFrame() {
+        stack.clear();
+        stack.pop_base();
+    }
+    Stack &stack;
+};
+}  // namespace
+
+// ---------------------------------------------------------------- quantize
+Quantize::Quantize() { field(name::quantize_scale, REQUIRED); }
+
+void Quantize::init() {
+    supper::init();
+    m_quantize_scales = tensor::array::to_float(get(name::quantize_scale));
+}
+
+int Quantize::infer(Stack &stack, std::vector<Tensor::Prototype> &output) {
+    TS_AUTO_CHECK(stack.size() == 1);
+    auto &x = stack[0];
+    TS_AUTO_CHECK(x.dims() >= 1);
+    // one scale per first-dimension slice
+    TS_AUTO_CHECK(int(m_quantize_scales.size()) == x.sizes()[0]);
+    output.resize(1);
+    output[0] = Tensor::Prototype(INT8, x.sizes());
+    return 1;
+}
+
+int Quantize::run(Stack &stack) {
+    std::vector<Tensor::Prototype> protos;
+    infer(stack, protos);
+    auto memory_device = running_memory_device();
+    auto x = stack[0].view(memory_device);
+    auto out = *stack.push(protos[0], memory_device);
+    quantize(x, m_quantize_scales, out);
+    return 1;
+}
+
+// ---------------------------------------------------------------- conv parameter block
+void Conv2DParams::declare_conv_fields(Operator &op, bool with_stride) {
+    op.field(name::format, Operator::REQUIRED);
+    op.field(name::padding, Operator::REQUIRED);
+    op.field(name::padding_value, Operator::OPTIONAL, tensor::from(0.0f));
+    if (with_stride) {
+        op.field(name::stride, Operator::REQUIRED);
+        op.field(name::dilation, Operator::OPTIONAL);
+        op.field(name::typo::dialations, Operator::OPTIONAL);
+    }
+}
+
+void Conv2DParams::parse_conv_fields(Operator &op, bool with_stride) {
+    auto format = tensor::to_string(op.get(name::format));
+    auto padding_tensor = tensor::cast(INT32, op.get(name::padding));
+    m_padding_value = tensor::to_float(op.get(name::padding_value));
+    TS_AUTO_CHECK(padding_tensor.has_shape({4, 2}));
+    if (format == name::NCHW) m_format = FORMAT_NCHW;
+    else if (format == name::NHWC) m_format = FORMAT_NHWC;
+    else TS_LOG_ERROR << op.op() << " do not support format: " << format << eject;
+    m_padding4x2 = tensor::array::to_int(padding_tensor);
+    m_stride4 = {1, 1, 1, 1};
+    m_dilation4 = {1, 1, 1, 1};
+    if (with_stride) {
+        auto stride_tensor = tensor::cast(INT32, op.get(name::stride));
+        Tensor dilation_tensor;
+        if (op.has(name::dilation)) dilation_tensor = tensor::cast(INT32, op.get(name::dilation));
+        else if (op.has(name::typo::dialations)) dilation_tensor = tensor::cast(INT32, op.get(name::typo::dialations));
+        if (dilation_tensor.empty())
+            TS_LOG_ERROR << op.op() << " must set " << name::dilation << " or " << name::typo::dialations << eject;
+        TS_AUTO_CHECK(stride_tensor.has_shape({4}));
+        TS_AUTO_CHECK(dilation_tensor.has_shape({4}));
+        m_stride4 = tensor::array::to_int(stride_tensor);
+        m_dilation4 = tensor::array::to_int(dilation_tensor);
+    }
+    // only the two spatial dimensions may be padded / strided / dilated
+    const int n = 0, c = m_format == FORMAT_NCHW ? 1 : 3;
+    if (m_padding4x2[2 * n] || m_padding4x2[2 * n + 1] || m_padding4x2[2 * c] || m_padding4x2[2 * c + 1])
+        TS_LOG_ERROR << op.op() << " do not support padding: " << list(m_padding4x2) << eject;
+    if (m_stride4[n] != 1 || m_stride4[c] != 1) TS_LOG_ERROR << op.op() << " do not support stride: " << list(m_stride4) << eject;
+    if (m_dilation4[n] != 1 || m_dilation4[c] != 1)
+        TS_LOG_ERROR << op.op() << " do not support dialations: " << list(m_dilation4) << eject;
+}
+
+Padding2D Conv2DParams::padding() const {
+    const int h = m_format == FORMAT_NCHW ? 2 : 1;
+    return Padding2D(m_padding4x2[2 * h], m_padding4x2[2 * h + 1], m_padding4x2[2 * h + 2], m_padding4x2[2 * h + 3]);
+}
+Stride2D Conv2DParams::stride() const {
+    const int h = m_format == FORMAT_NCHW ? 2 : 1;
+    return Stride2D(m_stride4[h], m_stride4[h + 1]);
+}
+Dilation2D Conv2DParams::dilation() const {
+    const int h = m_format == FORMAT_NCHW ? 2 : 1;
+    return Dilation2D(m_dilation4[h], m_dilation4[h + 1]);
+}
+
+namespace {
+Tensor::Prototype conv_out_proto(DTYPE dtype, Conv2DFormat format, const Tensor &x, const Tensor &w, const Padding2D &padding,
+                                 const Stride2D &stride, const Dilation2D &dilation) {
+    const bool nchw = format == FORMAT_NCHW;
+    Size2D xs(x.size(nchw ? 2 : 1), x.size(nchw ? 3 : 2));
+    KSize2D ks(w.size(nchw ? 2 : 1), w.size(nchw ? 3 : 2));
+    Size2D y = conv2d_forward(xs, padding, ks, stride, dilation);
+    if (nchw) return Tensor::Prototype(dtype, {x.size(0), w.size(0), y.height, y.width});
+    return Tensor::Prototype(dtype, {x.size(0), y.height, y.width, w.size(0)});
+}
+}  // namespace
+
+// ---------------------------------------------------------------- conv2d_quantized
+Conv2DQuantized::Conv2DQuantized() {
+    declare_conv_fields(*this, true);
+    field(name::dequantize_scales, REQUIRED);
+}
+
+void Conv2DQuantized::init() {
+    supper::init();
+    parse_conv_fields(*this, true);
+    m_dequantize_scales = tensor::array::to_float(get(name::dequantize_scales));
+}
+
+int Conv2DQuantized::infer(Stack &stack, std::vector<Tensor::Prototype> &output) {
+    TS_AUTO_CHECK(stack.size() == 2);
+    auto &x = stack[0];
+    auto &w = stack[1];
+    TS_AUTO_CHECK(x.dims() == 4);
+    TS_AUTO_CHECK(w.dims() == 4);
+    TS_AUTO_CHECK(x.dtype() == w.dtype());
+    TS_AUTO_CHECK(w.size(1) == x.size(1));
+    TS_AUTO_CHECK(x.dtype() == INT8);                                  // quantized input
+    TS_AUTO_CHECK(int(m_dequantize_scales.size()) == w.size(0));       // one scale per output channel
+    output.resize(1);
+    output[0] = conv_out_proto(FLOAT32, m_format, x, w, padding(), stride(), dilation());   // no requantize: fp32 out
+    return 1;
+}
+
+int Conv2DQuantized::run(Stack &stack) {
+    std::vector<Tensor::Prototype> protos;
+    infer(stack, protos);
+    auto memory_device = running_memory_device();
+    Tensor x = stack[0].view(memory_device);
+    Tensor w = stack[1].view(memory_device);
+    Tensor out = *stack.push(protos[0], memory_device);
+    {
+        ScratchFrame frame(stack, 3);
+        conv2d(x, padding(), m_padding_value, w, stride(), dilation(), m_format, m_dequantize_scales, out, stack);
+    }
+    return 1;
+}
+
+// ---------------------------------------------------------------- conv2d
+Conv2D::Conv2D() {
+    declare_conv_fields(*this, true);
+    field(name::kernel_packed, OPTIONAL, tensor::from<bool>(false));
+}
+
+void Conv2D::init() {
+    supper::init();
+    parse_conv_fields(*this, true);
+    if (has(name::kernel_packed)) m_kernel_packed = tensor::to_bool(get(name::kernel_packed));
+}
+
+int Conv2D::infer(Stack &stack, std::vector<Tensor::Prototype> &output) {
+    TS_AUTO_CHECK(stack.size() == 2);
+    auto &x = stack[0];
+    auto &w = stack[1];
+    TS_AUTO_CHECK(x.dims() == 4);
+    TS_AUTO_CHECK(w.dims() == 4);
+    TS_AUTO_CHECK(x.dtype() == w.dtype());
+    if (w.size(1) != x.size(1))
+        TS_LOG_ERROR << "Conv2D assert failed when x=" << to_string(x.sizes()) << ", w=" << to_string(w.sizes()) << eject;
+    output.resize(1);
+    output[0] = conv_out_proto(x.dtype(), m_format, x, w, padding(), stride(), dilation());
+    return 1;
+}
+
+int Conv2D::run(Stack &stack) {
+    std::vector<Tensor::Prototype> protos;
+    infer(stack, protos);
+    auto memory_device = running_memory_device();
+    Tensor x = stack[0].view(memory_device);
+    Tensor w = stack[1].view(memory_device);
+    Tensor out = *stack.push(protos[0], memory_device);
+    {
+        ScratchFrame frame(stack, 3);
+        conv2d(x, padding(), m_padding_value, w, stride(), dilation(), m_format, out, stack, m_kernel_packed);
+    }
+    return 1;
+}
+
+// ---------------------------------------------------------------- conv2d_winograd
+Conv2DWinograd::Conv2DWinograd() {
+    declare_conv_fields(*this, false);
+    field(name::kernel_winograd_transformed, OPTIONAL, tensor::from<bool>(false));
+}
+
+void Conv2DWinograd::init() {
+    supper::init();
+    parse_conv_fields(*this, false);
+    if (has(name::kernel_winograd_transformed)) m_kernel_transformed = tensor::to_bool(get(name::kernel_winograd_transformed));
+}
+
+int Conv2DWinograd::infer(Stack &stack, std::vector<Tensor::Prototype> &output) {
+    TS_AUTO_CHECK(stack.size() == 2);
+    auto &x = stack[0];
+    auto &k = stack[1];
+    TS_AUTO_CHECK(x.dims() == 4);
+    TS_AUTO_CHECK(k.dims() == 4);
+    const bool nchw = m_format == FORMAT_NCHW;
+    // 3x3, stride 1, dilation 1 whatever the kernel tensor's spatial extent says (it may hold
+    // a transformed kernel)
+    Size2D y = conv2d_forward(Size2D(x.size(nchw ? 2 : 1), x.size(nchw ? 3 : 2)), padding(), KSize2D(3, 3), Stride2D(1, 1),
+                              Dilation2D(1, 1));
+    output.resize(1);
+    if (nchw) output[0] = Tensor::Prototype(x.dtype(), {x.size(0), k.size(0), y.height, y.width});
+    else output[0] = Tensor::Prototype(x.dtype(), {x.size(0), y.height, y.width, k.size(0)});
+    return 1;
+}
+
+Shape Conv2DWinograd::transformed_kernel_shape(WinogradConv2DMode mode, const Tensor &kernel) {
+    const int tile = mode == F2X2_3X3 ? 4 : 8;
+    return Shape({kernel.size(0), kernel.size(1), tile, tile});
+}
+
+int Conv2DWinograd::run(Stack &stack) {
+    std::vector<Tensor::Prototype> protos;
+    infer(stack, protos);
+    auto memory_device = running_memory_device();
+    Tensor x = stack[0].view(memory_device);
+    Tensor kernel = stack[1].view(memory_device);
+    Tensor out = *stack.push(protos[0], memory_device);
+    // first run: pick the mode and transform the incoming (raw 3x3) weights; the cache is empty on
+    // the first run even when kernel_winograd_transformed was set (base_conv2d_winograd.cpp:146)
+    if (!m_kernel_transformed || m_k_transformed.empty()) {
+        // the reference selects F(6,3) only for Cin*Cout >= 256*256 on maps larger than 16x16 and
+        // F(2,3) otherwise (src/kernels/common/function.cpp:154-173); this backend implements the
+        // F(6,3) algorithm and uses it for every shape
+        m_winograd_mode = F6X6_3X3;
+        m_k_transformed = Tensor(memory_device, kernel.dtype(), transformed_kernel_shape(m_winograd_mode, kernel));
+        conv2d_tranform_kernel(m_winograd_mode, kernel, m_k_transformed);
+        m_kernel_transformed = true;
+    }
+    conv2d_winograd(x, m_winograd_mode, padding(), m_padding_value, m_k_transformed, m_format, out, m_kernel_transformed);
+    return 1;
+}
+
+// ---------------------------------------------------------------- inner_prod
+InnerProd::InnerProd() {
+    field("transpose", OPTIONAL, tensor::from<bool>(false));
+    field(name::kernel_packed, OPTIONAL, tensor::from<bool>(false));
+}
+
+void InnerProd::init() {
+    supper::init();
+    m_transpose = tensor::to_bool(get("transpose"));
+    if (has(name::kernel_packed)) m_kernel_packed = tensor::to_bool(get(name::kernel_packed));
+}
+
+namespace {
+void inner_prod_size(bool transpose, Tensor &lhs, const Tensor &rhs, std::vector<Tensor::Prototype> &output) {
+    if (lhs.dims() == 0) TS_LOG_ERROR << "InnerProd failed with LHS is scalar." << eject;
+    if (lhs.dims() != 2) lhs = lhs.reshape({lhs.size(0), -1});
+    const bool ok = rhs.dims() == 2 && lhs.size(1) == (transpose ? rhs.size(1) : rhs.size(0));
+    if (!ok)
+        TS_LOG_ERROR << "Can not inner-product between " << to_string(lhs.sizes()) << " and " << to_string(rhs.sizes())
+                     << (transpose ? "^T" : "") << eject;
+    TS_AUTO_CHECK(lhs.dtype() == rhs.dtype());
+    output.resize(1);
+    output[0] = Tensor::Prototype(lhs.dtype(), {lhs.size(0), transpose ? rhs.size(0) : rhs.size(1)});
+}
+}  // namespace
+
+int InnerProd::infer(Stack &stack, std::vector<Tensor::Prototype> &output) {
+    TS_AUTO_CHECK(stack.size() == 2);
+    auto lhs = stack[0];
+    inner_prod_size(m_transpose, lhs, stack[1], output);
+    return 1;
+}
+
+int InnerProd::run(Stack &stack) {
+    TS_AUTO_CHECK(stack.size() == 2);
+    std::vector<Tensor::Prototype> output;
+    auto lhs = stack[0];
+    auto rhs = stack[1];
+    inner_prod_size(m_transpose, lhs, rhs, output);
+    auto memory_device = running_memory_device();
+    lhs = lhs.view(memory_device);
+    rhs = rhs.view(memory_device);
+    auto &out = *stack.push(output[0], memory_device);
+    inner_prod(lhs, rhs, m_transpose, out, stack, m_kernel_packed);
+    return 1;
+}
+
+// ---------------------------------------------------------------- add_bias
+AddBias::AddBias() {
+    field(name::format, OPTIONAL);
+    field(name::dim, OPTIONAL);
+}
+
+void AddBias::init() {
+    supper::init();
+    const bool has_format = has(name::format), has_dim = has(name::dim);
+    TS_AUTO_CHECK(has_format || has_dim);
+    if (has_format) {
+        m_format = tensor::to_string(get(name::format));
+        TS_AUTO_CHECK(m_format == name::NCHW || m_format == name::NHWC);
+        m_dim = int(m_format.find('C'));
+    }
+    if (has_dim) m_dim = tensor::to_int(get(name::dim));
+    TS_AUTO_CHECK(m_dim >= 0);
+}
+
+bool AddBias::check_inputs(Stack &stack) const {
+    TS_AUTO_CHECK(stack.size() == 2);
+    auto &x = stack[0];
+    auto &b = stack[1];
+    TS_AUTO_CHECK(m_dim < int(x.dims()));
+    if (!b.has_shape(x.size(size_t(m_dim))))
+        TS_LOG_ERROR << "Miss matched: x:" << to_string(x.sizes()) << ", dim=" << m_dim << ", b:" << to_string(b.sizes()) << eject;
+    TS_AUTO_CHECK(x.dtype() == b.dtype());
+    return true;
+}
+
+int AddBias::infer(Stack &stack, std::vector<Tensor::Prototype> &output) {
+    check_inputs(stack);
+    output.resize(1);
+    output[0] = stack[0].proto();
+    return 1;
+}
+
+int AddBias::run(Stack &stack) {
+    check_inputs(stack);
+    auto memory_device = running_memory_device();
+    auto x = stack[0].view(memory_device);
+    auto b = stack[1].view(memory_device);
+    auto &out = *stack.push(x.proto(), memory_device);
+    add(x, b, m_dim, out);
+    return 1;
+}
+
+// ---------------------------------------------------------------- activations
+int Activation::infer(Stack &stack, std::vector<Tensor::Prototype> &output) {
+    TS_AUTO_CHECK(stack.size() == 1);
+    output.resize(1);
+    output[0] = stack[0].proto();
+    return 1;
+}
+
+int Activation::run(Stack &stack) {
+    TS_AUTO_CHECK(stack.size() == 1);
+    auto memory_device = running_memory_device();
+    auto x = stack[0].view(memory_device);
+    auto &out = *stack.push(x.proto(), memory_device);
+    active(x, out);
+    return 1;
+}
+
+LeakyReLU::LeakyReLU() { field(name::scale, REQUIRED); }
+
+void LeakyReLU::init() {
+    supper::init();
+    m_scale = tensor::to_float(get(name::scale));
+}
+
+int LeakyReLU::infer(Stack &stack, std::vector<Tensor::Prototype> &output) {
+    TS_AUTO_CHECK(stack.size() == 1);
+    output.resize(1);
+    output[0] = stack[0].proto();
+    return 1;
+}
+
+int LeakyReLU::run(Stack &stack) {
+    TS_AUTO_CHECK(stack.size() == 1);
+    auto memory_device = running_memory_device();
+    auto x = stack[0].view(memory_device);
+    auto &out = *stack.push(x.proto(), memory_device);
+    leaky_relu(x, m_scale, out);
+    return 1;
+}
+
+}  // namespace base
+}  // namespace ts

@@ -1,0 +1,155 @@
+// Device-agnostic operator skeletons of the hot path, restating the reference's
+// src/backend/base classes: parameter declaration and parsing in the constructor / init(),
+// shape inference in infer(), and run() = infer + view inputs on the running memory device +
+// push the output + call the pure-virtual device core.  A device backend overrides only the
+// core method and running_memory_device(), exactly as with TenniS's own skeletons:
+//   OperatorOnDevice      include/backend/base/operator_on_device.h:10-25
+//   base::Quantize        src/backend/base/base_quantize.cpp:12-50
+//   base::Conv2DQuantized src/backend/base/base_conv2d_quantized.cpp:13-219
+//   base::Conv2D          src/backend/base/base_conv2d.cpp:17-207
+//   base::Conv2DWinograd  src/backend/base/base_conv2d_winograd.cpp:15-169
+//   base::InnerProd       src/backend/base/base_inner_prod.cpp:14-93
+//   base::AddBias         src/backend/base/base_add_bias.cpp:15-90
+//   base::Activation      src/backend/base/base_activation.cpp (relu), base_leaky_relu.cpp
+#pragma once
+#include "ts_api.h"
+
+namespace ts {
+
+class OperatorOnDevice : public Operator {
+public:
+    // the memory device the core method's tensors live on
+    virtual MemoryDevice running_memory_device() = 0;
+};
+
+namespace base {
+
+class Quantize : public OperatorOnDevice {
+public:
+    using supper = OperatorOnDevice;
+    Quantize();
+    void init() override;
+    int run(Stack &stack) override;
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override;
+    virtual void quantize(const Tensor &x, std::vector<float> quantize_scales, Tensor &out) = 0;
+
+protected:
+    std::vector<float> m_quantize_scales;
+};
+
+// Shared parsing of format / padding / stride / dilation of the conv operators.
+class Conv2DParams {
+protected:
+    void declare_conv_fields(Operator &op, bool with_stride);
+    void parse_conv_fields(Operator &op, bool with_stride);
+    Padding2D padding() const;
+    Stride2D stride() const;
+    Dilation2D dilation() const;
+    Conv2DFormat m_format = FORMAT_NCHW;
+    std::vector<int32_t> m_padding4x2, m_stride4, m_dilation4;
+    float m_padding_value = 0;
+};
+
+class Conv2DQuantized : public OperatorOnDevice, protected Conv2DParams {
+public:
+    using supper = OperatorOnDevice;
+    Conv2DQuantized();
+    void init() override;
+    int run(Stack &stack) override;
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override;
+    virtual void conv2d(const Tensor &x, const Padding2D &padding, float padding_value, const Tensor &w,
+                        const Stride2D &stride, const Dilation2D &dilation, Conv2DFormat format,
+                        std::vector<float> dequantize_scale, Tensor &out, Stack &stack) = 0;
+
+protected:
+    std::vector<float> m_dequantize_scales;
+};
+
+class Conv2D : public OperatorOnDevice, protected Conv2DParams {
+public:
+    using supper = OperatorOnDevice;
+    Conv2D();
+    void init() override;
+    int run(Stack &stack) override;
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override;
+    virtual void conv2d(const Tensor &x, const Padding2D &padding, float padding_value, const Tensor &w,
+                        const Stride2D &stride, const Dilation2D &dilation, Conv2DFormat format, Tensor &out,
+                        Stack &stack, bool kernel_packed) = 0;
+
+protected:
+    bool m_kernel_packed = false;
+};
+
+class Conv2DWinograd : public OperatorOnDevice, protected Conv2DParams {
+public:
+    using supper = OperatorOnDevice;
+    Conv2DWinograd();
+    void init() override;
+    int run(Stack &stack) override;
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override;
+    virtual void conv2d_tranform_kernel(WinogradConv2DMode mode, const Tensor &kernel, Tensor &kernel_transformed) = 0;
+    virtual void conv2d_winograd(const Tensor &x, WinogradConv2DMode mode, const Padding2D &padding, float padding_value,
+                                 const Tensor &w, Conv2DFormat format, Tensor &out, bool kernel_transformed) = 0;
+    // shape of the device's transformed kernel for `kernel` (the reference allocates
+    // [cout, cin, 8, 8]; a backend is free to keep its own layout of the same size)
+    virtual Shape transformed_kernel_shape(WinogradConv2DMode mode, const Tensor &kernel);
+
+protected:
+    bool m_kernel_transformed = false;
+    WinogradConv2DMode m_winograd_mode = F6X6_3X3;
+    Tensor m_k_transformed;
+};
+
+class InnerProd : public OperatorOnDevice {
+public:
+    using supper = OperatorOnDevice;
+    InnerProd();
+    void init() override;
+    int run(Stack &stack) override;
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override;
+    virtual void inner_prod(const Tensor &lhs, const Tensor &rhs, bool transpose, Tensor &out, Stack &stack,
+                            bool kernel_packed) = 0;
+
+private:
+    bool m_transpose = false;
+    bool m_kernel_packed = false;
+};
+
+class AddBias : public OperatorOnDevice {
+public:
+    using supper = OperatorOnDevice;
+    AddBias();
+    void init() override;
+    int run(Stack &stack) override;
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override;
+    virtual void add(const Tensor &x, const Tensor &b, int dim, Tensor &out) = 0;
+
+private:
+    bool check_inputs(Stack &stack) const;
+    int m_dim = -1;
+    std::string m_format;
+};
+
+class Activation : public OperatorOnDevice {
+public:
+    using supper = OperatorOnDevice;
+    int run(Stack &stack) override;
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override;
+    virtual void active(const Tensor &x, Tensor &out) = 0;
+};
+
+class LeakyReLU : public OperatorOnDevice {
+public:
+    using supper = OperatorOnDevice;
+    LeakyReLU();
+    void init() override;
+    int run(Stack &stack) override;
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override;
+    virtual void leaky_relu(const Tensor &x, float scale, Tensor &out) = 0;
+
+private:
+    float m_scale = 0;
+};
+
+}  // namespace base
+}  // namespace ts

@@ -96,7 +96,27 @@ def build(verbose=True, jobs=8):
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
+    build_backend(verbose)
     return LIB_PATH
+
+
+BACKEND_DIR = os.path.join(HERE, "backend")
+BACKEND_LIB = os.path.join(LIB_DIR, "libtsx_backend.so")
+BACKEND_SOURCES = ["ts/ts_api.cpp", "ts/base_ops.cpp", "hip/hip_device.cpp", "hip/hip_operators.cpp", "capi_ops.cpp"]
+
+
+def build_backend(verbose=True):
+    """The C++ host side: TenniS-style operator classes for device "hip" over the C ABI (host code only;
+    linked against libtsx_hip.so and the HIP runtime)."""
+    cmd = [HIPCC, "-x", "c++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-D__HIP_PLATFORM_AMD__",
+           "-I" + os.path.join(ROOT, "include"), "-I/opt/rocm/include"]
+    cmd += [os.path.join(BACKEND_DIR, s) for s in BACKEND_SOURCES]
+    cmd += ["-o", BACKEND_LIB, "-L" + LIB_DIR, "-ltsx_hip", "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,$ORIGIN",
+            "-Wl,-rpath,/opt/rocm/lib"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return BACKEND_LIB
 
 
 if __name__ == "__main__":

@@ -64,6 +64,9 @@ SIGNATURES = {
     "tsx_gemm_i8": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, ctypes.POINTER(Epilogue), _vp, _vp, _vp, _vp, _sz, _vp]),
     "tsx_conv2d_f32_nchw": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, _f32, _vp, _i32, _f32, _vp, _vp]),
     "tsx_inner_prod_f32": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp]),
+    "tsx_add_bias_f32": (ctypes.c_int, [_vp, _i64, _i32, _i64, _vp, _vp, _vp]),
+    "tsx_relu_f32": (ctypes.c_int, [_vp, _i64, _vp, _vp]),
+    "tsx_leaky_relu_f32": (ctypes.c_int, [_vp, _i64, _f32, _vp, _vp]),
     "tsx_winograd_f63_kernel_bytes": (_sz, [_i32, _i32]),
     "tsx_winograd_f63_transform_kernel": (ctypes.c_int, [_i32, _i32, _vp, _vp, _vp]),
     "tsx_winograd_f63_workspace_bytes": (_sz, [ctypes.POINTER(ConvGeom)]),
@@ -290,3 +293,31 @@ class WinogradF63:
                                                  _ptr(bias), _ACT[act], float(slope), _ptr(out), _ptr(self._workspace),
                                                  nbytes, _stream()))
         return out
+
+
+def add_bias(x, bias, dim=1):
+    x = _dev(x, torch.float32)
+    bias = _dev(bias, torch.float32)
+    pre = 1
+    for d in x.shape[:dim]:
+        pre *= d
+    inner = 1
+    for d in x.shape[dim + 1:]:
+        inner *= d
+    out = torch.empty_like(x)
+    check(lib().tsx_add_bias_f32(_ptr(x), pre, x.shape[dim], inner, _ptr(bias), _ptr(out), _stream()))
+    return out
+
+
+def relu(x):
+    x = _dev(x, torch.float32)
+    out = torch.empty_like(x)
+    check(lib().tsx_relu_f32(_ptr(x), x.numel(), _ptr(out), _stream()))
+    return out
+
+
+def leaky_relu(x, scale):
+    x = _dev(x, torch.float32)
+    out = torch.empty_like(x)
+    check(lib().tsx_leaky_relu_f32(_ptr(x), x.numel(), float(scale), _ptr(out), _stream()))
+    return out

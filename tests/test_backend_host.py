@@ -1,0 +1,95 @@
+"""CPU-side checks of the boundary: the C-ABI library exports every symbol include/tsx_hip.h
+declares, the C++ operator layer registers the hot-path operators for device "hip", and its
+host logic (parameter checking, error behaviour) follows the reference.  No compute calls."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_c_abi_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "tsx_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(tsx_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 25
+    lib = ctypes.CDLL(os.path.join(ROOT, "tennis_amd", "lib", "libtsx_hip.so"))
+    missing = [name for name in sorted(declared) if not hasattr(lib, name)]
+    assert not missing, missing
+    from tennis_amd import capi
+    assert declared == set(capi.SIGNATURES), declared ^ set(capi.SIGNATURES)
+
+
+def test_argument_errors_need_no_device():
+    from tennis_amd import capi
+    L = capi.lib()
+    assert L.tsx_version() == 100
+    g = capi.ConvGeom(1, 8, 2, 2, 4, 3, 3, 0, 0, 0, 0, 1, 1, 1, 1)          # 3x3 on 2x2 without padding
+    assert L.tsx_conv2d_i8_workspace_bytes(ctypes.byref(g)) == 0
+    assert b"empty output" in L.tsx_last_error()
+    g = capi.ConvGeom(1, 8, 5, 5, 4, 3, 3, 1, 1, 1, 1, 0, 1, 1, 1)          # zero stride
+    assert L.tsx_conv2d_i8_packed_weight_bytes(ctypes.byref(g)) == 0
+    g = capi.ConvGeom(1, 8, 9, 9, 4, 5, 5, 1, 1, 1, 1, 1, 1, 1, 1)          # Winograd needs 3x3
+    assert L.tsx_winograd_f63_workspace_bytes(ctypes.byref(g)) == 0
+    assert L.tsx_quantize_f32_i8(None, -1, None, 1, None, None) == -1
+    # geometry bookkeeping of BASELINE config 2
+    g = capi.ConvGeom(32, 256, 28, 28, 256, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1)
+    assert L.tsx_conv2d_i8_workspace_bytes(ctypes.byref(g)) == 32 * 30 * 30 * 256
+    assert L.tsx_conv2d_i8_packed_weight_bytes(ctypes.byref(g)) == 256 * 256 * 9
+    ho, wo = capi.conv_out_size(g)
+    assert (ho, wo) == (28, 28)
+
+
+def test_hot_path_operators_are_registered_for_hip():
+    from tennis_amd import operators as ops
+    for name in ops.SYMBOLS:
+        assert hasattr(ops.lib(), name)
+    for op in ("quantize", "conv2d_quantized", "conv2d", "conv2d_winograd", "inner_prod", "add_bias", "relu", "leaky_relu"):
+        assert ops.is_registered("hip", op), op
+    assert not ops.is_registered("hip", "softmax")
+    assert not ops.is_registered("cpu", "conv2d")            # this library ships no host operators
+    with pytest.raises(ops.OperatorNotFound):
+        ops.check_params("softmax", {})                       # strict: no silent fallback
+
+
+def test_parameter_checking_follows_the_reference():
+    from tennis_amd import operators as ops
+    good = ops.conv_params((1, 1, 1, 1))
+    good["dequantize_scales"] = np.ones(4, np.float32)
+    ops.check_params("conv2d_quantized", good)
+    # required field missing (src/runtime/operator.cpp:174-193)
+    missing = dict(good)
+    del missing["dequantize_scales"]
+    with pytest.raises(ops.OperatorError, match="dequantize_scales"):
+        ops.check_params("conv2d_quantized", missing)
+    # unknown parameter names are rejected in strict mode (operator.cpp:26-38)
+    with pytest.raises(ops.OperatorError, match="Unidentified param"):
+        ops.check_params("conv2d_quantized", dict(good, quantize_scale=np.ones(1, np.float32)))
+    # the typo'd spelling of dilation is accepted, none at all is not (base_conv2d.cpp:51-60)
+    typo = dict(good)
+    typo["dialations"] = typo.pop("dilation")
+    ops.check_params("conv2d_quantized", typo)
+    none = dict(good)
+    del none["dilation"]
+    with pytest.raises(ops.OperatorError, match="must set dilation or dialations"):
+        ops.check_params("conv2d_quantized", none)
+    # padding / stride on batch or channel are refused
+    bad = dict(good, padding=np.array([[1, 0], [0, 0], [1, 1], [1, 1]], np.int32))
+    with pytest.raises(ops.OperatorError, match="do not support padding"):
+        ops.check_params("conv2d", {k: v for k, v in bad.items() if k != "dequantize_scales"})
+    bad = dict(good, stride=np.array([1, 2, 1, 1], np.int32))
+    with pytest.raises(ops.OperatorError, match="do not support stride"):
+        ops.check_params("conv2d_quantized", bad)
+    with pytest.raises(ops.OperatorError, match="do not support format"):
+        ops.check_params("conv2d_quantized", dict(good, format="NCDHW"))
+    with pytest.raises(ops.OperatorError):
+        ops.check_params("add_bias", {})                      # needs format or dim
+    ops.check_params("add_bias", {"dim": np.array([1], np.int32)})
+    ops.check_params("quantize", {"quantize_scale": np.ones(3, np.float32)})
+    with pytest.raises(ops.OperatorError, match="quantize_scale"):
+        ops.check_params("quantize", {})
+    with pytest.raises(ops.OperatorError, match="scale"):
+        ops.check_params("leaky_relu", {})

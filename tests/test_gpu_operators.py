@@ -1,0 +1,141 @@
+"""The C++ "hip" operators driven by name, like TenniS's operator test runner drives them
+(bench(device) -> create(op, params) -> run(inputs)), checked against the CPU oracle and -- where
+the compiled reference is present -- against the reference's own operator on device "cpu" given
+the very same parameters and inputs."""
+import numpy as np
+import pytest
+
+from _util import bits, c2_like
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from tennis_amd import operators
+    operators.lib()
+    return operators
+
+
+def _maybe_ref():
+    from oracle import ref as r
+    return r if r.available() else None
+
+
+def _close(a, b):
+    return np.all(np.abs(a.astype(np.float64) - b) <= 1e-5 + 1e-4 * np.abs(b))
+
+
+def test_quantize_operator(ops, port):
+    rng = np.random.default_rng(500)
+    for shape in [(1, 3, 7, 9), (4, 3, 7, 9), (32, 77)]:
+        x = (rng.standard_normal(shape) * 40).astype(np.float32)
+        x.ravel()[::3] = np.round(x.ravel()[::3]) + 0.5
+        s = rng.uniform(0.5, 2, shape[0]).astype(np.float32)
+        params = {"quantize_scale": s}
+        got = ops.run_op("quantize", params, [x])
+        assert got.dtype == np.int8 and got.shape == shape
+        assert np.array_equal(got, port.quantize(x, s))
+        ref = _maybe_ref()
+        if ref:
+            assert np.array_equal(got, ref.run_op("quantize", params, [x], x.size))
+    with pytest.raises(ops.OperatorError):        # one scale per batch item (base_quantize.cpp:26)
+        ops.run_op("quantize", {"quantize_scale": np.ones(3, np.float32)}, [np.zeros((2, 4), np.float32)])
+
+
+@pytest.mark.parametrize("case", [
+    (2, 8, 6, 6, 4, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),
+    (1, 5, 10, 9, 6, 3, 2, (2, 1, 0, 1), (1, 2), (2, 1)),
+    (2, 16, 5, 5, 8, 1, 1, (0, 0, 0, 0), (1, 1), (1, 1)),
+    (3, 64, 14, 14, 96, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),
+    (2, 3, 19, 19, 16, 7, 7, (3, 3, 3, 3), (2, 2), (1, 1)),
+])
+def test_conv2d_quantized_operator(ops, port, case):
+    n, c, h, w, cout, kh, kw, pads, st, dl = case
+    rng = np.random.default_rng(501)
+    x = rng.integers(-128, 128, (n, c, h, w)).astype(np.int8)
+    wt = rng.integers(-128, 128, (cout, c, kh, kw)).astype(np.int8)
+    params = ops.conv_params(pads, st, dl)
+    params["dequantize_scales"] = rng.uniform(1e-4, 1e-2, cout).astype(np.float32)
+    dtype, shape = ops.run_op("conv2d_quantized", params, [x, wt], infer_only=True)
+    got = ops.run_op("conv2d_quantized", params, [x, wt])
+    assert dtype == ops.FLOAT32 and tuple(shape) == got.shape          # no requantize: fp32 out
+    exp = port.conv2d_quantized(x, wt, params["dequantize_scales"], pads, st, dl)
+    assert np.array_equal(bits(got), bits(exp))
+    ref = _maybe_ref()
+    if ref:
+        r = ref.run_op("conv2d_quantized", params, [x, wt], got.nbytes, threads=1)
+        assert np.array_equal(bits(got), bits(r))
+
+
+def test_operator_chain_quantize_conv_bias_relu(ops, port):
+    """The graph fragment of BASELINE config 2 as four separate operators, small batch."""
+    rng = np.random.default_rng(502)
+    x, x_scales, wq, dq, bias = c2_like(rng, 3, 64, 14, 14, 64)
+    params = ops.conv_params((1, 1, 1, 1))
+    params["dequantize_scales"] = dq
+    xq = ops.run_op("quantize", {"quantize_scale": x_scales}, [x])
+    y = ops.run_op("conv2d_quantized", params, [xq, wq])
+    y = ops.run_op("add_bias", {"dim": np.array([1], np.int32)}, [y, bias])
+    y = ops.run_op("relu", {}, [y])
+    exp, _ = port.conv2d_i8_fused(port.quantize(x, x_scales), wq, dq, bias, "relu", pads=(1, 1, 1, 1))
+    assert np.array_equal(bits(y), bits(exp))
+    ref = _maybe_ref()
+    if ref:
+        r = ref.relu(ref.add_bias(ref.conv2d_quantized(ref.quantize(x, x_scales), wq, dq, pads=(1, 1, 1, 1)), bias))
+        assert np.array_equal(bits(y), bits(r))
+
+
+def test_conv2d_inner_prod_winograd_operators(ops, port):
+    rng = np.random.default_rng(503)
+    x = rng.uniform(-1, 1, (2, 16, 13, 11)).astype(np.float32)
+    wt = (rng.standard_normal((24, 16, 3, 3)) * 0.1).astype(np.float32)
+    params = ops.conv_params((1, 1, 1, 1))
+    got = ops.run_op("conv2d", params, [x, wt])
+    assert _close(got, port.conv2d_f32(x, wt, (1, 1, 1, 1)))
+    wparams = {k: params[k] for k in ("format", "padding", "padding_value")}
+    gotw = ops.run_op("conv2d_winograd", wparams, [x, wt])
+    assert np.array_equal(bits(gotw), bits(port.winograd_f63(x, wt, (1, 1, 1, 1))))
+    lhs = rng.standard_normal((5, 4, 6, 2)).astype(np.float32)          # flattened to [5, 48]
+    rhs = rng.standard_normal((48, 10)).astype(np.float32)
+    gotp = ops.run_op("inner_prod", {}, [lhs, rhs])
+    assert gotp.shape == (5, 10) and _close(gotp, port.inner_prod_f32(lhs.reshape(5, 48), rhs))
+    gott = ops.run_op("inner_prod", {"transpose": np.array([True])}, [lhs, np.ascontiguousarray(rhs.T)])
+    assert _close(gott, port.inner_prod_f32(lhs.reshape(5, 48), rhs))
+    ref = _maybe_ref()
+    if ref:
+        assert _close(got, ref.run_op("conv2d", params, [x, wt], got.nbytes))
+        assert _close(gotp, ref.run_op("inner_prod", {}, [lhs, rhs], gotp.nbytes))
+
+
+def test_elementwise_operators(ops, port):
+    rng = np.random.default_rng(504)
+    x = rng.standard_normal((2, 3, 5, 7)).astype(np.float32)
+    x.ravel()[:6] = [-1.0, -0.0, 0.0, np.nan, -1e-45, 2.0]
+    x.ravel()[-3:] = [-0.0, np.nan, -2.0]                               # 210 elements: last two are the scalar tail
+    b = rng.standard_normal(3).astype(np.float32)
+    assert np.array_equal(bits(ops.run_op("add_bias", {"format": "NCHW"}, [x, b])), bits(port.add_bias(x, b)))
+    assert np.array_equal(bits(ops.run_op("relu", {}, [x])), bits(port.relu(x)))
+    got = ops.run_op("leaky_relu", {"scale": np.array([0.1], np.float32)}, [x])
+    assert np.array_equal(bits(got), bits(port.leaky_relu(x, 0.1)))
+    ref = _maybe_ref()
+    if ref:
+        assert np.array_equal(bits(got), bits(ref.leaky_relu(x, 0.1)))
+    with pytest.raises(ops.OperatorError, match="Miss matched"):
+        ops.run_op("add_bias", {"dim": np.array([1], np.int32)}, [x, np.zeros(4, np.float32)])
+
+
+def test_operator_errors_at_run_time(ops):
+    params = ops.conv_params((1, 1, 1, 1))
+    params["dequantize_scales"] = np.ones(4, np.float32)
+    x = np.zeros((1, 8, 5, 5), np.int8)
+    with pytest.raises(ops.OperatorError):        # weight channels differ from input channels
+        ops.run_op("conv2d_quantized", params, [x, np.zeros((4, 7, 3, 3), np.int8)])
+    with pytest.raises(ops.OperatorError):        # one dequantize scale per output channel
+        ops.run_op("conv2d_quantized", params, [x, np.zeros((5, 8, 3, 3), np.int8)])
+    with pytest.raises(ops.OperatorError):        # input must be int8
+        ops.run_op("conv2d_quantized", params, [x.astype(np.float32), np.zeros((4, 8, 3, 3), np.float32)])
+    with pytest.raises(ops.OperatorNotFound):
+        ops.run_op("softmax", {}, [np.zeros((2, 2), np.float32)])
