@@ -90,6 +90,130 @@ __global__ __launch_bounds__(256) void stage_nchw_kernel(const void *__restrict_
     *reinterpret_cast<uint4 *>(xs + o) = make_uint4(words[0], words[1], words[2], words[3]);
 }
 
+// Row-at-a-time staging through LDS: one workgroup builds one staged row xs[n][hs][0..ws)[c0..c0+CG)
+// for a group of CG <= 256 channels.  Phase 1 reads the NCHW source coalesced along W (runs of
+// W elements per channel), quantizes (QUANT) and scatters bytes into an LDS tile [ws][CG+16]
+// pre-filled with the halo value; phase 2 writes the tile out as whole 16-byte chunks, a pixel's
+// channel group contiguous.  HBM traffic is exactly the algorithmic 4 B (or 1 B) read + 1 B
+// written per element; the older one-lane-per-chunk kernel remains for very wide rows.
+constexpr int STAGE_CG = 256;                 // channels per pass
+constexpr int STAGE_LROW = STAGE_CG + 16;     // LDS bytes per pixel: 16-byte aligned, bank-shifted
+constexpr int STAGE_MAX_WS = 232;             // ws * LROW <= 63 KiB
+
+template <bool QUANT>
+__global__ __launch_bounds__(256) void stage_rows_kernel(const void *__restrict__ src, StageGeom g,
+                                                        const float *__restrict__ scales, int n_scales,
+                                                        int64_t group_len, int64_t bulk8,
+                                                        int8_t *__restrict__ xs) {
+    extern __shared__ __attribute__((aligned(16))) int8_t tile[];   // [ws][STAGE_LROW]
+    const int tid = threadIdx.x;
+    const int hsi = blockIdx.x % g.hs, ni = blockIdx.x / g.hs;
+    const int hi = hsi - g.pad_top;
+    const bool row_inside = hi >= 0 && hi < g.h;
+    const uint32_t pad4 = uint32_t(g.pad_value & 0xff) * 0x01010101u;
+    // The scale group of element e is e / group_len (a 64-bit division).  With one scale, or one
+    // group per image (the usual case: the count divides evenly), it is uniform for this row.
+    const bool uniform_scale = QUANT && (n_scales == 1 || group_len == int64_t(g.c) * g.h * g.w);
+    const float row_scale = uniform_scale ? scales[n_scales == 1 ? 0 : ni] : 0.f;
+    for (int c0 = 0; c0 < g.cp; c0 += STAGE_CG) {
+        const int cg = min(STAGE_CG, g.cp - c0);        // multiple of 64
+        const int creal = max(0, min(cg, g.c - c0));    // channels that exist in the source
+        // pre-fill: halo value for real channels, zero for channel padding
+        for (int idx = tid; idx < g.ws * (cg / 4); idx += 256) {
+            const int pix = idx / (cg / 4), cw = idx - pix * (cg / 4);
+            uint32_t v = pad4;
+            if (cw * 4 + 4 > creal) {
+                v = 0;
+                for (int j = 0; j < 4; ++j)
+                    if (cw * 4 + j < creal) v |= uint32_t(g.pad_value & 0xff) << (8 * j);
+            }
+            *reinterpret_cast<uint32_t *>(&tile[pix * STAGE_LROW + cw * 4]) = v;
+        }
+        __syncthreads();
+        if (row_inside) {
+            // Lane = (w, channel quad): a lane loads the same pixel of 4 consecutive channels (each
+            // load coalesced along W across lanes), packs the 4 quantized bytes into one dword and
+            // writes it to the tile -- no byte-granular LDS traffic.  WL = power of two >= W keeps the
+            // mapping division-free; loads are issued in batches of NB quads before any is consumed.
+            int wl = 1, wl_shift = 0;
+            while (wl < g.w) {
+                wl <<= 1;
+                ++wl_shift;
+            }
+            if (wl <= 64) {
+                constexpr int NB = 4;
+                const int lane = tid & 63, wave = tid >> 6;
+                const int qpw = 64 >> wl_shift;                 // channel quads per wavefront per step
+                const int wi = lane & (wl - 1);
+                const int q_lane = wave * qpw + (lane >> wl_shift);
+                const int qstep = 4 * qpw;                      // quads per workgroup step
+                const bool lane_ok = wi < g.w;
+                const int64_t plane = int64_t(g.h) * g.w;
+                const int64_t row_base = (int64_t(ni) * g.c + c0) * plane + int64_t(hi) * g.w + wi;
+                const int quads = (creal + 3) / 4;
+                for (int qb = 0; qb < quads; qb += NB * qstep) {
+                    float fv[NB][4];
+                    int bv[NB][4];
+#pragma unroll
+                    for (int u = 0; u < NB; ++u) {
+                        const int c = (qb + u * qstep + q_lane) * 4;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const bool ok = lane_ok && c + j < creal;
+                            const int64_t e = row_base + int64_t(c + j) * plane;
+                            if (QUANT) fv[u][j] = ok ? static_cast<const float *>(src)[e] : 0.f;
+                            else bv[u][j] = ok ? static_cast<const int8_t *>(src)[e] : 0;
+                        }
+                    }
+#pragma unroll
+                    for (int u = 0; u < NB; ++u) {
+                        const int c = (qb + u * qstep + q_lane) * 4;
+                        if (!(lane_ok && c < creal)) continue;
+                        uint32_t word = 0;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            int q = 0;
+                            if (c + j < creal) {
+                                if (QUANT) {
+                                    const int64_t e = row_base + int64_t(c + j) * plane;
+                                    const float sc = uniform_scale ? row_scale : scales[e / group_len];
+                                    q = tsx::quantize_value(__fmul_rn(fv[u][j], sc), n_scales == 1 && e < bulk8);
+                                } else {
+                                    q = bv[u][j];
+                                }
+                            }
+                            word |= uint32_t(q & 0xff) << (8 * j);
+                        }
+                        *reinterpret_cast<uint32_t *>(&tile[(wi + g.pad_left) * STAGE_LROW + c]) = word;
+                    }
+                }
+            } else {
+                for (int idx = tid; idx < creal * g.w; idx += 256) {
+                    const int c = idx / g.w, wi = idx - c * g.w;
+                    const int64_t e = ((int64_t(ni) * g.c + c0 + c) * g.h + hi) * g.w + wi;
+                    int q;
+                    if (QUANT) {
+                        const float sc = uniform_scale ? row_scale : scales[e / group_len];
+                        q = tsx::quantize_value(__fmul_rn(static_cast<const float *>(src)[e], sc), n_scales == 1 && e < bulk8);
+                    } else {
+                        q = static_cast<const int8_t *>(src)[e];
+                    }
+                    tile[(wi + g.pad_left) * STAGE_LROW + c] = int8_t(q);
+                }
+            }
+        }
+        __syncthreads();
+        const int chunks = cg / 16;
+        int8_t *dst = xs + ((int64_t(ni) * g.hs + hsi) * g.ws) * g.cp + c0;
+        for (int idx = tid; idx < g.ws * chunks; idx += 256) {
+            const int pix = idx / chunks, ch = idx - pix * chunks;
+            *reinterpret_cast<v4i *>(dst + int64_t(pix) * g.cp + ch * 16) =
+                *reinterpret_cast<const v4i *>(&tile[pix * STAGE_LROW + ch * 16]);
+        }
+        __syncthreads();
+    }
+}
+
 // ------------------------------------------------------------------ weight packing
 
 // packed[ks][frag][half][lane][16]: ks = tap * cblocks + cb (tap = kh*KW + kw),
@@ -411,18 +535,30 @@ int run_stage(const tsx_conv2d_geom *g, const Plan &pl, const void *x, bool x_is
                  int(int8_t(padding_value))};  // T(padding_value), conv2d_quantized_core.cpp:72
     const int64_t stage_threads = int64_t(g->n) * pl.hs * pl.ws * (pl.cp / 16);
     const unsigned stage_blocks = unsigned(tsx::ceil_div(stage_threads, 256));
+    const bool by_rows = pl.ws <= STAGE_MAX_WS;
+    const unsigned row_blocks = unsigned(g->n) * unsigned(pl.hs);
+    const size_t row_lds = size_t(pl.ws) * STAGE_LROW;
     if (x_is_f32) {
         TSX_REQUIRE(x_scales && n_x_scales >= 1, "quantize_conv2d_i8: missing quantize scales");
         // base_quantize.cpp:26
         TSX_REQUIRE(n_x_scales == g->n, "quantize_conv2d_i8: n_x_scales (%d) must equal the batch (%d)", n_x_scales, g->n);
         const int64_t count = int64_t(g->n) * g->c * g->h * g->w;
         const int64_t group_len = int64_t(std::ceil(static_cast<float>(count) / static_cast<float>(n_x_scales)));
-        hipLaunchKernelGGL(stage_nchw_kernel<true>, dim3(stage_blocks), dim3(256), 0, stream, x, sg, x_scales,
-                           n_x_scales, group_len, (count >> 3) << 3, static_cast<int8_t *>(staged));
+        if (by_rows)
+            hipLaunchKernelGGL(stage_rows_kernel<true>, dim3(row_blocks), dim3(256), row_lds, stream, x, sg, x_scales,
+                               n_x_scales, group_len, (count >> 3) << 3, static_cast<int8_t *>(staged));
+        else
+            hipLaunchKernelGGL(stage_nchw_kernel<true>, dim3(stage_blocks), dim3(256), 0, stream, x, sg, x_scales,
+                               n_x_scales, group_len, (count >> 3) << 3, static_cast<int8_t *>(staged));
     } else {
-        hipLaunchKernelGGL(stage_nchw_kernel<false>, dim3(stage_blocks), dim3(256), 0, stream, x, sg,
-                           static_cast<const float *>(nullptr), 1, int64_t(1), int64_t(0),
-                           static_cast<int8_t *>(staged));
+        if (by_rows)
+            hipLaunchKernelGGL(stage_rows_kernel<false>, dim3(row_blocks), dim3(256), row_lds, stream, x, sg,
+                               static_cast<const float *>(nullptr), 1, int64_t(1), int64_t(0),
+                               static_cast<int8_t *>(staged));
+        else
+            hipLaunchKernelGGL(stage_nchw_kernel<false>, dim3(stage_blocks), dim3(256), 0, stream, x, sg,
+                               static_cast<const float *>(nullptr), 1, int64_t(1), int64_t(0),
+                               static_cast<int8_t *>(staged));
     }
     TSX_LAUNCH_CHECK("stage_nchw_kernel");
     return 0;
