@@ -155,6 +155,30 @@ def main():
     t_mfma = event_time(mfma_only, reps)
     t_stage = event_time(stage_only, reps)
 
+    # Same MFMA kernel with the requantized int8 output a following quantized layer would consume
+    # (quarter of the output bytes): reported beside the fp32-output figure, not instead of it.
+    qs = torch.full((cfg["n"],), 20.0, dtype=torch.float32, device=dev)
+    ep_q = capi._EpilogueArgs(torch.from_numpy(dq).to(dev), torch.from_numpy(bias).to(dev), "relu", q_scales=qs)
+    out_q = torch.empty((cfg["n"], cfg["cout"], ho, wo), dtype=torch.int8, device=dev)
+
+    def mfma_int8_out():
+        capi.check(L.tsx_conv2d_i8_staged(g, capi._ptr(ws), capi._ptr(packed), ctypes.byref(ep_q.c), None, capi._ptr(out_q),
+                                          None, stream))
+
+    t_mfma_q = event_time(mfma_int8_out, reps)
+
+    # The int8 MFMA rate this part sustains with operands of the same statistics (register-only loop):
+    # the practical ceiling below the nominal 5.0 POP/s.
+    operands = torch.randint(-128, 128, (32768,), dtype=torch.int8, device=dev)
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    probe_iters, probe_blocks = 20000, 512
+
+    def probe():
+        capi.check(L.tsx_probe_mfma_i8(capi._ptr(operands), probe_iters, probe_blocks, capi._ptr(sink), stream))
+
+    t_probe = event_time(probe, 3)
+    sustained_tops = probe_blocks * 4 * probe_iters * 8 * 65536.0 / t_probe / 1e12
+
     macs = cfg["n"] * cfg["cout"] * ho * wo * cfg["c"] * cfg["k"] * cfg["k"]
     ops = 2.0 * macs
     tops = ops / (ms_per_step * 1e-3) / 1e12
@@ -177,11 +201,16 @@ def main():
         "config": {"workload": "BASELINE config 2: int8 conv2d 32x256x28x28 * 256x256x3x3 s1 p1, fp32 dequant+bias+ReLU "
                                "out; step = quantize+stage kernel + i8-MFMA implicit-GEMM kernel",
                    "algorithmic_ops_per_step": ops, "pct_of_int8_mfma_peak_whole_step": 100.0 * tops / PEAK_INT8_TOPS},
-        "roofline": {"bound": "mfma", "kernel": "igemm_i8_kernel", "achieved": kernel_tops, "peak": PEAK_INT8_TOPS,
+        "roofline": {"bound": "mfma", "kernel": "conv_i8_ws_kernel", "achieved": kernel_tops, "peak": PEAK_INT8_TOPS,
                      "unit": "TFLOP/s", "frac": kernel_tops / PEAK_INT8_TOPS, "traffic": None,
                      "note": "int8 multiply-accumulate ops (TOP/s); 2*N*Cout*Ho*Wo*Cin*9 = %.4g ops per launch, "
                              "avg launch %.2f us over %d back-to-back launches" % (ops, t_mfma * 1e6, reps)},
-        "stage_kernel": {"bound": "hbm", "kernel": "stage_nchw_kernel<quantize>", "achieved": stage_bytes / t_stage / 1e9,
+        "sustained_mfma": {"value": sustained_tops, "unit": "TOPS", "frac_of_it": kernel_tops / sustained_tops,
+                           "note": "register-only v_mfma_i32_32x32x32_i8 loop on random int8 operands, measured in this "
+                                   "run: the rate the part sustains under load (clocks drop with operand activity)"},
+        "int8_output_variant": {"achieved": ops / t_mfma_q / 1e12, "unit": "TOPS", "us": t_mfma_q * 1e6,
+                                "note": "same kernel, epilogue requantizes to int8 for a following quantized layer"},
+        "stage_kernel": {"bound": "hbm", "kernel": "stage_rows_kernel<quantize>", "achieved": stage_bytes / t_stage / 1e9,
                          "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": stage_bytes / t_stage / 1e9 / PEAK_HBM_GBS,
                          "us": t_stage * 1e6, "bytes": stage_bytes},
     }

@@ -35,6 +35,13 @@ int tsx_version(void);
 /* Number of compute units of the current device (for launch heuristics and roofline peaks). */
 int tsx_device_cu_count(void);
 
+/* Diagnostic with no counterpart in the reference: launches `blocks` workgroups of 4 wavefronts, each
+ * issuing iters * 8 register-only v_mfma_i32_32x32x32_i8 (65536 ops each) on operands read once from
+ * operands_dev (32 KiB).  Timed by the caller, it gives the int8 MFMA rate this part sustains for the
+ * given operand data -- the practical ceiling of the contraction kernels (clocks drop under the power
+ * of random operands, so it is well below the nominal peak).  ops = blocks * 4 * iters * 8 * 65536. */
+int tsx_probe_mfma_i8(const void *operands_dev, int32_t iters, int32_t blocks, int32_t *sink_dev, void *stream);
+
 /* Geometry of one 2-D convolution, as base::Conv2D / base::Conv2DQuantized hand it to
  * their core: x [n,c,h,w], w [cout,c,kh,kw], Padding2D{top,bottom,left,right},
  * Stride2D, Dilation2D (include/backend/common_structure.h:10-62).  Output size follows

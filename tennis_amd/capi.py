@@ -46,6 +46,7 @@ SIGNATURES = {
     "tsx_last_error": (ctypes.c_char_p, []),
     "tsx_version": (ctypes.c_int, []),
     "tsx_device_cu_count": (ctypes.c_int, []),
+    "tsx_probe_mfma_i8": (ctypes.c_int, [_vp, _i32, _i32, _vp, _vp]),
     "tsx_conv2d_out_size": (ctypes.c_int, [ctypes.POINTER(ConvGeom), ctypes.POINTER(_i32), ctypes.POINTER(_i32)]),
     "tsx_quantize_f32_i8": (ctypes.c_int, [_vp, _i64, _vp, _i32, _vp, _vp]),
     "tsx_conv2d_i8_packed_weight_bytes": (_sz, [ctypes.POINTER(ConvGeom)]),

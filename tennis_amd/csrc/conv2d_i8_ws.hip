@@ -208,9 +208,14 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p) {
     const int tile_pos = p.th * p.wo;
     const int howo = p.ho * p.wo;
     const int64_t count = int64_t(gridDim.x / p.tiles_per_image) * p.cout * howo;
-    // hot case: fp32 output only, every element inside the activation's SIMD-body range, and
-    // a tensor small enough for 32-bit lane offsets
-    const bool fast = p.out_f32 && !p.out_i8 && !p.out_acc && p.act_body == count && count < (int64_t(1) << 30);
+    // hot case: no raw accumulators wanted, every element inside the activation's SIMD-body range,
+    // a tensor small enough for 32-bit lane offsets, and -- for the requantized output -- one
+    // quantize group per image (or a single scale whose round-half-even bulk covers everything),
+    // so the consumer's scale is uniform for this tile and needs no per-element division
+    const bool q_uniform = !p.out_i8 || (p.n_qscales == 1 ? p.q_bulk8 == count : p.q_group_len == int64_t(p.cout) * howo);
+    const bool fast = (p.out_f32 || p.out_i8) && !p.out_acc && p.act_body == count && count < (int64_t(1) << 30) && q_uniform;
+    const float q_scale = (fast && p.out_i8) ? p.q_scales[p.n_qscales == 1 ? 0 : img] : 0.f;
+    const bool q_even = p.n_qscales == 1;   // single-scale quantize rounds half to even in its bulk
     static_for<0, FM>([&](auto fc) {
         constexpr int f = decltype(fc)::value;
         const int cf = m0 + f * 32;   // first cout of this fragment (uniform)
@@ -229,7 +234,7 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p) {
             const bool pos_ok = pos < tile_pos && th0 + oh < p.ho;
             if (fast && cf + 32 <= p.cout) {
                 // uniform base in scalar registers + one 32-bit lane offset: no per-store address math
-                float *sbase = p.out_f32 + (int64_t(img) * p.cout + cf) * howo + int64_t(th0) * p.wo;
+                const int64_t tile_base = (int64_t(img) * p.cout + cf) * howo + int64_t(th0) * p.wo;
                 const unsigned lane_off = unsigned((4 * (lane / 32)) * howo + oh * p.wo + ow);
                 if (pos_ok) {
                     static_for<0, 16>([&](auto rc) {
@@ -237,7 +242,11 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p) {
                         constexpr int dco = 8 * (r / 4) + (r % 4);
                         float v = __fmul_rn(float(acc[f][j][r]), dq[r]);
                         if (p.bias) v = __fadd_rn(v, bias[r]);
-                        (sbase + int64_t(dco) * howo)[lane_off] = apply_act(v, p.act, p.slope, true);
+                        v = apply_act(v, p.act, p.slope, true);
+                        if (p.out_f32) (p.out_f32 + tile_base + int64_t(dco) * howo)[lane_off] = v;
+                        if (p.out_i8)
+                            (p.out_i8 + tile_base + int64_t(dco) * howo)[lane_off] =
+                                int8_t(quantize_value(__fmul_rn(v, q_scale), q_even));
                     });
                 }
             } else {
