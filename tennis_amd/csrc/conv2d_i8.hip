@@ -107,7 +107,13 @@ __global__ __launch_bounds__(256) void stage_rows_kernel(const void *__restrict_
                                                         int8_t *__restrict__ xs) {
     extern __shared__ __attribute__((aligned(16))) int8_t tile[];   // [ws][STAGE_LROW]
     const int tid = threadIdx.x;
-    const int hsi = blockIdx.x % g.hs, ni = blockIdx.x / g.hs;
+    // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Neighbouring rows of a
+    // channel plane share cache lines (a W-float run is rarely line-aligned), so give each XCD a
+    // contiguous run of rows: the shared lines are then fetched from HBM once, not once per XCD.
+    const unsigned total_rows = unsigned(g.n) * g.hs, per_xcd = (total_rows + 7) / 8;
+    const unsigned row_id = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (row_id >= total_rows) return;
+    const int hsi = row_id % g.hs, ni = row_id / g.hs;
     const int hi = hsi - g.pad_top;
     const bool row_inside = hi >= 0 && hi < g.h;
     const uint32_t pad4 = uint32_t(g.pad_value & 0xff) * 0x01010101u;
@@ -536,7 +542,7 @@ int run_stage(const tsx_conv2d_geom *g, const Plan &pl, const void *x, bool x_is
     const int64_t stage_threads = int64_t(g->n) * pl.hs * pl.ws * (pl.cp / 16);
     const unsigned stage_blocks = unsigned(tsx::ceil_div(stage_threads, 256));
     const bool by_rows = pl.ws <= STAGE_MAX_WS;
-    const unsigned row_blocks = unsigned(g->n) * unsigned(pl.hs);
+    const unsigned row_blocks = (unsigned(g->n) * unsigned(pl.hs) + 7) / 8 * 8;   // whole runs per XCD
     const size_t row_lds = size_t(pl.ws) * STAGE_LROW;
     if (x_is_f32) {
         TSX_REQUIRE(x_scales && n_x_scales >= 1, "quantize_conv2d_i8: missing quantize scales");
