@@ -182,6 +182,19 @@ int tsx_conv2d_winograd_f63_nchw(const tsx_conv2d_geom *g, const float *x_dev, c
                                  const float *bias_dev, int32_t act, float slope, float *out_dev, void *workspace_dev,
                                  size_t workspace_bytes, void *stream);
 
+/* ---------------------------------------------------------------- Winograd F(2x2, 3x3) fp32 conv2d
+ * Conv2dWinogradAlgorithm<float>::winograd_f23 (src/kernels/cpu/winograd_algorithm.cpp:347-459), the
+ * mode base::Conv2DWinograd picks unless Cin*Cout >= 256*256 on maps larger than 16x16
+ * (KernelCommonFunc::winograd_mode_select_on_arm, src/kernels/common/function.cpp:154-173).  Same
+ * contract as the F(6,3) calls above with 16 instead of 64 tile positions (u_dev is [16][cout][cin]);
+ * results match the reference's F(2,3) to the bit. */
+size_t tsx_winograd_f23_kernel_bytes(int32_t cout, int32_t cin);
+int tsx_winograd_f23_transform_kernel(int32_t cout, int32_t cin, const float *w_oihw_dev, float *u_dev, void *stream);
+size_t tsx_winograd_f23_workspace_bytes(const tsx_conv2d_geom *g);
+int tsx_conv2d_winograd_f23_nchw(const tsx_conv2d_geom *g, const float *x_dev, const float *u_dev, float padding_value,
+                                 const float *bias_dev, int32_t act, float slope, float *out_dev, void *workspace_dev,
+                                 size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

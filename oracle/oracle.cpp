@@ -13,8 +13,8 @@
 //   orc_add_bias/relu/leaky_relu  closed forms incl. signed-zero cases + compiled reference
 //   orc_epilogue / orc_conv2d_i8_fused / orc_gemm_i8_dequant   composition of the above
 //   orc_gemm_f32 / orc_conv2d_f32 / orc_inner_prod_f32  fp64 brute force (tolerance) +
-//                         compiled reference (bit-exact when M%8==0 && N%8==0)
-//   orc_winograd_f63      fp64 direct conv (tolerance) + compiled reference (tolerance 1e-5 abs)
+//                         compiled reference (bit-exact, remainder paths included)
+//   orc_winograd_f63 / orc_winograd_f23  fp64 direct conv (tolerance) + compiled reference (bit-exact)
 #include <algorithm>
 #include <cmath>
 #include <cstdint>
@@ -524,4 +524,96 @@ void orc_winograd_f63(const float *x, int n, int c, int h, int w, const float *w
     }
 }
 
+// ---------------------------------------------------------------------------
+// Winograd F(2,3): src/kernels/cpu/winograd_algorithm.cpp:57-459, the 4x4-tile twin of F(6,3)
+// (output rounded up to a multiple of 2, 16 GEMMs).  B^T and A^T hold only 0/+-1, so those
+// transforms are sums and differences written exactly as the reference groups them; the kernel
+// transform G (4x3, entries 0, 1, +-1/2) has the same a*g0 + b*g1 + c*g2 shape as F(6,3)'s and
+// is contracted by the reference's build the same way.
+// ---------------------------------------------------------------------------
+static void wino_f23_kernel(const float *g, float u[16]) {
+    static const float G[4][3] = {{1.f, 0.f, 0.f}, {0.5f, 0.5f, 0.5f}, {0.5f, -0.5f, 0.5f}, {0.f, 0.f, 1.f}};
+    float tmp[3][4];
+    for (int i = 0; i < 4; ++i)
+        for (int r = 0; r < 3; ++r)
+            tmp[r][i] = std::fmaf(g[r * 3 + 2], G[i][2], std::fmaf(g[r * 3 + 0], G[i][0], g[r * 3 + 1] * G[i][1]));
+    for (int i = 0; i < 4; ++i)
+        for (int j = 0; j < 4; ++j) u[i * 4 + j] = std::fmaf(tmp[2][j], G[i][2], std::fmaf(tmp[0][j], G[i][0], tmp[1][j] * G[i][1]));
+}
+
+void orc_winograd_f23(const float *x, int n, int c, int h, int w, const float *wt, int cout, int pt, int pb,
+                      int pl, int pr, float padding_value, float *out) {
+    const int ho = h + pt + pb - 2, wo = w + pl + pr - 2;
+    const int hop = (ho + 1) / 2 * 2, wop = (wo + 1) / 2 * 2;
+    const int hip = hop + 2, wip = wop + 2;
+    const int th = hop / 2, tw = wop / 2, tiles = th * tw;
+
+    std::vector<float> u(size_t(16) * cout * c);   // [16][Cout][Cin]
+#pragma omp parallel for num_threads(g_threads)
+    for (int p = 0; p < cout; ++p)
+        for (int q = 0; q < c; ++q) {
+            float tmp[16];
+            wino_f23_kernel(wt + (int64_t(p) * c + q) * 9, tmp);
+            for (int t = 0; t < 16; ++t) u[(size_t(t) * cout + p) * c + q] = tmp[t];
+        }
+
+    std::vector<float> xp(size_t(c) * hip * wip);
+    std::vector<float> v(size_t(16) * c * tiles);
+    std::vector<float> mm(size_t(16) * cout * tiles);
+    std::vector<float> yp(size_t(cout) * hop * wop);
+    for (int img = 0; img < n; ++img) {
+        std::fill(xp.begin(), xp.end(), padding_value);
+        for (int ch = 0; ch < c; ++ch)
+            for (int y = 0; y < h; ++y)
+                std::memcpy(&xp[(size_t(ch) * hip + y + pt) * wip + pl], x + ((int64_t(img) * c + ch) * h + y) * w,
+                            sizeof(float) * size_t(w));
+        // V = B^T d B (:181-243): rows first as (i_a -+ i_b), then the column combination
+#pragma omp parallel for num_threads(g_threads)
+        for (int ch = 0; ch < c; ++ch)
+            for (int ty = 0; ty < th; ++ty)
+                for (int tx = 0; tx < tw; ++tx) {
+                    const float *i0 = &xp[(size_t(ch) * hip + ty * 2) * wip + tx * 2];
+                    const float *i1 = i0 + wip, *i2 = i1 + wip, *i3 = i2 + wip;
+                    float r[4][4];   // r[k][j]: row combination k at column j
+                    for (int j = 0; j < 4; ++j) {
+                        r[0][j] = i0[j] - i2[j];
+                        r[1][j] = i1[j] + i2[j];
+                        r[2][j] = i2[j] - i1[j];
+                        r[3][j] = i1[j] - i3[j];
+                    }
+                    const int tile = ty * tw + tx;
+                    for (int k = 0; k < 4; ++k) {
+                        const float t[4] = {r[k][0] - r[k][2], r[k][1] + r[k][2], r[k][2] - r[k][1], r[k][1] - r[k][3]};
+                        for (int j = 0; j < 4; ++j) v[(size_t(k * 4 + j) * c + ch) * tiles + tile] = t[j];
+                    }
+                }
+        for (int t = 0; t < 16; ++t)
+            orc_gemm_f32(cout, tiles, c, &u[size_t(t) * cout * c], &v[size_t(t) * c * tiles],
+                         &mm[size_t(t) * cout * tiles]);
+        // Y = A^T M A (:262-330)
+#pragma omp parallel for num_threads(g_threads)
+        for (int p = 0; p < cout; ++p)
+            for (int ty = 0; ty < th; ++ty)
+                for (int tx = 0; tx < tw; ++tx) {
+                    const int tile = ty * tw + tx;
+                    float m[16], a[8];
+                    for (int t = 0; t < 16; ++t) m[t] = mm[(size_t(t) * cout + p) * tiles + tile];
+                    for (int k = 0; k < 4; ++k) {
+                        a[2 * k] = m[4 * k] + m[4 * k + 1] + m[4 * k + 2];
+                        a[2 * k + 1] = m[4 * k + 1] - m[4 * k + 2] - m[4 * k + 3];
+                    }
+                    float *o = &yp[(size_t(p) * hop + ty * 2) * wop + tx * 2];
+                    o[0] = a[0] + a[2] + a[4];
+                    o[1] = a[1] + a[3] + a[5];
+                    o[wop] = a[2] - a[4] - a[6];
+                    o[wop + 1] = a[3] - a[5] - a[7];
+                }
+        for (int p = 0; p < cout; ++p)
+            for (int y = 0; y < ho; ++y)
+                std::memcpy(out + ((int64_t(img) * cout + p) * ho + y) * wo, &yp[(size_t(p) * hop + y) * wop],
+                            sizeof(float) * size_t(wo));
+    }
+}
+
 }  // extern "C"
+

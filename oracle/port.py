@@ -44,6 +44,7 @@ def lib():
         L.orc_conv2d_f32.argtypes = [_vp, _i, _i, _i, _i, _vp] + [_i] * 11 + [_f, _vp]
         L.orc_inner_prod_f32.argtypes = [_vp, _i, _i, _vp, _i, _i, _vp]
         L.orc_winograd_f63.argtypes = [_vp, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _f, _vp]
+        L.orc_winograd_f23.argtypes = [_vp, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _f, _vp]
         _lib = L
     return _lib
 
@@ -229,4 +230,16 @@ def winograd_f63(x, w, pads, padding_value=0.0):
     ho, wo = out_hw(h, wd, 3, 3, pads, (1, 1), (1, 1))
     out = np.empty((n, cout, ho, wo), np.float32)
     lib().orc_winograd_f63(_p(x), n, c, h, wd, _p(w), cout, *pads, padding_value, _p(out))
+    return out
+
+
+def winograd_f23(x, w, pads, padding_value=0.0):
+    """Conv2dWinogradAlgorithm<float>::winograd_f23 (winograd_algorithm.cpp:347-459): 3x3, stride 1."""
+    x = _c(x, np.float32)
+    w = _c(w, np.float32)
+    n, c, h, wd = x.shape
+    cout = w.shape[0]
+    ho, wo = out_hw(h, wd, 3, 3, pads, (1, 1), (1, 1))
+    out = np.empty((n, cout, ho, wo), np.float32)
+    lib().orc_winograd_f23(_p(x), n, c, h, wd, _p(w), cout, *pads, padding_value, _p(out))
     return out

@@ -54,6 +54,43 @@ def _check(rc):
         raise RuntimeError("reference raised: " + lib().ref_last_error().decode(errors="replace"))
 
 
+# ---- the reference built WITH this repository's "hip" device backend inside it (ref.mk `intree`):
+# TenniS's own Workbench / Stack / Tensor / operator factory running the backend's operators.
+_INTREE_PATH = os.path.join(_HERE, "_ref", "libref_driver_hip.so")
+_intree = None
+
+
+def intree_available():
+    return os.path.exists(_INTREE_PATH)
+
+
+def intree_lib():
+    global _intree
+    if _intree is None:
+        if not intree_available():
+            raise RuntimeError("in-tree build absent: run `make -C oracle -f ref.mk intree`")
+        _intree = ctypes.CDLL(_INTREE_PATH)   # RTLD_LOCAL: its TenniS copy stays apart from lib()'s
+        _intree.ref_last_error.restype = ctypes.c_char_p
+    return _intree
+
+
+def run_op_intree(device, op, params, inputs, out_bytes, threads=1, strict=True):
+    """Run operator ``op`` in a TenniS Workbench on ``device`` ("cpu" or "hip") of the in-tree build."""
+    L = intree_lib()
+    keep = []
+    p = (_Tensor * max(len(params), 1))(*[_pack(k, v, keep) for k, v in params.items()])
+    i = (_Tensor * max(len(inputs), 1))(*[_pack("", v, keep) for v in inputs])
+    buf = np.empty(out_bytes, dtype=np.uint8)
+    out = _Output()
+    out.data = buf.ctypes.data
+    out.capacity = out_bytes
+    rc = L.ref_run_op_on(device.encode(), int(strict), op.encode(), len(params), p, len(inputs), i, int(threads), ctypes.byref(out))
+    if rc != 0:
+        raise RuntimeError("TenniS raised: " + L.ref_last_error().decode(errors="replace"))
+    shape = tuple(out.shape[k] for k in range(out.ndim))
+    return buf[:out.bytes].view(_TS2NP[out.dtype]).reshape(shape).copy()
+
+
 def _pack(name, value, keep):
     """Turn a python value into a _Tensor; ``keep`` holds the buffers alive."""
     if isinstance(value, str):

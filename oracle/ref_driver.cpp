@@ -16,6 +16,9 @@
 #include <vector>
 #include <memory>
 #include <exception>
+#include <map>
+#include <stdexcept>
+#include <dlfcn.h>
 
 #include "runtime/workbench.h"
 #include "module/bubble.h"
@@ -70,11 +73,12 @@ struct Bench {
     int threads = -1;
 };
 
-Bench &bench_for(int threads) {
-    static thread_local Bench b;
+Bench &bench_for(int threads, const std::string &device = ts::CPU) {
+    static thread_local std::map<std::string, Bench> benches;
+    Bench &b = benches[device];
     if (!b.bench) {
         ts::setup();
-        b.bench = std::make_shared<ts::Workbench>(ts::ComputingDevice(ts::CPU, 0));
+        b.bench = std::make_shared<ts::Workbench>(ts::ComputingDevice(device, 0));
     }
     if (b.threads != threads) {
         b.bench->runtime().set_computing_thread_number(threads);
@@ -113,15 +117,36 @@ int guarded(F f) {
 
 extern "C" {
 
+// Load a device plugin (a shared library whose static initialisers register operators and
+// device plumbing with this process's TenniS registries, e.g. the "hip" backend compiled
+// against the real TenniS headers).
+int ref_load_plugin(const char *path) {
+    return guarded([&] {
+        if (!dlopen(path, RTLD_NOW | RTLD_GLOBAL)) throw std::runtime_error(dlerror());
+    });
+}
+
+int ref_run_op_on(const char *device, int strict, const char *op, int nparams, const ref_tensor *params, int ninputs,
+                  const ref_tensor *inputs, int threads, ref_output *out);
+
 // Run one reference operator on the CPU device.  Returns 0 on success.
 int ref_run_op(const char *op, int nparams, const ref_tensor *params, int ninputs,
                const ref_tensor *inputs, int threads, ref_output *out) {
+    return ref_run_op_on(ts::CPU, 1, op, nparams, params, ninputs, inputs, threads, out);
+}
+
+// Same, on a Workbench of the named computing device: the operator is looked up the way the
+// runtime does it: strict = this device only; otherwise device -> its memory device -> cpu, the
+// order a compiled graph uses (src/global/operator_factory.cpp:60-81).
+int ref_run_op_on(const char *device, int strict, const char *op, int nparams, const ref_tensor *params, int ninputs,
+                  const ref_tensor *inputs, int threads, ref_output *out) {
     return guarded([&] {
-        Bench &b = bench_for(threads);
+        Bench &b = bench_for(threads, device);
         ts::ctx::bind<ts::RuntimeContext> bind_rt(b.bench->runtime());
         ts::Bubble bubble(op, op, 1);
         for (int i = 0; i < nparams; ++i) bubble.set(params[i].name, make_tensor(params[i]));
-        auto oper = b.bench->offline_create(bubble, true);
+        auto oper = b.bench->offline_create(bubble, strict != 0);
+        if (!oper) throw std::runtime_error(std::string("no operator ") + op);
         std::vector<ts::Tensor> in, res;
         for (int i = 0; i < ninputs; ++i) in.push_back(make_tensor(inputs[i]));
         b.bench->offline_run(oper, in, res);

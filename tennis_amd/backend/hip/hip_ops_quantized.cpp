@@ -1,0 +1,82 @@
+// The quantized "hip" device operators of the convolution hot path.  Each class inherits the
+// device-agnostic skeleton (parameter parsing, infer, run) and implements only the core method,
+// which hands raw device pointers to the C ABI in include/tsx_hip.h -- the structure of TenniS's
+// own device backends (src/kernels/cpu/quantize.cpp:147,
+// src/kernels/cpu/quantized/conv2d_quantized.cpp:7).
+//
+// Registered (device "hip"): quantize, conv2d_quantized.  They live in their own translation
+// unit because TenniS's base_conv2d_core.h and base_conv2d_quantized_core.h both define a
+// template named Conv2DWithCore and cannot be included together.
+#define TSX_TS_QUANTIZED_OPS
+#include "hip_ops_common.h"
+
+namespace ts {
+namespace hip {
+
+// ---------------------------------------------------------------- quantize
+class Quantize : public OperatorOnHip<base::Quantize> {
+public:
+    void quantize(const Tensor &x, std::vector<float> quantize_scales, Tensor &out) override {
+        if (x.dtype() != FLOAT32)
+            TS_LOG_ERROR << this->op() << " not support this data type: " << type_str(x.dtype()) << eject;
+        const float *scales = m_scales.get(quantize_scales, out.device());
+        check(tsx_quantize_f32_i8(x.data<float>(), x.count(), scales, int32_t(quantize_scales.size()), out.data<int8_t>(),
+                                  current_stream()),
+              "tsx_quantize_f32_i8");
+    }
+
+private:
+    DeviceFloats m_scales;
+};
+
+// ---------------------------------------------------------------- conv2d_quantized
+class Conv2DQuantized : public OperatorOnHip<base::Conv2DQuantized> {
+public:
+    void conv2d(const Tensor &x, const Padding2D &padding, float padding_value, const Tensor &w, const Stride2D &stride,
+                const Dilation2D &dilation, Conv2DFormat format, std::vector<float> dequantize_scale, Tensor &out,
+                Stack &stack) override {
+        if (format != FORMAT_NCHW) TS_LOG_ERROR << "Conv2D_quantized only support NCHW" << eject;
+        if (x.dtype() != INT8) TS_LOG_ERROR << "Conv2D_quantized not support this data type: " << type_str(x.dtype()) << eject;
+        const tsx_conv2d_geom g = make_geom(x, w, padding, stride, dilation);
+        void *stream = current_stream();
+        // Weights are constant graph data: pack them into MFMA operand tiles once per weight
+        // tensor and geometry, on first use (the pack translator leaves them unpacked for a
+        // device that registers its own operator).
+        const size_t packed_bytes = tsx_conv2d_i8_packed_weight_bytes(&g);
+        if (packed_bytes == 0) TS_LOG_ERROR << "[hip] conv2d_quantized: " << tsx_last_error() << eject;
+        if (m_packed.empty() || m_packed_from != w.data() || size_t(m_packed.count()) != packed_bytes || m_packed_cin != g.c) {
+            m_packed = Tensor(out.device(), INT8, Shape({int32_t(packed_bytes)}));
+            check(tsx_conv2d_i8_pack_weights(&g, w.data<int8_t>(), m_packed.data(), stream), "tsx_conv2d_i8_pack_weights");
+            m_packed_from = w.data();
+            m_packed_cin = g.c;
+        }
+        // staging scratch for the activations: kept across runs instead of taken from the stack's
+        // scratch frame, so the steady state allocates nothing
+        const size_t ws_bytes = tsx_conv2d_i8_workspace_bytes(&g);
+        if (m_workspace.empty() || size_t(m_workspace.count()) < ws_bytes || m_workspace.device() != out.device())
+            m_workspace = Tensor(out.device(), INT8, Shape({int32_t(ws_bytes ? ws_bytes : 16)}));
+        Tensor &workspace = m_workspace;
+        (void) stack;
+        tsx_epilogue ep{};
+        ep.dq_dev = m_dq.get(dequantize_scale, out.device());
+        ep.act = TSX_ACT_NONE;
+        check(tsx_conv2d_i8_nchw(&g, x.data<int8_t>(), m_packed.data(), padding_value, &ep, out.data<float>(), nullptr,
+                                 nullptr, workspace.data(), ws_bytes, stream),
+              "tsx_conv2d_i8_nchw");
+    }
+
+private:
+    Tensor m_packed;
+    Tensor m_workspace;
+    const void *m_packed_from = nullptr;
+    int m_packed_cin = 0;
+    DeviceFloats m_dq;
+};
+
+}  // namespace hip
+}  // namespace ts
+
+using namespace ts;
+using namespace ts::hip;
+TS_REGISTER_OPERATOR(Quantize, ts::hip::DEVICE, name::layer::quantize())
+TS_REGISTER_OPERATOR(Conv2DQuantized, ts::hip::DEVICE, name::layer::conv2d_quantized())

@@ -1,16 +1,23 @@
 // Chooses the TenniS API the "hip" backend is compiled against: the real TenniS headers
 // (integration build, -DTSX_WITH_TENNIS with the TenniS include/ and src/ directories on the
 // include path) or this repository's self-contained restatement of the same interfaces.
+// A translation unit defines TSX_TS_QUANTIZED_OPS or TSX_TS_FLOAT_OPS before including this to
+// get the operator skeletons it derives from (TenniS's two conv2d core headers clash).
 #pragma once
 #ifdef TSX_WITH_TENNIS
+#ifdef TSX_TS_QUANTIZED_OPS
+#include <backend/base/base_conv2d_quantized.h>
+#include <backend/base/base_quantize.h>
+#endif
+#ifdef TSX_TS_FLOAT_OPS
 #include <backend/base/base_add_bias.h>
 #include <backend/base/base_activation.h>
 #include <backend/base/base_conv2d.h>
-#include <backend/base/base_conv2d_quantized.h>
 #include <backend/base/base_conv2d_winograd.h>
 #include <backend/base/base_inner_prod.h>
 #include <backend/base/base_leaky_relu.h>
-#include <backend/base/base_quantize.h>
+#endif
+#include <backend/base/operator_on_device.h>
 #include <backend/name.h>
 #include <core/device_context.h>
 #include <core/tensor_builder.h>

@@ -237,9 +237,12 @@ int Conv2DWinograd::infer(Stack &stack, std::vector<Tensor::Prototype> &output) 
     return 1;
 }
 
-Shape Conv2DWinograd::transformed_kernel_shape(WinogradConv2DMode mode, const Tensor &kernel) {
-    const int tile = mode == F2X2_3X3 ? 4 : 8;
-    return Shape({kernel.size(0), kernel.size(1), tile, tile});
+// KernelCommonFunc<float>::winograd_mode_select_on_arm (src/kernels/common/function.cpp:154-173):
+// F(6,3) only for Cin*Cout >= 256*256 on maps larger than 16x16, F(2,3) otherwise.
+static WinogradConv2DMode select_winograd_mode(const Shape &input_shape, int out_channels) {
+    const int input_channels = input_shape[1], input_height = input_shape[2], input_width = input_shape[3];
+    if (input_channels * out_channels >= 256 * 256 && input_height > 16 && input_width > 16) return F6X6_3X3;
+    return F2X2_3X3;
 }
 
 int Conv2DWinograd::run(Stack &stack) {
@@ -249,14 +252,14 @@ int Conv2DWinograd::run(Stack &stack) {
     Tensor x = stack[0].view(memory_device);
     Tensor kernel = stack[1].view(memory_device);
     Tensor out = *stack.push(protos[0], memory_device);
-    // first run: pick the mode and transform the incoming (raw 3x3) weights; the cache is empty on
-    // the first run even when kernel_winograd_transformed was set (base_conv2d_winograd.cpp:146)
+    // first run: pick the mode and transform the incoming weights; the cache is empty on the first
+    // run even when kernel_winograd_transformed was set, and the transformed-kernel tensor is a HOST
+    // tensor whatever the device (base_conv2d_winograd.cpp:144-164) -- a device backend keeps its
+    // own transformed copy and treats this tensor as opaque
     if (!m_kernel_transformed || m_k_transformed.empty()) {
-        // the reference selects F(6,3) only for Cin*Cout >= 256*256 on maps larger than 16x16 and
-        // F(2,3) otherwise (src/kernels/common/function.cpp:154-173); this backend implements the
-        // F(6,3) algorithm and uses it for every shape
-        m_winograd_mode = F6X6_3X3;
-        m_k_transformed = Tensor(memory_device, kernel.dtype(), transformed_kernel_shape(m_winograd_mode, kernel));
+        m_winograd_mode = select_winograd_mode(x.sizes(), kernel.size(0));
+        const int tile = m_winograd_mode == F2X2_3X3 ? 4 : 8;
+        m_k_transformed = Tensor(MemoryDevice(CPU), kernel.dtype(), Shape({kernel.size(0), kernel.size(1), tile, tile}));
         conv2d_tranform_kernel(m_winograd_mode, kernel, m_k_transformed);
         m_kernel_transformed = true;
     }

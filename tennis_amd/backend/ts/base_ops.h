@@ -90,9 +90,6 @@ public:
     virtual void conv2d_tranform_kernel(WinogradConv2DMode mode, const Tensor &kernel, Tensor &kernel_transformed) = 0;
     virtual void conv2d_winograd(const Tensor &x, WinogradConv2DMode mode, const Padding2D &padding, float padding_value,
                                  const Tensor &w, Conv2DFormat format, Tensor &out, bool kernel_transformed) = 0;
-    // shape of the device's transformed kernel for `kernel` (the reference allocates
-    // [cout, cin, 8, 8]; a backend is free to keep its own layout of the same size)
-    virtual Shape transformed_kernel_shape(WinogradConv2DMode mode, const Tensor &kernel);
 
 protected:
     bool m_kernel_transformed = false;

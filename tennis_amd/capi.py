@@ -71,6 +71,11 @@ SIGNATURES = {
     "tsx_winograd_f63_kernel_bytes": (_sz, [_i32, _i32]),
     "tsx_winograd_f63_transform_kernel": (ctypes.c_int, [_i32, _i32, _vp, _vp, _vp]),
     "tsx_winograd_f63_workspace_bytes": (_sz, [ctypes.POINTER(ConvGeom)]),
+    "tsx_winograd_f23_kernel_bytes": (_sz, [_i32, _i32]),
+    "tsx_winograd_f23_transform_kernel": (ctypes.c_int, [_i32, _i32, _vp, _vp, _vp]),
+    "tsx_winograd_f23_workspace_bytes": (_sz, [ctypes.POINTER(ConvGeom)]),
+    "tsx_conv2d_winograd_f23_nchw": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, _f32, _vp, _i32, _f32, _vp, _vp,
+                                                    _sz, _vp]),
     "tsx_conv2d_winograd_f63_nchw": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, _f32, _vp, _i32, _f32, _vp, _vp,
                                                     _sz, _vp]),
 }
@@ -265,18 +270,24 @@ def inner_prod_f32(lhs, rhs, transpose=False):
     return out
 
 
-class WinogradF63:
-    """Winograd F(6,3) conv2d: the state of a `conv2d_winograd` operator instance (transformed kernel
-    cached at first use, base_conv2d_winograd.cpp:146-164)."""
+class Winograd:
+    """Winograd conv2d, mode "f63" or "f23": the state of a `conv2d_winograd` operator instance
+    (transformed kernel cached at first use, base_conv2d_winograd.cpp:146-164)."""
 
-    def __init__(self, w, pads=(0, 0, 0, 0), padding_value=0.0):
+    def __init__(self, w, pads=(0, 0, 0, 0), padding_value=0.0, mode="f63"):
+        assert mode in ("f63", "f23")
+        self.mode = mode
         self.w = _dev(w, torch.float32)
         self.pads = tuple(pads)
         self.padding_value = float(padding_value)
         cout, cin = self.w.shape[0], self.w.shape[1]
-        self.u = torch.empty(lib().tsx_winograd_f63_kernel_bytes(cout, cin) // 4, dtype=torch.float32,
-                             device=self.w.device)
-        check(lib().tsx_winograd_f63_transform_kernel(cout, cin, _ptr(self.w), _ptr(self.u), _stream()))
+        L = lib()
+        self._kernel_bytes = getattr(L, "tsx_winograd_%s_kernel_bytes" % mode)
+        self._transform = getattr(L, "tsx_winograd_%s_transform_kernel" % mode)
+        self._workspace_bytes = getattr(L, "tsx_winograd_%s_workspace_bytes" % mode)
+        self._conv = getattr(L, "tsx_conv2d_winograd_%s_nchw" % mode)
+        self.u = torch.empty(self._kernel_bytes(cout, cin) // 4, dtype=torch.float32, device=self.w.device)
+        check(self._transform(cout, cin, _ptr(self.w), _ptr(self.u), _stream()))
         self._workspace = None
 
     def __call__(self, x, bias=None, act=None, slope=0.0):
@@ -284,16 +295,25 @@ class WinogradF63:
         bias = _dev(bias, torch.float32)
         geom = make_geom(tuple(x.shape), tuple(self.w.shape), self.pads)
         ho, wo = conv_out_size(geom)
-        nbytes = lib().tsx_winograd_f63_workspace_bytes(ctypes.byref(geom))
+        nbytes = self._workspace_bytes(ctypes.byref(geom))
         if nbytes == 0:
             raise TsxError("winograd: " + lib().tsx_last_error().decode())
         if self._workspace is None or self._workspace.numel() < nbytes:
             self._workspace = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
         out = torch.empty((x.shape[0], self.w.shape[0], ho, wo), dtype=torch.float32, device=x.device)
-        check(lib().tsx_conv2d_winograd_f63_nchw(ctypes.byref(geom), _ptr(x), _ptr(self.u), self.padding_value,
-                                                 _ptr(bias), _ACT[act], float(slope), _ptr(out), _ptr(self._workspace),
-                                                 nbytes, _stream()))
+        check(self._conv(ctypes.byref(geom), _ptr(x), _ptr(self.u), self.padding_value, _ptr(bias), _ACT[act],
+                         float(slope), _ptr(out), _ptr(self._workspace), nbytes, _stream()))
         return out
+
+
+class WinogradF63(Winograd):
+    def __init__(self, w, pads=(0, 0, 0, 0), padding_value=0.0):
+        super().__init__(w, pads, padding_value, "f63")
+
+
+class WinogradF23(Winograd):
+    def __init__(self, w, pads=(0, 0, 0, 0), padding_value=0.0):
+        super().__init__(w, pads, padding_value, "f23")
 
 
 def add_bias(x, bias, dim=1):

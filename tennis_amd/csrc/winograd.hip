@@ -1,7 +1,9 @@
-// Winograd F(6x6, 3x3) fp32 convolution, restating
-// Conv2dWinogradAlgorithm<float>::winograd_f63 (src/kernels/cpu/winograd_algorithm.cpp:504-947)
-// with the padding rule of KernelCommonFunc::in_out_pad_and_fix_size
-// (src/kernels/common/function.cpp:14-78).
+// Winograd F(6x6, 3x3) and F(2x2, 3x3) fp32 convolution, restating
+// Conv2dWinogradAlgorithm<float>::winograd_f63 / winograd_f23
+// (src/kernels/cpu/winograd_algorithm.cpp:504-947 / :57-459) with the padding rule of
+// KernelCommonFunc::in_out_pad_and_fix_size (src/kernels/common/function.cpp:14-78).
+// F(6,3) is described below; F(2,3) is its twin with 4x4 patches (stride 2), 16 GEMMs and
+// transforms made of sums and differences only.
 //
 //   U = G g G^T      kernel transform, once per weight tensor          -> u[64][Cout][Cin]
 //   V = B^T d B      input transform of every 8x8 patch (stride 6)      -> v[N][64][Cin][tiles]
@@ -154,17 +156,18 @@ __global__ __launch_bounds__(256) void wino_input_transform_kernel(const float *
     }
 }
 
-// C[b][m][n] = A[b % 64][m][k] * B[b][k][n] in the reference's accumulation order
+// C[b][m][n] = A[b % a_batches][m][k] * B[b][k][n] in the reference's accumulation order
 // (math_cpu.cpp:386-700 as restated by the CPU oracle): m8/n8 = extents rounded down to 8.
 __global__ __launch_bounds__(256) void gemm_f32_seq_kernel(const float *__restrict__ a, const float *__restrict__ b,
-                                                          float *__restrict__ c, int m, int n, int k, int batches) {
+                                                          float *__restrict__ c, int m, int n, int k, int batches,
+                                                          int a_batches) {
     const int64_t total = int64_t(batches) * m * n;
     const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
     if (id >= total) return;
     const int j = int(id % n);
     const int i = int((id / n) % m);
     const int bt = int(id / n / m);
-    const float *ar = a + (int64_t(bt % 64) * m + i) * k;
+    const float *ar = a + (int64_t(bt % a_batches) * m + i) * k;
     const float *bc = b + int64_t(bt) * k * n + j;
     const int m8 = m / 8 * 8, n8 = n / 8 * 8, k4 = k / 4 * 4;
     float r;
@@ -239,14 +242,123 @@ __global__ __launch_bounds__(256) void wino_output_transform_kernel(const float 
     }
 }
 
-int make_geom(const tsx_conv2d_geom *q, float padding_value, WinoGeom *g) {
-    TSX_REQUIRE(q, "winograd_f63: null geometry");
+// ---------------------------------------------------------------- F(2,3)
+
+// U[t = i*4+j][cout][cin] = (G g G^T)[i][j], G = {1,0,0; 1/2,1/2,1/2; 1/2,-1/2,1/2; 0,0,1}
+// (winograd_algorithm.cpp:57-105, before its pack8_A); same contraction as the F(6,3) transform.
+__global__ __launch_bounds__(256) void wino23_kernel_transform_kernel(const float *__restrict__ w, int cout, int cin,
+                                                                     float *__restrict__ u) {
+    const int id = blockIdx.x * blockDim.x + threadIdx.x;
+    if (id >= cout * cin) return;
+    const float G[4][3] = {{1.f, 0.f, 0.f}, {0.5f, 0.5f, 0.5f}, {0.5f, -0.5f, 0.5f}, {0.f, 0.f, 1.f}};
+    float g[9];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) g[i] = w[int64_t(id) * 9 + i];
+    float tmp[3][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 3; ++r)
+            tmp[r][i] = fmaf(g[r * 3 + 2], G[i][2], fmaf(g[r * 3 + 0], G[i][0], g[r * 3 + 1] * G[i][1]));
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            u[int64_t(i * 4 + j) * cout * cin + id] =
+                fmaf(tmp[2][j], G[i][2], fmaf(tmp[0][j], G[i][0], tmp[1][j] * G[i][1]));
+}
+
+// V = B^T d B (winograd_algorithm.cpp:181-243): row combinations (i0-i2, i1+i2, i2-i1, i1-i3) first,
+// then the same combination across columns, in the reference's grouping.
+__global__ __launch_bounds__(256) void wino23_input_transform_kernel(const float *__restrict__ x, WinoGeom g,
+                                                                    float *__restrict__ v) {
+    const int64_t total = int64_t(g.n) * g.c * g.tiles;
+    const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id >= total) return;
+    const int tile = int(id % g.tiles);
+    const int ch = int((id / g.tiles) % g.c);
+    const int img = int(id / g.tiles / g.c);
+    const int ty = tile / g.tw, tx = tile - ty * g.tw;
+    const float *src = x + (int64_t(img) * g.c + ch) * g.h * g.w;
+    float d[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int hh = ty * 2 + i - g.pad_top;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int ww = tx * 2 + j - g.pad_left;
+            d[i][j] = (hh >= 0 && hh < g.h && ww >= 0 && ww < g.w) ? src[hh * g.w + ww] : g.padding_value;
+        }
+    }
+    float *dst = v + (int64_t(img) * 16 * g.c + ch) * g.tiles + tile;
+    const int64_t stride = int64_t(g.c) * g.tiles;
+    float r[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        r[0][j] = d[0][j] - d[2][j];
+        r[1][j] = d[1][j] + d[2][j];
+        r[2][j] = d[2][j] - d[1][j];
+        r[3][j] = d[1][j] - d[3][j];
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        dst[(k * 4 + 0) * stride] = r[k][0] - r[k][2];
+        dst[(k * 4 + 1) * stride] = r[k][1] + r[k][2];
+        dst[(k * 4 + 2) * stride] = r[k][2] - r[k][1];
+        dst[(k * 4 + 3) * stride] = r[k][1] - r[k][3];
+    }
+}
+
+// Y = A^T M A (winograd_algorithm.cpp:262-330), cut to the true output, + optional bias / activation.
+__global__ __launch_bounds__(256) void wino23_output_transform_kernel(const float *__restrict__ mm, WinoGeom g,
+                                                                     const float *__restrict__ bias, int act,
+                                                                     float slope, int64_t act_body,
+                                                                     float *__restrict__ out) {
+    const int64_t total = int64_t(g.n) * g.cout * g.tiles;
+    const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id >= total) return;
+    const int tile = int(id % g.tiles);
+    const int co = int((id / g.tiles) % g.cout);
+    const int img = int(id / g.tiles / g.cout);
+    const int ty = tile / g.tw, tx = tile - ty * g.tw;
+    const float *src = mm + (int64_t(img) * 16 * g.cout + co) * g.tiles + tile;
+    const int64_t stride = int64_t(g.cout) * g.tiles;
+    float m[16], a[8], o[4];
+#pragma unroll
+    for (int t = 0; t < 16; ++t) m[t] = src[t * stride];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        a[2 * k] = m[4 * k] + m[4 * k + 1] + m[4 * k + 2];
+        a[2 * k + 1] = m[4 * k + 1] - m[4 * k + 2] - m[4 * k + 3];
+    }
+    o[0] = a[0] + a[2] + a[4];
+    o[1] = a[1] + a[3] + a[5];
+    o[2] = a[2] - a[4] - a[6];
+    o[3] = a[3] - a[5] - a[7];
+    const float bv = bias ? bias[co] : 0.f;
+    const int64_t plane = (int64_t(img) * g.cout + co) * g.ho * g.wo;
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int hh = ty * 2 + r, ww = tx * 2 + i;
+            if (hh < g.ho && ww < g.wo) {
+                float val = o[r * 2 + i];
+                if (bias) val = __fadd_rn(val, bv);
+                const int64_t idx = plane + hh * g.wo + ww;
+                out[idx] = apply_act(val, act, slope, idx < act_body);
+            }
+        }
+}
+
+int make_geom(const tsx_conv2d_geom *q, float padding_value, WinoGeom *g, int tile = 6) {
+    TSX_REQUIRE(q, "winograd: null geometry");
     TSX_REQUIRE(q->kh == 3 && q->kw == 3 && q->stride_h == 1 && q->stride_w == 1 && q->dilation_h == 1 &&
                     q->dilation_w == 1,
-                "winograd_f63: needs a 3x3 kernel with stride 1 and dilation 1");
-    TSX_REQUIRE(q->n > 0 && q->c > 0 && q->h > 0 && q->w > 0 && q->cout > 0, "winograd_f63: non-positive extent");
+                "winograd: needs a 3x3 kernel with stride 1 and dilation 1");
+    TSX_REQUIRE(q->n > 0 && q->c > 0 && q->h > 0 && q->w > 0 && q->cout > 0, "winograd: non-positive extent");
     TSX_REQUIRE(q->pad_top >= 0 && q->pad_bottom >= 0 && q->pad_left >= 0 && q->pad_right >= 0,
-                "winograd_f63: negative padding is not supported");
+                "winograd: negative padding is not supported");
     g->n = q->n;
     g->c = q->c;
     g->h = q->h;
@@ -254,11 +366,11 @@ int make_geom(const tsx_conv2d_geom *q, float padding_value, WinoGeom *g) {
     g->cout = q->cout;
     g->ho = q->h + q->pad_top + q->pad_bottom - 2;
     g->wo = q->w + q->pad_left + q->pad_right - 2;
-    TSX_REQUIRE(g->ho > 0 && g->wo > 0, "winograd_f63: empty output %dx%d", g->ho, g->wo);
+    TSX_REQUIRE(g->ho > 0 && g->wo > 0, "winograd: empty output %dx%d", g->ho, g->wo);
     g->pad_top = q->pad_top;
     g->pad_left = q->pad_left;
-    g->th = (g->ho + 5) / 6;
-    g->tw = (g->wo + 5) / 6;
+    g->th = (g->ho + tile - 1) / tile;
+    g->tw = (g->wo + tile - 1) / tile;
     g->tiles = g->th * g->tw;
     g->padding_value = padding_value;
     return 0;
@@ -295,11 +407,11 @@ int tsx_conv2d_winograd_f63_nchw(const tsx_conv2d_geom *q, const float *x_dev, c
     tsx::WinoGeom g;
     int rc = tsx::make_geom(q, padding_value, &g);
     if (rc) return rc;
-    TSX_REQUIRE(x_dev && u_dev && out_dev, "winograd_f63: null argument");
-    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_LEAKY_RELU, "winograd_f63: unknown activation %d", act);
+    TSX_REQUIRE(x_dev && u_dev && out_dev, "winograd: null argument");
+    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_LEAKY_RELU, "winograd: unknown activation %d", act);
     const size_t need = tsx_winograd_f63_workspace_bytes(q);
     if (!workspace_dev || workspace_bytes < need)
-        return tsx::fail(TSX_E_WORKSPACE, "winograd_f63: workspace %zu < %zu bytes", workspace_bytes, need);
+        return tsx::fail(TSX_E_WORKSPACE, "winograd: workspace %zu < %zu bytes", workspace_bytes, need);
     hipStream_t stream = tsx::as_stream(stream_);
     float *v = static_cast<float *>(workspace_dev);
     float *mm = v + size_t(g.n) * 64 * g.c * g.tiles;
@@ -312,7 +424,7 @@ int tsx_conv2d_winograd_f63_nchw(const tsx_conv2d_geom *q, const float *x_dev, c
     const int batches = g.n * 64;
     const int64_t gemm_threads = int64_t(batches) * g.cout * g.tiles;
     hipLaunchKernelGGL(tsx::gemm_f32_seq_kernel, dim3(unsigned(tsx::ceil_div(gemm_threads, 256))), dim3(256), 0, stream,
-                       u_dev, v, mm, g.cout, g.tiles, g.c, batches);
+                       u_dev, v, mm, g.cout, g.tiles, g.c, batches, 64);
     TSX_LAUNCH_CHECK("gemm_f32_seq_kernel");
 
     const int64_t out_threads = int64_t(g.n) * g.cout * g.tiles;
@@ -320,6 +432,60 @@ int tsx_conv2d_winograd_f63_nchw(const tsx_conv2d_geom *q, const float *x_dev, c
     hipLaunchKernelGGL(tsx::wino_output_transform_kernel, dim3(unsigned(tsx::ceil_div(out_threads, 256))), dim3(256), 0,
                        stream, mm, g, bias_dev, act, slope, count / 4 * 4, out_dev);
     TSX_LAUNCH_CHECK("wino_output_transform_kernel");
+    return 0;
+}
+
+size_t tsx_winograd_f23_kernel_bytes(int32_t cout, int32_t cin) {
+    if (cout <= 0 || cin <= 0) return 0;
+    return size_t(16) * size_t(cout) * size_t(cin) * sizeof(float);
+}
+
+int tsx_winograd_f23_transform_kernel(int32_t cout, int32_t cin, const float *w_oihw_dev, float *u_dev, void *stream) {
+    TSX_REQUIRE(cout > 0 && cin > 0 && w_oihw_dev && u_dev, "winograd_f23_transform_kernel: bad argument");
+    const int total = cout * cin;
+    hipLaunchKernelGGL(tsx::wino23_kernel_transform_kernel, dim3(unsigned(tsx::ceil_div(total, 256))), dim3(256), 0,
+                       tsx::as_stream(stream), w_oihw_dev, cout, cin, u_dev);
+    TSX_LAUNCH_CHECK("wino23_kernel_transform_kernel");
+    return 0;
+}
+
+size_t tsx_winograd_f23_workspace_bytes(const tsx_conv2d_geom *q) {
+    tsx::WinoGeom g;
+    if (tsx::make_geom(q, 0.f, &g, 2)) return 0;
+    return size_t(g.n) * 16 * g.tiles * (size_t(g.c) + size_t(g.cout)) * sizeof(float);
+}
+
+int tsx_conv2d_winograd_f23_nchw(const tsx_conv2d_geom *q, const float *x_dev, const float *u_dev, float padding_value,
+                                 const float *bias_dev, int32_t act, float slope, float *out_dev, void *workspace_dev,
+                                 size_t workspace_bytes, void *stream_) {
+    tsx::WinoGeom g;
+    int rc = tsx::make_geom(q, padding_value, &g, 2);
+    if (rc) return rc;
+    TSX_REQUIRE(x_dev && u_dev && out_dev, "winograd_f23: null argument");
+    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_LEAKY_RELU, "winograd_f23: unknown activation %d", act);
+    const size_t need = tsx_winograd_f23_workspace_bytes(q);
+    if (!workspace_dev || workspace_bytes < need)
+        return tsx::fail(TSX_E_WORKSPACE, "winograd_f23: workspace %zu < %zu bytes", workspace_bytes, need);
+    hipStream_t stream = tsx::as_stream(stream_);
+    float *v = static_cast<float *>(workspace_dev);
+    float *mm = v + size_t(g.n) * 16 * g.c * g.tiles;
+
+    const int64_t in_threads = int64_t(g.n) * g.c * g.tiles;
+    hipLaunchKernelGGL(tsx::wino23_input_transform_kernel, dim3(unsigned(tsx::ceil_div(in_threads, 256))), dim3(256), 0,
+                       stream, x_dev, g, v);
+    TSX_LAUNCH_CHECK("wino23_input_transform_kernel");
+
+    const int batches = g.n * 16;
+    const int64_t gemm_threads = int64_t(batches) * g.cout * g.tiles;
+    hipLaunchKernelGGL(tsx::gemm_f32_seq_kernel, dim3(unsigned(tsx::ceil_div(gemm_threads, 256))), dim3(256), 0, stream,
+                       u_dev, v, mm, g.cout, g.tiles, g.c, batches, 16);
+    TSX_LAUNCH_CHECK("gemm_f32_seq_kernel");
+
+    const int64_t out_threads = int64_t(g.n) * g.cout * g.tiles;
+    const int64_t count = int64_t(g.n) * g.cout * g.ho * g.wo;
+    hipLaunchKernelGGL(tsx::wino23_output_transform_kernel, dim3(unsigned(tsx::ceil_div(out_threads, 256))), dim3(256), 0,
+                       stream, mm, g, bias_dev, act, slope, count / 4 * 4, out_dev);
+    TSX_LAUNCH_CHECK("wino23_output_transform_kernel");
     return 0;
 }
 

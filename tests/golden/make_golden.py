@@ -80,6 +80,9 @@ def main():
     v["wg_x"], v["wg_w"] = x, w
     v["wg_y"] = ref.winograd(x, w, (1, 1, 1, 1), True, 0.0)
     v["wg_y_pv"] = ref.winograd(x, w, (1, 1, 1, 1), True, 0.25)
+    # ... and F(2,3) (:57-459) on the same input
+    v["wg23_y"] = ref.winograd(x, w, (1, 1, 1, 1), False, 0.0)
+    v["wg23_y_pv"] = ref.winograd(x, w, (1, 1, 1, 1), False, 0.25)
 
     # int8 GEMM (math_cpu.cpp:143-244)
     a8 = rng.integers(-128, 128, (7, 45)).astype(np.int8)

@@ -54,6 +54,8 @@ def test_oracle_fp32(port):
     assert np.array_equal(bits(port.inner_prod_f32(G["ip_a"], np.ascontiguousarray(G["ip_b"].T), True)), bits(G["ip_yt"]))
     assert np.array_equal(bits(port.winograd_f63(G["wg_x"], G["wg_w"], (1, 1, 1, 1), 0.0)), bits(G["wg_y"]))
     assert np.array_equal(bits(port.winograd_f63(G["wg_x"], G["wg_w"], (1, 1, 1, 1), 0.25)), bits(G["wg_y_pv"]))
+    assert np.array_equal(bits(port.winograd_f23(G["wg_x"], G["wg_w"], (1, 1, 1, 1), 0.0)), bits(G["wg23_y"]))
+    assert np.array_equal(bits(port.winograd_f23(G["wg_x"], G["wg_w"], (1, 1, 1, 1), 0.25)), bits(G["wg23_y_pv"]))
     assert np.array_equal(port.gemm_i8(G["g8_a"], G["g8_b"]), G["g8_c"])
     assert np.array_equal(port.gemm_i8(G["g8_a"], G["g8_b"], faithful=True), G["g8_c"])
 
@@ -127,6 +129,10 @@ def test_hip_fp32(tsx):
     assert np.array_equal(bits(wg(_dev(G["wg_x"])).cpu().numpy()), bits(G["wg_y"]))
     wg = tsx.WinogradF63(_dev(G["wg_w"]), (1, 1, 1, 1), 0.25)
     assert np.array_equal(bits(wg(_dev(G["wg_x"])).cpu().numpy()), bits(G["wg_y_pv"]))
+    wg = tsx.WinogradF23(_dev(G["wg_w"]), (1, 1, 1, 1))
+    assert np.array_equal(bits(wg(_dev(G["wg_x"])).cpu().numpy()), bits(G["wg23_y"]))
+    wg = tsx.WinogradF23(_dev(G["wg_w"]), (1, 1, 1, 1), 0.25)
+    assert np.array_equal(bits(wg(_dev(G["wg_x"])).cpu().numpy()), bits(G["wg23_y_pv"]))
     g = tsx.GemmI8(_dev(G["g8_b"]))
     _, _, acc = g(_dev(G["g8_a"]), want_acc=True)
     assert np.array_equal(acc.cpu().numpy(), G["g8_c"])

@@ -100,28 +100,30 @@ WINO_CASES = [
 ]
 
 
+@pytest.mark.parametrize("mode", ["f63", "f23"])
 @pytest.mark.parametrize("case", WINO_CASES)
-def test_winograd_f63(tsx, port, case):
+def test_winograd(tsx, port, case, mode):
     n, c, h, w, cout, pads = case
     rng = np.random.default_rng(403)
     x = rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)
     wt = (rng.standard_normal((cout, c, 3, 3)) * np.sqrt(2.0 / (c * 9))).astype(np.float32)
-    op = tsx.WinogradF63(_dev(wt), pads)
+    op = tsx.Winograd(_dev(wt), pads, mode=mode)
     got = op(_dev(x)).cpu().numpy()
-    exp = port.winograd_f63(x, wt, pads)
+    exp = getattr(port, "winograd_" + mode)(x, wt, pads)
     assert _close(got, exp), np.abs(got - exp).max()
     # same operations in the same order as the reference's AVX2/FMA build: equal bits
     assert np.array_equal(bits(got), bits(exp)), (bits(got) != bits(exp)).mean()
 
 
-def test_winograd_f63_padding_value_bias_relu(tsx, port):
+@pytest.mark.parametrize("mode", ["f63", "f23"])
+def test_winograd_padding_value_bias_relu(tsx, port, mode):
     rng = np.random.default_rng(404)
     x = rng.uniform(-1, 1, (2, 8, 9, 9)).astype(np.float32)
     wt = (rng.standard_normal((8, 8, 3, 3)) * 0.1).astype(np.float32)
     bias = rng.standard_normal(8).astype(np.float32) * 0.1
-    op = tsx.WinogradF63(_dev(wt), (1, 1, 1, 1), padding_value=0.5)
+    op = tsx.Winograd(_dev(wt), (1, 1, 1, 1), padding_value=0.5, mode=mode)
     got = op(_dev(x), bias=_dev(bias), act="relu").cpu().numpy()
-    exp = port.relu(port.add_bias(port.winograd_f63(x, wt, (1, 1, 1, 1), padding_value=0.5), bias))
+    exp = port.relu(port.add_bias(getattr(port, "winograd_" + mode)(x, wt, (1, 1, 1, 1), padding_value=0.5), bias))
     assert np.array_equal(bits(got), bits(exp))
 
 

@@ -1,0 +1,102 @@
+"""The "hip" backend inside the real TenniS runtime: oracle/ref.mk's `intree` target compiles
+tennis_amd/backend/hip/*.cpp against TenniS's own headers and links them into the reference
+library, as TenniS does with its own device backends.  Each operator is then created and run by
+TenniS's Workbench on ComputingDevice("hip") and on ComputingDevice("cpu") -- same process, same
+operator factory, same Tensor/SyncMemory machinery -- and the two outputs compared.
+
+Bar: bitwise for the int8 operators, the elementwise operators and Winograd F(6,3); 1e-4
+relative + 1e-5 absolute for the fp32 MFMA GEMM paths.  Skipped where the in-tree build is absent
+(it needs the reference tree at build time).
+"""
+import numpy as np
+import pytest
+
+from _util import bits
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ts():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from oracle import ref
+    if not ref.intree_available():
+        pytest.skip("oracle/_ref/libref_driver_hip.so not built in this tree")
+    ref.intree_lib()
+    return ref
+
+
+def conv_params(ref, pads, strides=(1, 1), dil=(1, 1), pv=0.0):
+    return ref._conv_params(pads, strides, dil, pv)
+
+
+def both(ts, op, params, inputs, out_bytes):
+    cpu = ts.run_op_intree("cpu", op, params, inputs, out_bytes)
+    hip = ts.run_op_intree("hip", op, params, inputs, out_bytes)
+    assert cpu.shape == hip.shape and cpu.dtype == hip.dtype
+    return cpu, hip
+
+
+def close(a, b):
+    return np.all(np.abs(a.astype(np.float64) - b) <= 1e-4 * np.abs(b) + 1e-5)
+
+
+def test_quantized_chain_in_tennis_workbench(ts):
+    rng = np.random.default_rng(900)
+    n, c, h, w, cout = 3, 70, 12, 11, 37
+    x = (rng.standard_normal((n, c, h, w)) * 30).astype(np.float32)
+    scales = np.array([1.3, 0.7, 2.1], np.float32)
+    cpu, hip = both(ts, "quantize", {"quantize_scale": scales}, [x], x.size)
+    assert np.array_equal(cpu, hip)
+    xq = cpu
+    wq = rng.integers(-127, 128, (cout, c, 3, 3)).astype(np.int8)
+    dq = rng.uniform(1e-4, 1e-3, cout).astype(np.float32)
+    for pads, strides, dil, pv in (((1, 1, 1, 1), (1, 1), (1, 1), 0.0), ((2, 0, 1, 2), (2, 1), (1, 2), 3.0)):
+        p = conv_params(ts, pads, strides, dil, pv)
+        p["dequantize_scales"] = dq
+        cpu, hip = both(ts, "conv2d_quantized", p, [xq, wq], 4 * n * cout * (h + 4) * (w + 4))
+        assert np.array_equal(bits(cpu), bits(hip)), (pads, strides, dil)
+    bias = rng.standard_normal(cout).astype(np.float32)
+    y = cpu
+    cpu, hip = both(ts, "add_bias", {"dim": np.array([1], np.int32)}, [y, bias], y.nbytes)
+    assert np.array_equal(bits(cpu), bits(hip))
+    yb = cpu
+    cpu, hip = both(ts, "relu", {}, [yb], yb.nbytes)
+    assert np.array_equal(bits(cpu), bits(hip))
+    cpu, hip = both(ts, "leaky_relu", {"scale": np.array([0.1], np.float32)}, [yb], yb.nbytes)
+    assert np.array_equal(bits(cpu), bits(hip))
+
+
+def test_fp32_operators_in_tennis_workbench(ts):
+    rng = np.random.default_rng(901)
+    x = rng.uniform(-1, 1, (2, 16, 20, 19)).astype(np.float32)
+    w = (rng.standard_normal((24, 16, 3, 3)) * 0.1).astype(np.float32)
+    p = conv_params(ts, (1, 1, 1, 1))
+    cpu, hip = both(ts, "conv2d", p, [x, w], 4 * 2 * 24 * 20 * 19)
+    assert close(hip, cpu)
+    # TenniS's skeleton picks F(2,3) for this shape and F(6,3) for the 256x256-channel one
+    # (src/kernels/common/function.cpp:154-173); both are bit-exact restatements on the device
+    wp = {"format": "NCHW", "padding": p["padding"], "padding_value": p["padding_value"]}
+    cpu, hip = both(ts, "conv2d_winograd", wp, [x, w], 4 * 2 * 24 * 20 * 19)
+    assert np.array_equal(bits(cpu), bits(hip))
+    xb = rng.uniform(-1, 1, (1, 256, 18, 17)).astype(np.float32)
+    wb = (rng.standard_normal((256, 256, 3, 3)) * 0.02).astype(np.float32)
+    cpu, hip = both(ts, "conv2d_winograd", wp, [xb, wb], 4 * 256 * 18 * 17)
+    assert np.array_equal(bits(cpu), bits(hip))
+    a = rng.standard_normal((5, 70)).astype(np.float32)
+    b = rng.standard_normal((70, 33)).astype(np.float32)
+    cpu, hip = both(ts, "inner_prod", {"transpose": np.array([False], np.bool_)}, [a, b], 4 * 5 * 33)
+    assert close(hip, cpu)
+
+
+def test_unregistered_operator_falls_back_to_cpu(ts):
+    """An operator the backend does not register runs through TenniS's device -> cpu lookup order
+    (src/global/operator_factory.cpp:60-81) on a "hip" Workbench, with the tensors copied by the
+    backend's converters."""
+    x = np.linspace(-3, 3, 24, dtype=np.float32).reshape(2, 3, 4)
+    with pytest.raises(RuntimeError):
+        ts.run_op_intree("hip", "sigmoid", {}, [x], x.nbytes, strict=True)
+    cpu = ts.run_op_intree("cpu", "sigmoid", {}, [x], x.nbytes)
+    hip = ts.run_op_intree("hip", "sigmoid", {}, [x], x.nbytes, strict=False)
+    assert np.array_equal(bits(cpu), bits(hip))

@@ -96,8 +96,14 @@ def test_conv2d_inner_prod_winograd_operators(ops, port):
     got = ops.run_op("conv2d", params, [x, wt])
     assert _close(got, port.conv2d_f32(x, wt, (1, 1, 1, 1)))
     wparams = {k: params[k] for k in ("format", "padding", "padding_value")}
+    # the skeleton picks the mode as the reference does: F(2,3) here, F(6,3) for Cin*Cout >= 256*256
+    # on maps larger than 16x16 (src/kernels/common/function.cpp:154-173)
     gotw = ops.run_op("conv2d_winograd", wparams, [x, wt])
-    assert np.array_equal(bits(gotw), bits(port.winograd_f63(x, wt, (1, 1, 1, 1))))
+    assert np.array_equal(bits(gotw), bits(port.winograd_f23(x, wt, (1, 1, 1, 1))))
+    xb = rng.uniform(-1, 1, (1, 256, 18, 17)).astype(np.float32)
+    wb = (rng.standard_normal((256, 256, 3, 3)) * 0.02).astype(np.float32)
+    gotb = ops.run_op("conv2d_winograd", wparams, [xb, wb])
+    assert np.array_equal(bits(gotb), bits(port.winograd_f63(xb, wb, (1, 1, 1, 1))))
     lhs = rng.standard_normal((5, 4, 6, 2)).astype(np.float32)          # flattened to [5, 48]
     rhs = rng.standard_normal((48, 10)).astype(np.float32)
     gotp = ops.run_op("inner_prod", {}, [lhs, rhs])

@@ -114,24 +114,38 @@ WINO_CASES = [
 ]
 
 
+@pytest.mark.parametrize("mode", ["f63", "f23"])
 @pytest.mark.parametrize("case", WINO_CASES)
-def test_winograd_f63(port, ref, case):
+def test_winograd(port, ref, case, mode):
     n, c, h, w, cout, pads = case
     rng = np.random.default_rng(26)
     x = rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)
     wt = (rng.standard_normal((cout, c, 3, 3)) * np.sqrt(2.0 / (c * 9))).astype(np.float32)
-    got = port.winograd_f63(x, wt, pads)
+    got = getattr(port, "winograd_" + mode)(x, wt, pads)
     # F(6,3) in fp32 is itself ~5e-5 off an exact convolution at these sizes
     assert np.abs(got - _conv_fp64(x, wt, pads)).max() < 2e-4
-    exp = ref.winograd(x, wt, pads, f63=True, threads=1)
+    exp = ref.winograd(x, wt, pads, f63=mode == "f63", threads=1)
     assert np.array_equal(got.view(np.int32), exp.view(np.int32))
 
 
-def test_winograd_f63_padding_value(port, ref):
+@pytest.mark.parametrize("mode", ["f63", "f23"])
+def test_winograd_padding_value(port, ref, mode):
     rng = np.random.default_rng(27)
     x = rng.uniform(-1, 1, (1, 8, 9, 9)).astype(np.float32)
     wt = rng.standard_normal((8, 8, 3, 3)).astype(np.float32) * 0.1
-    got = port.winograd_f63(x, wt, (1, 1, 1, 1), padding_value=0.5)
-    exp = ref.winograd(x, wt, (1, 1, 1, 1), f63=True, padding_value=0.5, threads=1)
+    got = getattr(port, "winograd_" + mode)(x, wt, (1, 1, 1, 1), padding_value=0.5)
+    exp = ref.winograd(x, wt, (1, 1, 1, 1), f63=mode == "f63", padding_value=0.5, threads=1)
     assert np.array_equal(got.view(np.int32), exp.view(np.int32))
     assert np.abs(got - _conv_fp64(x, wt, (1, 1, 1, 1), pad_value=0.5)).max() < 2e-4
+
+
+def test_winograd_all_ones_kernel_is_a_box_sum(port):
+    """Reference-independent anchor (the reference's own test/winograd.cpp uses the same input): an
+    all-ones 3x3 kernel on small integers makes every transform exact, so both modes must equal the
+    3x3 box sum."""
+    rng = np.random.default_rng(28)
+    x = rng.integers(-4, 5, (1, 2, 9, 10)).astype(np.float32)
+    wt = np.ones((3, 2, 3, 3), np.float32)
+    box = _conv_fp64(x, wt, (1, 1, 1, 1)).astype(np.float32)
+    assert np.array_equal(port.winograd_f23(x, wt, (1, 1, 1, 1)), box)
+    assert np.abs(port.winograd_f63(x, wt, (1, 1, 1, 1)) - box).max() < 1e-4
