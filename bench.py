@@ -31,6 +31,11 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, 8 TB/s
 
 CFG = dict(n=32, c=256, h=28, w=28, cout=256, k=3, pad=1)
 
+# HBM bytes per launch of the two kernels on this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a
+# known-size copy (profiles/conv2d_i8_config2_hbm_traffic.txt); a profiler figure, not measured by this script.
+TRAFFIC_CONV_BYTES = 41.68e6
+TRAFFIC_STAGE_BYTES = 33.38e6
+
 
 def make_inputs(cfg, seed=1234):
     rng = np.random.default_rng(seed)
@@ -89,6 +94,10 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--cpu-images", type=int, default=32, help="images of the batch timed on the CPU (0 = skip)")
+    ap.add_argument("--profile", action="store_true",
+                    help="for runs under a profiler: skip the int8-output variant (same kernel name as the roofline "
+                         "kernel), the MFMA-rate probe and the CPU baseline, so per-kernel statistics cover the timed "
+                         "kernels only")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
@@ -165,7 +174,7 @@ def main():
         capi.check(L.tsx_conv2d_i8_staged(g, capi._ptr(ws), capi._ptr(packed), ctypes.byref(ep_q.c), None, capi._ptr(out_q),
                                           None, stream))
 
-    t_mfma_q = event_time(mfma_int8_out, reps)
+    t_mfma_q = None if args.profile else event_time(mfma_int8_out, reps)
 
     # The int8 MFMA rate this part sustains with operands of the same statistics (register-only loop):
     # the practical ceiling below the nominal 5.0 POP/s.
@@ -176,8 +185,8 @@ def main():
     def probe():
         capi.check(L.tsx_probe_mfma_i8(capi._ptr(operands), probe_iters, probe_blocks, capi._ptr(sink), stream))
 
-    t_probe = event_time(probe, 3)
-    sustained_tops = probe_blocks * 4 * probe_iters * 8 * 65536.0 / t_probe / 1e12
+    t_probe = None if args.profile else event_time(probe, 3)
+    sustained_tops = None if args.profile else probe_blocks * 4 * probe_iters * 8 * 65536.0 / t_probe / 1e12
 
     # One device copy of known size: the dispatch the HBM counters of a profiler run are scaled by.
     calib_src = torch.empty(64 << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -209,19 +218,22 @@ def main():
                                "out; step = quantize+stage kernel + i8-MFMA implicit-GEMM kernel",
                    "algorithmic_ops_per_step": ops, "pct_of_int8_mfma_peak_whole_step": 100.0 * tops / PEAK_INT8_TOPS},
         "roofline": {"bound": "mfma", "kernel": "conv_i8_ws_kernel", "achieved": kernel_tops, "peak": PEAK_INT8_TOPS,
-                     "unit": "TFLOP/s", "frac": kernel_tops / PEAK_INT8_TOPS, "traffic": None,
+                     "unit": "TFLOP/s", "frac": kernel_tops / PEAK_INT8_TOPS, "traffic": TRAFFIC_CONV_BYTES,
+                     "traffic_unit": "HBM bytes per launch (rocprofv3 counters; algorithmic 33.65e6)",
                      "note": "int8 multiply-accumulate ops (TOP/s); 2*N*Cout*Ho*Wo*Cin*9 = %.4g ops per launch, "
                              "avg launch %.2f us over %d back-to-back launches" % (ops, t_mfma * 1e6, reps)},
-        "sustained_mfma": {"value": sustained_tops, "unit": "TOPS", "frac_of_it": kernel_tops / sustained_tops,
-                           "note": "register-only v_mfma_i32_32x32x32_i8 loop on random int8 operands, measured in this "
-                                   "run: the rate the part sustains under load (clocks drop with operand activity)"},
-        "int8_output_variant": {"achieved": ops / t_mfma_q / 1e12, "unit": "TOPS", "us": t_mfma_q * 1e6,
-                                "note": "same kernel, epilogue requantizes to int8 for a following quantized layer"},
+        "sustained_mfma": None if args.profile else {
+            "value": sustained_tops, "unit": "TOPS", "frac_of_it": kernel_tops / sustained_tops,
+            "note": "register-only v_mfma_i32_32x32x32_i8 loop on random int8 operands, measured in this "
+                    "run: the rate the part sustains under load (clocks drop with operand activity)"},
+        "int8_output_variant": None if args.profile else {
+            "achieved": ops / t_mfma_q / 1e12, "unit": "TOPS", "us": t_mfma_q * 1e6,
+            "note": "same kernel, epilogue requantizes to int8 for a following quantized layer"},
         "stage_kernel": {"bound": "hbm", "kernel": "stage_rows_kernel<quantize>", "achieved": stage_bytes / t_stage / 1e9,
                          "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": stage_bytes / t_stage / 1e9 / PEAK_HBM_GBS,
-                         "us": t_stage * 1e6, "bytes": stage_bytes},
+                         "us": t_stage * 1e6, "bytes": stage_bytes, "traffic": TRAFFIC_STAGE_BYTES},
     }
-    if args.cpu_images > 0:
+    if args.cpu_images > 0 and not args.profile:
         result["cpu_baseline"] = cpu_baseline(x, x_scales, wq, dq, bias, pad, min(args.cpu_images, cfg["n"]))
     print(json.dumps(result))
 

@@ -172,6 +172,10 @@ def test_conv2d_i8_baseline_config2_full(tsx, port):
     _, _, acc2 = conv(_dev((xq // 2).astype(np.int8)), want_acc=True)
     _, _, acc3 = conv(_dev((xq - xq // 2).astype(np.int8)), want_acc=True)
     assert np.array_equal((acc2 + acc3).cpu().numpy(), exp_acc)
+    # ... and a zero input leaves exactly the activation of the bias in every position of a channel
+    out0, _, _ = conv(_dev(np.zeros_like(xq)), dq=_dev(dq), bias=_dev(bias), act="relu")
+    exp0 = np.broadcast_to(np.maximum(bias, 0)[None, :, None, None], exp.shape)
+    assert np.array_equal(out0.cpu().numpy(), exp0)
 
 
 def test_conv2d_i8_rejects_bad_arguments(tsx):
