@@ -243,7 +243,9 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p) {
                         float v = __fmul_rn(float(acc[f][j][r]), dq[r]);
                         if (p.bias) v = __fadd_rn(v, bias[r]);
                         v = apply_act(v, p.act, p.slope, true);
-                        if (p.out_f32) (p.out_f32 + tile_base + int64_t(dco) * howo)[lane_off] = v;
+                        // streaming store: the output is not read again by this kernel, and lines that never become dirty
+                        // in L2 need no write-back burst when the kernel ends
+                        if (p.out_f32) __builtin_nontemporal_store(v, &(p.out_f32 + tile_base + int64_t(dco) * howo)[lane_off]);
                         if (p.out_i8)
                             (p.out_i8 + tile_base + int64_t(dco) * howo)[lane_off] =
                                 int8_t(quantize_value(__fmul_rn(v, q_scale), q_even));
