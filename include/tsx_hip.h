@@ -164,6 +164,27 @@ int tsx_add_bias_f32(const float *x_dev, int64_t pre, int32_t channels, int64_t 
 int tsx_relu_f32(const float *x_dev, int64_t count, float *out_dev, void *stream);
 int tsx_leaky_relu_f32(const float *x_dev, int64_t count, float scale, float *out_dev, void *stream);
 
+/* ---------------------------------------------------------------- glue between convolutions
+ * The HBM-bound operators that sit between the convolutions of whole networks, so that a graph stays
+ * on the device:
+ *   tsx_add_f32        cpu::Add on equal shapes (src/kernels/cpu/add.cpp; a residual join), optionally
+ *                      followed by relu / leaky_relu in the same pass (same semantics as the separate
+ *                      activation operator on the sum)
+ *   tsx_pooling2d_f32  cpu::Pooling2DCore::pooling2d (src/kernels/cpu/pooling2d_core.cpp:48-186) behind
+ *                      base::Pooling2D and base::GlobalPooling2D (base_global_pooling2d.cpp:58-79: window =
+ *                      whole map, stride 1, no padding).  type 0 = MAX, 1 = AVG (Pooling2DType,
+ *                      include/backend/common_structure.h:84-87); white_padding selects Padding2DType WHITE
+ *                      (AVG divides by kh*kw) instead of BLACK (by the valid count).  planes = N*C.
+ *   tsx_pooling2d_out_size  pooling2d_forward (include/backend/common_function.h:14-20): ceil mode. */
+int tsx_add_f32(const float *a_dev, const float *b_dev, int64_t count, int32_t act, float slope, float *out_dev,
+                void *stream);
+int tsx_pooling2d_out_size(int32_t h, int32_t w, int32_t kh, int32_t kw, int32_t pad_top, int32_t pad_bottom,
+                           int32_t pad_left, int32_t pad_right, int32_t stride_h, int32_t stride_w, int32_t *out_h,
+                           int32_t *out_w);
+int tsx_pooling2d_f32(const float *x_dev, int64_t planes, int32_t h, int32_t w, int32_t type, int32_t pad_top,
+                      int32_t pad_left, int32_t kh, int32_t kw, int32_t stride_h, int32_t stride_w, int32_t white_padding,
+                      float *out_dev, int32_t out_h, int32_t out_w, void *stream);
+
 /* ---------------------------------------------------------------- Winograd F(6x6, 3x3) fp32 conv2d
  * Conv2dWinogradAlgorithm<float>::winograd_f63 (src/kernels/cpu/winograd_algorithm.cpp:846-947),
  * reached in the reference through base::Conv2DWinograd's two core calls

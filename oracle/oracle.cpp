@@ -15,6 +15,8 @@
 //   orc_gemm_f32 / orc_conv2d_f32 / orc_inner_prod_f32  fp64 brute force (tolerance) +
 //                         compiled reference (bit-exact, remainder paths included)
 //   orc_winograd_f63 / orc_winograd_f23  fp64 direct conv (tolerance) + compiled reference (bit-exact)
+//   orc_add_f32 / orc_pooling2d_f32      numpy closed forms (max / mean of clipped windows) + compiled
+//                         reference operators add, pooling2d, global_pooling2d (bit-exact)
 #include <algorithm>
 #include <cmath>
 #include <cstdint>
@@ -615,5 +617,55 @@ void orc_winograd_f23(const float *x, int n, int c, int h, int w, const float *w
     }
 }
 
-}  // extern "C"
+// ---------------------------------------------------------------------------
+// Glue operators between convolutions in whole networks.
+// ---------------------------------------------------------------------------
 
+// cpu::Add on equal shapes (src/kernels/cpu/add.cpp: x = lhs + rhs per element).
+void orc_add_f32(const float *a, const float *b, int64_t count, float *out) {
+#pragma omp parallel for num_threads(g_threads)
+    for (int64_t i = 0; i < count; ++i) out[i] = a[i] + b[i];
+}
+
+// cpu::Pooling2DCore (src/kernels/cpu/pooling2d_core.cpp:48-186), NCHW fp32.  Output size is the
+// caller's (pooling2d_forward, include/backend/common_function.h:14-20: ceil).  The window is
+// clipped to the image; MAX (type 0) starts from the first valid element; AVG (type 1) sums the
+// valid elements in row-major order in fp32 and divides by their count (BLACK padding, white = 0)
+// or by kh*kw (WHITE padding, white = 1).  planes = N*C.
+void orc_pooling2d_f32(const float *x, int64_t planes, int h, int w, int type, int pt, int pl, int kh, int kw, int sh,
+                       int sw, int white, float *out, int ho, int wo) {
+#pragma omp parallel for num_threads(g_threads)
+    for (int64_t pc = 0; pc < planes; ++pc) {
+        const float *in = x + pc * h * w;
+        float *o = out + pc * ho * wo;
+        for (int oh = 0; oh < ho; ++oh) {
+            int hs = oh * sh - pt;
+            const int he = std::min(hs + kh, h);
+            hs = std::max(hs, 0);
+            for (int ow = 0; ow < wo; ++ow) {
+                int ws = ow * sw - pl;
+                const int we = std::min(ws + kw, w);
+                ws = std::max(ws, 0);
+                if (type == 0) {
+                    float m = in[hs * w + ws];
+                    for (int ih = hs; ih < he; ++ih)
+                        for (int iw = ws; iw < we; ++iw)
+                            if (in[ih * w + iw] > m) m = in[ih * w + iw];
+                    o[oh * wo + ow] = m;
+                } else {
+                    float sum = 0.f;
+                    int count = 0;
+                    for (int ih = hs; ih < he; ++ih)
+                        for (int iw = ws; iw < we; ++iw) {
+                            sum += in[ih * w + iw];
+                            ++count;
+                        }
+                    if (white) o[oh * wo + ow] = sum / float(kh * kw);
+                    else o[oh * wo + ow] = count == 0 ? 0.f : sum / float(count);
+                }
+            }
+        }
+    }
+}
+
+}  // extern "C"

@@ -44,6 +44,8 @@ def lib():
         L.orc_conv2d_f32.argtypes = [_vp, _i, _i, _i, _i, _vp] + [_i] * 11 + [_f, _vp]
         L.orc_inner_prod_f32.argtypes = [_vp, _i, _i, _vp, _i, _i, _vp]
         L.orc_winograd_f63.argtypes = [_vp, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _f, _vp]
+        L.orc_add_f32.argtypes = [_vp, _vp, ctypes.c_int64, _vp]
+        L.orc_pooling2d_f32.argtypes = [_vp, ctypes.c_int64] + [_i] * 10 + [_vp, _i, _i]
         L.orc_winograd_f23.argtypes = [_vp, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _f, _vp]
         _lib = L
     return _lib
@@ -243,3 +245,36 @@ def winograd_f23(x, w, pads, padding_value=0.0):
     out = np.empty((n, cout, ho, wo), np.float32)
     lib().orc_winograd_f23(_p(x), n, c, h, wd, _p(w), cout, *pads, padding_value, _p(out))
     return out
+
+
+def add(a, b):
+    """cpu::Add on equal shapes (src/kernels/cpu/add.cpp)."""
+    a = _c(a, np.float32)
+    b = _c(b, np.float32)
+    assert a.shape == b.shape
+    out = np.empty_like(a)
+    lib().orc_add_f32(_p(a), _p(b), a.size, _p(out))
+    return out
+
+
+def pool_out_hw(h, w, ksize, pads, strides):
+    """pooling2d_forward (include/backend/common_function.h:14-20): ceil, evaluated in fp32 like the reference."""
+    ho = int(np.ceil(np.float32(h + pads[0] + pads[1] - ksize[0]) / np.float32(strides[0]) + np.float32(1)))
+    wo = int(np.ceil(np.float32(w + pads[2] + pads[3] - ksize[1]) / np.float32(strides[1]) + np.float32(1)))
+    return ho, wo
+
+
+def pooling2d(x, kind, ksize, strides, pads=(0, 0, 0, 0), white=False):
+    """cpu::Pooling2D (pooling2d_core.cpp:48-186): kind "max" or "avg"; pads = (top, bottom, left, right)."""
+    x = _c(x, np.float32)
+    n, c, h, w = x.shape
+    ho, wo = pool_out_hw(h, w, ksize, pads, strides)
+    out = np.empty((n, c, ho, wo), np.float32)
+    lib().orc_pooling2d_f32(_p(x), n * c, h, w, {"max": 0, "avg": 1}[kind], pads[0], pads[2], ksize[0], ksize[1],
+                            strides[0], strides[1], int(white), _p(out), ho, wo)
+    return out
+
+
+def global_pooling2d(x, kind):
+    """base::GlobalPooling2D (base_global_pooling2d.cpp:58-79) = pooling2d over the whole map, BLACK padding."""
+    return pooling2d(x, kind, x.shape[2:], (1, 1))

@@ -172,6 +172,24 @@ def leaky_relu(x, scale, threads=1):
     return run_op("leaky_relu", {"scale": np.array([scale], np.float32)}, [x], x.nbytes, threads)
 
 
+def add(a, b, threads=1):
+    return run_op("add", {}, [a, b], max(a.nbytes, b.nbytes), threads)
+
+
+def pooling2d(x, kind, ksize, strides, pads=(0, 0, 0, 0), white=False, threads=1):
+    p = {"format": "NCHW", "type": np.array([{"max": 0, "avg": 1}[kind]], np.int32),
+         "padding": np.array([[0, 0], [0, 0], [pads[0], pads[1]], [pads[2], pads[3]]], np.int32),
+         "padding_type": np.array([3 if white else 0], np.int32),
+         "ksize": np.array([1, 1, ksize[0], ksize[1]], np.int32),
+         "stride": np.array([1, 1, strides[0], strides[1]], np.int32)}
+    return run_op("pooling2d", p, [x], 4 * x.size + 4096, threads)
+
+
+def global_pooling2d(x, kind, threads=1):
+    p = {"format": "NCHW", "type": np.array([{"max": 0, "avg": 1}[kind]], np.int32)}
+    return run_op("global_pooling2d", p, [x], 4 * x.shape[0] * x.shape[1], threads)
+
+
 def inner_prod(lhs, rhs, transpose=False, threads=1):
     n = rhs.shape[0] if transpose else rhs.shape[1]
     return run_op("inner_prod", {"transpose": np.array([transpose], np.bool_)}, [lhs, rhs],

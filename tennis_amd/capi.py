@@ -68,6 +68,9 @@ SIGNATURES = {
     "tsx_add_bias_f32": (ctypes.c_int, [_vp, _i64, _i32, _i64, _vp, _vp, _vp]),
     "tsx_relu_f32": (ctypes.c_int, [_vp, _i64, _vp, _vp]),
     "tsx_leaky_relu_f32": (ctypes.c_int, [_vp, _i64, _f32, _vp, _vp]),
+    "tsx_add_f32": (ctypes.c_int, [_vp, _vp, _i64, _i32, _f32, _vp, _vp]),
+    "tsx_pooling2d_out_size": (ctypes.c_int, [_i32] * 10 + [ctypes.POINTER(_i32), ctypes.POINTER(_i32)]),
+    "tsx_pooling2d_f32": (ctypes.c_int, [_vp, _i64] + [_i32] * 10 + [_vp, _i32, _i32, _vp]),
     "tsx_winograd_f63_kernel_bytes": (_sz, [_i32, _i32]),
     "tsx_winograd_f63_transform_kernel": (ctypes.c_int, [_i32, _i32, _vp, _vp, _vp]),
     "tsx_winograd_f63_workspace_bytes": (_sz, [ctypes.POINTER(ConvGeom)]),
@@ -342,3 +345,36 @@ def leaky_relu(x, scale):
     out = torch.empty_like(x)
     check(lib().tsx_leaky_relu_f32(_ptr(x), x.numel(), float(scale), _ptr(out), _stream()))
     return out
+
+
+def add(a, b, act=None, slope=0.0, out=None):
+    """tsx_add_f32: act(a + b) on equal shapes."""
+    a = _dev(a, torch.float32)
+    b = _dev(b, torch.float32)
+    assert a.shape == b.shape
+    if out is None:
+        out = torch.empty_like(a)
+    check(lib().tsx_add_f32(_ptr(a), _ptr(b), a.numel(), _ACT[act], float(slope), _ptr(out), _stream()))
+    return out
+
+
+def pool_out_size(h, w, ksize, pads, strides):
+    oh, ow = _i32(), _i32()
+    check(lib().tsx_pooling2d_out_size(h, w, ksize[0], ksize[1], pads[0], pads[1], pads[2], pads[3], strides[0],
+                                       strides[1], ctypes.byref(oh), ctypes.byref(ow)))
+    return oh.value, ow.value
+
+
+def pooling2d(x, kind, ksize, strides, pads=(0, 0, 0, 0), white=False):
+    """tsx_pooling2d_f32: kind "max" | "avg", pads = (top, bottom, left, right)."""
+    x = _dev(x, torch.float32)
+    n, c, h, w = x.shape
+    ho, wo = pool_out_size(h, w, ksize, pads, strides)
+    out = torch.empty((n, c, ho, wo), dtype=torch.float32, device=x.device)
+    check(lib().tsx_pooling2d_f32(_ptr(x), n * c, h, w, {"max": 0, "avg": 1}[kind], pads[0], pads[2], ksize[0], ksize[1],
+                                  strides[0], strides[1], int(white), _ptr(out), ho, wo, _stream()))
+    return out
+
+
+def global_pooling2d(x, kind):
+    return pooling2d(x, kind, tuple(x.shape[2:]), (1, 1))

@@ -3,6 +3,8 @@
 //   cpu::AddBias    src/kernels/cpu/add_bias.cpp:47-85      y = x + b[c]
 //   cpu::ReLU       src/kernels/cpu/relu.cpp:30-52          SIMD body max(x,0), scalar tail std::max
 //   cpu::LeakyReLU  src/kernels/cpu/leaky_relu.cpp:41-66    body fma(scale, min(x,0), max(x,0)), tail x>0?x:x*scale
+//   cpu::Add        src/kernels/cpu/add.cpp                 y = a + b on equal shapes (a residual join), optionally
+//                                                           followed by the activation operator in the same pass
 // Each lane handles 4 consecutive elements (16-byte accesses) in a grid-stride loop.
 #include "tsx_common.hpp"
 
@@ -10,26 +12,36 @@ namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-// MODE 0: add_bias (layout [pre][channels][inner]); 1: relu; 2: leaky_relu
+// MODE 0: add_bias (layout [pre][channels][inner]); 1: relu; 2: leaky_relu; 3: add (second operand in `bias`) + act
 template <int MODE>
 __global__ __launch_bounds__(256) void elementwise_kernel(const float *__restrict__ x, int64_t count,
                                                          const float *__restrict__ bias, int channels, int64_t inner,
-                                                         float slope, int64_t body, float *__restrict__ out, bool vec) {
+                                                         float slope, int64_t body, float *__restrict__ out, bool vec,
+                                                         int act) {
     const int64_t stride = int64_t(gridDim.x) * blockDim.x * 4;
     for (int64_t base = (int64_t(blockIdx.x) * blockDim.x + threadIdx.x) * 4; base < count; base += stride) {
         float v[4];
         const bool full = vec && base + 4 <= count;
+        float u[4] = {0.f, 0.f, 0.f, 0.f};
         if (full) {
             const v4f in = *reinterpret_cast<const v4f *>(x + base);
             v[0] = in[0]; v[1] = in[1]; v[2] = in[2]; v[3] = in[3];
+            if (MODE == 3) {
+                const v4f in2 = *reinterpret_cast<const v4f *>(bias + base);
+                u[0] = in2[0]; u[1] = in2[1]; u[2] = in2[2]; u[3] = in2[3];
+            }
         } else {
             for (int j = 0; j < 4; ++j) v[j] = base + j < count ? x[base + j] : 0.f;
+            if (MODE == 3)
+                for (int j = 0; j < 4; ++j) u[j] = base + j < count ? bias[base + j] : 0.f;
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int64_t i = base + j;
             if (MODE == 0) {
                 if (i < count) v[j] = __fadd_rn(v[j], bias[(i / inner) % channels]);
+            } else if (MODE == 3) {
+                v[j] = tsx::apply_act(__fadd_rn(v[j], u[j]), act, slope, i < body);
             } else {
                 v[j] = tsx::apply_act(v[j], MODE == 1 ? TSX_ACT_RELU : TSX_ACT_LEAKY_RELU, slope, i < body);
             }
@@ -46,14 +58,15 @@ __global__ __launch_bounds__(256) void elementwise_kernel(const float *__restric
 
 template <int MODE>
 int launch(const float *x, int64_t count, const float *bias, int channels, int64_t inner, float slope, float *out,
-           void *stream) {
+           void *stream, int act = TSX_ACT_NONE) {
     if (count == 0) return 0;
     TSX_REQUIRE(x && out, "elementwise: null pointer");
-    const bool vec = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    const bool vec = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
+                     (MODE != 3 || reinterpret_cast<uintptr_t>(bias) % 16 == 0);
     int64_t blocks = tsx::ceil_div(tsx::ceil_div(count, 4), 256);
     if (blocks > 256 * 8) blocks = 256 * 8;
     hipLaunchKernelGGL(elementwise_kernel<MODE>, dim3(unsigned(blocks)), dim3(256), 0, tsx::as_stream(stream), x, count,
-                       bias, channels, inner, slope, count / 4 * 4, out, vec);
+                       bias, channels, inner, slope, count / 4 * 4, out, vec, act);
     TSX_LAUNCH_CHECK("elementwise_kernel");
     return 0;
 }
@@ -76,6 +89,13 @@ int tsx_relu_f32(const float *x_dev, int64_t count, float *out_dev, void *stream
 int tsx_leaky_relu_f32(const float *x_dev, int64_t count, float scale, float *out_dev, void *stream) {
     TSX_REQUIRE(count >= 0, "leaky_relu: negative count");
     return launch<2>(x_dev, count, nullptr, 1, 1, scale, out_dev, stream);
+}
+
+int tsx_add_f32(const float *a_dev, const float *b_dev, int64_t count, int32_t act, float slope, float *out_dev,
+                void *stream) {
+    TSX_REQUIRE(count >= 0 && (count == 0 || b_dev), "add: bad argument");
+    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_LEAKY_RELU, "add: unknown activation %d", act);
+    return launch<3>(a_dev, count, b_dev, 1, 1, slope, out_dev, stream, act);
 }
 
 }  // extern "C"
