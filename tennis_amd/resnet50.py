@@ -1,0 +1,210 @@
+"""A ResNet-50-shaped int8 network on the MI355X convolution path.
+
+Topology (random-init; the shape is what matters): 7x7/2 stem -> 3x3/2 max pool -> [3, 4, 6, 3]
+bottleneck blocks (1x1 -> 3x3 -> 1x1, stride 2 on the 3x3 of the first block of stages 2-4, 1x1
+projection shortcuts) with 64..2048 channels, BN folded into conv (so conv + bias), ReLU, residual
+add, global average pool, FC 2048 -> 1000.  Per-output-channel int8 weights, per-tensor int8
+activations calibrated on a batch.
+
+Every layer is the TenniS operator chain the reference would run for a quantized graph --
+    quantize(x, s) -> conv2d_quantized(w_q, dq) -> add_bias -> relu        (src/kernels/cpu/quantize.cpp,
+    quantized/conv2d_quantized_core.cpp, add_bias.cpp, relu.cpp)
+    add -> relu (residual join), pooling2d, global_pooling2d, and for the classifier
+    quantize -> int8 gemm -> dequant -> add_bias
+-- executed with the chain fused into the kernels' epilogues, which reproduce the separate operators
+rounding for rounding.  `layers()` describes the network independently of the device so that the same
+description can be evaluated by a CPU checker.
+
+Activation scales follow the reference's quantize operator: `quantize_scale` holds one multiplier per
+image (its length must equal the batch); per-tensor calibration passes N equal values.
+"""
+import numpy as np
+import torch
+
+from . import capi
+
+STAGES = ((64, 3, 1), (128, 4, 2), (256, 6, 2), (512, 3, 2))   # (mid channels, blocks, stride of the first block)
+
+
+class ConvSpec:
+    def __init__(self, name, cin, cout, k, stride, pad, relu):
+        self.name, self.cin, self.cout, self.k, self.stride, self.pad, self.relu = name, cin, cout, k, stride, pad, relu
+
+
+def layers(width=1.0, blocks=None, classes=1000):
+    """The network as data: stem spec, list of blocks (conv1, conv2, conv3, projection-or-None), fc (cin, cout).
+    `width` scales every channel count and `blocks` overrides the per-stage block counts (small test nets)."""
+    ch = lambda c: max(8, int(c * width))
+    stem = ConvSpec("stem", 3, ch(64), 7, 2, 3, True)
+    net, cin = [], ch(64)
+    for si, (mid, count, stride) in enumerate(STAGES):
+        count = blocks[si] if blocks else count
+        for bi in range(count):
+            s = stride if bi == 0 else 1
+            m, cout = ch(mid), ch(mid * 4)
+            name = "s%db%d" % (si + 1, bi)
+            proj = ConvSpec(name + ".proj", cin, cout, 1, s, 0, False) if bi == 0 else None
+            net.append((ConvSpec(name + ".c1", cin, m, 1, 1, 0, True), ConvSpec(name + ".c2", m, m, 3, s, 1, True),
+                        ConvSpec(name + ".c3", m, cout, 1, 1, 0, False), proj))
+            cin = cout
+    return stem, net, (cin, classes)
+
+
+def quantize_weights(w):
+    """Per-output-channel symmetric int8, round half away from zero (offline weight quantization)."""
+    flat = w.reshape(w.shape[0], -1)
+    s = (np.float32(127.0) / np.maximum(np.abs(flat).max(axis=1), np.float32(1e-12))).astype(np.float32)
+    q = flat * s[:, None]
+    q = np.clip(np.sign(q) * np.floor(np.abs(q) + np.float32(0.5)), -127, 127).astype(np.int8)
+    return q.reshape(w.shape), s
+
+
+def make_parameters(seed=0, width=1.0, blocks=None, classes=1000):
+    """Random Kaiming-normal weights quantized per channel; small random biases.  Host arrays only."""
+    rng = np.random.default_rng(seed)
+    stem, net, fc = layers(width, blocks, classes)
+    params = {}
+
+    def conv(spec):
+        fan_in = spec.cin * spec.k * spec.k
+        w = (rng.standard_normal((spec.cout, spec.cin, spec.k, spec.k)) * np.sqrt(2.0 / fan_in)).astype(np.float32)
+        wq, sw = quantize_weights(w)
+        params[spec.name] = {"wq": wq, "sw": sw, "bias": (rng.standard_normal(spec.cout) * 0.05).astype(np.float32)}
+
+    conv(stem)
+    for c1, c2, c3, proj in net:
+        for spec in (c1, c2, c3, proj):
+            if spec is not None:
+                conv(spec)
+    w = (rng.standard_normal((fc[0], fc[1])) * np.sqrt(1.0 / fc[0])).astype(np.float32)   # [k][n]
+    wq_t, sw = quantize_weights(np.ascontiguousarray(w.T))                                  # per output column
+    params["fc"] = {"wq": np.ascontiguousarray(wq_t.T), "sw": sw, "bias": (rng.standard_normal(fc[1]) * 0.05).astype(np.float32)}
+    return (stem, net, fc), params
+
+
+def total_macs(desc, batch, size):
+    """Multiply-accumulates of one forward pass (convolutions + classifier)."""
+    stem, net, fc = desc
+
+    def out(h, spec):
+        return (h + 2 * spec.pad - spec.k) // spec.stride + 1
+
+    h = out(size, stem)
+    macs = batch * stem.cout * h * h * stem.cin * stem.k * stem.k
+    h = int(np.ceil((h + 1 - 3) / 2.0 + 1))
+    for c1, c2, c3, proj in net:
+        h2 = out(h, c2)
+        macs += batch * c1.cout * h * h * c1.cin
+        macs += batch * c2.cout * h2 * h2 * c2.cin * 9
+        macs += batch * c3.cout * h2 * h2 * c3.cin
+        if proj is not None:
+            macs += batch * proj.cout * h2 * h2 * proj.cin
+        h = h2
+    return macs + batch * fc[0] * fc[1]
+
+
+class ResNet50Int8:
+    """The network on the device.  calibrate(x) fixes the activation scales; forward(x) runs the fused path."""
+
+    POOL = ((3, 3), (2, 2), (0, 1, 0, 1))   # ksize, stride, pads: 112 -> 56 under TenniS's ceil-mode size rule
+
+    def __init__(self, desc, params, device="cuda:0"):
+        self.desc, self.host = desc, params
+        self.dev = torch.device(device)
+        self.conv, self.bias, self.sw = {}, {}, {}
+        stem, net, fc = desc
+        specs = [stem] + [s for blk in net for s in blk if s is not None]
+        for spec in specs:
+            p = params[spec.name]
+            self.conv[spec.name] = capi.Conv2dI8(torch.from_numpy(p["wq"]).to(self.dev), (spec.pad,) * 4,
+                                                 (spec.stride, spec.stride))
+            self.bias[spec.name] = torch.from_numpy(p["bias"]).to(self.dev)
+            self.sw[spec.name] = p["sw"]
+        self.fc = capi.GemmI8(torch.from_numpy(params["fc"]["wq"]).to(self.dev))
+        self.bias["fc"] = torch.from_numpy(params["fc"]["bias"]).to(self.dev)
+        self.sw["fc"] = params["fc"]["sw"]
+        self.scales = None      # name -> python float (multiplier applied before rounding)
+        self._dq, self._sx = {}, {}
+
+    # ---- calibration: per-tensor scale = 127 / max|input of the layer| on this batch, measured on the
+    # activations of the quantized network itself, layer by layer
+    @staticmethod
+    def _scale_of(t):
+        m = float(t.abs().max().item())
+        return float(np.float32(127.0) / np.float32(m if m > 0 else 1.0))
+
+    def calibrate(self, x):
+        n = x.shape[0]
+        self.scales = {}
+        self._forward(x, n, calibrating=True)
+        self._dq = {k: torch.from_numpy((np.float32(1.0) / (np.float32(s) * self.sw[k])).astype(np.float32)).to(self.dev)
+                    for k, s in self.scales.items()}
+        return dict(self.scales)
+
+    def set_scales(self, scales, n):
+        self.scales = dict(scales)
+        self._dq = {k: torch.from_numpy((np.float32(1.0) / (np.float32(s) * self.sw[k])).astype(np.float32)).to(self.dev)
+                    for k, s in self.scales.items()}
+        self._sx = {}
+        self._batch_scales(n)
+
+    def _batch_scales(self, n):
+        """quantize_scale tensors: one equal multiplier per image (base_quantize.cpp:26)."""
+        if self._sx.get("_n") != n:
+            self._sx = {k: torch.full((n,), s, dtype=torch.float32, device=self.dev) for k, s in self.scales.items()}
+            self._sx["_n"] = n
+        return self._sx
+
+    def forward(self, x):
+        assert self.scales is not None, "calibrate() or set_scales() first"
+        return self._forward(x, x.shape[0], calibrating=False)
+
+    def _forward(self, x, n, calibrating):
+        stem, net, fc = self.desc
+
+        def dq_of(name, s):
+            return torch.from_numpy((np.float32(1.0) / (np.float32(s) * self.sw[name])).astype(np.float32)).to(self.dev)
+
+        def conv_from_f32(spec, t, out_scale_name=None):
+            """quantize(t) -> conv -> bias -> relu?; int8 requantized output when the consumer's scale is known."""
+            if calibrating:
+                self.scales[spec.name] = self._scale_of(t)
+                sx = torch.full((n,), self.scales[spec.name], dtype=torch.float32, device=self.dev)
+                dq = dq_of(spec.name, self.scales[spec.name])
+                return self.conv[spec.name](t, dq=dq, bias=self.bias[spec.name], act="relu" if spec.relu else None, x_scales=sx)[0]
+            sxs = self._batch_scales(n)
+            qs = sxs[out_scale_name] if out_scale_name else None
+            f, q, _ = self.conv[spec.name](t, dq=self._dq[spec.name], bias=self.bias[spec.name],
+                                           act="relu" if spec.relu else None, x_scales=sxs[spec.name], q_scales=qs,
+                                           want_f32=qs is None)
+            return q if qs is not None else f
+
+        def conv_from_i8(spec, t8, out_scale_name=None):
+            sxs = self._batch_scales(n)
+            qs = sxs[out_scale_name] if out_scale_name else None
+            f, q, _ = self.conv[spec.name](t8, dq=self._dq[spec.name], bias=self.bias[spec.name],
+                                           act="relu" if spec.relu else None, q_scales=qs, want_f32=qs is None)
+            return q if qs is not None else f
+
+        y = conv_from_f32(stem, x)
+        y = capi.pooling2d(y, "max", *self.POOL)
+        for c1, c2, c3, proj in net:
+            if calibrating:
+                a = conv_from_f32(c1, y)
+                b = conv_from_f32(c2, a)
+                c = conv_from_f32(c3, b)
+            else:
+                a8 = conv_from_f32(c1, y, out_scale_name=c2.name)
+                b8 = conv_from_i8(c2, a8, out_scale_name=c3.name)
+                c = conv_from_i8(c3, b8)
+            sc = conv_from_f32(proj, y) if proj is not None else y
+            y = capi.add(c, sc, "relu")
+        pooled = capi.global_pooling2d(y, "avg").reshape(n, fc[0])
+        if calibrating:
+            self.scales["fc"] = self._scale_of(pooled)
+            sx = torch.full((n,), self.scales["fc"], dtype=torch.float32, device=self.dev)
+            dq = dq_of("fc", self.scales["fc"])
+        else:
+            sx, dq = self._batch_scales(n)["fc"], self._dq["fc"]
+        p8 = capi.quantize(pooled, sx)
+        return self.fc(p8, dq=dq, bias=self.bias["fc"])[0]
