@@ -88,12 +88,48 @@ def cpu_baseline(x, x_scales, wq, dq, bias, pad, images):
             "host_cpus": os.cpu_count()}
 
 
+def resnet_leg(steps=20):
+    """ResNet-50-shaped int8 network, batch 32 at 3x224x224 (BASELINE config 4): img/s of the whole forward pass,
+    replayed from a captured HIP graph (the pass is ~130 short kernels; capture removes the host launch cost)."""
+    import torch
+    from tennis_amd import resnet50
+    n, size = 32, 224
+    desc, params = resnet50.make_parameters(seed=0)
+    net = resnet50.ResNet50Int8(desc, params)
+    x = torch.rand((n, 3, size, size), device="cuda")
+    net.set_scales(net.calibrate(x), n)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        net.forward(x)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        logits = net.forward(x)
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    macs = resnet50.total_macs(desc, n, size)
+    return {"workload": "BASELINE config 4: ResNet-50-shaped int8 network, batch 32, 3x224x224, random-init weights, "
+                        "per-channel int8 weights, per-tensor int8 activations calibrated on the batch",
+            "img_per_s": n / dt, "ms_per_batch": dt * 1e3, "TOPS": 2.0 * macs / dt / 1e12,
+            "pct_of_int8_mfma_peak": 100.0 * 2.0 * macs / dt / 1e12 / PEAK_INT8_TOPS, "gmac_per_image": macs / n / 1e9,
+            "steps": steps, "logits_finite": bool(torch.isfinite(logits).all().item())}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--cpu-images", type=int, default=32, help="images of the batch timed on the CPU (0 = skip)")
+    ap.add_argument("--no-resnet", action="store_true", help="skip the ResNet-50-shaped network leg")
     ap.add_argument("--profile", action="store_true",
                     help="for runs under a profiler: skip the int8-output variant (same kernel name as the roofline "
                          "kernel), the MFMA-rate probe and the CPU baseline, so per-kernel statistics cover the timed "
@@ -233,6 +269,8 @@ def main():
                          "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": stage_bytes / t_stage / 1e9 / PEAK_HBM_GBS,
                          "us": t_stage * 1e6, "bytes": stage_bytes, "traffic": TRAFFIC_STAGE_BYTES},
     }
+    if not args.no_resnet and not args.profile:
+        result["resnet50_int8_bs32"] = resnet_leg()
     if args.cpu_images > 0 and not args.profile:
         result["cpu_baseline"] = cpu_baseline(x, x_scales, wq, dq, bias, pad, min(args.cpu_images, cfg["n"]))
     print(json.dumps(result))
