@@ -100,6 +100,103 @@ constexpr int STAGE_CG = 256;                 // channels per pass
 constexpr int STAGE_LROW = STAGE_CG + 16;     // LDS bytes per pixel: 16-byte aligned, bank-shifted
 constexpr int STAGE_MAX_WS = 232;             // ws * LROW <= 63 KiB
 
+struct StageRow {
+    const void *src;
+    const float *scales;
+    int n_scales;
+    int64_t group_len, bulk8;
+    bool uniform_scale;
+    float row_scale;
+    int ni, hi, c0, creal;
+};
+
+// Phase 1 of stage_rows_kernel for one source row and one channel group.  Lane = (run of VW pixels
+// along W, channel quad): a lane loads the same VW pixels of 4 consecutive channels (one VW-wide load
+// per channel, coalesced along W across lanes), packs the 4 quantized bytes of each pixel into one
+// dword and writes VW dwords to the tile -- no byte-granular LDS traffic.  WL = power of two >= W/VW
+// keeps the mapping division-free; loads are issued in batches of NB quads before any is consumed.
+template <bool QUANT, int VW>
+__device__ __forceinline__ void stage_quads(const StageGeom &g, const StageRow &r, int8_t *tile, int tid) {
+    typedef float vf __attribute__((ext_vector_type(VW == 1 ? 2 : VW)));   // VW == 1 uses scalars
+    constexpr int NB = VW == 4 ? 2 : 4;
+    const int pw = g.w / VW;
+    int wl = 1, wl_shift = 0;
+    while (wl < pw) {
+        wl <<= 1;
+        ++wl_shift;
+    }
+    const int lane = tid & 63, wave = tid >> 6;
+    const int qpw = 64 >> wl_shift;                 // channel quads per wavefront per step
+    const int pi = lane & (wl - 1);
+    const int wi = pi * VW;
+    const int q_lane = wave * qpw + (lane >> wl_shift);
+    const int qstep = 4 * qpw;                      // quads per workgroup step
+    const bool lane_ok = pi < pw;
+    const int64_t plane = int64_t(g.h) * g.w;
+    const int64_t row_base = (int64_t(r.ni) * g.c + r.c0) * plane + int64_t(r.hi) * g.w + wi;
+    const int quads = (r.creal + 3) / 4;
+    for (int qb = 0; qb < quads; qb += NB * qstep) {
+        float fv[NB][4][VW];
+        int bv[NB][4][VW];
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int c = (qb + u * qstep + q_lane) * 4;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool ok = lane_ok && c + j < r.creal;
+                const int64_t e = row_base + int64_t(c + j) * plane;
+                if (QUANT) {
+                    const float *p = static_cast<const float *>(r.src) + e;
+                    if (VW == 1) {
+                        fv[u][j][0] = ok ? *p : 0.f;
+                    } else {
+                        vf t;
+#pragma unroll
+                        for (int v = 0; v < VW; ++v) t[v] = 0.f;
+                        if (ok) t = *reinterpret_cast<const vf *>(p);
+#pragma unroll
+                        for (int v = 0; v < VW; ++v) fv[u][j][v] = t[v];
+                    }
+                } else {
+                    const int8_t *p = static_cast<const int8_t *>(r.src) + e;
+                    uint32_t t = 0;
+                    if (ok) {
+                        if (VW == 4) t = *reinterpret_cast<const uint32_t *>(p);
+                        else if (VW == 2) t = *reinterpret_cast<const uint16_t *>(p);
+                        else t = uint8_t(*p);
+                    }
+#pragma unroll
+                    for (int v = 0; v < VW; ++v) bv[u][j][v] = int8_t(t >> (8 * v));
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int c = (qb + u * qstep + q_lane) * 4;
+            if (!(lane_ok && c < r.creal)) continue;
+#pragma unroll
+            for (int v = 0; v < VW; ++v) {
+                uint32_t word = 0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    int q = 0;
+                    if (c + j < r.creal) {
+                        if (QUANT) {
+                            const int64_t e = row_base + int64_t(c + j) * plane + v;
+                            const float sc = r.uniform_scale ? r.row_scale : r.scales[e / r.group_len];
+                            q = tsx::quantize_value(__fmul_rn(fv[u][j][v], sc), r.n_scales == 1 && e < r.bulk8);
+                        } else {
+                            q = bv[u][j][v];
+                        }
+                    }
+                    word |= uint32_t(q & 0xff) << (8 * j);
+                }
+                *reinterpret_cast<uint32_t *>(&tile[(wi + v + g.pad_left) * STAGE_LROW + c]) = word;
+            }
+        }
+    }
+}
+
 template <bool QUANT>
 __global__ __launch_bounds__(256) void stage_rows_kernel(const void *__restrict__ src, StageGeom g,
                                                         const float *__restrict__ scales, int n_scales,
@@ -137,62 +234,20 @@ __global__ __launch_bounds__(256) void stage_rows_kernel(const void *__restrict_
         }
         __syncthreads();
         if (row_inside) {
-            // Lane = (w, channel quad): a lane loads the same pixel of 4 consecutive channels (each
-            // load coalesced along W across lanes), packs the 4 quantized bytes into one dword and
-            // writes it to the tile -- no byte-granular LDS traffic.  WL = power of two >= W keeps the
-            // mapping division-free; loads are issued in batches of NB quads before any is consumed.
-            int wl = 1, wl_shift = 0;
-            while (wl < g.w) {
-                wl <<= 1;
-                ++wl_shift;
-            }
+            // Lane = (run of VW pixels along W, channel quad): see stage_quads.  The widest run the
+            // row length and the source alignment allow keeps the number of load instructions down.
+            const uintptr_t addr = reinterpret_cast<uintptr_t>(src);
+            const int esz = QUANT ? 4 : 1;
+            int vw = 1;
+            if (g.w % 4 == 0 && addr % (4 * esz) == 0) vw = 4;
+            else if (g.w % 2 == 0 && addr % (2 * esz) == 0) vw = 2;
+            int wl = 1;
+            while (wl * vw < g.w) wl <<= 1;
             if (wl <= 64) {
-                constexpr int NB = 4;
-                const int lane = tid & 63, wave = tid >> 6;
-                const int qpw = 64 >> wl_shift;                 // channel quads per wavefront per step
-                const int wi = lane & (wl - 1);
-                const int q_lane = wave * qpw + (lane >> wl_shift);
-                const int qstep = 4 * qpw;                      // quads per workgroup step
-                const bool lane_ok = wi < g.w;
-                const int64_t plane = int64_t(g.h) * g.w;
-                const int64_t row_base = (int64_t(ni) * g.c + c0) * plane + int64_t(hi) * g.w + wi;
-                const int quads = (creal + 3) / 4;
-                for (int qb = 0; qb < quads; qb += NB * qstep) {
-                    float fv[NB][4];
-                    int bv[NB][4];
-#pragma unroll
-                    for (int u = 0; u < NB; ++u) {
-                        const int c = (qb + u * qstep + q_lane) * 4;
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            const bool ok = lane_ok && c + j < creal;
-                            const int64_t e = row_base + int64_t(c + j) * plane;
-                            if (QUANT) fv[u][j] = ok ? static_cast<const float *>(src)[e] : 0.f;
-                            else bv[u][j] = ok ? static_cast<const int8_t *>(src)[e] : 0;
-                        }
-                    }
-#pragma unroll
-                    for (int u = 0; u < NB; ++u) {
-                        const int c = (qb + u * qstep + q_lane) * 4;
-                        if (!(lane_ok && c < creal)) continue;
-                        uint32_t word = 0;
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            int q = 0;
-                            if (c + j < creal) {
-                                if (QUANT) {
-                                    const int64_t e = row_base + int64_t(c + j) * plane;
-                                    const float sc = uniform_scale ? row_scale : scales[e / group_len];
-                                    q = tsx::quantize_value(__fmul_rn(fv[u][j], sc), n_scales == 1 && e < bulk8);
-                                } else {
-                                    q = bv[u][j];
-                                }
-                            }
-                            word |= uint32_t(q & 0xff) << (8 * j);
-                        }
-                        *reinterpret_cast<uint32_t *>(&tile[(wi + g.pad_left) * STAGE_LROW + c]) = word;
-                    }
-                }
+                const StageRow r{src, scales, n_scales, group_len, bulk8, uniform_scale, row_scale, ni, hi, c0, creal};
+                if (vw == 4) stage_quads<QUANT, 4>(g, r, tile, tid);
+                else if (vw == 2) stage_quads<QUANT, 2>(g, r, tile, tid);
+                else stage_quads<QUANT, 1>(g, r, tile, tid);
             } else {
                 for (int idx = tid; idx < creal * g.w; idx += 256) {
                     const int c = idx / g.w, wi = idx - c * g.w;
