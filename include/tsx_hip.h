@@ -66,6 +66,8 @@ int tsx_conv2d_out_size(const tsx_conv2d_geom *g, int32_t *out_h, int32_t *out_w
  *   y = float(acc) * dq[channel]            conv2d_quantized_core.cpp:81-106
  *   y = y * row_scale[row]    if row_scale  (GEMM only: per-row activation dequant)
  *   y = y + bias[channel]     if bias       add_bias.cpp:47-85
+ *   y = y + residual[i]       if residual   add.cpp on equal shapes (a residual join: the
+ *                                           other branch of the block, same shape as the output)
  *   y = act(y)                              relu.cpp / leaky_relu.cpp (incl. their SIMD-body /
  *                                           scalar-tail difference in signed zero and NaN)
  *   q = quantize(y)           if out_i8     quantize.cpp:70-125 with q_scales[n_qscales]
@@ -79,6 +81,7 @@ typedef struct tsx_epilogue {
     const float *q_scales_dev;  /* [n_qscales] quantize_scale of the consumer, or NULL */
     int32_t n_qscales;          /* must equal n (or rows) when q_scales_dev != NULL, as
                                    base_quantize.cpp:26 requires of the consumer */
+    const float *residual_dev;  /* fp32 tensor of the output's shape added before the activation, or NULL */
 } tsx_epilogue;
 
 /* ---------------------------------------------------------------- quantize

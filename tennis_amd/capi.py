@@ -32,7 +32,7 @@ class ConvGeom(ctypes.Structure):
 class Epilogue(ctypes.Structure):
     """tsx_epilogue."""
     _fields_ = [("dq_dev", _vp), ("row_scale_dev", _vp), ("bias_dev", _vp), ("act", _i32), ("slope", _f32),
-                ("q_scales_dev", _vp), ("n_qscales", _i32)]
+                ("q_scales_dev", _vp), ("n_qscales", _i32), ("residual_dev", _vp)]
 
 
 class TsxError(RuntimeError):
@@ -147,13 +147,15 @@ def quantize(x, scales):
 class _EpilogueArgs:
     """Keeps the device tensors of an epilogue alive next to the C struct."""
 
-    def __init__(self, dq, bias=None, act=None, slope=0.0, q_scales=None, row_scale=None):
+    def __init__(self, dq, bias=None, act=None, slope=0.0, q_scales=None, row_scale=None, residual=None):
         self.dq = _dev(dq, torch.float32)
         self.bias = _dev(bias, torch.float32)
         self.q_scales = _dev(q_scales, torch.float32)
         self.row_scale = _dev(row_scale, torch.float32)
+        self.residual = _dev(residual, torch.float32)
         self.c = Epilogue(_ptr(self.dq), _ptr(self.row_scale), _ptr(self.bias), _ACT[act], float(slope),
-                          _ptr(self.q_scales), 0 if self.q_scales is None else self.q_scales.numel())
+                          _ptr(self.q_scales), 0 if self.q_scales is None else self.q_scales.numel(),
+                          _ptr(self.residual))
 
 
 class Conv2dI8:
@@ -186,8 +188,9 @@ class Conv2dI8:
         return geom, self._packed[key], ws_bytes
 
     def __call__(self, x, dq=None, bias=None, act=None, slope=0.0, q_scales=None, x_scales=None,
-                 want_f32=True, want_acc=False):
-        """x: int8 NCHW device tensor, or fp32 NCHW with x_scales (fused quantize).
+                 want_f32=True, want_acc=False, residual=None):
+        """x: int8 NCHW device tensor, or fp32 NCHW with x_scales (fused quantize); residual: fp32 tensor of
+        the output's shape added before the activation.
 
         Returns (out_f32 or None, out_i8 or None, acc_i32 or None)."""
         fused_quant = x_scales is not None
@@ -195,7 +198,9 @@ class Conv2dI8:
         geom, packed, ws_bytes = self._plan(tuple(x.shape))
         ho, wo = conv_out_size(geom)
         shape = (x.shape[0], self.w.shape[0], ho, wo)
-        ep = _EpilogueArgs(dq, bias, act, slope, q_scales) if dq is not None else None
+        ep = _EpilogueArgs(dq, bias, act, slope, q_scales, residual=residual) if dq is not None else None
+        if residual is not None and tuple(residual.shape) != shape:
+            raise TsxError("residual shape %s != output shape %s" % (tuple(residual.shape), shape))
         out_f32 = torch.empty(shape, dtype=torch.float32, device=x.device) if (want_f32 and ep) else None
         out_i8 = torch.empty(shape, dtype=torch.int8, device=x.device) if (ep and q_scales is not None) else None
         acc = torch.empty(shape, dtype=torch.int32, device=x.device) if want_acc else None

@@ -237,11 +237,19 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p) {
                 const int64_t tile_base = (int64_t(img) * p.cout + cf) * howo + int64_t(th0) * p.wo;
                 const unsigned lane_off = unsigned((4 * (lane / 32)) * howo + oh * p.wo + ow);
                 if (pos_ok) {
+                    // the other branch of a residual join: all 16 loads in flight before the first use
+                    float res[16];
+                    static_for<0, 16>([&](auto rc) {
+                        constexpr int r = decltype(rc)::value;
+                        constexpr int dco = 8 * (r / 4) + (r % 4);
+                        res[r] = p.residual ? __builtin_nontemporal_load(&(p.residual + tile_base + int64_t(dco) * howo)[lane_off]) : 0.f;
+                    });
                     static_for<0, 16>([&](auto rc) {
                         constexpr int r = decltype(rc)::value;
                         constexpr int dco = 8 * (r / 4) + (r % 4);
                         float v = __fmul_rn(float(acc[f][j][r]), dq[r]);
                         if (p.bias) v = __fadd_rn(v, bias[r]);
+                        if (p.residual) v = __fadd_rn(v, res[r]);
                         v = apply_act(v, p.act, p.slope, true);
                         // streaming store: the output is not read again by this kernel, and lines that never become dirty
                         // in L2 need no write-back burst when the kernel ends

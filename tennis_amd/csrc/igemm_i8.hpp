@@ -1,5 +1,5 @@
 // Shared device-side pieces of the int8 MFMA kernels: epilogue parameters and the
-// per-accumulator epilogue (dequant -> row scale -> bias -> activation -> requantize).
+// per-accumulator epilogue (dequant -> row scale -> bias -> residual -> activation -> requantize).
 #pragma once
 #include "tsx_common.hpp"
 
@@ -10,6 +10,7 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 struct EpiParams {
     const float *dq, *row_scale, *bias, *q_scales;
+    const float *residual;
     int act;
     float slope;
     int n_qscales;
@@ -26,6 +27,7 @@ __device__ __forceinline__ void emit(const EpiParams &p, int acc, int64_t idx, f
     float v = __fmul_rn(float(acc), dq);
     if (p.row_scale) v = __fmul_rn(v, row_scale);
     if (p.bias) v = __fadd_rn(v, bias);
+    if (p.residual) v = __fadd_rn(v, p.residual[idx]);
     v = apply_act(v, p.act, p.slope, idx < p.act_body);
     if (p.out_f32) p.out_f32[idx] = v;
     if (p.out_i8) {

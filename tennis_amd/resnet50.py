@@ -179,11 +179,13 @@ class ResNet50Int8:
                                            want_f32=qs is None)
             return q if qs is not None else f
 
-        def conv_from_i8(spec, t8, out_scale_name=None):
+        def conv_from_i8(spec, t8, out_scale_name=None, residual=None):
+            """conv -> bias (-> + residual -> relu: the block's join, fused behind the last convolution)."""
             sxs = self._batch_scales(n)
             qs = sxs[out_scale_name] if out_scale_name else None
-            f, q, _ = self.conv[spec.name](t8, dq=self._dq[spec.name], bias=self.bias[spec.name],
-                                           act="relu" if spec.relu else None, q_scales=qs, want_f32=qs is None)
+            act = "relu" if (spec.relu or residual is not None) else None
+            f, q, _ = self.conv[spec.name](t8, dq=self._dq[spec.name], bias=self.bias[spec.name], act=act, q_scales=qs,
+                                           want_f32=qs is None, residual=residual)
             return q if qs is not None else f
 
         y = conv_from_f32(stem, x)
@@ -193,12 +195,13 @@ class ResNet50Int8:
                 a = conv_from_f32(c1, y)
                 b = conv_from_f32(c2, a)
                 c = conv_from_f32(c3, b)
+                sc = conv_from_f32(proj, y) if proj is not None else y
+                y = capi.add(c, sc, "relu")
             else:
+                sc = conv_from_f32(proj, y) if proj is not None else y
                 a8 = conv_from_f32(c1, y, out_scale_name=c2.name)
                 b8 = conv_from_i8(c2, a8, out_scale_name=c3.name)
-                c = conv_from_i8(c3, b8)
-            sc = conv_from_f32(proj, y) if proj is not None else y
-            y = capi.add(c, sc, "relu")
+                y = conv_from_i8(c3, b8, residual=sc)
         pooled = capi.global_pooling2d(y, "avg").reshape(n, fc[0])
         if calibrating:
             self.scales["fc"] = self._scale_of(pooled)

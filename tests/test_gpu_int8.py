@@ -143,6 +143,28 @@ def test_conv2d_i8_epilogue_signed_zero_and_tail(tsx, port):
     assert np.signbit(exp.ravel()[-1])        # 27 elements: the last three are the scalar tail
 
 
+@pytest.mark.parametrize("strides", [(1, 1), (2, 2)])     # window-stationary kernel / generic implicit GEMM
+def test_conv2d_i8_residual_join_in_epilogue(tsx, port, strides):
+    """conv -> add_bias -> add(residual) -> relu (-> quantize) fused, against the separate operators."""
+    rng = np.random.default_rng(204)
+    x, _, wq, dq, bias = c2_like(rng, 3, 70, 12, 11, 37)
+    xq = rng.integers(-128, 128, x.shape).astype(np.int8)
+    conv = tsx.Conv2dI8(_dev(wq), (1, 1, 1, 1), strides)
+    plain = port.conv2d_i8_fused(xq, wq, dq, bias, None, pads=(1, 1, 1, 1), strides=strides)[0]
+    res = (rng.standard_normal(plain.shape) * np.abs(plain).mean()).astype(np.float32)
+    res.ravel()[::5] = -plain.ravel()[::5]                    # exact zeros before the activation
+    qs = np.full(3, 0.05, np.float32)
+    for act in (None, "relu"):
+        out, q, _ = conv(_dev(xq), dq=_dev(dq), bias=_dev(bias), act=act, q_scales=_dev(qs), residual=_dev(res))
+        exp = port.add(plain, res)
+        if act:
+            exp = port.relu(exp)
+        assert np.array_equal(bits(out.cpu().numpy()), bits(exp)), act
+        assert np.array_equal(q.cpu().numpy(), port.quantize(exp, qs))
+    with pytest.raises(tsx.TsxError):
+        conv(_dev(xq), dq=_dev(dq), residual=_dev(res[:, :, :-1]))
+
+
 def test_quantize_conv2d_fused_input(tsx, port):
     rng = np.random.default_rng(203)
     for n in (1, 4):
