@@ -82,6 +82,13 @@ typedef struct tsx_epilogue {
     int32_t n_qscales;          /* must equal n (or rows) when q_scales_dev != NULL, as
                                    base_quantize.cpp:26 requires of the consumer */
     const float *residual_dev;  /* fp32 tensor of the output's shape added before the activation, or NULL */
+    /* Convolutions only: write the requantized int8 output straight into the staged (channel-blocked,
+     * padded) input of the convolution that consumes it, [n][staged_hs][staged_ws][staged_cp] with output
+     * pixel (oh, ow) at (oh + staged_pad_top, ow + staged_pad_left), instead of NCHW -- the consumer then
+     * runs tsx_conv2d_i8_staged_at without a staging pass.  Needs q_scales_dev; the buffer's halo and
+     * channel padding are written once by tsx_conv2d_i8_stage_fill.  NULL = not used. */
+    int8_t *staged_out_dev;
+    int32_t staged_hs, staged_ws, staged_cp, staged_pad_top, staged_pad_left;
 } tsx_epilogue;
 
 /* ---------------------------------------------------------------- quantize
@@ -126,6 +133,21 @@ int tsx_conv2d_i8_stage(const tsx_conv2d_geom *g, const void *x_dev, int32_t x_i
 int tsx_conv2d_i8_staged(const tsx_conv2d_geom *g, const void *staged_dev, const void *packed_w_dev,
                          const tsx_epilogue *ep, float *out_f32_dev, int8_t *out_i8_dev, int32_t *out_acc_dev,
                          void *stream);
+
+/* Chaining quantized convolutions without staging passes (no counterpart in the reference, whose operators
+ * exchange NCHW tensors; values are those of quantize(relu(add_bias(conv))) either way):
+ *   staged_dims : extents [hs][ws][cp] of the staged input the convolution `g` reads (bytes = n*hs*ws*cp);
+ *   stage_fill  : writes the halo value T(padding_value) to every real channel and 0 to the channel padding
+ *                 of a whole staged buffer -- once per buffer; producers only overwrite the interior;
+ *   staged_at   : tsx_conv2d_i8_staged on a staged buffer whose row/column extents are larger than the
+ *                 convolution needs (a buffer shared with another consumer of the same tensor, e.g. a
+ *                 stride-2 1x1 projection reading the staged input of a stride-1 1x1 convolution). */
+int tsx_conv2d_i8_staged_dims(const tsx_conv2d_geom *g, int32_t *hs, int32_t *ws, int32_t *cp);
+int tsx_conv2d_i8_stage_fill(const tsx_conv2d_geom *g, float padding_value, void *staged_dev, size_t staged_bytes,
+                             void *stream);
+int tsx_conv2d_i8_staged_at(const tsx_conv2d_geom *g, const void *staged_dev, int32_t staged_hs, int32_t staged_ws,
+                            const void *packed_w_dev, const tsx_epilogue *ep, float *out_f32_dev, int8_t *out_i8_dev,
+                            int32_t *out_acc_dev, void *stream);
 
 /* ---------------------------------------------------------------- int8 GEMM (quantized inner_prod)
  * cpu::math<int8_t,int32_t>::gemm (src/kernels/cpu/math_cpu.cpp:238-244) followed by the

@@ -32,7 +32,9 @@ class ConvGeom(ctypes.Structure):
 class Epilogue(ctypes.Structure):
     """tsx_epilogue."""
     _fields_ = [("dq_dev", _vp), ("row_scale_dev", _vp), ("bias_dev", _vp), ("act", _i32), ("slope", _f32),
-                ("q_scales_dev", _vp), ("n_qscales", _i32), ("residual_dev", _vp)]
+                ("q_scales_dev", _vp), ("n_qscales", _i32), ("residual_dev", _vp), ("staged_out_dev", _vp),
+                ("staged_hs", _i32), ("staged_ws", _i32), ("staged_cp", _i32), ("staged_pad_top", _i32),
+                ("staged_pad_left", _i32)]
 
 
 class TsxError(RuntimeError):
@@ -59,6 +61,11 @@ SIGNATURES = {
     "tsx_conv2d_i8_stage": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _i32, _vp, _i32, _f32, _vp, _sz, _vp]),
     "tsx_conv2d_i8_staged": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, ctypes.POINTER(Epilogue), _vp, _vp,
                                             _vp, _vp]),
+    "tsx_conv2d_i8_staged_dims": (ctypes.c_int, [ctypes.POINTER(ConvGeom), ctypes.POINTER(_i32), ctypes.POINTER(_i32),
+                                                 ctypes.POINTER(_i32)]),
+    "tsx_conv2d_i8_stage_fill": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _f32, _vp, _sz, _vp]),
+    "tsx_conv2d_i8_staged_at": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _i32, _i32, _vp, ctypes.POINTER(Epilogue), _vp,
+                                               _vp, _vp, _vp]),
     "tsx_gemm_i8_packed_weight_bytes": (_sz, [_i32, _i32]),
     "tsx_gemm_i8_pack_weights": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, _vp]),
     "tsx_gemm_i8_workspace_bytes": (_sz, [_i32, _i32]),
@@ -147,7 +154,7 @@ def quantize(x, scales):
 class _EpilogueArgs:
     """Keeps the device tensors of an epilogue alive next to the C struct."""
 
-    def __init__(self, dq, bias=None, act=None, slope=0.0, q_scales=None, row_scale=None, residual=None):
+    def __init__(self, dq, bias=None, act=None, slope=0.0, q_scales=None, row_scale=None, residual=None, staged_out=None):
         self.dq = _dev(dq, torch.float32)
         self.bias = _dev(bias, torch.float32)
         self.q_scales = _dev(q_scales, torch.float32)
@@ -156,6 +163,26 @@ class _EpilogueArgs:
         self.c = Epilogue(_ptr(self.dq), _ptr(self.row_scale), _ptr(self.bias), _ACT[act], float(slope),
                           _ptr(self.q_scales), 0 if self.q_scales is None else self.q_scales.numel(),
                           _ptr(self.residual))
+        self.staged_out = staged_out     # StagedInput of the consuming convolution
+        if staged_out is not None:
+            self.c.staged_out_dev = staged_out.buf.data_ptr()
+            self.c.staged_hs, self.c.staged_ws, self.c.staged_cp = staged_out.hs, staged_out.ws, staged_out.cp
+            self.c.staged_pad_top, self.c.staged_pad_left = staged_out.pad_top, staged_out.pad_left
+
+
+class StagedInput:
+    """The staged (channel-blocked, padded) int8 input of one convolution for one input shape: producers write
+    their requantized output straight into it, the convolution (and other consumers of the same tensor) read it."""
+
+    def __init__(self, conv, x_shape):
+        geom, _, ws_bytes = conv._plan(tuple(x_shape))
+        hs, ws, cp = _i32(), _i32(), _i32()
+        check(lib().tsx_conv2d_i8_staged_dims(ctypes.byref(geom), ctypes.byref(hs), ctypes.byref(ws), ctypes.byref(cp)))
+        self.x_shape = tuple(x_shape)
+        self.hs, self.ws, self.cp = hs.value, ws.value, cp.value
+        self.pad_top, self.pad_left = conv.pads[0], conv.pads[2]
+        self.buf = torch.empty(max(ws_bytes, 16), dtype=torch.int8, device=conv.w.device)
+        check(lib().tsx_conv2d_i8_stage_fill(ctypes.byref(geom), conv.padding_value, _ptr(self.buf), ws_bytes, _stream()))
 
 
 class Conv2dI8:
@@ -187,8 +214,35 @@ class Conv2dI8:
             self._workspace = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=self.w.device)
         return geom, self._packed[key], ws_bytes
 
+    def stage(self, x, staged, x_scales=None):
+        """Fill a StagedInput from an NCHW tensor: int8, or fp32 quantized with x_scales on the way."""
+        fused_quant = x_scales is not None
+        x = _dev(x, torch.float32 if fused_quant else torch.int8)
+        geom, _, ws_bytes = self._plan(tuple(x.shape))
+        xs = _dev(x_scales, torch.float32)
+        check(lib().tsx_conv2d_i8_stage(ctypes.byref(geom), _ptr(x), int(fused_quant), _ptr(xs),
+                                        0 if xs is None else xs.numel(), self.padding_value, _ptr(staged.buf), ws_bytes,
+                                        _stream()))
+
+    def run_staged(self, staged, dq, bias=None, act=None, slope=0.0, q_scales=None, want_f32=True, residual=None,
+                   staged_out=None):
+        """The convolution on a StagedInput (its own, or another consumer's of the same tensor).  Returns
+        (out_f32 or None, out_i8 or None); with staged_out the int8 output goes to that StagedInput instead."""
+        geom, packed, _ = self._plan(staged.x_shape)
+        ho, wo = conv_out_size(geom)
+        shape = (staged.x_shape[0], self.w.shape[0], ho, wo)
+        if residual is not None and tuple(residual.shape) != shape:
+            raise TsxError("residual shape %s != output shape %s" % (tuple(residual.shape), shape))
+        ep = _EpilogueArgs(dq, bias, act, slope, q_scales, residual=residual, staged_out=staged_out)
+        out_f32 = torch.empty(shape, dtype=torch.float32, device=self.w.device) if want_f32 else None
+        out_i8 = (torch.empty(shape, dtype=torch.int8, device=self.w.device)
+                  if (q_scales is not None and staged_out is None) else None)
+        check(lib().tsx_conv2d_i8_staged_at(ctypes.byref(geom), _ptr(staged.buf), staged.hs, staged.ws, _ptr(packed),
+                                            ctypes.byref(ep.c), _ptr(out_f32), _ptr(out_i8), None, _stream()))
+        return out_f32, out_i8
+
     def __call__(self, x, dq=None, bias=None, act=None, slope=0.0, q_scales=None, x_scales=None,
-                 want_f32=True, want_acc=False, residual=None):
+                 want_f32=True, want_acc=False, residual=None, staged_out=None):
         """x: int8 NCHW device tensor, or fp32 NCHW with x_scales (fused quantize); residual: fp32 tensor of
         the output's shape added before the activation.
 
@@ -198,11 +252,12 @@ class Conv2dI8:
         geom, packed, ws_bytes = self._plan(tuple(x.shape))
         ho, wo = conv_out_size(geom)
         shape = (x.shape[0], self.w.shape[0], ho, wo)
-        ep = _EpilogueArgs(dq, bias, act, slope, q_scales, residual=residual) if dq is not None else None
+        ep = _EpilogueArgs(dq, bias, act, slope, q_scales, residual=residual, staged_out=staged_out) if dq is not None else None
         if residual is not None and tuple(residual.shape) != shape:
             raise TsxError("residual shape %s != output shape %s" % (tuple(residual.shape), shape))
         out_f32 = torch.empty(shape, dtype=torch.float32, device=x.device) if (want_f32 and ep) else None
-        out_i8 = torch.empty(shape, dtype=torch.int8, device=x.device) if (ep and q_scales is not None) else None
+        out_i8 = (torch.empty(shape, dtype=torch.int8, device=x.device)
+                  if (ep and q_scales is not None and staged_out is None) else None)
         acc = torch.empty(shape, dtype=torch.int32, device=x.device) if want_acc else None
         epp = ctypes.byref(ep.c) if ep else None
         if fused_quant:

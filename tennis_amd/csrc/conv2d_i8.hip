@@ -275,6 +275,23 @@ __global__ __launch_bounds__(256) void stage_rows_kernel(const void *__restrict_
     }
 }
 
+// Whole staged buffer = halo: T(padding_value) in the real channels, 0 in the channel padding.
+__global__ __launch_bounds__(256) void stage_fill_kernel(int8_t *__restrict__ xs, int64_t chunks, int cp, int c, int pad_value) {
+    const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id >= chunks) return;
+    const int c0 = int((id * 16) % cp);
+    uint32_t words[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (c0 + v * 4 + j < c) word |= uint32_t(pad_value & 0xff) << (8 * j);
+        words[v] = word;
+    }
+    *reinterpret_cast<uint4 *>(xs + id * 16) = make_uint4(words[0], words[1], words[2], words[3]);
+}
+
 // ------------------------------------------------------------------ weight packing
 
 // packed[ks][frag][half][lane][16]: ks = tap * cblocks + cb (tap = kh*KW + kw),
@@ -546,8 +563,19 @@ int make_plan(const tsx_conv2d_geom *g, Plan *pl) {
 }
 
 int check_epilogue(const tsx_epilogue *ep, const float *out_f32, const int8_t *out_i8, const int32_t *out_acc,
-                   int64_t groups) {
-    TSX_REQUIRE(out_f32 || out_i8 || out_acc, "no output requested");
+                   int64_t groups, int cout = 0, int ho = 0, int wo = 0) {
+    const bool staged_out = ep && ep->staged_out_dev;
+    TSX_REQUIRE(out_f32 || out_i8 || out_acc || staged_out, "no output requested");
+    if (staged_out) {
+        TSX_REQUIRE(cout > 0, "staged output is a convolution-only epilogue term");
+        TSX_REQUIRE(ep->dq_dev && ep->q_scales_dev && ep->n_qscales == groups,
+                    "staged output needs dequantize scales and one consumer quantize scale per image");
+        TSX_REQUIRE(ep->staged_pad_top >= 0 && ep->staged_pad_left >= 0 && ep->staged_cp >= cout && ep->staged_cp % 64 == 0 &&
+                        ho + ep->staged_pad_top <= ep->staged_hs && wo + ep->staged_pad_left <= ep->staged_ws,
+                    "staged output: %dx%dx%d does not fit [%d][%d][%d] at (%d,%d)", ho, wo, cout, ep->staged_hs,
+                    ep->staged_ws, ep->staged_cp, ep->staged_pad_top, ep->staged_pad_left);
+        TSX_REQUIRE(reinterpret_cast<uintptr_t>(ep->staged_out_dev) % 16 == 0, "staged output must be 16-byte aligned");
+    }
     if (out_f32 || out_i8) {
         TSX_REQUIRE(ep && ep->dq_dev, "epilogue with dequantize scales required for fp32/int8 output");
         TSX_REQUIRE(ep->act >= TSX_ACT_NONE && ep->act <= TSX_ACT_LEAKY_RELU, "unknown activation %d", ep->act);
@@ -577,6 +605,14 @@ void fill_epilogue(tsx::EpiParams &p, const tsx_epilogue *ep, int64_t count, flo
     p.out_f32 = out_f32;
     p.out_i8 = out_i8;
     p.out_acc = out_acc;
+    p.st_out = ep ? ep->staged_out_dev : nullptr;
+    if (p.st_out) {
+        p.st_hs = ep->staged_hs;
+        p.st_ws = ep->staged_ws;
+        p.st_cp = ep->staged_cp;
+        p.st_pt = ep->staged_pad_top;
+        p.st_pl = ep->staged_pad_left;
+    }
 }
 
 template <bool SWAP>
@@ -628,7 +664,7 @@ int run_stage(const tsx_conv2d_geom *g, const Plan &pl, const void *x, bool x_is
 
 int run_staged(const tsx_conv2d_geom *g, const Plan &pl, const void *staged, const void *packed_w,
                const tsx_epilogue *ep, float *out_f32, int8_t *out_i8, int32_t *out_acc, hipStream_t stream) {
-    int rc = check_epilogue(ep, out_f32, out_i8, out_acc, g->n);
+    int rc = check_epilogue(ep, out_f32, out_i8, out_acc, g->n, g->cout, pl.ho, pl.wo);
     if (rc) return rc;
     TSX_REQUIRE(staged && packed_w, "conv2d_i8: null input");
     TSX_REQUIRE(!(ep && ep->row_scale_dev), "conv2d_i8: row_scale is a GEMM-only epilogue term");
@@ -653,6 +689,9 @@ int run_staged(const tsx_conv2d_geom *g, const Plan &pl, const void *staged, con
     p.cout = g->cout;
     p.coutp = pl.coutp;
     fill_epilogue(p, ep, int64_t(g->n) * g->cout * pl.ho * pl.wo, out_f32, out_i8, out_acc);
+    p.o_c = g->cout;
+    p.o_h = pl.ho;
+    p.o_w = pl.wo;
     if (pl.use_ws)
         return tsx::ws_launch(pl.wsg, pl.wsp, p.xs, p.wp, static_cast<const tsx::EpiParams &>(p), stream);
     return launch_igemm<false>(p, stream);
@@ -665,7 +704,7 @@ int run_conv(const tsx_conv2d_geom *g, const void *x, bool x_is_f32, const float
     int rc = make_plan(g, &pl);
     if (rc) return rc;
     // validate the second half before launching the first
-    rc = check_epilogue(ep, out_f32, out_i8, out_acc, g->n);
+    rc = check_epilogue(ep, out_f32, out_i8, out_acc, g->n, g->cout, pl.ho, pl.wo);
     if (rc) return rc;
     TSX_REQUIRE(packed_w, "conv2d_i8: null packed weights");
     hipStream_t stream = tsx::as_stream(stream_);
@@ -735,6 +774,57 @@ int tsx_conv2d_i8_staged(const tsx_conv2d_geom *g, const void *staged_dev, const
     Plan pl;
     int rc = make_plan(g, &pl);
     if (rc) return rc;
+    return run_staged(g, pl, staged_dev, packed_w_dev, ep, out_f32_dev, out_i8_dev, out_acc_dev, tsx::as_stream(stream));
+}
+
+int tsx_conv2d_i8_staged_dims(const tsx_conv2d_geom *g, int32_t *hs, int32_t *ws, int32_t *cp) {
+    Plan pl;
+    int rc = make_plan(g, &pl);
+    if (rc) return rc;
+    TSX_REQUIRE(hs && ws && cp, "staged_dims: null output");
+    *hs = pl.hs;
+    *ws = pl.ws;
+    *cp = pl.cp;
+    return 0;
+}
+
+int tsx_conv2d_i8_stage_fill(const tsx_conv2d_geom *g, float padding_value, void *staged_dev, size_t staged_bytes,
+                             void *stream) {
+    Plan pl;
+    int rc = make_plan(g, &pl);
+    if (rc) return rc;
+    TSX_REQUIRE(staged_dev && reinterpret_cast<uintptr_t>(staged_dev) % 16 == 0, "stage_fill: buffer must be 16-byte aligned");
+    TSX_REQUIRE(staged_bytes >= 16 && staged_bytes % size_t(pl.cp) == 0, "stage_fill: size is not a whole number of pixels");
+    const int64_t chunks = int64_t(staged_bytes / 16);
+    hipLaunchKernelGGL(stage_fill_kernel, dim3(unsigned(tsx::ceil_div(chunks, 256))), dim3(256), 0, tsx::as_stream(stream),
+                       static_cast<int8_t *>(staged_dev), chunks, pl.cp, g->c, int(int8_t(padding_value)));
+    TSX_LAUNCH_CHECK("stage_fill_kernel");
+    return 0;
+}
+
+int tsx_conv2d_i8_staged_at(const tsx_conv2d_geom *g, const void *staged_dev, int32_t staged_hs, int32_t staged_ws,
+                            const void *packed_w_dev, const tsx_epilogue *ep, float *out_f32_dev, int8_t *out_i8_dev,
+                            int32_t *out_acc_dev, void *stream) {
+    Plan pl;
+    int rc = make_plan(g, &pl);
+    if (rc) return rc;
+    TSX_REQUIRE(staged_hs >= pl.hs && staged_ws >= pl.ws, "staged_at: buffer rows/columns %dx%d smaller than the %dx%d read",
+                staged_hs, staged_ws, pl.hs, pl.ws);
+    // same kernels, with the buffer's own pitches; the window-stationary plan is re-derived for them
+    pl.hs = staged_hs;
+    pl.ws = staged_ws;
+    if (pl.use_ws) {
+        pl.wsg.hs = staged_hs;
+        pl.wsg.ws = staged_ws;
+        const tsx::WsPlan wide = tsx::ws_plan(pl.wsg);
+        if (wide.ok && wide.packed_bytes == pl.wsp.packed_bytes) {
+            pl.wsp = wide;
+        } else {
+            // weights were packed for the window-stationary kernel: only that kernel can read them
+            return tsx::fail(TSX_E_INVALID, "staged_at: a %dx%d staged buffer does not fit this layer's kernel", staged_hs,
+                             staged_ws);
+        }
+    }
     return run_staged(g, pl, staged_dev, packed_w_dev, ep, out_f32_dev, out_i8_dev, out_acc_dev, tsx::as_stream(stream));
 }
 

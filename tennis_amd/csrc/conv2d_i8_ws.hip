@@ -212,9 +212,10 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p) {
     // a tensor small enough for 32-bit lane offsets, and -- for the requantized output -- one
     // quantize group per image (or a single scale whose round-half-even bulk covers everything),
     // so the consumer's scale is uniform for this tile and needs no per-element division
-    const bool q_uniform = !p.out_i8 || (p.n_qscales == 1 ? p.q_bulk8 == count : p.q_group_len == int64_t(p.cout) * howo);
-    const bool fast = (p.out_f32 || p.out_i8) && !p.out_acc && p.act_body == count && count < (int64_t(1) << 30) && q_uniform;
-    const float q_scale = (fast && p.out_i8) ? p.q_scales[p.n_qscales == 1 ? 0 : img] : 0.f;
+    const bool want_q = p.out_i8 || p.st_out;
+    const bool q_uniform = !want_q || (p.n_qscales == 1 ? p.q_bulk8 == count : p.q_group_len == int64_t(p.cout) * howo);
+    const bool fast = (p.out_f32 || want_q) && !p.out_acc && p.act_body == count && count < (int64_t(1) << 30) && q_uniform;
+    const float q_scale = (fast && want_q) ? p.q_scales[p.n_qscales == 1 ? 0 : img] : 0.f;
     const bool q_even = p.n_qscales == 1;   // single-scale quantize rounds half to even in its bulk
     static_for<0, FM>([&](auto fc) {
         constexpr int f = decltype(fc)::value;
@@ -244,6 +245,7 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p) {
                         constexpr int dco = 8 * (r / 4) + (r % 4);
                         res[r] = p.residual ? __builtin_nontemporal_load(&(p.residual + tile_base + int64_t(dco) * howo)[lane_off]) : 0.f;
                     });
+                    int qv[16];
                     static_for<0, 16>([&](auto rc) {
                         constexpr int r = decltype(rc)::value;
                         constexpr int dco = 8 * (r / 4) + (r % 4);
@@ -254,10 +256,21 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p) {
                         // streaming store: the output is not read again by this kernel, and lines that never become dirty
                         // in L2 need no write-back burst when the kernel ends
                         if (p.out_f32) __builtin_nontemporal_store(v, &(p.out_f32 + tile_base + int64_t(dco) * howo)[lane_off]);
-                        if (p.out_i8)
-                            (p.out_i8 + tile_base + int64_t(dco) * howo)[lane_off] =
-                                int8_t(quantize_value(__fmul_rn(v, q_scale), q_even));
+                        qv[r] = want_q ? quantize_value(__fmul_rn(v, q_scale), q_even) : 0;
+                        if (p.out_i8) (p.out_i8 + tile_base + int64_t(dco) * howo)[lane_off] = int8_t(qv[r]);
                     });
+                    if (p.st_out) {
+                        // consumer's staged layout: accumulator registers 4g..4g+3 of a lane are 4 consecutive
+                        // channels of one pixel -> one dword per group
+                        int8_t *dst = p.st_out + ((int64_t(img) * p.st_hs + th0 + oh + p.st_pt) * p.st_ws + ow + p.st_pl) * p.st_cp +
+                                      cf + 4 * (lane / 32);
+                        static_for<0, 4>([&](auto gc) {
+                            constexpr int g4 = decltype(gc)::value;
+                            const uint32_t word = uint32_t(qv[4 * g4] & 0xff) | (uint32_t(qv[4 * g4 + 1] & 0xff) << 8) |
+                                                  (uint32_t(qv[4 * g4 + 2] & 0xff) << 16) | (uint32_t(qv[4 * g4 + 3] & 0xff) << 24);
+                            *reinterpret_cast<uint32_t *>(dst + 8 * g4) = word;
+                        });
+                    }
                 }
             } else {
                 const int co0 = cf + 4 * (lane / 32);

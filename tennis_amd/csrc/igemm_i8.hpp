@@ -18,21 +18,35 @@ struct EpiParams {
     float *out_f32;
     int8_t *out_i8;
     int32_t *out_acc;
+    // int8 output in the consumer's staged layout [n][st_hs][st_ws][st_cp] (convolutions only)
+    int8_t *st_out;
+    int st_hs, st_ws, st_cp, st_pt, st_pl;
+    int o_c, o_h, o_w;   // NCHW extents of the output, to decode a linear index
 };
 
 // Epilogue of one accumulator; idx is the linear index in the output tensor.
 __device__ __forceinline__ void emit(const EpiParams &p, int acc, int64_t idx, float dq, float bias, float row_scale) {
     if (p.out_acc) p.out_acc[idx] = acc;
-    if (!p.out_f32 && !p.out_i8) return;
+    if (!p.out_f32 && !p.out_i8 && !p.st_out) return;
     float v = __fmul_rn(float(acc), dq);
     if (p.row_scale) v = __fmul_rn(v, row_scale);
     if (p.bias) v = __fadd_rn(v, bias);
     if (p.residual) v = __fadd_rn(v, p.residual[idx]);
     v = apply_act(v, p.act, p.slope, idx < p.act_body);
     if (p.out_f32) p.out_f32[idx] = v;
-    if (p.out_i8) {
+    if (p.out_i8 || p.st_out) {
         const float s = p.n_qscales == 1 ? p.q_scales[0] : p.q_scales[idx / p.q_group_len];
-        p.out_i8[idx] = int8_t(quantize_value(__fmul_rn(v, s), p.n_qscales == 1 && idx < p.q_bulk8));
+        const int8_t q = int8_t(quantize_value(__fmul_rn(v, s), p.n_qscales == 1 && idx < p.q_bulk8));
+        if (p.out_i8) p.out_i8[idx] = q;
+        if (p.st_out) {
+            const int ow = int(idx % p.o_w);
+            const int64_t t1 = idx / p.o_w;
+            const int oh = int(t1 % p.o_h);
+            const int64_t t2 = t1 / p.o_h;
+            const int co = int(t2 % p.o_c);
+            const int64_t n = t2 / p.o_c;
+            p.st_out[((n * p.st_hs + oh + p.st_pt) * p.st_ws + ow + p.st_pl) * p.st_cp + co] = q;
+        }
     }
 }
 

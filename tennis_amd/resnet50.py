@@ -125,6 +125,7 @@ class ResNet50Int8:
         self.sw["fc"] = params["fc"]["sw"]
         self.scales = None      # name -> python float (multiplier applied before rounding)
         self._dq, self._sx = {}, {}
+        self._staged = {}      # (conv name, input shape) -> StagedInput
 
     # ---- calibration: per-tensor scale = 127 / max|input of the layer| on this batch, measured on the
     # activations of the quantized network itself, layer by layer
@@ -157,7 +158,52 @@ class ResNet50Int8:
 
     def forward(self, x):
         assert self.scales is not None, "calibrate() or set_scales() first"
-        return self._forward(x, x.shape[0], calibrating=False)
+        return self._forward_chained(x)
+
+    def _staged_input(self, spec, x_shape):
+        key = (spec.name, tuple(x_shape))
+        if key not in self._staged:
+            self._staged[key] = capi.StagedInput(self.conv[spec.name], x_shape)
+        return self._staged[key]
+
+    def _forward_chained(self, x):
+        """Inference path: between quantized convolutions the activations stay int8 in the consumer's staged
+        layout (written by the producer's epilogue); block outputs are also kept as fp32 NCHW, which the
+        residual join of the next block reads.  Values are those of the operator chain in _forward."""
+        stem, net, fc = self.desc
+        n = x.shape[0]
+        sxs = self._batch_scales(n)
+        relu = lambda spec: "relu" if spec.relu else None
+
+        y = self.conv[stem.name](x, dq=self._dq[stem.name], bias=self.bias[stem.name], act=relu(stem),
+                                 x_scales=sxs[stem.name])[0]
+        y = capi.pooling2d(y, "max", *self.POOL)
+        c1 = net[0][0]
+        s_in = self._staged_input(c1, y.shape)
+        self.conv[c1.name].stage(y, s_in, x_scales=sxs[c1.name])     # the only staging pass after the stem
+        for bi, (c1, c2, c3, proj) in enumerate(net):
+            conv1, conv2, conv3 = self.conv[c1.name], self.conv[c2.name], self.conv[c3.name]
+            in_shape = s_in.x_shape
+            sc = y if proj is None else self.conv[proj.name].run_staged(s_in, self._dq[proj.name], self.bias[proj.name])[0]
+            s2 = self._staged_input(c2, (n, c1.cout, in_shape[2], in_shape[3]))
+            conv1.run_staged(s_in, self._dq[c1.name], self.bias[c1.name], relu(c1), q_scales=sxs[c2.name], want_f32=False,
+                             staged_out=s2)
+            h2 = (in_shape[2] + 2 * c2.pad - c2.k) // c2.stride + 1
+            w2 = (in_shape[3] + 2 * c2.pad - c2.k) // c2.stride + 1
+            s3 = self._staged_input(c3, (n, c2.cout, h2, w2))
+            conv2.run_staged(s2, self._dq[c2.name], self.bias[c2.name], relu(c2), q_scales=sxs[c3.name], want_f32=False,
+                             staged_out=s3)
+            if bi + 1 < len(net):
+                nxt = net[bi + 1][0]
+                s_next = self._staged_input(nxt, (n, c3.cout, h2, w2))
+                y = conv3.run_staged(s3, self._dq[c3.name], self.bias[c3.name], "relu", q_scales=sxs[nxt.name],
+                                     residual=sc, staged_out=s_next)[0]
+                s_in = s_next
+            else:
+                y = conv3.run_staged(s3, self._dq[c3.name], self.bias[c3.name], "relu", residual=sc)[0]
+        pooled = capi.global_pooling2d(y, "avg").reshape(n, fc[0])
+        p8 = capi.quantize(pooled, sxs["fc"])
+        return self.fc(p8, dq=self._dq["fc"], bias=self.bias["fc"])[0]
 
     def _forward(self, x, n, calibrating):
         stem, net, fc = self.desc

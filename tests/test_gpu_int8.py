@@ -165,6 +165,55 @@ def test_conv2d_i8_residual_join_in_epilogue(tsx, port, strides):
         conv(_dev(xq), dq=_dev(dq), residual=_dev(res[:, :, :-1]))
 
 
+@pytest.mark.parametrize("cmid", [64, 37])          # packed dword stores / per-element path (cout not a multiple of 32)
+@pytest.mark.parametrize("a_strides", [(1, 1), (2, 2)])   # producer: window-stationary kernel / generic implicit GEMM
+def test_conv2d_i8_staged_hand_over(tsx, port, cmid, a_strides):
+    """Producer writes its requantized output straight into the consumers' staged input; results must equal
+    the NCHW int8 hand-over (and the oracle) bit for bit.  Two consumers share one staged buffer: a 3x3 p1
+    convolution and -- through its own padded buffer's interior being a superset -- a strided 1x1."""
+    import torch
+    rng = np.random.default_rng(205)
+    n, cin, h, w = 3, 70, 13, 12
+    xq = rng.integers(-128, 128, (n, cin, h, w)).astype(np.int8)
+    wa = rng.integers(-127, 128, (cmid, cin, 3, 3)).astype(np.int8)
+    dqa = rng.uniform(1e-4, 3e-4, cmid).astype(np.float32)
+    ba = rng.standard_normal(cmid).astype(np.float32)
+    qs = np.full(n, 3.0, np.float32)
+    A = tsx.Conv2dI8(_dev(wa), (1, 1, 1, 1), a_strides)
+    ya_f, ya_q, _ = A(_dev(xq), dq=_dev(dqa), bias=_dev(ba), act="relu", q_scales=_dev(qs))
+    exp_f, exp_q = port.conv2d_i8_fused(xq, wa, dqa, ba, "relu", 0.0, qs, (1, 1, 1, 1), a_strides)
+    assert np.array_equal(ya_q.cpu().numpy(), exp_q)
+
+    wb = rng.integers(-127, 128, (48, cmid, 3, 3)).astype(np.int8)
+    wc = rng.integers(-127, 128, (40, cmid, 1, 1)).astype(np.int8)
+    dqb = rng.uniform(1e-4, 3e-4, 48).astype(np.float32)
+    dqc = rng.uniform(1e-4, 3e-4, 40).astype(np.float32)
+    B = tsx.Conv2dI8(_dev(wb), (1, 1, 1, 1))
+    C1 = tsx.Conv2dI8(_dev(wc))                      # 1x1 stride 1: owns the un-padded staged buffer
+    C2 = tsx.Conv2dI8(_dev(wc), strides=(2, 2))      # 1x1 stride 2 reading C1's buffer
+    sb = tsx.StagedInput(B, tuple(ya_q.shape))
+    sc = tsx.StagedInput(C1, tuple(ya_q.shape))
+    for staged in (sb, sc):
+        f, q, _ = A(_dev(xq), dq=_dev(dqa), bias=_dev(ba), act="relu", q_scales=_dev(qs), staged_out=staged)
+        assert q is None and np.array_equal(bits(f.cpu().numpy()), bits(exp_f))
+    got_b = B.run_staged(sb, _dev(dqb))[0].cpu().numpy()
+    assert np.array_equal(bits(got_b), bits(port.conv2d_quantized(exp_q, wb, dqb, (1, 1, 1, 1))))
+    got_c1 = C1.run_staged(sc, _dev(dqc))[0].cpu().numpy()
+    assert np.array_equal(bits(got_c1), bits(port.conv2d_quantized(exp_q, wc, dqc)))
+    sc2 = tsx.StagedInput.__new__(tsx.StagedInput)   # C2's view of C1's buffer
+    sc2.__dict__.update(sc.__dict__)
+    got_c2 = C2.run_staged(sc2, _dev(dqc))[0].cpu().numpy()
+    assert np.array_equal(bits(got_c2), bits(port.conv2d_quantized(exp_q, wc, dqc, strides=(2, 2))))
+    # a second run overwrites only the interior: the halo written once stays valid
+    A(_dev((xq // 2).astype(np.int8)), dq=_dev(dqa), bias=_dev(ba), act="relu", q_scales=_dev(qs), staged_out=sb)
+    exp_q2 = port.conv2d_i8_fused((xq // 2).astype(np.int8), wa, dqa, ba, "relu", 0.0, qs, (1, 1, 1, 1), a_strides)[1]
+    got_b2 = B.run_staged(sb, _dev(dqb))[0].cpu().numpy()
+    assert np.array_equal(bits(got_b2), bits(port.conv2d_quantized(exp_q2, wb, dqb, (1, 1, 1, 1))))
+    with pytest.raises(tsx.TsxError):                # a buffer too small for the producer's output
+        small = tsx.StagedInput(tsx.Conv2dI8(_dev(wb)), (n, cmid, 4, 4))
+        A(_dev(xq), dq=_dev(dqa), q_scales=_dev(qs), staged_out=small)
+
+
 def test_quantize_conv2d_fused_input(tsx, port):
     rng = np.random.default_rng(203)
     for n in (1, 4):
