@@ -24,15 +24,21 @@ struct EpiParams {
     int o_c, o_h, o_w;   // NCHW extents of the output, to decode a linear index
 };
 
-// Epilogue of one accumulator; idx is the linear index in the output tensor.
-__device__ __forceinline__ void emit(const EpiParams &p, int acc, int64_t idx, float dq, float bias, float row_scale) {
-    if (p.out_acc) p.out_acc[idx] = acc;
-    if (!p.out_f32 && !p.out_i8 && !p.st_out) return;
+// fp32 value of one accumulator after dequant -> row scale -> bias -> residual -> activation;
+// idx is the linear index in the output tensor.
+__device__ __forceinline__ float epi_value(const EpiParams &p, int acc, int64_t idx, float dq, float bias, float row_scale) {
     float v = __fmul_rn(float(acc), dq);
     if (p.row_scale) v = __fmul_rn(v, row_scale);
     if (p.bias) v = __fadd_rn(v, bias);
     if (p.residual) v = __fadd_rn(v, p.residual[idx]);
-    v = apply_act(v, p.act, p.slope, idx < p.act_body);
+    return apply_act(v, p.act, p.slope, idx < p.act_body);
+}
+
+// Epilogue of one accumulator: every requested output of element idx.
+__device__ __forceinline__ void emit(const EpiParams &p, int acc, int64_t idx, float dq, float bias, float row_scale) {
+    if (p.out_acc) p.out_acc[idx] = acc;
+    if (!p.out_f32 && !p.out_i8 && !p.st_out) return;
+    const float v = epi_value(p, acc, idx, dq, bias, row_scale);
     if (p.out_f32) p.out_f32[idx] = v;
     if (p.out_i8 || p.st_out) {
         const float s = p.n_qscales == 1 ? p.q_scales[0] : p.q_scales[idx / p.q_group_len];
