@@ -275,6 +275,61 @@ __global__ __launch_bounds__(256) void stage_rows_kernel(const void *__restrict_
     }
 }
 
+// Explicit im2col staging for layers with very few input channels and a large kernel (a 7x7 stem on
+// 3 channels): padding 3 channels to a 64-byte K block per tap would make 95 % of the MFMA work
+// zeros, so the K axis is packed as the reference's im2col does (k = (c*KH + kh)*KW + kw,
+// src/kernels/cpu/im2col.cpp:37-111) and the layer runs as a 1x1 convolution over
+// [n][ho][wo][round_up(C*KH*KW, 64)].  One lane = one 16-byte K chunk of one output pixel; lanes of a
+// pixel are adjacent, so stores are contiguous and the gathered loads stay inside one small patch.
+struct Im2colGeom {
+    int n, c, h, w, ho, wo, kh, kw, sh, sw, dh, dw, pad_top, pad_left, kk, cp, pad_value;
+};
+
+template <bool QUANT>
+__global__ __launch_bounds__(256) void stage_im2col_kernel(const void *__restrict__ src, Im2colGeom g,
+                                                          const float *__restrict__ scales, int n_scales,
+                                                          int64_t group_len, int64_t bulk8, int8_t *__restrict__ xs) {
+    const int chunks = g.cp / 16;
+    const int64_t total = int64_t(g.n) * g.ho * g.wo * chunks;
+    const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id >= total) return;
+    const int chunk = int(id % chunks);
+    int64_t rest = id / chunks;
+    const int ow = int(rest % g.wo);
+    rest /= g.wo;
+    const int oh = int(rest % g.ho);
+    const int ni = int(rest / g.ho);
+    const int taps = g.kh * g.kw;
+    uint32_t words[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int k = chunk * 16 + v * 4 + j;
+            int q = 0;   // K padding: the packed weights are zero there as well
+            if (k < g.kk) {
+                const int ci = k / taps, tap = k - ci * taps;
+                const int kh = tap / g.kw, kw = tap - kh * g.kw;
+                const int hi = oh * g.sh - g.pad_top + kh * g.dh, wi = ow * g.sw - g.pad_left + kw * g.dw;
+                q = g.pad_value;
+                if (hi >= 0 && hi < g.h && wi >= 0 && wi < g.w) {
+                    const int64_t e = ((int64_t(ni) * g.c + ci) * g.h + hi) * g.w + wi;
+                    if (QUANT) {
+                        const float sc = n_scales == 1 ? scales[0] : scales[e / group_len];
+                        q = tsx::quantize_value(__fmul_rn(static_cast<const float *>(src)[e], sc), n_scales == 1 && e < bulk8);
+                    } else {
+                        q = static_cast<const int8_t *>(src)[e];
+                    }
+                }
+            }
+            word |= uint32_t(q & 0xff) << (8 * j);
+        }
+        words[v] = word;
+    }
+    *reinterpret_cast<uint4 *>(xs + id * 16) = make_uint4(words[0], words[1], words[2], words[3]);
+}
+
 // Whole staged buffer = halo: T(padding_value) in the real channels, 0 in the channel padding.
 __global__ __launch_bounds__(256) void stage_fill_kernel(int8_t *__restrict__ xs, int64_t chunks, int cp, int c, int pad_value) {
     const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -566,6 +621,9 @@ struct Plan {
     int ho, wo, hs, ws, cp, cblocks, taps, coutp;
     int64_t positions;
     size_t staged_bytes, packed_bytes;
+    // few input channels x large kernel: K packed by explicit im2col, the layer runs as a 1x1 convolution
+    bool im2col;
+    int kk;   // C*KH*KW
     // stride-1 layers whose tap window fits LDS take the window-stationary kernel
     bool use_ws;
     tsx::WsGeom wsg;
@@ -589,15 +647,26 @@ int make_plan(const tsx_conv2d_geom *g, Plan *pl) {
     pl->cp = int(tsx::round_up(g->c, KSTEP));
     pl->cblocks = pl->cp / KSTEP;
     pl->taps = g->kh * g->kw;
+    pl->kk = g->c * pl->taps;
+    // padding C to 64 per tap wastes (64-C)/64 of the MFMA work; packing K costs a larger staged copy
+    pl->im2col = pl->taps > 1 && g->c <= 8 && pl->kk <= 512;
+    if (pl->im2col) {
+        pl->hs = pl->ho;
+        pl->ws = pl->wo;
+        pl->cp = int(tsx::round_up(pl->kk, KSTEP));
+        pl->cblocks = pl->cp / KSTEP;
+        pl->taps = 1;
+    }
     pl->coutp = int(tsx::round_up(g->cout, BM));
     pl->positions = int64_t(g->n) * pl->ho * pl->wo;
     TSX_REQUIRE(pl->positions < (int64_t(1) << 31), "conv2d_i8: too many output positions");
     pl->staged_bytes = size_t(g->n) * pl->hs * pl->ws * pl->cp;
     pl->packed_bytes = size_t(pl->taps) * pl->cblocks * pl->coutp * KSTEP;
     pl->use_ws = false;
-    if (g->stride_h == 1 && g->stride_w == 1) {
-        pl->wsg = tsx::WsGeom{g->n, g->cout, pl->ho, pl->wo, pl->hs, pl->ws, pl->cp, pl->cblocks, g->kh, g->kw,
-                              g->dilation_h, g->dilation_w};
+    if (pl->im2col || (g->stride_h == 1 && g->stride_w == 1)) {
+        pl->wsg = tsx::WsGeom{g->n, g->cout, pl->ho, pl->wo, pl->hs, pl->ws, pl->cp, pl->cblocks,
+                              pl->im2col ? 1 : g->kh, pl->im2col ? 1 : g->kw,
+                              pl->im2col ? 1 : g->dilation_h, pl->im2col ? 1 : g->dilation_w};
         pl->wsp = tsx::ws_plan(pl->wsg);
         if (pl->wsp.ok) {
             pl->use_ws = true;
@@ -674,6 +743,25 @@ int run_stage(const tsx_conv2d_geom *g, const Plan &pl, const void *x, bool x_is
     if (!staged || staged_bytes < pl.staged_bytes)
         return tsx::fail(TSX_E_WORKSPACE, "conv2d_i8: workspace %zu < %zu bytes", staged_bytes, pl.staged_bytes);
     TSX_REQUIRE(reinterpret_cast<uintptr_t>(staged) % 16 == 0, "conv2d_i8: workspace must be 16-byte aligned");
+    if (pl.im2col) {
+        const Im2colGeom ig{g->n, g->c, g->h, g->w, pl.ho, pl.wo, g->kh, g->kw, g->stride_h, g->stride_w, g->dilation_h,
+                            g->dilation_w, g->pad_top, g->pad_left, pl.kk, pl.cp, int(int8_t(padding_value))};
+        const int64_t threads = int64_t(pl.staged_bytes / 16);
+        const dim3 grid(unsigned(tsx::ceil_div(threads, 256)));
+        if (x_is_f32) {
+            TSX_REQUIRE(x_scales && n_x_scales >= 1, "quantize_conv2d_i8: missing quantize scales");
+            TSX_REQUIRE(n_x_scales == g->n, "quantize_conv2d_i8: n_x_scales (%d) must equal the batch (%d)", n_x_scales, g->n);
+            const int64_t count = int64_t(g->n) * g->c * g->h * g->w;
+            const int64_t group_len = int64_t(std::ceil(static_cast<float>(count) / static_cast<float>(n_x_scales)));
+            hipLaunchKernelGGL(stage_im2col_kernel<true>, grid, dim3(256), 0, stream, x, ig, x_scales, n_x_scales, group_len,
+                               (count >> 3) << 3, static_cast<int8_t *>(staged));
+        } else {
+            hipLaunchKernelGGL(stage_im2col_kernel<false>, grid, dim3(256), 0, stream, x, ig,
+                               static_cast<const float *>(nullptr), 1, int64_t(1), int64_t(0), static_cast<int8_t *>(staged));
+        }
+        TSX_LAUNCH_CHECK("stage_im2col_kernel");
+        return 0;
+    }
     StageGeom sg{g->n, g->c, g->h, g->w, pl.hs, pl.ws, pl.cp, g->pad_top, g->pad_left,
                  int(int8_t(padding_value))};  // T(padding_value), conv2d_quantized_core.cpp:72
     const int64_t stage_threads = int64_t(g->n) * pl.hs * pl.ws * (pl.cp / 16);
@@ -724,11 +812,11 @@ int run_staged(const tsx_conv2d_geom *g, const Plan &pl, const void *staged, con
     p.hs = pl.hs;
     p.ws = pl.ws;
     p.cp = pl.cp;
-    p.stride_h = g->stride_h;
-    p.stride_w = g->stride_w;
-    p.dil_h = g->dilation_h;
-    p.dil_w = g->dilation_w;
-    p.kw = g->kw;
+    p.stride_h = pl.im2col ? 1 : g->stride_h;
+    p.stride_w = pl.im2col ? 1 : g->stride_w;
+    p.dil_h = pl.im2col ? 1 : g->dilation_h;
+    p.dil_w = pl.im2col ? 1 : g->dilation_w;
+    p.kw = pl.im2col ? 1 : g->kw;
     p.taps = pl.taps;
     p.cblocks = pl.cblocks;
     p.cout = g->cout;
@@ -778,12 +866,14 @@ int tsx_conv2d_i8_pack_weights(const tsx_conv2d_geom *g, const int8_t *w_oihw_de
     if (rc) return rc;
     TSX_REQUIRE(w_oihw_dev && packed_dev, "pack_weights: null pointer");
     TSX_REQUIRE(reinterpret_cast<uintptr_t>(packed_dev) % 16 == 0, "pack_weights: packed buffer must be 16-byte aligned");
+    // im2col plans see OIHW weights as [cout][C*KH*KW][1][1]: the same bytes, K in the reference's im2col order
+    const int c_eff = pl.im2col ? pl.kk : g->c;
     if (pl.use_ws)
-        return tsx::ws_pack_weights(pl.wsg, pl.wsp, w_oihw_dev, g->c, static_cast<int8_t *>(packed_dev),
+        return tsx::ws_pack_weights(pl.wsg, pl.wsp, w_oihw_dev, c_eff, static_cast<int8_t *>(packed_dev),
                                     tsx::as_stream(stream));
     const int64_t threads = int64_t(pl.packed_bytes / 16);
     hipLaunchKernelGGL(pack_weights_kernel, dim3(unsigned(tsx::ceil_div(threads, 256))), dim3(256), 0,
-                       tsx::as_stream(stream), w_oihw_dev, g->cout, g->c, pl.taps, int64_t(g->c) * pl.taps,
+                       tsx::as_stream(stream), w_oihw_dev, g->cout, c_eff, pl.taps, int64_t(c_eff) * pl.taps,
                        int64_t(pl.taps), int64_t(1), pl.coutp, pl.cblocks, static_cast<int8_t *>(packed_dev));
     TSX_LAUNCH_CHECK("pack_weights_kernel");
     return 0;
@@ -827,6 +917,7 @@ int tsx_conv2d_i8_staged_dims(const tsx_conv2d_geom *g, int32_t *hs, int32_t *ws
     int rc = make_plan(g, &pl);
     if (rc) return rc;
     TSX_REQUIRE(hs && ws && cp, "staged_dims: null output");
+    TSX_REQUIRE(!pl.im2col, "staged_dims: this layer stages by im2col; a producer cannot write its input");
     *hs = pl.hs;
     *ws = pl.ws;
     *cp = pl.cp;
@@ -838,6 +929,7 @@ int tsx_conv2d_i8_stage_fill(const tsx_conv2d_geom *g, float padding_value, void
     Plan pl;
     int rc = make_plan(g, &pl);
     if (rc) return rc;
+    TSX_REQUIRE(!pl.im2col, "stage_fill: this layer stages by im2col; a producer cannot write its input");
     TSX_REQUIRE(staged_dev && reinterpret_cast<uintptr_t>(staged_dev) % 16 == 0, "stage_fill: buffer must be 16-byte aligned");
     TSX_REQUIRE(staged_bytes >= 16 && staged_bytes % size_t(pl.cp) == 0, "stage_fill: size is not a whole number of pixels");
     const int64_t chunks = int64_t(staged_bytes / 16);
@@ -853,6 +945,7 @@ int tsx_conv2d_i8_staged_at(const tsx_conv2d_geom *g, const void *staged_dev, in
     Plan pl;
     int rc = make_plan(g, &pl);
     if (rc) return rc;
+    TSX_REQUIRE(!pl.im2col || (staged_hs == pl.hs && staged_ws == pl.ws), "staged_at: im2col layers read their own buffer only");
     TSX_REQUIRE(staged_hs >= pl.hs && staged_ws >= pl.ws, "staged_at: buffer rows/columns %dx%d smaller than the %dx%d read",
                 staged_hs, staged_ws, pl.hs, pl.ws);
     // same kernels, with the buffer's own pitches; the window-stationary plan is re-derived for them
