@@ -300,23 +300,29 @@ __global__ __launch_bounds__(256) void stage_im2col_kernel(const void *__restric
     const int oh = int(rest % g.ho);
     const int ni = int(rest / g.ho);
     const int taps = g.kh * g.kw;
+    // one quantize group per image (the usual case) or a single scale: no per-element 64-bit division
+    const bool uniform_scale = QUANT && (n_scales == 1 || group_len == int64_t(g.c) * g.h * g.w);
+    const float img_scale = uniform_scale ? scales[n_scales == 1 ? 0 : ni] : 0.f;
+    // (ci, kh, kw) of the chunk's first K index, then stepped without divisions
+    int k = chunk * 16;
+    int ci = k / taps;
+    int kh = (k - ci * taps) / g.kw;
+    int kw = k - ci * taps - kh * g.kw;
+    const int h0 = oh * g.sh - g.pad_top, w0 = ow * g.sw - g.pad_left;
     uint32_t words[4];
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
         uint32_t word = 0;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int k = chunk * 16 + v * 4 + j;
             int q = 0;   // K padding: the packed weights are zero there as well
             if (k < g.kk) {
-                const int ci = k / taps, tap = k - ci * taps;
-                const int kh = tap / g.kw, kw = tap - kh * g.kw;
-                const int hi = oh * g.sh - g.pad_top + kh * g.dh, wi = ow * g.sw - g.pad_left + kw * g.dw;
+                const int hi = h0 + kh * g.dh, wi = w0 + kw * g.dw;
                 q = g.pad_value;
                 if (hi >= 0 && hi < g.h && wi >= 0 && wi < g.w) {
                     const int64_t e = ((int64_t(ni) * g.c + ci) * g.h + hi) * g.w + wi;
                     if (QUANT) {
-                        const float sc = n_scales == 1 ? scales[0] : scales[e / group_len];
+                        const float sc = uniform_scale ? img_scale : scales[e / group_len];
                         q = tsx::quantize_value(__fmul_rn(static_cast<const float *>(src)[e], sc), n_scales == 1 && e < bulk8);
                     } else {
                         q = static_cast<const int8_t *>(src)[e];
@@ -324,6 +330,14 @@ __global__ __launch_bounds__(256) void stage_im2col_kernel(const void *__restric
                 }
             }
             word |= uint32_t(q & 0xff) << (8 * j);
+            ++k;
+            if (++kw == g.kw) {
+                kw = 0;
+                if (++kh == g.kh) {
+                    kh = 0;
+                    ++ci;
+                }
+            }
         }
         words[v] = word;
     }

@@ -69,8 +69,15 @@ __global__ __launch_bounds__(256) void ws_pack_kernel(const int8_t *__restrict__
     *reinterpret_cast<uint4 *>(packed + id * 16) = make_uint4(words[0], words[1], words[2], words[3]);
 }
 
-template <int NT, int FM>
-__global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p) {
+// EXTRA = false compiles the residual input and the staged-layout output out of the epilogue (fewer
+// registers for the plain dequant + bias + activation case).
+template <int NT, int FM, bool EXTRA>
+__global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
+    WsParams p = p_in;
+    if (!EXTRA) {
+        p.residual = nullptr;
+        p.st_out = nullptr;
+    }
     extern __shared__ __attribute__((aligned(16))) int8_t lds[];   // 2 x wpix x PIX
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const int img = blockIdx.x / p.tiles_per_image;
@@ -228,6 +235,23 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p) {
             dq[r] = (in && p.dq) ? p.dq[co] : 0.f;
             bias[r] = (in && p.bias) ? p.bias[co] : 0.f;
         });
+        // the other branch of a residual join: the loads of every fragment are in flight before the first use
+        float res[NT][16];
+        if (fast && cf + 32 <= p.cout && p.residual) {
+            const int64_t tile_base = (int64_t(img) * p.cout + cf) * howo + int64_t(th0) * p.wo;
+            static_for<0, NT>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                const int pos = j * 32 + lane % 32;
+                const int oh = pos / p.wo, ow = pos - oh * p.wo;
+                const bool pos_ok = pos < tile_pos && th0 + oh < p.ho;
+                const unsigned lane_off = unsigned((4 * (lane / 32)) * howo + oh * p.wo + ow);
+                static_for<0, 16>([&](auto rc) {
+                    constexpr int r = decltype(rc)::value;
+                    constexpr int dco = 8 * (r / 4) + (r % 4);
+                    res[j][r] = pos_ok ? __builtin_nontemporal_load(&(p.residual + tile_base + int64_t(dco) * howo)[lane_off]) : 0.f;
+                });
+            });
+        }
         static_for<0, NT>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
             const int pos = j * 32 + lane % 32;
@@ -238,26 +262,24 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p) {
                 const int64_t tile_base = (int64_t(img) * p.cout + cf) * howo + int64_t(th0) * p.wo;
                 const unsigned lane_off = unsigned((4 * (lane / 32)) * howo + oh * p.wo + ow);
                 if (pos_ok) {
-                    // the other branch of a residual join: all 16 loads in flight before the first use
-                    float res[16];
-                    static_for<0, 16>([&](auto rc) {
-                        constexpr int r = decltype(rc)::value;
-                        constexpr int dco = 8 * (r / 4) + (r % 4);
-                        res[r] = p.residual ? __builtin_nontemporal_load(&(p.residual + tile_base + int64_t(dco) * howo)[lane_off]) : 0.f;
-                    });
                     int qv[16];
                     static_for<0, 16>([&](auto rc) {
                         constexpr int r = decltype(rc)::value;
                         constexpr int dco = 8 * (r / 4) + (r % 4);
                         float v = __fmul_rn(float(acc[f][j][r]), dq[r]);
                         if (p.bias) v = __fadd_rn(v, bias[r]);
-                        if (p.residual) v = __fadd_rn(v, res[r]);
+                        if (p.residual) v = __fadd_rn(v, res[j][r]);
                         v = apply_act(v, p.act, p.slope, true);
                         // streaming store: the output is not read again by this kernel, and lines that never become dirty
                         // in L2 need no write-back burst when the kernel ends
                         if (p.out_f32) __builtin_nontemporal_store(v, &(p.out_f32 + tile_base + int64_t(dco) * howo)[lane_off]);
-                        qv[r] = want_q ? quantize_value(__fmul_rn(v, q_scale), q_even) : 0;
-                        if (p.out_i8) (p.out_i8 + tile_base + int64_t(dco) * howo)[lane_off] = int8_t(qv[r]);
+                        if (EXTRA) {
+                            qv[r] = want_q ? quantize_value(__fmul_rn(v, q_scale), q_even) : 0;
+                            if (p.out_i8) (p.out_i8 + tile_base + int64_t(dco) * howo)[lane_off] = int8_t(qv[r]);
+                        } else if (p.out_i8) {
+                            (p.out_i8 + tile_base + int64_t(dco) * howo)[lane_off] =
+                                int8_t(quantize_value(__fmul_rn(v, q_scale), q_even));
+                        }
                     });
                     if (p.st_out) {
                         // consumer's staged layout: accumulator registers 4g..4g+3 of a lane are 4 consecutive
@@ -290,7 +312,10 @@ template <int NT>
 int launch_nt(const WsParams &p, dim3 grid, size_t lds_bytes, hipStream_t stream) {
     // 32 cout per wavefront (128 per workgroup): two workgroups share a CU, so one
     // wavefront's LDS/L2 waits are covered by the other on the same SIMD.
-    hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM>), grid, dim3(WS_THREADS), lds_bytes, stream, p);
+    if (p.residual || p.st_out)
+        hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, true>), grid, dim3(WS_THREADS), lds_bytes, stream, p);
+    else
+        hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, false>), grid, dim3(WS_THREADS), lds_bytes, stream, p);
     TSX_LAUNCH_CHECK("conv_i8_ws_kernel");
     return 0;
 }
