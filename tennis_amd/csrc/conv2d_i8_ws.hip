@@ -39,6 +39,7 @@ struct WsParams : EpiParams {
     const int8_t *wp;   // packed weights [ks_p][coutp/32][2 halves][64 lanes][16]
     int cout, coutp, ho, wo, hs, ws, cp, cblocks, kh, kw, dil_h, dil_w;
     int th, tiles_per_image, wr, wc, wpix, ksteps_p;
+    int stream_out;   // fp32 output written with streaming stores
 };
 
 // packed[ks][frag][half][lane][16]: ks = cb*taps + tap; frag = cout/32; lane l: cout frag*32 + l%32,
@@ -70,8 +71,8 @@ __global__ __launch_bounds__(256) void ws_pack_kernel(const int8_t *__restrict__
 }
 
 // EXTRA = false compiles the residual input and the staged-layout output out of the epilogue (fewer
-// registers for the plain dequant + bias + activation case).
-template <int NT, int FM, bool EXTRA>
+// registers for the plain dequant + bias + activation case); STREAM selects streaming fp32 stores.
+template <int NT, int FM, bool EXTRA, bool STREAM>
 __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
     WsParams p = p_in;
     if (!EXTRA) {
@@ -270,9 +271,13 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
                         if (p.bias) v = __fadd_rn(v, bias[r]);
                         if (p.residual) v = __fadd_rn(v, res[j][r]);
                         v = apply_act(v, p.act, p.slope, true);
-                        // streaming store: the output is not read again by this kernel, and lines that never become dirty
-                        // in L2 need no write-back burst when the kernel ends
-                        if (p.out_f32) __builtin_nontemporal_store(v, &(p.out_f32 + tile_base + int64_t(dco) * howo)[lane_off]);
+                        // streaming store for large plain outputs: lines that never become dirty in L2 need no
+                        // write-back burst when the kernel ends; outputs a following kernel reads stay cached
+                        if (p.out_f32) {
+                            float *o = &(p.out_f32 + tile_base + int64_t(dco) * howo)[lane_off];
+                            if (STREAM) __builtin_nontemporal_store(v, o);
+                            else *o = v;
+                        }
                         if (EXTRA) {
                             qv[r] = want_q ? quantize_value(__fmul_rn(v, q_scale), q_even) : 0;
                             if (p.out_i8) (p.out_i8 + tile_base + int64_t(dco) * howo)[lane_off] = int8_t(qv[r]);
@@ -313,9 +318,11 @@ int launch_nt(const WsParams &p, dim3 grid, size_t lds_bytes, hipStream_t stream
     // 32 cout per wavefront (128 per workgroup): two workgroups share a CU, so one
     // wavefront's LDS/L2 waits are covered by the other on the same SIMD.
     if (p.residual || p.st_out)
-        hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, true>), grid, dim3(WS_THREADS), lds_bytes, stream, p);
+        hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, true, false>), grid, dim3(WS_THREADS), lds_bytes, stream, p);
+    else if (p.stream_out)
+        hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, false, true>), grid, dim3(WS_THREADS), lds_bytes, stream, p);
     else
-        hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, false>), grid, dim3(WS_THREADS), lds_bytes, stream, p);
+        hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, false, false>), grid, dim3(WS_THREADS), lds_bytes, stream, p);
     TSX_LAUNCH_CHECK("conv_i8_ws_kernel");
     return 0;
 }
@@ -387,6 +394,8 @@ int ws_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t 
     p.wc = pl.wc;
     p.wpix = pl.wp;
     p.ksteps_p = pl.ksteps_p;
+    // an output of L2 size or more that no fused consumer reads: stream it
+    p.stream_out = (!ep.residual && !ep.st_out && ep.out_f32 && int64_t(g.n) * g.cout * g.ho * g.wo * 4 >= (int64_t(16) << 20)) ? 1 : 0;
     const dim3 grid(unsigned(g.n) * pl.tiles_per_image, unsigned(pl.coutp / WS_BM));
     const size_t lds_bytes = size_t(2) * pl.wp * PIX;
     switch (pl.nt) {
