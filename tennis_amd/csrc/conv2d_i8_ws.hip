@@ -263,40 +263,69 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
                 const int64_t tile_base = (int64_t(img) * p.cout + cf) * howo + int64_t(th0) * p.wo;
                 const unsigned lane_off = unsigned((4 * (lane / 32)) * howo + oh * p.wo + ow);
                 if (pos_ok) {
-                    int qv[16];
+                    // One pass per epilogue term over the fragment's 16 accumulators, each behind a single
+                    // uniform branch: testing the (uniform) options per element costs more instructions than
+                    // the arithmetic itself.
+                    float v[16];
                     static_for<0, 16>([&](auto rc) {
                         constexpr int r = decltype(rc)::value;
+                        v[r] = __fmul_rn(float(acc[f][j][r]), dq[r]);
+                    });
+                    if (p.bias) static_for<0, 16>([&](auto rc) {
+                        constexpr int r = decltype(rc)::value;
+                        v[r] = __fadd_rn(v[r], bias[r]);
+                    });
+                    if (EXTRA && p.residual) static_for<0, 16>([&](auto rc) {
+                        constexpr int r = decltype(rc)::value;
+                        v[r] = __fadd_rn(v[r], res[j][r]);
+                    });
+                    if (p.act == TSX_ACT_RELU) {
+                        static_for<0, 16>([&](auto rc) {
+                            constexpr int r = decltype(rc)::value;
+                            v[r] = v[r] > 0.f ? v[r] : 0.f;
+                        });
+                    } else if (p.act == TSX_ACT_LEAKY_RELU) {
+                        static_for<0, 16>([&](auto rc) {
+                            constexpr int r = decltype(rc)::value;
+                            v[r] = apply_act(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
+                        });
+                    }
+                    if (p.out_f32) static_for<0, 16>([&](auto rc) {
+                        constexpr int r = decltype(rc)::value;
                         constexpr int dco = 8 * (r / 4) + (r % 4);
-                        float v = __fmul_rn(float(acc[f][j][r]), dq[r]);
-                        if (p.bias) v = __fadd_rn(v, bias[r]);
-                        if (p.residual) v = __fadd_rn(v, res[j][r]);
-                        v = apply_act(v, p.act, p.slope, true);
                         // streaming store for large plain outputs: lines that never become dirty in L2 need no
                         // write-back burst when the kernel ends; outputs a following kernel reads stay cached
-                        if (p.out_f32) {
-                            float *o = &(p.out_f32 + tile_base + int64_t(dco) * howo)[lane_off];
-                            if (STREAM) __builtin_nontemporal_store(v, o);
-                            else *o = v;
-                        }
-                        if (EXTRA) {
-                            qv[r] = want_q ? quantize_value(__fmul_rn(v, q_scale), q_even) : 0;
-                            if (p.out_i8) (p.out_i8 + tile_base + int64_t(dco) * howo)[lane_off] = int8_t(qv[r]);
-                        } else if (p.out_i8) {
-                            (p.out_i8 + tile_base + int64_t(dco) * howo)[lane_off] =
-                                int8_t(quantize_value(__fmul_rn(v, q_scale), q_even));
-                        }
+                        float *o = &(p.out_f32 + tile_base + int64_t(dco) * howo)[lane_off];
+                        if (STREAM) __builtin_nontemporal_store(v[r], o);
+                        else *o = v[r];
                     });
-                    if (p.st_out) {
-                        // consumer's staged layout: accumulator registers 4g..4g+3 of a lane are 4 consecutive
-                        // channels of one pixel -> one dword per group
-                        int8_t *dst = p.st_out + ((int64_t(img) * p.st_hs + th0 + oh + p.st_pt) * p.st_ws + ow + p.st_pl) * p.st_cp +
-                                      cf + 4 * (lane / 32);
-                        static_for<0, 4>([&](auto gc) {
-                            constexpr int g4 = decltype(gc)::value;
-                            const uint32_t word = uint32_t(qv[4 * g4] & 0xff) | (uint32_t(qv[4 * g4 + 1] & 0xff) << 8) |
-                                                  (uint32_t(qv[4 * g4 + 2] & 0xff) << 16) | (uint32_t(qv[4 * g4 + 3] & 0xff) << 24);
-                            *reinterpret_cast<uint32_t *>(dst + 8 * g4) = word;
+                    if (want_q) {
+                        int qv[16];
+                        if (q_even) static_for<0, 16>([&](auto rc) {
+                            constexpr int r = decltype(rc)::value;
+                            qv[r] = quantize_value(__fmul_rn(v[r], q_scale), true);
                         });
+                        else static_for<0, 16>([&](auto rc) {
+                            constexpr int r = decltype(rc)::value;
+                            qv[r] = quantize_value(__fmul_rn(v[r], q_scale), false);
+                        });
+                        if (p.out_i8) static_for<0, 16>([&](auto rc) {
+                            constexpr int r = decltype(rc)::value;
+                            constexpr int dco = 8 * (r / 4) + (r % 4);
+                            (p.out_i8 + tile_base + int64_t(dco) * howo)[lane_off] = int8_t(qv[r]);
+                        });
+                        if (EXTRA && p.st_out) {
+                            // consumer's staged layout: accumulator registers 4g..4g+3 of a lane are 4 consecutive
+                            // channels of one pixel -> one dword per group
+                            int8_t *dst = p.st_out + ((int64_t(img) * p.st_hs + th0 + oh + p.st_pt) * p.st_ws + ow + p.st_pl) * p.st_cp +
+                                          cf + 4 * (lane / 32);
+                            static_for<0, 4>([&](auto gc) {
+                                constexpr int g4 = decltype(gc)::value;
+                                const uint32_t word = uint32_t(qv[4 * g4] & 0xff) | (uint32_t(qv[4 * g4 + 1] & 0xff) << 8) |
+                                                      (uint32_t(qv[4 * g4 + 2] & 0xff) << 16) | (uint32_t(qv[4 * g4 + 3] & 0xff) << 24);
+                                *reinterpret_cast<uint32_t *>(dst + 8 * g4) = word;
+                            });
+                        }
                     }
                 }
             } else {

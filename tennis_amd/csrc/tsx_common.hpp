@@ -64,13 +64,12 @@ __device__ __forceinline__ void static_for(F &&f) {
 // NaN and |v| >= 2^31 convert to INT_MIN, i.e. -128 after the clamp
 // (src/kernels/cpu/quantize.cpp:15-29,83-96).
 __device__ __forceinline__ int quantize_value(float v, bool half_even) {
-    if (!(__builtin_fabsf(v) < 2147483648.0f)) return -128;
     // rintf = round half to even (_mm256_cvtps_epi32); roundf = half away from zero (round()).
     const float r = half_even ? __builtin_rintf(v) : __builtin_roundf(v);
-    int q = int(r);
-    q = q > 127 ? 127 : q;
-    q = q < -128 ? -128 : q;
-    return q;
+    // selects, not branches: this runs once per output element in the epilogues
+    const float c = __builtin_fminf(__builtin_fmaxf(r, -128.f), 127.f);
+    const bool in_range = __builtin_fabsf(v) < 2147483648.0f;   // false for NaN as well
+    return in_range ? int(c) : -128;
 }
 
 // relu / leaky_relu of element `in_body` (= linear index < 4*floor(count/4) of the whole
