@@ -545,63 +545,56 @@ __global__ __launch_bounds__(WGM *WGN * 64) void igemm_i8_kernel(GemmParams p) {
             const int n = pos / p.howo;
             base[j] = int64_t(n) * p.cout * p.howo + (pos - n * p.howo);
         }
-        // The consumer's staged layout wants 4 consecutive channels of a pixel per dword, which is what
-        // accumulator registers 4g..4g+3 of a lane hold.  Taken when the consumer's quantize scale is
-        // uniform per image (one group per image, or a single scale whose half-even bulk covers all).
+        // Fast path per 32-channel fragment: taken when no raw accumulators are wanted, every element is in
+        // the activation's SIMD-body range and the consumer's quantize scale is uniform per image (one
+        // group per image, or a single scale whose half-even bulk covers everything).
         const int64_t count = int64_t(p.positions) * p.cout;
-        const bool st_fast = p.st_out && (p.n_qscales == 1 ? p.q_bulk8 == count : p.q_group_len == int64_t(p.cout) * p.howo);
-        GemmParams q = p;
-        if (st_fast) q.st_out = nullptr;   // emit() then handles the other outputs only
-        if (q.out_acc || q.out_f32 || q.out_i8 || q.st_out) {
-#pragma unroll
-            for (int i = 0; i < FM; ++i)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int co = m0 + (wm * FM + i) * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
-                    if (co >= p.cout) continue;
-                    const float dq = p.dq ? p.dq[co] : 0.f;
-                    const float bias = p.bias ? p.bias[co] : 0.f;
-#pragma unroll
-                    for (int j = 0; j < FN; ++j)
-                        if (ok[j]) emit(q, acc[i][j][r], base[j] + int64_t(co) * p.howo, dq, bias, 0.f);
-                }
-        }
-        if (st_fast) {
-#pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                if (!ok[j]) continue;
-                const int pos = n0 + (wn * FN + j) * 32 + lane % 32;
-                const int n = pos / p.howo, rem = pos - n * p.howo;
-                const int oh = rem / p.wo, ow = rem - oh * p.wo;
-                int8_t *dst = p.st_out + ((int64_t(n) * p.st_hs + oh + p.st_pt) * p.st_ws + ow + p.st_pl) * p.st_cp;
-                const float qs = p.q_scales[p.n_qscales == 1 ? 0 : n];
-                const bool even = p.n_qscales == 1;
-#pragma unroll
-                for (int i = 0; i < FM; ++i)
-#pragma unroll
-                    for (int g4 = 0; g4 < 4; ++g4) {
-                        const int co0 = m0 + (wm * FM + i) * 32 + 8 * g4 + 4 * (lane / 32);
-                        uint32_t word = 0;
-#pragma unroll
-                        for (int t = 0; t < 4; ++t) {
-                            const int co = co0 + t;
-                            int qv = 0;
-                            if (co < p.cout) {
-                                const float v = tsx::epi_value(p, acc[i][j][4 * g4 + t], base[j] + int64_t(co) * p.howo,
-                                                               p.dq[co], p.bias ? p.bias[co] : 0.f, 0.f);
-                                qv = tsx::quantize_value(__fmul_rn(v, qs), even);
-                            }
-                            word |= uint32_t(qv & 0xff) << (8 * t);
+        const bool want_q = p.out_i8 || p.st_out;
+        const bool q_uniform = !want_q || (p.n_qscales == 1 ? p.q_bulk8 == count : p.q_group_len == int64_t(p.cout) * p.howo);
+        const bool fast = (p.out_f32 || want_q) && !p.out_acc && p.act_body == count && q_uniform;
+        tsx::static_for<0, FM>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            const int cf = m0 + (wm * FM + i) * 32;            // first channel of the fragment (uniform)
+            if (fast && cf + 32 <= p.cout) {
+                const int co0 = cf + 4 * (lane / 32);
+                float dq[16], bias[16];
+                tsx::static_for<0, 16>([&](auto rc) {
+                    constexpr int r = decltype(rc)::value;
+                    const int co = co0 + 8 * (r / 4) + (r % 4);
+                    dq[r] = p.dq[co];
+                    bias[r] = p.bias ? p.bias[co] : 0.f;
+                });
+                tsx::static_for<0, FN>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value;
+                    if (ok[j]) {
+                        const int pos = n0 + (wn * FN + j) * 32 + lane % 32;
+                        const int n = pos / p.howo;
+                        int8_t *st_dst = nullptr;
+                        if (p.st_out) {
+                            const int rem = pos - n * p.howo;
+                            const int oh = rem / p.wo, ow = rem - oh * p.wo;
+                            st_dst = p.st_out + ((int64_t(n) * p.st_hs + oh + p.st_pt) * p.st_ws + ow + p.st_pl) * p.st_cp + co0;
                         }
-                        if (co0 + 3 < p.cout) {
-                            *reinterpret_cast<uint32_t *>(dst + co0) = word;
-                        } else {
-                            for (int t = 0; t < 4; ++t)
-                                if (co0 + t < p.cout) dst[co0 + t] = int8_t(word >> (8 * t));
-                        }
+                        const float qs = want_q ? p.q_scales[p.n_qscales == 1 ? 0 : n] : 0.f;
+                        tsx::epilogue_rows16(p, acc[i][j], dq, bias, base[j] + int64_t(co0) * p.howo, p.howo, qs,
+                                             p.n_qscales == 1, st_dst);
                     }
+                });
+            } else {
+                tsx::static_for<0, 16>([&](auto rc) {
+                    constexpr int r = decltype(rc)::value;
+                    const int co = cf + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
+                    if (co < p.cout) {
+                        const float dq = p.dq ? p.dq[co] : 0.f;
+                        const float bias = p.bias ? p.bias[co] : 0.f;
+                        tsx::static_for<0, FN>([&](auto jc) {
+                            constexpr int j = decltype(jc)::value;
+                            if (ok[j]) emit(p, acc[i][j][r], base[j] + int64_t(co) * p.howo, dq, bias, 0.f);
+                        });
+                    }
+                });
             }
-        }
+        });
     } else {
         // columns = cout (one per lane and i), rows = positions; output is [positions][cout]
         float dq[FM], bias[FM];

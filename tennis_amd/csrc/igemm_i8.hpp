@@ -56,6 +56,63 @@ __device__ __forceinline__ void emit(const EpiParams &p, int acc, int64_t idx, f
     }
 }
 
+// Epilogue of one 32x32 accumulator fragment for one lane, rows = output channels: accumulator r is
+// channel row 8*(r/4) + (r%4) relative to the lane's first row, at linear index idx0 + row * row_stride.
+// One pass per epilogue term behind a single uniform branch each (testing the uniform options per
+// element costs more instructions than the arithmetic).  Caller guarantees: no raw-accumulator
+// output, every element in the activation's SIMD-body range, one quantize scale for this lane's
+// image (q_scale, rounding half to even iff q_even).  st_dst = the lane's pixel in the consumer's
+// staged layout at its first channel row, or null.
+__device__ __forceinline__ void epilogue_rows16(const EpiParams &p, const v16i &acc, const float (&dq)[16],
+                                                const float (&bias)[16], int64_t idx0, int64_t row_stride, float q_scale,
+                                                bool q_even, int8_t *st_dst) {
+    float v[16];
+    static_for<0, 16>([&](auto rc) { constexpr int r = decltype(rc)::value; v[r] = __fmul_rn(float(acc[r]), dq[r]); });
+    if (p.bias) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) v[r] = __fadd_rn(v[r], bias[r]);
+    }
+    if (p.residual) {
+        float res[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) res[r] = p.residual[idx0 + int64_t(8 * (r / 4) + (r % 4)) * row_stride];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) v[r] = __fadd_rn(v[r], res[r]);
+    }
+    if (p.act == TSX_ACT_RELU) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) v[r] = v[r] > 0.f ? v[r] : 0.f;
+    } else if (p.act == TSX_ACT_LEAKY_RELU) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) v[r] = apply_act(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
+    }
+    if (p.out_f32) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) p.out_f32[idx0 + int64_t(8 * (r / 4) + (r % 4)) * row_stride] = v[r];
+    }
+    if (p.out_i8 || st_dst) {
+        int qv[16];
+        if (q_even) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) qv[r] = quantize_value(__fmul_rn(v[r], q_scale), true);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) qv[r] = quantize_value(__fmul_rn(v[r], q_scale), false);
+        }
+        if (p.out_i8) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) p.out_i8[idx0 + int64_t(8 * (r / 4) + (r % 4)) * row_stride] = int8_t(qv[r]);
+        }
+        if (st_dst) {
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4)
+                *reinterpret_cast<uint32_t *>(st_dst + 8 * g4) =
+                    uint32_t(qv[4 * g4] & 0xff) | (uint32_t(qv[4 * g4 + 1] & 0xff) << 8) |
+                    (uint32_t(qv[4 * g4 + 2] & 0xff) << 16) | (uint32_t(qv[4 * g4 + 3] & 0xff) << 24);
+        }
+    }
+}
+
 // ---- window-stationary stride-1 convolution kernel (conv2d_i8_ws.hip) ----
 
 struct WsPlan {
