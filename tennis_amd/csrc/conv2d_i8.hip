@@ -620,6 +620,68 @@ __global__ __launch_bounds__(WGM *WGN * 64) void igemm_i8_kernel(GemmParams p) {
     }
 }
 
+// ------------------------------------------------------------------ skinny int8 GEMM (m <= 32 rows)
+// With at most 32 activation rows the whole left operand is ONE MFMA B fragment and the GEMM is a
+// stream over the packed weights: HBM-bound (K*N bytes), not MFMA-bound.  The 128x128-tile kernel
+// would launch N/128 workgroups and walk K serially; here one workgroup owns 32 output columns and
+// its 8 wavefronts split K (interleaved K-steps, 4 in flight each), then add their int32 partial
+// sums through LDS -- exact, so results equal the tiled kernel's and the oracle's.
+// acc register r of lane l: column (weight row) 8*(r/4) + 4*(l/32) + r%4 of the fragment, activation row l%32.
+constexpr int SK_WAVES = 8;
+constexpr int SK_BATCH = 4;
+
+__global__ __launch_bounds__(SK_WAVES * 64) void gemm_i8_skinny_kernel(GemmParams p) {
+    __shared__ int red[SK_WAVES][16][64];
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const int frag = blockIdx.x;
+    const int frags = p.coutp / 32;
+    const int ksteps = p.cblocks;
+    const int row = lane % 32;
+    const bool row_ok = row < p.positions;
+    // B operand: activation row `row`, the 16 K bytes of group lane/32 of each half K-step
+    const int8_t *b_ptr = p.xs + int64_t(row_ok ? row : 0) * p.cp + (lane / 32) * 16;
+    // A operand: packed[ks][frag][half][lane][16]
+    const int8_t *a_ptr = p.wp + (int64_t(frag) * 128 + lane) * 16;
+    const int64_t a_kstride = int64_t(frags) * 2048;
+    v16i acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0;
+    const v4i zero = {0, 0, 0, 0};
+    for (int ks0 = wave; ks0 < ksteps; ks0 += SK_WAVES * SK_BATCH) {
+        v4i a[SK_BATCH][2], b[SK_BATCH][2];
+        tsx::static_for<0, SK_BATCH>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            const int ks = ks0 + u * SK_WAVES;
+            const bool on = ks < ksteps;
+            const int kk = on ? ks : 0;
+            tsx::static_for<0, 2>([&](auto hc) {
+                constexpr int h = decltype(hc)::value;
+                a[u][h] = on ? *reinterpret_cast<const v4i *>(a_ptr + kk * a_kstride + h * 1024) : zero;
+                b[u][h] = (on && row_ok) ? *reinterpret_cast<const v4i *>(b_ptr + kk * 64 + h * 32) : zero;
+            });
+        });
+        tsx::static_for<0, SK_BATCH>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[u][0], b[u][0], acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[u][1], b[u][1], acc, 0, 0, 0);
+        });
+    }
+    tsx::static_for<0, 16>([&](auto rc) { red[wave][decltype(rc)::value][lane] = acc[decltype(rc)::value]; });
+    __syncthreads();
+    // wavefront w finishes accumulator registers 2w and 2w+1
+    tsx::static_for<0, 2>([&](auto tc) {
+        const int r = wave * 2 + decltype(tc)::value;
+        int sum = 0;
+#pragma unroll
+        for (int w = 0; w < SK_WAVES; ++w) sum += red[w][r][lane];
+        const int co = frag * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
+        if (row_ok && co < p.cout) {
+            const float rs = p.row_scale ? p.row_scale[row] : 0.f;
+            emit(p, sum, int64_t(row) * p.cout + co, p.dq ? p.dq[co] : 0.f, p.bias ? p.bias[co] : 0.f, rs);
+        }
+    });
+}
+
 // ------------------------------------------------------------------ host side
 
 constexpr int BM = 128, BN = 128;
@@ -1038,6 +1100,11 @@ int tsx_gemm_i8(int32_t m, int32_t n, int32_t k, const int8_t *a_dev, const void
     p.cout = n;
     p.coutp = int(tsx::round_up(n, BM));
     fill_epilogue(p, ep, int64_t(m) * n, out_f32_dev, out_i8_dev, out_acc_dev);
+    if (m <= 32) {
+        hipLaunchKernelGGL(gemm_i8_skinny_kernel, dim3(unsigned(tsx::ceil_div(n, 32))), dim3(SK_WAVES * 64), 0, stream, p);
+        TSX_LAUNCH_CHECK("gemm_i8_skinny_kernel");
+        return 0;
+    }
     return launch_igemm<true>(p, stream);
 }
 
