@@ -60,6 +60,10 @@ int tsx_conv2d_out_size(const tsx_conv2d_geom *g, int32_t *out_h, int32_t *out_w
 #define TSX_ACT_NONE       0
 #define TSX_ACT_RELU       1  /* cpu::ReLU      src/kernels/cpu/relu.cpp:30-52 */
 #define TSX_ACT_LEAKY_RELU 2  /* cpu::LeakyReLU src/kernels/cpu/leaky_relu.cpp:41-66 */
+#define TSX_ACT_MISH       3  /* x * tanh(softplus(x)) as the operators softplus, tanh, mul compose it
+                                 (src/kernels/cpu/softplus.cpp:30-39, tanh.cpp:14-23, mul.cpp); the only
+                                 epilogue term that is not bit-exact: device expf/log differ from the host's
+                                 by a few ulp */
 
 /* Fused epilogue applied to the int32 accumulators.  It reproduces, rounding for
  * rounding, the reference's chain of separate operators on the fp32 tensor:
@@ -203,6 +207,21 @@ int tsx_leaky_relu_f32(const float *x_dev, int64_t count, float scale, float *ou
  *   tsx_pooling2d_out_size  pooling2d_forward (include/backend/common_function.h:14-20): ceil mode. */
 int tsx_add_f32(const float *a_dev, const float *b_dev, int64_t count, int32_t act, float slope, float *out_dev,
                 void *stream);
+/*   tsx_mish_f32       mul(x, tanh(softplus(x))) in one pass (TSX_ACT_MISH above)
+ *   tsx_concat_channels_f32  cpu::Concat (src/kernels/cpu/concat.cpp) on dim 1 of NCHW, one call per input:
+ *                      copies src [n][c_src][inner] into channels [c_offset, c_offset + c_src) of dst [n][c_dst][inner]
+ *   tsx_resize_nearest_f32   cpu::Resize2D, Resize2DType::NEAREST, on [planes][h][w] (src/kernels/cpu/resize2d.cpp:186-215:
+ *                      source index round(scale * d + scale/2 - 0.5) in double, clamped)
+ *   tsx_depthwise_conv2d_f32 cpu::DepthwiseConv2D (src/kernels/cpu/depthwise_conv2d_algorithm.cpp:44-85), weights
+ *                      [1][C][KH][KW] (base_depthwise_conv2d.cpp:11-24), geometry as tsx_conv2d_geom with cout == c;
+ *                      optional add_bias + activation fused behind it; same fused-multiply-add order as the reference */
+int tsx_mish_f32(const float *x_dev, int64_t count, float *out_dev, void *stream);
+int tsx_concat_channels_f32(const float *src_dev, int64_t n, int32_t c_src, int64_t inner, float *dst_dev, int32_t c_dst,
+                            int32_t c_offset, void *stream);
+int tsx_resize_nearest_f32(const float *x_dev, int64_t planes, int32_t h, int32_t w, float *out_dev, int32_t out_h,
+                           int32_t out_w, void *stream);
+int tsx_depthwise_conv2d_f32(const tsx_conv2d_geom *g, const float *x_dev, const float *w_dev, float padding_value,
+                             const float *bias_dev, int32_t act, float slope, float *out_dev, void *stream);
 int tsx_pooling2d_out_size(int32_t h, int32_t w, int32_t kh, int32_t kw, int32_t pad_top, int32_t pad_bottom,
                            int32_t pad_left, int32_t pad_right, int32_t stride_h, int32_t stride_w, int32_t *out_h,
                            int32_t *out_w);

@@ -15,6 +15,10 @@
 //   orc_gemm_f32 / orc_conv2d_f32 / orc_inner_prod_f32  fp64 brute force (tolerance) +
 //                         compiled reference (bit-exact, remainder paths included)
 //   orc_winograd_f63 / orc_winograd_f23  fp64 direct conv (tolerance) + compiled reference (bit-exact)
+//   orc_depthwise_conv2d_f32   fp64 brute force (tolerance) + compiled reference depthwise_conv2d (bit-exact on its
+//                         general path, tolerance on its 3x3 SIMD paths)
+//   orc_resize_nearest_f32     index closed form + compiled reference resize2d (bit-exact: a copy)
+//   orc_softplus/tanh/mish     closed forms in fp64 (tolerance) + compiled reference softplus, tanh, mul (bit-exact)
 //   orc_add_f32 / orc_pooling2d_f32      numpy closed forms (max / mean of clipped windows) + compiled
 //                         reference operators add, pooling2d, global_pooling2d (bit-exact)
 #include <algorithm>
@@ -665,6 +669,71 @@ void orc_pooling2d_f32(const float *x, int64_t planes, int h, int w, int type, i
                 }
             }
         }
+    }
+}
+
+// cpu::DepthwiseConv2dAlgorithm<float>::depthwise_general
+// (src/kernels/cpu/depthwise_conv2d_algorithm.cpp:44-85): one filter per channel (multiplier 1),
+// value += w * x over (kh, kw) in order, padding contributing w * padding_value; the reference's
+// FMA build contracts each step to one fused multiply-add.  Its 3x3 stride-1/2 SIMD paths sum the
+// same terms in another order and agree with this to fp32 rounding (tolerance, not bits).
+void orc_depthwise_conv2d_f32(const float *x, int n, int c, int h, int w, const float *wt, int kh, int kw, int pt,
+                              int pb, int pl, int pr, int sh, int sw, int dh, int dw, float padding_value, float *out) {
+    // conv2d_forward (include/backend/common_function.h:30-40)
+    const int ho = (h + pt + pb - (dh * (kh - 1) + 1)) / sh + 1, wo = (w + pl + pr - (dw * (kw - 1) + 1)) / sw + 1;
+#pragma omp parallel for collapse(2) num_threads(g_threads)
+    for (int ni = 0; ni < n; ++ni)
+        for (int ci = 0; ci < c; ++ci) {
+            const float *in = x + (int64_t(ni) * c + ci) * h * w;
+            const float *k = wt + int64_t(ci) * kh * kw;
+            float *o = out + (int64_t(ni) * c + ci) * ho * wo;
+            for (int oh = 0; oh < ho; ++oh)
+                for (int ow = 0; ow < wo; ++ow) {
+                    float value = 0.f;
+                    for (int i = 0; i < kh; ++i)
+                        for (int j = 0; j < kw; ++j) {
+                            const int hi = -pt + oh * sh + i * dh, wi = -pl + ow * sw + j * dw;
+                            const float v = (hi >= 0 && hi < h && wi >= 0 && wi < w) ? in[hi * w + wi] : padding_value;
+                            value = std::fmaf(k[i * kw + j], v, value);
+                        }
+                    o[oh * wo + ow] = value;
+                }
+        }
+}
+
+// Nearest-neighbour resize of [planes][h][w] (src/kernels/cpu/resize2d.cpp:186-215): source index
+// round(scale * d + scale/2 - 0.5) in double, scale = src/dst, clamped to the image.
+void orc_resize_nearest_f32(const float *x, int64_t planes, int h, int w, float *out, int ho, int wo) {
+    const double sx = double(w) / wo, sy = double(h) / ho;
+    const double bx = sx / 2 - 0.5, by = sy / 2 - 0.5;
+#pragma omp parallel for num_threads(g_threads)
+    for (int64_t p = 0; p < planes; ++p)
+        for (int y = 0; y < ho; ++y)
+            for (int xd = 0; xd < wo; ++xd) {
+                int xs = int(std::round(sx * xd + bx)), ys = int(std::round(sy * y + by));
+                xs = xs >= 0 ? xs : 0;
+                xs = xs < w - 1 ? xs : w - 1;
+                ys = ys >= 0 ? ys : 0;
+                ys = ys < h - 1 ? ys : h - 1;
+                out[(p * ho + y) * wo + xd] = (h == ho && w == wo) ? x[(p * h + y) * w + xd] : x[(p * h + ys) * w + xs];
+            }
+}
+
+// Mish as TenniS graphs compose it: x * tanh(softplus(x)) with
+//   softplus  y = float(log(double(expf(x)) + 1.0))        src/kernels/cpu/softplus.cpp:30-39
+//   tanh      2 * (1 / (1 + expf(-2y))) - 1 in float         src/kernels/cpu/tanh.cpp:14-23
+//   mul       x * t                                          src/kernels/cpu/mul.cpp
+void orc_softplus_f32(const float *x, int64_t count, float *out) {
+    for (int64_t i = 0; i < count; ++i) out[i] = static_cast<float>(std::log(std::exp(x[i]) + 1.));
+}
+void orc_tanh_f32(const float *x, int64_t count, float *out) {
+    for (int64_t i = 0; i < count; ++i) out[i] = 2.f * (1.f / (1.f + std::exp(-(2.f * x[i])))) - 1.f;
+}
+void orc_mish_f32(const float *x, int64_t count, float *out) {
+    for (int64_t i = 0; i < count; ++i) {
+        const float sp = static_cast<float>(std::log(std::exp(x[i]) + 1.));
+        const float t = 2.f * (1.f / (1.f + std::exp(-(2.f * sp)))) - 1.f;
+        out[i] = x[i] * t;
     }
 }
 

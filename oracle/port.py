@@ -44,6 +44,10 @@ def lib():
         L.orc_conv2d_f32.argtypes = [_vp, _i, _i, _i, _i, _vp] + [_i] * 11 + [_f, _vp]
         L.orc_inner_prod_f32.argtypes = [_vp, _i, _i, _vp, _i, _i, _vp]
         L.orc_winograd_f63.argtypes = [_vp, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _f, _vp]
+        L.orc_depthwise_conv2d_f32.argtypes = [_vp, _i, _i, _i, _i, _vp] + [_i] * 10 + [_f, _vp]
+        L.orc_resize_nearest_f32.argtypes = [_vp, ctypes.c_int64, _i, _i, _vp, _i, _i]
+        for _n in ('orc_softplus_f32', 'orc_tanh_f32', 'orc_mish_f32'):
+            getattr(L, _n).argtypes = [_vp, ctypes.c_int64, _vp]
         L.orc_add_f32.argtypes = [_vp, _vp, ctypes.c_int64, _vp]
         L.orc_pooling2d_f32.argtypes = [_vp, ctypes.c_int64] + [_i] * 10 + [_vp, _i, _i]
         L.orc_winograd_f23.argtypes = [_vp, _i, _i, _i, _i, _vp, _i, _i, _i, _i, _i, _f, _vp]
@@ -278,3 +282,50 @@ def pooling2d(x, kind, ksize, strides, pads=(0, 0, 0, 0), white=False):
 def global_pooling2d(x, kind):
     """base::GlobalPooling2D (base_global_pooling2d.cpp:58-79) = pooling2d over the whole map, BLACK padding."""
     return pooling2d(x, kind, x.shape[2:], (1, 1))
+
+
+def depthwise_conv2d(x, w, pads=(0, 0, 0, 0), strides=(1, 1), dilations=(1, 1), padding_value=0.0):
+    """cpu::DepthwiseConv2D, general form (depthwise_conv2d_algorithm.cpp:44-85); w is [1, C, KH, KW]."""
+    x = _c(x, np.float32)
+    w = _c(w, np.float32)
+    n, c, h, wd = x.shape
+    assert w.shape[0] == 1 and w.shape[1] == c
+    kh, kw = w.shape[2], w.shape[3]
+    ho, wo = out_hw(h, wd, kh, kw, pads, strides, dilations)
+    out = np.empty((n, c, ho, wo), np.float32)
+    lib().orc_depthwise_conv2d_f32(_p(x), n, c, h, wd, _p(w), kh, kw, *pads, *strides, *dilations, padding_value, _p(out))
+    return out
+
+
+def resize_nearest(x, ho, wo):
+    """cpu::Resize2D, NEAREST, on the two last axes of NCHW (resize2d.cpp:186-215)."""
+    x = _c(x, np.float32)
+    n, c, h, w = x.shape
+    out = np.empty((n, c, ho, wo), np.float32)
+    lib().orc_resize_nearest_f32(_p(x), n * c, h, w, _p(out), ho, wo)
+    return out
+
+
+def _unary(name, x):
+    x = _c(x, np.float32)
+    out = np.empty_like(x)
+    getattr(lib(), name)(_p(x), x.size, _p(out))
+    return out
+
+
+def softplus(x):
+    return _unary("orc_softplus_f32", x)
+
+
+def tanh(x):
+    return _unary("orc_tanh_f32", x)
+
+
+def mish(x):
+    """x * tanh(softplus(x)) with TenniS's softplus and tanh (softplus.cpp:30-39, tanh.cpp:14-23)."""
+    return _unary("orc_mish_f32", x)
+
+
+def concat(tensors, dim=1):
+    """cpu::Concat (src/kernels/cpu/concat.cpp): a copy."""
+    return np.concatenate([np.asarray(t) for t in tensors], axis=dim)

@@ -190,6 +190,23 @@ def global_pooling2d(x, kind, threads=1):
     return run_op("global_pooling2d", p, [x], 4 * x.shape[0] * x.shape[1], threads)
 
 
+def unary(op, x, threads=1):
+    return run_op(op, {}, [x], x.nbytes, threads)
+
+
+def mul(a, b, threads=1):
+    return run_op("mul", {}, [a, b], max(a.nbytes, b.nbytes), threads)
+
+
+def concat(tensors, dim=1, threads=1):
+    return run_op("concat", {"dim": np.array([dim], np.int32)}, list(tensors), sum(t.nbytes for t in tensors), threads)
+
+
+def resize_nearest(x, ho, wo, threads=1):
+    size = np.array([-1, -1, ho, wo], np.int32)
+    return run_op("_resize2d", {"type": np.array([2], np.int32)}, [x, size], 4 * x.shape[0] * x.shape[1] * ho * wo, threads)
+
+
 def inner_prod(lhs, rhs, transpose=False, threads=1):
     n = rhs.shape[0] if transpose else rhs.shape[1]
     return run_op("inner_prod", {"transpose": np.array([transpose], np.bool_)}, [lhs, rhs],

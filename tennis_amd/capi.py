@@ -20,7 +20,7 @@ _f32 = ctypes.c_float
 _sz = ctypes.c_size_t
 
 ACT_NONE, ACT_RELU, ACT_LEAKY_RELU = 0, 1, 2
-_ACT = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "leaky_relu": ACT_LEAKY_RELU}
+_ACT = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "leaky_relu": ACT_LEAKY_RELU, "mish": 3}
 
 
 class ConvGeom(ctypes.Structure):
@@ -76,6 +76,10 @@ SIGNATURES = {
     "tsx_relu_f32": (ctypes.c_int, [_vp, _i64, _vp, _vp]),
     "tsx_leaky_relu_f32": (ctypes.c_int, [_vp, _i64, _f32, _vp, _vp]),
     "tsx_add_f32": (ctypes.c_int, [_vp, _vp, _i64, _i32, _f32, _vp, _vp]),
+    "tsx_mish_f32": (ctypes.c_int, [_vp, _i64, _vp, _vp]),
+    "tsx_concat_channels_f32": (ctypes.c_int, [_vp, _i64, _i32, _i64, _vp, _i32, _i32, _vp]),
+    "tsx_resize_nearest_f32": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32, _i32, _vp]),
+    "tsx_depthwise_conv2d_f32": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, _f32, _vp, _i32, _f32, _vp, _vp]),
     "tsx_pooling2d_out_size": (ctypes.c_int, [_i32] * 10 + [ctypes.POINTER(_i32), ctypes.POINTER(_i32)]),
     "tsx_pooling2d_f32": (ctypes.c_int, [_vp, _i64] + [_i32] * 10 + [_vp, _i32, _i32, _vp]),
     "tsx_winograd_f63_kernel_bytes": (_sz, [_i32, _i32]),
@@ -438,3 +442,51 @@ def pooling2d(x, kind, ksize, strides, pads=(0, 0, 0, 0), white=False):
 
 def global_pooling2d(x, kind):
     return pooling2d(x, kind, tuple(x.shape[2:]), (1, 1))
+
+
+def mish(x):
+    x = _dev(x, torch.float32)
+    out = torch.empty_like(x)
+    check(lib().tsx_mish_f32(_ptr(x), x.numel(), _ptr(out), _stream()))
+    return out
+
+
+def concat_channels(tensors):
+    """cpu::Concat on dim 1 of NCHW tensors."""
+    tensors = [_dev(t, torch.float32) for t in tensors]
+    n, inner = tensors[0].shape[0], 1
+    for d in tensors[0].shape[2:]:
+        inner *= int(d)
+    ctot = sum(t.shape[1] for t in tensors)
+    out = torch.empty((n, ctot) + tuple(tensors[0].shape[2:]), dtype=torch.float32, device=tensors[0].device)
+    off = 0
+    for t in tensors:
+        if t.shape[0] != n or tuple(t.shape[2:]) != tuple(tensors[0].shape[2:]):
+            raise TsxError("concat: shapes differ outside dim 1")
+        check(lib().tsx_concat_channels_f32(_ptr(t), n, t.shape[1], inner, _ptr(out), ctot, off, _stream()))
+        off += t.shape[1]
+    return out
+
+
+def resize_nearest(x, ho, wo):
+    x = _dev(x, torch.float32)
+    n, c, h, w = x.shape
+    out = torch.empty((n, c, ho, wo), dtype=torch.float32, device=x.device)
+    check(lib().tsx_resize_nearest_f32(_ptr(x), n * c, h, w, _ptr(out), ho, wo, _stream()))
+    return out
+
+
+def depthwise_conv2d(x, w, pads=(0, 0, 0, 0), strides=(1, 1), dilations=(1, 1), padding_value=0.0, bias=None, act=None,
+                     slope=0.0):
+    """tsx_depthwise_conv2d_f32: w is [1, C, KH, KW]."""
+    x = _dev(x, torch.float32)
+    w = _dev(w, torch.float32)
+    bias = _dev(bias, torch.float32)
+    n, c, h, wd = x.shape
+    geom = ConvGeom(n, c, h, wd, c, w.shape[2], w.shape[3], pads[0], pads[1], pads[2], pads[3], strides[0], strides[1],
+                    dilations[0], dilations[1])
+    ho, wo = conv_out_size(geom)
+    out = torch.empty((n, c, ho, wo), dtype=torch.float32, device=x.device)
+    check(lib().tsx_depthwise_conv2d_f32(ctypes.byref(geom), _ptr(x), _ptr(w), float(padding_value), _ptr(bias), _ACT[act],
+                                         float(slope), _ptr(out), _stream()))
+    return out

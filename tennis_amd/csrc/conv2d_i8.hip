@@ -606,17 +606,20 @@ __global__ __launch_bounds__(WGM *WGN * 64) void igemm_i8_kernel(GemmParams p) {
             dq[i] = (in && p.dq) ? p.dq[co[i]] : 0.f;
             bias[i] = (in && p.bias) ? p.bias[co[i]] : 0.f;
         }
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
+        tsx::static_for<0, FN>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            tsx::static_for<0, 16>([&](auto rc) {
+                constexpr int r = decltype(rc)::value;
                 const int pos = n0 + (wn * FN + j) * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
-                if (pos >= p.positions) continue;
-                const float rs = p.row_scale ? p.row_scale[pos] : 0.f;
-#pragma unroll
-                for (int i = 0; i < FM; ++i)
-                    if (co[i] < p.cout) emit(p, acc[i][j][r], int64_t(pos) * p.cout + co[i], dq[i], bias[i], rs);
-            }
+                if (pos < p.positions) {
+                    const float rs = p.row_scale ? p.row_scale[pos] : 0.f;
+                    tsx::static_for<0, FM>([&](auto ic) {
+                        constexpr int i = decltype(ic)::value;
+                        if (co[i] < p.cout) emit(p, acc[i][j][r], int64_t(pos) * p.cout + co[i], dq[i], bias[i], rs);
+                    });
+                }
+            });
+        });
     }
 }
 
@@ -761,7 +764,7 @@ int check_epilogue(const tsx_epilogue *ep, const float *out_f32, const int8_t *o
     }
     if (out_f32 || out_i8) {
         TSX_REQUIRE(ep && ep->dq_dev, "epilogue with dequantize scales required for fp32/int8 output");
-        TSX_REQUIRE(ep->act >= TSX_ACT_NONE && ep->act <= TSX_ACT_LEAKY_RELU, "unknown activation %d", ep->act);
+        TSX_REQUIRE(ep->act >= TSX_ACT_NONE && ep->act <= TSX_ACT_MISH, "unknown activation %d", ep->act);
     }
     if (out_i8) {
         TSX_REQUIRE(ep->q_scales_dev, "int8 output needs q_scales_dev");

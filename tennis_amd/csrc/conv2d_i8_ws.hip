@@ -289,6 +289,11 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
                             constexpr int r = decltype(rc)::value;
                             v[r] = apply_act(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
                         });
+                    } else if (p.act == TSX_ACT_MISH) {
+                        static_for<0, 16>([&](auto rc) {
+                            constexpr int r = decltype(rc)::value;
+                            v[r] = apply_act(v[r], TSX_ACT_MISH, 0.f, true);
+                        });
                     }
                     if (p.out_f32) static_for<0, 16>([&](auto rc) {
                         constexpr int r = decltype(rc)::value;

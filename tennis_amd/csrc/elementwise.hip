@@ -12,7 +12,8 @@ namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-// MODE 0: add_bias (layout [pre][channels][inner]); 1: relu; 2: leaky_relu; 3: add (second operand in `bias`) + act
+// MODE 0: add_bias (layout [pre][channels][inner]); 1: relu; 2: leaky_relu; 3: add (second operand in `bias`) + act;
+// 4: mish
 template <int MODE>
 __global__ __launch_bounds__(256) void elementwise_kernel(const float *__restrict__ x, int64_t count,
                                                          const float *__restrict__ bias, int channels, int64_t inner,
@@ -42,6 +43,8 @@ __global__ __launch_bounds__(256) void elementwise_kernel(const float *__restric
                 if (i < count) v[j] = __fadd_rn(v[j], bias[(i / inner) % channels]);
             } else if (MODE == 3) {
                 v[j] = tsx::apply_act(__fadd_rn(v[j], u[j]), act, slope, i < body);
+            } else if (MODE == 4) {
+                v[j] = tsx::apply_act(v[j], TSX_ACT_MISH, 0.f, true);
             } else {
                 v[j] = tsx::apply_act(v[j], MODE == 1 ? TSX_ACT_RELU : TSX_ACT_LEAKY_RELU, slope, i < body);
             }
@@ -94,8 +97,13 @@ int tsx_leaky_relu_f32(const float *x_dev, int64_t count, float scale, float *ou
 int tsx_add_f32(const float *a_dev, const float *b_dev, int64_t count, int32_t act, float slope, float *out_dev,
                 void *stream) {
     TSX_REQUIRE(count >= 0 && (count == 0 || b_dev), "add: bad argument");
-    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_LEAKY_RELU, "add: unknown activation %d", act);
+    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_MISH, "add: unknown activation %d", act);
     return launch<3>(a_dev, count, b_dev, 1, 1, slope, out_dev, stream, act);
+}
+
+int tsx_mish_f32(const float *x_dev, int64_t count, float *out_dev, void *stream) {
+    TSX_REQUIRE(count >= 0, "mish: negative count");
+    return launch<4>(x_dev, count, nullptr, 1, 1, 0.f, out_dev, stream);
 }
 
 }  // extern "C"

@@ -85,6 +85,9 @@ __device__ __forceinline__ void epilogue_rows16(const EpiParams &p, const v16i &
     } else if (p.act == TSX_ACT_LEAKY_RELU) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) v[r] = apply_act(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
+    } else if (p.act == TSX_ACT_MISH) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) v[r] = apply_act(v[r], TSX_ACT_MISH, 0.f, true);
     }
     if (p.out_f32) {
 #pragma unroll

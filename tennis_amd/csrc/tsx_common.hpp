@@ -88,6 +88,15 @@ __device__ __forceinline__ float apply_act(float v, int act, float slope, bool i
         }
         return v > 0.f ? v : __fmul_rn(v, slope);
     }
+    if (act == TSX_ACT_MISH) {
+        // x * tanh(softplus(x)) as TenniS graphs compose it: softplus = float(log(double(expf(x)) + 1.0))
+        // (src/kernels/cpu/softplus.cpp:30-39), tanh = 2 * (1 / (1 + expf(-2y))) - 1 in float
+        // (src/kernels/cpu/tanh.cpp:14-23), then mul.  Same formulas; expf/log are this device's
+        // library routines, so results agree with the host's to a few ulp, not bit for bit.
+        const float sp = float(log(double(expf(v)) + 1.0));
+        const float t = __fsub_rn(__fmul_rn(2.f, __fdiv_rn(1.f, __fadd_rn(1.f, expf(-__fmul_rn(2.f, sp))))), 1.f);
+        return __fmul_rn(v, t);
+    }
     return v;
 }
 

@@ -408,7 +408,7 @@ int tsx_conv2d_winograd_f63_nchw(const tsx_conv2d_geom *q, const float *x_dev, c
     int rc = tsx::make_geom(q, padding_value, &g);
     if (rc) return rc;
     TSX_REQUIRE(x_dev && u_dev && out_dev, "winograd: null argument");
-    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_LEAKY_RELU, "winograd: unknown activation %d", act);
+    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_MISH, "winograd: unknown activation %d", act);
     const size_t need = tsx_winograd_f63_workspace_bytes(q);
     if (!workspace_dev || workspace_bytes < need)
         return tsx::fail(TSX_E_WORKSPACE, "winograd: workspace %zu < %zu bytes", workspace_bytes, need);
@@ -462,7 +462,7 @@ int tsx_conv2d_winograd_f23_nchw(const tsx_conv2d_geom *q, const float *x_dev, c
     int rc = tsx::make_geom(q, padding_value, &g, 2);
     if (rc) return rc;
     TSX_REQUIRE(x_dev && u_dev && out_dev, "winograd_f23: null argument");
-    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_LEAKY_RELU, "winograd_f23: unknown activation %d", act);
+    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_MISH, "winograd_f23: unknown activation %d", act);
     const size_t need = tsx_winograd_f23_workspace_bytes(q);
     if (!workspace_dev || workspace_bytes < need)
         return tsx::fail(TSX_E_WORKSPACE, "winograd_f23: workspace %zu < %zu bytes", workspace_bytes, need);
