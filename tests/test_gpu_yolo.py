@@ -1,0 +1,75 @@
+"""YOLOv4-shaped int8 network: the device runner (tennis_amd/yolov4.py) against the CPU oracle interpreting
+the same layer list operator by operator.
+
+Every operator on the path is bit-exact except Mish (device expf/log), whose few-ulp differences can move a
+value across an int8 rounding boundary of the next quantize; the bar is therefore 2e-3 of the head's largest
+magnitude, with Mish-free (LeakyReLU-only) networks required to match bit for bit.
+"""
+import numpy as np
+import pytest
+
+from _util import bits
+
+pytestmark = pytest.mark.gpu
+
+
+def oracle_forward(port, L, heads, srcs, params, scales, x):
+    n = x.shape[0]
+    outs = []
+    for i, l in enumerate(L):
+        src = [x if j < 0 else outs[j] for j in srcs[i]]
+        if l["type"] == "conv":
+            p, s = params[i], np.float32(scales[i])
+            tq = port.quantize(src[0], np.full(n, s, np.float32))
+            dq = (np.float32(1.0) / (s * p["sw"])).astype(np.float32)
+            pad = l["size"] // 2
+            y = port.add_bias(port.conv2d_quantized(tq, p["wq"], dq, (pad,) * 4, (l["stride"],) * 2), p["bias"])
+            if l["act"] == "mish":
+                y = port.mish(y)
+            elif l["act"] == "leaky_relu":
+                y = port.leaky_relu(y, 0.1)
+        elif l["type"] == "route":
+            y = src[0] if len(src) == 1 else port.concat(src, 1)
+        elif l["type"] == "shortcut":
+            y = port.add(src[0], src[1])
+        elif l["type"] == "maxpool":
+            k = l["size"]
+            y = port.pooling2d(src[0], "max", (k, k), (1, 1), (k // 2,) * 4)
+        elif l["type"] == "upsample":
+            y = port.resize_nearest(src[0], src[0].shape[2] * 2, src[0].shape[3] * 2)
+        outs.append(y)
+    return [outs[h] for h in heads]
+
+
+@pytest.mark.parametrize("mish", [True, False])
+def test_yolov4_shaped_network(port, mish):
+    import torch
+    from tennis_amd import yolov4
+    L, heads = yolov4.layers(width=0.125, classes=3)
+    if not mish:
+        for l in L:
+            if l["type"] == "conv" and l["act"] == "mish":
+                l["act"] = "leaky_relu"
+    params = yolov4.make_parameters(L, seed=5)
+    net = yolov4.YoloV4Int8(L, heads, params)
+    x = np.random.default_rng(6).uniform(0, 1, (2, 3, 64, 64)).astype(np.float32)
+    xd = torch.from_numpy(x).cuda()
+    scales = net.calibrate(xd)
+    got = [t.cpu().numpy() for t in net.forward(xd)]
+    srcs, _ = yolov4.resolve(L)
+    exp = oracle_forward(port, L, heads, srcs, params, scales, x)
+    assert [g.shape for g in got] == [(2, 24, 8, 8), (2, 24, 4, 4), (2, 24, 2, 2)]
+    for g, e in zip(got, exp):
+        assert g.shape == e.shape and np.isfinite(e).all() and np.abs(e).max() > 0
+        if mish:
+            assert np.abs(g - e).max() <= 2e-3 * np.abs(e).max()
+        else:
+            assert np.array_equal(bits(g), bits(e))
+
+
+def test_layer_list_matches_yolov4():
+    from tennis_amd import yolov4
+    L, heads = yolov4.layers()
+    assert sum(1 for l in L if l["type"] == "conv") == 110          # the 110 convolutions of yolov4.cfg
+    macs = yolov4.total_macs(L, 1, 608)
+    assert 60e9 < macs < 68e9                                        # ~64 GMAC per 608x608 image
