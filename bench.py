@@ -123,6 +123,39 @@ def resnet_leg(steps=20):
             "steps": steps, "logits_finite": bool(torch.isfinite(logits).all().item())}
 
 
+def yolo_leg(steps=5):
+    """YOLOv4-shaped int8 network, batch 8 at 3x608x608 (BASELINE config 5): img/s of the whole forward pass
+    (three head tensors), replayed from a captured HIP graph."""
+    import torch
+    from tennis_amd import yolov4
+    n, size = 8, 608
+    L, heads = yolov4.layers()
+    net = yolov4.YoloV4Int8(L, heads, yolov4.make_parameters(L, seed=0))
+    x = torch.rand((n, 3, size, size), device="cuda")
+    net.calibrate(x)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        net.forward(x)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = net.forward(x)
+    graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    macs = yolov4.total_macs(L, n, size)
+    return {"workload": "BASELINE config 5: YOLOv4-shaped int8 network (CSPDarknet53 + SPP + PANet, Mish / LeakyReLU), "
+                        "batch 8, 3x608x608, random-init weights, per-channel int8 weights, per-tensor int8 activations",
+            "img_per_s": n / dt, "ms_per_batch": dt * 1e3, "TOPS": 2.0 * macs / dt / 1e12, "gmac_per_image": macs / n / 1e9,
+            "steps": steps, "outputs_finite": bool(all(torch.isfinite(o).all().item() for o in outs))}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -130,6 +163,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--cpu-images", type=int, default=32, help="images of the batch timed on the CPU (0 = skip)")
     ap.add_argument("--no-resnet", action="store_true", help="skip the ResNet-50-shaped network leg")
+    ap.add_argument("--no-yolo", action="store_true", help="skip the YOLOv4-shaped network leg")
     ap.add_argument("--profile", action="store_true",
                     help="for runs under a profiler: skip the int8-output variant (same kernel name as the roofline "
                          "kernel), the MFMA-rate probe and the CPU baseline, so per-kernel statistics cover the timed "
@@ -271,6 +305,8 @@ def main():
     }
     if not args.no_resnet and not args.profile:
         result["resnet50_int8_bs32"] = resnet_leg()
+    if not args.no_yolo and not args.profile:
+        result["yolov4_int8_bs8"] = yolo_leg()
     if args.cpu_images > 0 and not args.profile:
         result["cpu_baseline"] = cpu_baseline(x, x_scales, wq, dq, bias, pad, min(args.cpu_images, cfg["n"]))
     print(json.dumps(result))
