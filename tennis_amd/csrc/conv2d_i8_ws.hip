@@ -5,8 +5,12 @@
 // Same arithmetic as the generic implicit GEMM in conv2d_i8.hip (exact int32 sums of
 // cpu::Conv2DQuantizedCore, src/kernels/cpu/quantized/conv2d_quantized_core.cpp:18-147), but
 // a different data movement:
-//   * one workgroup (4 wavefronts) owns TH full output rows of one image x 256 output
-//     channels; wavefront w owns channels [64w, 64w+64) and all positions of the tile;
+//   * one workgroup (4 wavefronts) owns TH full output rows x 128 output channels; wavefront w
+//     owns channels [32w, 32w+32) and all positions of the tile.  Rows are counted across the
+//     whole batch (image n's rows follow image n-1's), so a tile may straddle two images: their
+//     staged rows are contiguous in memory, and a position in the second image just reads the
+//     window (KH-1)*dilation rows further down.  Tiles therefore need not divide the image
+//     height (28 rows = 3.5 tiles of 8 rows = 7 position fragments with no padding);
 //   * per 64-channel block the input *window* that all KH*KW taps of the tile read
 //     ((TH + (KH-1)*dil) rows x staged width) is copied once into LDS (double buffered,
 //     one block ahead, 80-byte pixel stride = bank-conflict-free 16-byte reads); every tap is
@@ -37,8 +41,8 @@ constexpr int MAX_WP = MAX_FILL * WS_THREADS / 4;   // 448 window pixels
 struct WsParams : EpiParams {
     const int8_t *xs;   // staged activations [n][hs][ws][cp]
     const int8_t *wp;   // packed weights [ks_p][coutp/32][2 halves][64 lanes][16]
-    int cout, coutp, ho, wo, hs, ws, cp, cblocks, kh, kw, dil_h, dil_w;
-    int th, tiles_per_image, wr, wc, wpix, ksteps_p;
+    int n, cout, coutp, ho, wo, hs, ws, cp, cblocks, kh, kw, dil_h, dil_w;
+    int th, wr, wc, wpix, ksteps_p;
     int stream_out;   // fp32 output written with streaming stores
 };
 
@@ -81,8 +85,11 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
     }
     extern __shared__ __attribute__((aligned(16))) int8_t lds[];   // 2 x wpix x PIX
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
-    const int img = blockIdx.x / p.tiles_per_image;
-    const int th0 = (blockIdx.x - img * p.tiles_per_image) * p.th;   // first output row of the tile
+    const int row0 = blockIdx.x * p.th;      // first output row of the tile, counted over the whole batch
+    const int img = row0 / p.ho;             // image of the tile's first row
+    const int th0 = row0 - img * p.ho;       // ... and that row inside it
+    const int rows_total = p.n * p.ho;
+    const int wrap = p.hs - p.ho;            // staged rows between the last output row of an image and the next image's first
     const int m0 = (blockIdx.y * 4 + wave) * (32 * FM);             // first cout of this wavefront
     const int taps = p.kh * p.kw;
     const int win_bytes = p.wpix * PIX;
@@ -98,9 +105,10 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
         if (pix >= p.wpix) pix = p.wpix - 1;   // duplicates rewrite the same bytes
         int wrow = pix / p.wc;
         const int wcol = pix - wrow * p.wc;
-        int row = th0 + wrow;                  // stride 1: window row r is staged row th0 + r
-        if (row >= p.hs) row = p.hs - 1;       // partial last tile: rows never used by stored outputs
-        fill_src[i] = p.xs + ((int64_t(img) * p.hs + row) * p.ws + wcol) * p.cp + chunk * 16;
+        // stride 1: window row r is staged row (img * hs + th0) + r of the batch-wide staged row sequence
+        int64_t row = int64_t(img) * p.hs + th0 + wrow;
+        if (row >= int64_t(p.n) * p.hs) row = int64_t(p.n) * p.hs - 1;   // last tile: rows no stored output uses
+        fill_src[i] = p.xs + (row * p.ws + wcol) * p.cp + chunk * 16;
         fill_dst[i] = pix * PIX + chunk * 16;
     });
     const int n_fill = (p.wpix * 4 + WS_THREADS - 1) / WS_THREADS;   // <= MAX_FILL, uniform
@@ -125,8 +133,9 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
         constexpr int j = decltype(jc)::value;
         int pos = j * 32 + lane % 32;
         if (pos >= p.th * p.wo) pos = 0;       // padding positions: computed, never stored
-        const int oh = pos / p.wo, ow = pos - oh * p.wo;
-        b_base[j] = (oh * p.wc + ow) * PIX + (lane / 32) * 16;
+        const int r = pos / p.wo, ow = pos - r * p.wo;
+        const int wrow = r + (th0 + r >= p.ho ? wrap : 0);   // positions of the next image sit below its halo rows
+        b_base[j] = (wrow * p.wc + ow) * PIX + (lane / 32) * 16;
     });
 
     // ---- A ring: the wavefront's FM fragments (32 cout each) x 2 halves of K-step ks, 1 KiB each
@@ -215,7 +224,7 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
     // ---- epilogue: accumulator register r of lane l = cout 8*(r/4) + 4*(l/32) + r%4, position l%32
     const int tile_pos = p.th * p.wo;
     const int howo = p.ho * p.wo;
-    const int64_t count = int64_t(gridDim.x / p.tiles_per_image) * p.cout * howo;
+    const int64_t count = int64_t(p.n) * p.cout * howo;
     // hot case: no raw accumulators wanted, every element inside the activation's SIMD-body range,
     // a tensor small enough for 32-bit lane offsets, and -- for the requantized output -- one
     // quantize group per image (or a single scale whose round-half-even bulk covers everything),
@@ -223,7 +232,9 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
     const bool want_q = p.out_i8 || p.st_out;
     const bool q_uniform = !want_q || (p.n_qscales == 1 ? p.q_bulk8 == count : p.q_group_len == int64_t(p.cout) * howo);
     const bool fast = (p.out_f32 || want_q) && !p.out_acc && p.act_body == count && count < (int64_t(1) << 30) && q_uniform;
-    const float q_scale = (fast && want_q) ? p.q_scales[p.n_qscales == 1 ? 0 : img] : 0.f;
+    // a tile may end in the next image: one consumer scale per image, selected per lane
+    const float q_scale_a = (fast && want_q) ? p.q_scales[p.n_qscales == 1 ? 0 : img] : 0.f;
+    const float q_scale_b = (fast && want_q) ? p.q_scales[p.n_qscales == 1 ? 0 : min(img + 1, p.n - 1)] : 0.f;
     const bool q_even = p.n_qscales == 1;   // single-scale quantize rounds half to even in its bulk
     static_for<0, FM>([&](auto fc) {
         constexpr int f = decltype(fc)::value;
@@ -239,13 +250,15 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
         // the other branch of a residual join: the loads of every fragment are in flight before the first use
         float res[NT][16];
         if (fast && cf + 32 <= p.cout && p.residual) {
-            const int64_t tile_base = (int64_t(img) * p.cout + cf) * howo + int64_t(th0) * p.wo;
+            const int64_t tile_base = (int64_t(img) * p.cout + cf) * howo;
             static_for<0, NT>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
                 const int pos = j * 32 + lane % 32;
-                const int oh = pos / p.wo, ow = pos - oh * p.wo;
-                const bool pos_ok = pos < tile_pos && th0 + oh < p.ho;
-                const unsigned lane_off = unsigned((4 * (lane / 32)) * howo + oh * p.wo + ow);
+                const int tr = pos / p.wo, ow = pos - tr * p.wo;
+                const bool wrapped = th0 + tr >= p.ho;
+                const int oh = th0 + tr - (wrapped ? p.ho : 0);
+                const bool pos_ok = pos < tile_pos && row0 + tr < rows_total;
+                const unsigned lane_off = unsigned((wrapped ? p.cout * howo : 0) + (4 * (lane / 32)) * howo + oh * p.wo + ow);
                 static_for<0, 16>([&](auto rc) {
                     constexpr int r = decltype(rc)::value;
                     constexpr int dco = 8 * (r / 4) + (r % 4);
@@ -256,12 +269,15 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
         static_for<0, NT>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
             const int pos = j * 32 + lane % 32;
-            const int oh = pos / p.wo, ow = pos - oh * p.wo;
-            const bool pos_ok = pos < tile_pos && th0 + oh < p.ho;
+            const int tr = pos / p.wo, ow = pos - tr * p.wo;
+            const bool wrapped = th0 + tr >= p.ho;                 // this position belongs to the next image
+            const int oh = th0 + tr - (wrapped ? p.ho : 0);
+            const bool pos_ok = pos < tile_pos && row0 + tr < rows_total;
+            const float q_scale = wrapped ? q_scale_b : q_scale_a;
             if (fast && cf + 32 <= p.cout) {
                 // uniform base in scalar registers + one 32-bit lane offset: no per-store address math
-                const int64_t tile_base = (int64_t(img) * p.cout + cf) * howo + int64_t(th0) * p.wo;
-                const unsigned lane_off = unsigned((4 * (lane / 32)) * howo + oh * p.wo + ow);
+                const int64_t tile_base = (int64_t(img) * p.cout + cf) * howo;
+                const unsigned lane_off = unsigned((wrapped ? p.cout * howo : 0) + (4 * (lane / 32)) * howo + oh * p.wo + ow);
                 if (pos_ok) {
                     // One pass per epilogue term over the fragment's 16 accumulators, each behind a single
                     // uniform branch: testing the (uniform) options per element costs more instructions than
@@ -322,7 +338,7 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
                         if (EXTRA && p.st_out) {
                             // consumer's staged layout: accumulator registers 4g..4g+3 of a lane are 4 consecutive
                             // channels of one pixel -> one dword per group
-                            int8_t *dst = p.st_out + ((int64_t(img) * p.st_hs + th0 + oh + p.st_pt) * p.st_ws + ow + p.st_pl) * p.st_cp +
+                            int8_t *dst = p.st_out + ((int64_t(img + (wrapped ? 1 : 0)) * p.st_hs + oh + p.st_pt) * p.st_ws + ow + p.st_pl) * p.st_cp +
                                           cf + 4 * (lane / 32);
                             static_for<0, 4>([&](auto gc) {
                                 constexpr int g4 = decltype(gc)::value;
@@ -335,7 +351,7 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
                 }
             } else {
                 const int co0 = cf + 4 * (lane / 32);
-                const int64_t base = (int64_t(img) * p.cout + co0) * howo + (th0 + oh) * p.wo + ow;
+                const int64_t base = (int64_t(img + (wrapped ? 1 : 0)) * p.cout + co0) * howo + oh * p.wo + ow;
                 static_for<0, 16>([&](auto rc) {
                     constexpr int r = decltype(rc)::value;
                     constexpr int dco = 8 * (r / 4) + (r % 4);
@@ -366,31 +382,46 @@ int launch_nt(const WsParams &p, dim3 grid, size_t lds_bytes, hipStream_t stream
 WsPlan ws_plan(const WsGeom &g) {
     WsPlan pl{};
     pl.ok = false;
-    // stride-1 only (the caller checks strides); positions of a tile must fit 8 fragments
-    if (g.wo > 128 || g.wo < 1) return pl;
-    int th = 128 / g.wo;
-    if (th > g.ho) th = g.ho;
-    // prefer the row count with the least padding per fragment group
-    int best = th, best_waste = 1 << 30;
-    for (int t = th; t >= 1 && t * 2 > th; --t) {
+    // stride-1 only (the caller checks strides).  A tile is TH output rows of the batch-wide row
+    // sequence, at most MAX_NT fragments of 32 positions.  Candidates are ranked by a model of the
+    // busiest CU's time in units of one fragment's work,
+    //     (workgroups per CU) x (0.5 + fragments x slow),
+    // where 0.5 is the per-workgroup fixed cost and slow = 1.45 for tiles of more than 4 fragments
+    // (one workgroup per CU, so one wavefront per SIMD with nothing to hide its LDS/L2 waits).  The two
+    // constants come from a sweep over 32x256x28x28 (1/2/4/8-row tiles: 35 / 30.5 / 23.0 / 23.4 us) and the
+    // layers of a ResNet-50-shaped network, whose small maps want many small workgroups.  Ties go to the
+    // fewest total fragments (least padding).
+    constexpr int MAX_NT = 7;
+    if (g.wo < 1 || g.wo > 32 * MAX_NT) return pl;
+    const int wrap = g.hs - g.ho;
+    const int coutp = (g.cout + WS_BM - 1) / WS_BM * WS_BM;
+    const int ksteps_p = (g.cblocks * g.kh * g.kw + RING - 1) / RING * RING;
+    double best_cost = -1;
+    int64_t best_frags = 0;
+    for (int t = 1; t <= g.ho && t * g.wo <= 32 * MAX_NT; ++t) {
         const int nt = (t * g.wo + 31) / 32;
-        const int tiles = (g.ho + t - 1) / t;
-        const int waste = tiles * nt * 32 - g.ho * g.wo;
-        if (waste < best_waste) {
-            best_waste = waste;
-            best = t;
+        const int64_t tiles = (int64_t(g.n) * g.ho + t - 1) / t;
+        const bool straddle = g.ho % t != 0;
+        const int wr = t + (g.kh - 1) * g.dil_h + (straddle ? wrap : 0);
+        const int wp = wr * g.ws;
+        if (wp > MAX_WP || size_t(2) * wp * PIX > 65536) continue;   // two windows must fit 64 KiB of LDS
+        const int64_t wgs = tiles * (coutp / WS_BM);
+        const int64_t frags = tiles * nt;
+        const double cost = double((wgs + 255) / 256) * (0.5 + nt * (nt > 4 ? 1.45 : 1.0));
+        if (best_cost < 0 || cost < best_cost || (cost == best_cost && frags < best_frags)) {
+            best_cost = cost;
+            best_frags = frags;
+            pl.th = t;
+            pl.nt = nt;
+            pl.tiles = tiles;
+            pl.wr = wr;
+            pl.wp = wp;
         }
     }
-    pl.th = best;
-    pl.nt = (pl.th * g.wo + 31) / 32;
-    pl.tiles_per_image = (g.ho + pl.th - 1) / pl.th;
-    pl.wr = pl.th + (g.kh - 1) * g.dil_h;
+    if (best_cost < 0 || pl.tiles >= (int64_t(1) << 31)) return pl;
     pl.wc = g.ws;
-    pl.wp = pl.wr * pl.wc;
-    if (pl.wp > MAX_WP || size_t(2) * pl.wp * PIX > 65536) return pl;   // two windows must fit 64 KiB of LDS
-    const int ksteps = g.cblocks * g.kh * g.kw;
-    pl.ksteps_p = (ksteps + RING - 1) / RING * RING;
-    pl.coutp = (g.cout + WS_BM - 1) / WS_BM * WS_BM;
+    pl.ksteps_p = ksteps_p;
+    pl.coutp = coutp;
     pl.packed_bytes = size_t(pl.ksteps_p) * pl.coutp * 64;
     pl.ok = true;
     return pl;
@@ -410,6 +441,7 @@ int ws_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t 
     static_cast<EpiParams &>(p) = ep;
     p.xs = xs;
     p.wp = packed;
+    p.n = g.n;
     p.cout = g.cout;
     p.coutp = pl.coutp;
     p.ho = g.ho;
@@ -423,20 +455,22 @@ int ws_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t 
     p.dil_h = g.dil_h;
     p.dil_w = g.dil_w;
     p.th = pl.th;
-    p.tiles_per_image = pl.tiles_per_image;
     p.wr = pl.wr;
     p.wc = pl.wc;
     p.wpix = pl.wp;
     p.ksteps_p = pl.ksteps_p;
     // an output of L2 size or more that no fused consumer reads: stream it
     p.stream_out = (!ep.residual && !ep.st_out && ep.out_f32 && int64_t(g.n) * g.cout * g.ho * g.wo * 4 >= (int64_t(16) << 20)) ? 1 : 0;
-    const dim3 grid(unsigned(g.n) * pl.tiles_per_image, unsigned(pl.coutp / WS_BM));
+    const dim3 grid(unsigned(pl.tiles), unsigned(pl.coutp / WS_BM));
     const size_t lds_bytes = size_t(2) * pl.wp * PIX;
     switch (pl.nt) {
         case 1: return launch_nt<1>(p, grid, lds_bytes, stream);
         case 2: return launch_nt<2>(p, grid, lds_bytes, stream);
         case 3: return launch_nt<3>(p, grid, lds_bytes, stream);
         case 4: return launch_nt<4>(p, grid, lds_bytes, stream);
+        case 5: return launch_nt<5>(p, grid, lds_bytes, stream);
+        case 6: return launch_nt<6>(p, grid, lds_bytes, stream);
+        case 7: return launch_nt<7>(p, grid, lds_bytes, stream);
     }
     return fail(TSX_E_INVALID, "conv_i8_ws: unsupported fragment count %d", pl.nt);
 }

@@ -121,7 +121,7 @@ __device__ __forceinline__ void epilogue_rows16(const EpiParams &p, const v16i &
 struct WsPlan {
     bool ok;            // geometry supported
     int th, nt;         // output rows per tile, 32-position fragments per tile
-    int tiles_per_image;
+    int64_t tiles;      // tiles over the batch-wide row sequence
     int wr, wc, wp;     // window rows, cols, pixels
     int ksteps_p;       // K-steps padded to the A-ring size
     int coutp;          // cout padded to the workgroup's 256
