@@ -207,6 +207,12 @@ int tsx_leaky_relu_f32(const float *x_dev, int64_t count, float scale, float *ou
  *   tsx_pooling2d_out_size  pooling2d_forward (include/backend/common_function.h:14-20): ceil mode. */
 int tsx_add_f32(const float *a_dev, const float *b_dev, int64_t count, int32_t act, float slope, float *out_dev,
                 void *stream);
+/*   tsx_add_broadcast_f32   cpu::Add::reduce_with_broadcast (src/kernels/cpu/add.cpp) for operands whose shapes,
+ *                      already aligned to `dims` axes (at most 8) as ElementWiseReduce::reduce leaves them
+ *                      (src/backend/base/element_wise_reduce.cpp:150-206), differ: an extent of 1 repeats.  The
+ *                      shape arrays are host memory. */
+int tsx_add_broadcast_f32(const float *lhs_dev, const int32_t *lhs_shape, const float *rhs_dev, const int32_t *rhs_shape,
+                          int32_t dims, float *out_dev, void *stream);
 /*   tsx_mish_f32       mul(x, tanh(softplus(x))) in one pass (TSX_ACT_MISH above)
  *   tsx_concat_channels_f32  cpu::Concat (src/kernels/cpu/concat.cpp) on dim 1 of NCHW, one call per input:
  *                      copies src [n][c_src][inner] into channels [c_offset, c_offset + c_src) of dst [n][c_dst][inner]

@@ -1,0 +1,101 @@
+// The "hip" device operators that sit between the convolutions of whole networks, so that a graph
+// running on the device does not bounce through host memory between two convolutions: pooling2d,
+// global_pooling2d, add (a residual join, with the general broadcast behind it) and depthwise_conv2d.
+// Each class inherits TenniS's device-agnostic skeleton and implements the core method over the
+// C ABI in include/tsx_hip.h, as TenniS's own device backends do (src/kernels/gpu/pooling2d.cu,
+// add.cu, depthwise_conv2d.cu).
+#define TSX_TS_GLUE_OPS
+#include "hip_ops_common.h"
+
+namespace ts {
+namespace hip {
+
+namespace {
+// The pooling kernel works on [planes][h][w]: only NCHW maps fold into that.
+void pool_nchw(const char *who, const Tensor &x, Pooling2DType type, const Padding2D &padding, Padding2DType padding_type,
+               const Size2D &ksize, const Stride2D &stride, Conv2DFormat format, Tensor &out) {
+    if (format != FORMAT_NCHW) TS_LOG_ERROR << who << " only support NCHW" << eject;
+    if (x.dtype() != FLOAT32) TS_LOG_ERROR << who << " not support data type(" << x.dtype() << "): " << type_str(x.dtype()) << eject;
+    if (type != Pooling2DType::MAX && type != Pooling2DType::AVG)
+        TS_LOG_ERROR << who << " not support pooling type: " << int(type) << eject;
+    // cpu::Pooling2DCore (src/kernels/cpu/pooling2d_core.cpp:48-186) knows BLACK and WHITE only
+    if (padding_type != Padding2DType::BLACK && padding_type != Padding2DType::WHITE)
+        TS_LOG_ERROR << who << " not support padding type: " << int(padding_type) << eject;
+    check(tsx_pooling2d_f32(x.data<float>(), int64_t(x.size(0)) * x.size(1), x.size(2), x.size(3), int(type), padding.top,
+                            padding.left, ksize.height, ksize.width, stride.height, stride.width,
+                            padding_type == Padding2DType::WHITE ? 1 : 0, out.data<float>(), out.size(2), out.size(3),
+                            current_stream()),
+          "tsx_pooling2d_f32");
+}
+}  // namespace
+
+class Pooling2D : public OperatorOnHip<base::Pooling2D> {
+public:
+    void pooling2d(const Tensor &x, Pooling2DType type, const Padding2D &padding, Padding2DType padding_type,
+                   const Size2D &ksize, const Stride2D &stride, Conv2DFormat format, Tensor &out) override {
+        pool_nchw("Pooling2D", x, type, padding, padding_type, ksize, stride, format, out);
+    }
+};
+
+class GlobalPooling2D : public OperatorOnHip<base::GlobalPooling2D> {
+public:
+    void pooling2d(const Tensor &x, Pooling2DType type, const Padding2D &padding, Padding2DType padding_type,
+                   const Size2D &ksize, const Stride2D &stride, Conv2DFormat format, Tensor &out) override {
+        pool_nchw("GlobalPooling2D", x, type, padding, padding_type, ksize, stride, format, out);
+    }
+};
+
+// add: equal shapes take the vectorised pass; every other case of ElementWiseReduce::run (scalar,
+// bias along one axis, general broadcast, either operand) is one broadcast kernel, so the
+// specialised hooks keep the skeleton's default (which forwards to reduce_with_broadcast).
+class Add : public OperatorOnHip<base::Add> {
+public:
+    void reduce_with_same_shape(const Tensor &lhs, const Tensor &rhs, Tensor &out) override {
+        check_type(out);
+        check(tsx_add_f32(lhs.data<float>(), rhs.data<float>(), out.count(), TSX_ACT_NONE, 0.f, out.data<float>(), current_stream()),
+              "tsx_add_f32");
+    }
+
+    void reduce_with_broadcast(const Tensor &lhs, const Tensor &rhs, Tensor &out) override {
+        check_type(out);
+        const Shape &ls = lhs.sizes(), &rs = rhs.sizes();
+        if (ls.size() != rs.size() || ls.size() > 8)
+            TS_LOG_ERROR << "[hip] add: can not broadcast " << to_string(ls) << " with " << to_string(rs) << eject;
+        const std::vector<int32_t> l(ls.begin(), ls.end()), r(rs.begin(), rs.end());
+        check(tsx_add_broadcast_f32(lhs.data<float>(), l.data(), rhs.data<float>(), r.data(), int32_t(l.size()), out.data<float>(),
+                                    current_stream()),
+              "tsx_add_broadcast_f32");
+    }
+
+private:
+    static void check_type(const Tensor &out) {
+        if (out.dtype() != FLOAT32) TS_LOG_ERROR << "[hip] add not support data type(" << out.dtype() << "): " << type_str(out.dtype()) << eject;
+    }
+};
+
+// depthwise_conv2d: weights [1, C, KH, KW]; the core signature is base::Conv2D's.
+class DepthwiseConv2D : public OperatorOnHip<base::DepthwiseConv2D> {
+public:
+    void conv2d(const Tensor &x, const Padding2D &padding, float padding_value, const Tensor &w, const Stride2D &stride,
+                const Dilation2D &dilation, Conv2DFormat format, Tensor &out, Stack &, bool kernel_packed) override {
+        if (format != FORMAT_NCHW) TS_LOG_ERROR << "DepthwiseConv2D only support NCHW" << eject;
+        if (out.dtype() != FLOAT32)
+            TS_LOG_ERROR << "DepthwiseConv2D not support data type(" << out.dtype() << "): " << type_str(out.dtype()) << eject;
+        if (kernel_packed) TS_LOG_ERROR << "[hip] depthwise_conv2d expects [1, C, KH, KW] weights (kernel_packed=false)" << eject;
+        tsx_conv2d_geom g = make_geom(x, w, padding, stride, dilation);
+        g.cout = x.size(1);
+        check(tsx_depthwise_conv2d_f32(&g, x.data<float>(), w.data<float>(), padding_value, nullptr, TSX_ACT_NONE, 0.f,
+                                       out.data<float>(), current_stream()),
+              "tsx_depthwise_conv2d_f32");
+    }
+};
+
+}  // namespace hip
+}  // namespace ts
+
+using namespace ts;
+using namespace ts::hip;
+TS_REGISTER_OPERATOR(Pooling2D, ts::hip::DEVICE, name::layer::pooling2d())
+TS_REGISTER_OPERATOR(GlobalPooling2D, ts::hip::DEVICE, name::layer::global_pooling2d())
+TS_REGISTER_OPERATOR(Add, ts::hip::DEVICE, name::layer::add())
+TS_REGISTER_OPERATOR(DepthwiseConv2D, ts::hip::DEVICE, name::layer::depthwise_conv2d())

@@ -1,7 +1,7 @@
 // Chooses the TenniS API the "hip" backend is compiled against: the real TenniS headers
 // (integration build, -DTSX_WITH_TENNIS with the TenniS include/ and src/ directories on the
 // include path) or this repository's self-contained restatement of the same interfaces.
-// A translation unit defines TSX_TS_QUANTIZED_OPS or TSX_TS_FLOAT_OPS before including this to
+// A translation unit defines TSX_TS_QUANTIZED_OPS, TSX_TS_FLOAT_OPS or TSX_TS_GLUE_OPS before including this to
 // get the operator skeletons it derives from (TenniS's two conv2d core headers clash).
 #pragma once
 #ifdef TSX_WITH_TENNIS
@@ -16,6 +16,12 @@
 #include <backend/base/base_conv2d_winograd.h>
 #include <backend/base/base_inner_prod.h>
 #include <backend/base/base_leaky_relu.h>
+#endif
+#ifdef TSX_TS_GLUE_OPS
+#include <backend/base/base_add.h>
+#include <backend/base/base_depthwise_conv2d.h>
+#include <backend/base/base_global_pooling2d.h>
+#include <backend/base/base_pooling2d.h>
 #endif
 #include <backend/base/operator_on_device.h>
 #include <backend/name.h>

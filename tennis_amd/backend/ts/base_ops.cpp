@@ -267,6 +267,124 @@ int Conv2DWinograd::run(Stack &stack) {
     return 1;
 }
 
+// ---------------------------------------------------------------- depthwise_conv2d
+int DepthwiseConv2D::infer(Stack &stack, std::vector<Tensor::Prototype> &output) {
+    supper::infer(stack, output);
+    auto &x = stack[0];
+    auto &w = stack[1];
+    TS_AUTO_CHECK(w.size(0) == 1);
+    Shape output_shape = output[0].sizes();
+    output_shape[1] = x.size(1) * w.size(0);
+    output[0] = Tensor::Prototype(output[0].dtype(), output_shape);
+    return 1;
+}
+
+// ---------------------------------------------------------------- pooling2d / global_pooling2d
+static std::string ints_str(const std::vector<int32_t> &v) {
+    std::string s = "[";
+    for (size_t i = 0; i < v.size(); ++i) s += (i ? ", " : "") + std::to_string(v[i]);
+    return s + "]";
+}
+
+Pooling2D::Pooling2D() {
+    field(name::format, REQUIRED);
+    field(name::type, REQUIRED);
+    field(name::padding, REQUIRED);
+    field(name::padding_type, OPTIONAL, tensor::from(int(Padding2DType::BLACK)));
+    field(name::ksize, REQUIRED);
+    field(name::stride, REQUIRED);
+}
+
+void Pooling2D::init() {
+    supper::init();
+    const std::string format = tensor::to_string(get(name::format));
+    m_type = static_cast<Pooling2DType>(tensor::to_int(get(name::type)));
+    Tensor padding_tensor = tensor::cast(INT32, get(name::padding));
+    m_padding_type = static_cast<Padding2DType>(tensor::to_int(get(name::padding_type)));
+    Tensor ksize_tensor = tensor::cast(INT32, get(name::ksize));
+    Tensor stride_tensor = tensor::cast(INT32, get(name::stride));
+    TS_AUTO_CHECK(padding_tensor.has_shape({4, 2}));
+    TS_AUTO_CHECK(ksize_tensor.has_shape({4}));
+    TS_AUTO_CHECK(stride_tensor.has_shape({4}));
+    if (format == name::NCHW) m_format = FORMAT_NCHW;
+    else if (format == name::NHWC) m_format = FORMAT_NHWC;
+    else TS_LOG_ERROR << this->op() << " do not support format: " << format << eject;
+    m_padding4x2.assign(padding_tensor.data<int32_t>(), padding_tensor.data<int32_t>() + 8);
+    m_ksize4.assign(ksize_tensor.data<int32_t>(), ksize_tensor.data<int32_t>() + 4);
+    m_stride4.assign(stride_tensor.data<int32_t>(), stride_tensor.data<int32_t>() + 4);
+    // only the two image axes may be pooled (base_pooling2d.cpp:66-98)
+    const int a = m_format == FORMAT_NCHW ? 1 : 3;   // the channel axis
+    if (m_padding4x2[0] || m_padding4x2[1] || m_padding4x2[2 * a] || m_padding4x2[2 * a + 1])
+        TS_LOG_ERROR << this->op() << " do not support padding: " << ints_str(m_padding4x2) << eject;
+    if (m_ksize4[0] != 1 || m_ksize4[a] != 1) TS_LOG_ERROR << this->op() << " do not support ksize: " << ints_str(m_ksize4) << eject;
+    if (m_stride4[0] != 1 || m_stride4[a] != 1) TS_LOG_ERROR << this->op() << " do not support stride: " << ints_str(m_stride4) << eject;
+}
+
+int Pooling2D::infer(Stack &stack, std::vector<Tensor::Prototype> &output) {
+    TS_AUTO_CHECK(stack.size() == 1);
+    auto &x_tensor = stack[0];
+    TS_AUTO_CHECK(x_tensor.dims() == 4);
+    const int hd = m_format == FORMAT_NCHW ? 2 : 1;
+    const Size2D x(x_tensor.size(hd), x_tensor.size(hd + 1));
+    const Size2D ksize(m_ksize4[hd], m_ksize4[hd + 1]);
+    const Padding2D padding(m_padding4x2[2 * hd], m_padding4x2[2 * hd + 1], m_padding4x2[2 * hd + 2], m_padding4x2[2 * hd + 3]);
+    const Stride2D stride(m_stride4[hd], m_stride4[hd + 1]);
+    const Size2D y = pooling2d_forward(x, padding, ksize, stride);
+    output.resize(1);
+    if (m_format == FORMAT_NCHW) output[0] = Tensor::Prototype(x_tensor.dtype(), {x_tensor.size(0), x_tensor.size(1), y.height, y.width});
+    else output[0] = Tensor::Prototype(x_tensor.dtype(), {x_tensor.size(0), y.height, y.width, x_tensor.size(3)});
+    return 1;
+}
+
+int Pooling2D::run(Stack &stack) {
+    std::vector<Tensor::Prototype> protos;
+    infer(stack, protos);
+    auto memory_device = running_memory_device();
+    Tensor x = stack[0].view(memory_device);
+    Tensor out = *stack.push(protos[0], memory_device);
+    const int hd = m_format == FORMAT_NCHW ? 2 : 1;
+    const Size2D ksize(m_ksize4[hd], m_ksize4[hd + 1]);
+    const Padding2D padding(m_padding4x2[2 * hd], m_padding4x2[2 * hd + 1], m_padding4x2[2 * hd + 2], m_padding4x2[2 * hd + 3]);
+    const Stride2D stride(m_stride4[hd], m_stride4[hd + 1]);
+    pooling2d(x, m_type, padding, m_padding_type, ksize, stride, m_format, out);
+    return 1;
+}
+
+GlobalPooling2D::GlobalPooling2D() {
+    field(name::format, REQUIRED);
+    field(name::type, REQUIRED);
+}
+
+void GlobalPooling2D::init() {
+    supper::init();
+    const std::string format = tensor::to_string(get(name::format));
+    m_type = static_cast<Pooling2DType>(tensor::to_int(get(name::type)));
+    if (format == name::NCHW) m_format = FORMAT_NCHW;
+    else if (format == name::NHWC) m_format = FORMAT_NHWC;
+    else TS_LOG_ERROR << this->op() << " do not support format: " << format << eject;
+}
+
+int GlobalPooling2D::infer(Stack &stack, std::vector<Tensor::Prototype> &output) {
+    TS_AUTO_CHECK(stack.size() == 1);
+    auto &x = stack[0];
+    TS_AUTO_CHECK(x.dims() == 4);
+    output.resize(1);
+    if (m_format == FORMAT_NCHW) output[0] = Tensor::Prototype(x.dtype(), {x.size(0), x.size(1), 1, 1});
+    else output[0] = Tensor::Prototype(x.dtype(), {x.size(0), 1, 1, x.size(3)});
+    return 1;
+}
+
+int GlobalPooling2D::run(Stack &stack) {
+    std::vector<Tensor::Prototype> protos;
+    infer(stack, protos);
+    auto memory_device = running_memory_device();
+    Tensor x = stack[0].view(memory_device);
+    Tensor out = *stack.push(protos[0], memory_device);
+    const int hd = m_format == FORMAT_NCHW ? 2 : 1;
+    pooling2d(x, m_type, Padding2D(0, 0, 0, 0), Padding2DType::BLACK, Size2D(x.size(hd), x.size(hd + 1)), Stride2D(1, 1), m_format, out);
+    return 1;
+}
+
 // ---------------------------------------------------------------- inner_prod
 InnerProd::InnerProd() {
     field("transpose", OPTIONAL, tensor::from<bool>(false));
@@ -402,4 +520,125 @@ int LeakyReLU::run(Stack &stack) {
 }
 
 }  // namespace base
+
+// ---------------------------------------------------------------- element-wise reduce (add ...)
+bool ElementWiseReduce::reduce(Operator *op, Shape &_lhs_shape, Shape &_rhs_shape, Shape &_out_shape, bool broadcast) {
+    if (_lhs_shape == _rhs_shape) {
+        _out_shape = _lhs_shape;
+        return false;
+    }
+    if (!broadcast)
+        TS_LOG_ERROR << "[" << op->op() << ":" << op->name() << "] Can not reduce shape: " << to_string(_lhs_shape) << " vs. " << to_string(_rhs_shape) << eject;
+    Shape lhs_shape = _lhs_shape, rhs_shape = _rhs_shape;
+    while (lhs_shape.size() < rhs_shape.size()) lhs_shape.insert(lhs_shape.begin(), 1);
+    while (rhs_shape.size() < lhs_shape.size()) rhs_shape.insert(rhs_shape.begin(), 1);
+    const size_t dims = lhs_shape.size();
+    Shape out_shape;
+    out_shape.resize(dims);
+    bool do_broadcast = false;
+    for (size_t i = 0; i < dims; ++i) {
+        int size = lhs_shape[i];
+        if (lhs_shape[i] != rhs_shape[i]) {
+            if (lhs_shape[i] != 1 && rhs_shape[i] != 1)
+                TS_LOG_ERROR << "[" << op->op() << ":" << op->name() << "] Can not reduce shape: " << to_string(_lhs_shape) << " vs. " << to_string(_rhs_shape) << eject;
+            do_broadcast = true;
+            size = lhs_shape[i] * rhs_shape[i];
+        }
+        out_shape[i] = size;
+    }
+    _lhs_shape = lhs_shape;
+    _rhs_shape = rhs_shape;
+    _out_shape = out_shape;
+    return do_broadcast;
+}
+
+static int shape_count(const Shape &s, size_t b, size_t e) {
+    int c = 1;
+    for (size_t i = b; i < e; ++i) c *= s[i];
+    return c;
+}
+
+bool ElementWiseReduce::is_scalar(const Shape &shape) { return shape_count(shape, 0, shape.size()) == 1; }
+
+bool ElementWiseReduce::is_bias(Shape &lhs_shape, Shape &rhs_shape, int &dim) {
+    const int count = shape_count(rhs_shape, 0, rhs_shape.size());
+    for (size_t i = 0; i < rhs_shape.size(); ++i)
+        if (rhs_shape[i] == count && lhs_shape[i] == count) {
+            dim = int(i);
+            return true;
+        }
+    return false;
+}
+
+// collapses runs of axes on which both operands behave alike (element_wise_reduce.cpp:226-273)
+bool ElementWiseReduce::reduce_shape(Shape &lhs, Shape &rhs, Shape &out) {
+    bool reduced = false;
+    for (size_t i = 0; i < out.size();) {
+        bool lhs_ones = lhs[i] == 1, rhs_ones = rhs[i] == 1, same = lhs[i] == rhs[i];
+        if (!(lhs_ones || rhs_ones || same)) {
+            ++i;
+            continue;
+        }
+        size_t j = i + 1;
+        for (; j < out.size(); ++j) {
+            if (lhs_ones) lhs_ones = lhs[j] == 1;
+            if (rhs_ones) rhs_ones = rhs[j] == 1;
+            if (same) same = lhs[j] == rhs[j];
+            if (!(lhs_ones || rhs_ones || same)) break;
+        }
+        if (j - i > 1) {
+            const int a = shape_count(lhs, i, j), b = shape_count(rhs, i, j), c = shape_count(out, i, j);
+            lhs.erase(lhs.begin() + i, lhs.begin() + j);
+            rhs.erase(rhs.begin() + i, rhs.begin() + j);
+            out.erase(out.begin() + i, out.begin() + j);
+            lhs.insert(lhs.begin() + i, a);
+            rhs.insert(rhs.begin() + i, b);
+            out.insert(out.begin() + i, c);
+            reduced = true;
+            ++i;
+        } else {
+            i = j + 1;
+        }
+    }
+    return reduced;
+}
+
+int ElementWiseReduce::infer(Stack &stack, std::vector<Tensor::Prototype> &output) {
+    TS_AUTO_CHECK(stack.size() == 2);
+    auto &lhs = stack[0];
+    auto &rhs = stack[1];
+    if (lhs.dtype() != rhs.dtype())
+        TS_LOG_ERROR << "[" << this->op() << ":" << this->name() << "] Can not reduce mismatch type: " << type_str(lhs.dtype())
+                     << " vs. " << type_str(rhs.dtype()) << eject;
+    Shape lhs_shape = lhs.sizes(), rhs_shape = rhs.sizes(), out_shape;
+    reduce(this, lhs_shape, rhs_shape, out_shape, true);
+    output.resize(1);
+    output[0] = Tensor::Prototype(lhs.dtype(), out_shape);
+    return 1;
+}
+
+int ElementWiseReduce::run(Stack &stack) {
+    std::vector<Tensor::Prototype> output;
+    infer(stack, output);
+    Shape lhs_shape = stack[0].sizes(), rhs_shape = stack[1].sizes(), out_shape;
+    const bool do_broadcast = reduce(this, lhs_shape, rhs_shape, out_shape, true);
+    auto memory_device = running_memory_device();
+    Tensor lhs = stack[0].view(memory_device).reshape(lhs_shape);
+    Tensor rhs = stack[1].view(memory_device).reshape(rhs_shape);
+    Tensor out = *stack.push(output[0], memory_device);
+    if (reduce_shape(lhs_shape, rhs_shape, out_shape)) {
+        lhs = lhs.reshape(lhs_shape);
+        rhs = rhs.reshape(rhs_shape);
+        out = out.reshape(out_shape);
+    }
+    int dim;
+    if (!do_broadcast) reduce_with_same_shape(lhs, rhs, out);
+    else if (is_scalar(rhs_shape)) reduce_with_scalar(lhs, rhs, out);
+    else if (is_scalar(lhs_shape)) reduce_with_scalar_cross(lhs, rhs, out);
+    else if (is_bias(lhs_shape, rhs_shape, dim)) reduce_with_bias(lhs, rhs, out, dim);
+    else if (is_bias(rhs_shape, lhs_shape, dim)) reduce_with_bias_cross(lhs, rhs, out, dim);
+    else reduce_with_broadcast(lhs, rhs, out);
+    return 1;
+}
+
 }  // namespace ts

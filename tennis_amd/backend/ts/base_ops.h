@@ -97,6 +97,51 @@ protected:
     Tensor m_k_transformed;
 };
 
+// base::DepthwiseConv2D (include/backend/base/base_depthwise_conv2d.h:12): base::Conv2D with weights
+// [1, C, KH, KW] and C * 1 output channels.
+class DepthwiseConv2D : public Conv2D {
+public:
+    using supper = Conv2D;
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override;
+};
+
+// base::Pooling2DCore / Pooling2D / GlobalPooling2D (include/backend/base/base_pooling2d_core.h:12-21,
+// base_pooling2d.h:16-41, base_global_pooling2d.h:16)
+class Pooling2DCore {
+public:
+    virtual ~Pooling2DCore() = default;
+    virtual void pooling2d(const Tensor &x, Pooling2DType type, const Padding2D &padding, Padding2DType padding_type,
+                           const Size2D &ksize, const Stride2D &stride, Conv2DFormat format, Tensor &out) = 0;
+};
+
+class Pooling2D : public OperatorOnDevice, public Pooling2DCore {
+public:
+    using supper = OperatorOnDevice;
+    Pooling2D();
+    void init() override;
+    int run(Stack &stack) override;
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override;
+
+private:
+    Conv2DFormat m_format = FORMAT_NCHW;
+    Pooling2DType m_type = Pooling2DType::MAX;
+    Padding2DType m_padding_type = Padding2DType::BLACK;
+    std::vector<int32_t> m_padding4x2, m_ksize4, m_stride4;
+};
+
+class GlobalPooling2D : public OperatorOnDevice, public Pooling2DCore {
+public:
+    using supper = OperatorOnDevice;
+    GlobalPooling2D();
+    void init() override;
+    int run(Stack &stack) override;
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override;
+
+private:
+    Conv2DFormat m_format = FORMAT_NCHW;
+    Pooling2DType m_type = Pooling2DType::MAX;
+};
+
 class InnerProd : public OperatorOnDevice {
 public:
     using supper = OperatorOnDevice;
@@ -149,4 +194,29 @@ private:
 };
 
 }  // namespace base
+
+// ts::ElementWiseReduce (include/backend/base/element_wise_reduce.h:12-118; src/backend/base/
+// element_wise_reduce.cpp): the skeleton of add / sub / mul / div.  Shapes are aligned, broadcast and
+// collapsed as in the reference and the matching core method is called; this slice has no `_cast`
+// operator, so operands of different dtype are rejected instead of up-cast.
+class ElementWiseReduce : public OperatorOnDevice {
+public:
+    using supper = OperatorOnDevice;
+    int run(Stack &stack) override;
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override;
+    virtual void reduce_with_broadcast(const Tensor &lhs, const Tensor &rhs, Tensor &out) = 0;
+    virtual void reduce_with_same_shape(const Tensor &lhs, const Tensor &rhs, Tensor &out) { reduce_with_broadcast(lhs, rhs, out); }
+    virtual void reduce_with_bias(const Tensor &lhs, const Tensor &rhs, Tensor &out, int) { reduce_with_broadcast(lhs, rhs, out); }
+    virtual void reduce_with_scalar(const Tensor &lhs, const Tensor &rhs, Tensor &out) { reduce_with_broadcast(lhs, rhs, out); }
+    virtual void reduce_with_bias_cross(const Tensor &lhs, const Tensor &rhs, Tensor &out, int) { reduce_with_broadcast(lhs, rhs, out); }
+    virtual void reduce_with_scalar_cross(const Tensor &lhs, const Tensor &rhs, Tensor &out) { reduce_with_broadcast(lhs, rhs, out); }
+    static bool reduce(Operator *op, Shape &lhs_shape, Shape &rhs_shape, Shape &out_shape, bool broadcast = true);
+    static bool reduce_shape(Shape &lhs, Shape &rhs, Shape &out);
+    static bool is_scalar(const Shape &shape);
+    static bool is_bias(Shape &lhs_shape, Shape &rhs_shape, int &dim);
+};
+
+namespace base {
+using Add = ElementWiseReduce;   // include/backend/base/base_add.h:12
+}
 }  // namespace ts

@@ -448,7 +448,17 @@ Size2D conv2d_forward(const Size2D &x, const Padding2D &padding, const KSize2D &
     return y;
 }
 
+Size2D pooling2d_forward(const Size2D &x, const Padding2D &padding, const KSize2D &ksize, const Stride2D &stride) {
+    Size2D y;
+    y.height = int(std::ceil((x.height + padding.top + padding.bottom - ksize.height) / float(stride.height) + 1));
+    y.width = int(std::ceil((x.width + padding.left + padding.right - ksize.width) / float(stride.width) + 1));
+    return y;
+}
+
 namespace name {
+const char *const type = "type";
+const char *const padding_type = "padding_type";
+const char *const ksize = "ksize";
 const char *const NCHW = "NCHW";
 const char *const NHWC = "NHWC";
 const char *const format = "format";

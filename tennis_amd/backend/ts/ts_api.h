@@ -206,6 +206,18 @@ public:
     const int32_t &operator[](size_t i) const { return m_dims[i]; }
     const int32_t *begin() const { return m_dims; }
     const int32_t *end() const { return m_dims + m_size; }
+    void erase(const int32_t *first, const int32_t *last) {
+        const size_t b = size_t(first - m_dims), e = size_t(last - m_dims);
+        for (size_t i = e; i < m_size; ++i) m_dims[b + i - e] = m_dims[i];
+        m_size -= e - b;
+    }
+    void insert(const int32_t *pos, int32_t d) {
+        const size_t at = size_t(pos - m_dims);
+        if (m_size >= 7) TS_LOG_ERROR << "Shape holds at most 7 dims" << eject;
+        for (size_t i = m_size; i > at; --i) m_dims[i] = m_dims[i - 1];
+        m_dims[at] = d;
+        ++m_size;
+    }
     bool operator==(const Shape &rhs) const { return m_size == rhs.m_size && std::equal(begin(), end(), rhs.begin()); }
     bool operator!=(const Shape &rhs) const { return !(*this == rhs); }
     std::vector<int32_t> std() const { return std::vector<int32_t>(begin(), end()); }
@@ -436,6 +448,11 @@ using Dilation2D = Form2D<int32_t>;
 using Size2D = Form2D<int32_t>;
 enum Conv2DFormat { FORMAT_NCHW = 0, FORMAT_NHWC = 1 };
 enum WinogradConv2DMode { F6X6_3X3 = 0, F2X2_3X3 = 1 };
+// include/backend/common_structure.h:84-94
+enum class Pooling2DType : int { MAX = 0, AVG = 1 };
+enum class Padding2DType : int { BLACK = 0, COPY = 1, LOOP = 2, WHITE = 3 };
+// include/backend/common_function.h:14-20 (ceil of an fp32 quotient)
+Size2D pooling2d_forward(const Size2D &x, const Padding2D &padding, const KSize2D &ksize, const Stride2D &stride);
 Size2D conv2d_forward(const Size2D &x, const Padding2D &padding, const KSize2D &ksize, const Stride2D &stride,
                       const Dilation2D &dilation);
 
@@ -454,6 +471,9 @@ extern const char *const quantize_scale;
 extern const char *const dequantize_scales;
 extern const char *const winograd_mode;
 extern const char *const kernel_winograd_transformed;
+extern const char *const type;
+extern const char *const padding_type;
+extern const char *const ksize;
 namespace typo { extern const char *const dialations; }
 namespace layer {
 inline const char *conv2d() { return "conv2d"; }
@@ -465,6 +485,10 @@ inline const char *winograd_transform_kernel() { return "winograd_transform_kern
 inline const char *add_bias() { return "add_bias"; }
 inline const char *relu() { return "relu"; }
 inline const char *leaky_relu() { return "leaky_relu"; }
+inline const char *add() { return "add"; }
+inline const char *pooling2d() { return "pooling2d"; }
+inline const char *global_pooling2d() { return "global_pooling2d"; }
+inline const char *depthwise_conv2d() { return "depthwise_conv2d"; }
 }  // namespace layer
 }  // namespace name
 

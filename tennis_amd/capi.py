@@ -76,6 +76,7 @@ SIGNATURES = {
     "tsx_relu_f32": (ctypes.c_int, [_vp, _i64, _vp, _vp]),
     "tsx_leaky_relu_f32": (ctypes.c_int, [_vp, _i64, _f32, _vp, _vp]),
     "tsx_add_f32": (ctypes.c_int, [_vp, _vp, _i64, _i32, _f32, _vp, _vp]),
+    "tsx_add_broadcast_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32, _vp, _vp]),
     "tsx_mish_f32": (ctypes.c_int, [_vp, _i64, _vp, _vp]),
     "tsx_concat_channels_f32": (ctypes.c_int, [_vp, _i64, _i32, _i64, _vp, _i32, _i32, _vp]),
     "tsx_resize_nearest_f32": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32, _i32, _vp]),

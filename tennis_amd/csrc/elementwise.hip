@@ -74,6 +74,30 @@ int launch(const float *x, int64_t count, const float *bias, int channels, int64
     return 0;
 }
 
+// out = lhs + rhs with numpy-style broadcasting over up to 8 aligned axes (an extent of 1 repeats).
+// One lane per output element; an operand's stride is 0 on the axes it is broadcast along.
+struct BroadcastGeom {
+    int out_shape[8];   // right-aligned; leading unused axes have extent 1
+    int64_t lhs_stride[8], rhs_stride[8];
+};
+
+__global__ __launch_bounds__(256) void add_broadcast_kernel(const float *__restrict__ lhs, const float *__restrict__ rhs,
+                                                           BroadcastGeom g, int64_t count, float *__restrict__ out) {
+    const int64_t stride = int64_t(gridDim.x) * blockDim.x;
+    for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += stride) {
+        int64_t rest = i, lo = 0, ro = 0;
+#pragma unroll
+        for (int d = 7; d >= 0; --d) {
+            const int64_t q = rest / g.out_shape[d];
+            const int c = int(rest - q * g.out_shape[d]);
+            rest = q;
+            lo += c * g.lhs_stride[d];
+            ro += c * g.rhs_stride[d];
+        }
+        out[i] = __fadd_rn(lhs[lo], rhs[ro]);
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -99,6 +123,32 @@ int tsx_add_f32(const float *a_dev, const float *b_dev, int64_t count, int32_t a
     TSX_REQUIRE(count >= 0 && (count == 0 || b_dev), "add: bad argument");
     TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_MISH, "add: unknown activation %d", act);
     return launch<3>(a_dev, count, b_dev, 1, 1, slope, out_dev, stream, act);
+}
+
+int tsx_add_broadcast_f32(const float *lhs_dev, const int32_t *lhs_shape, const float *rhs_dev, const int32_t *rhs_shape,
+                          int32_t dims, float *out_dev, void *stream) {
+    TSX_REQUIRE(dims >= 1 && dims <= 8 && lhs_shape && rhs_shape, "add_broadcast: 1..8 axes, got %d", dims);
+    BroadcastGeom g{};
+    for (int d = 0; d < 8; ++d) g.out_shape[d] = 1;
+    int64_t count = 1, ls = 1, rs = 1;
+    for (int d = dims - 1; d >= 0; --d) {
+        const int l = lhs_shape[d], r = rhs_shape[d];
+        TSX_REQUIRE(l >= 0 && r >= 0 && (l == r || l == 1 || r == 1), "add_broadcast: axis %d: %d vs %d", d, l, r);
+        const int slot = d + 8 - dims;
+        g.out_shape[slot] = l == 1 ? r : l;
+        g.lhs_stride[slot] = l == 1 ? 0 : ls;
+        g.rhs_stride[slot] = r == 1 ? 0 : rs;
+        ls *= l;
+        rs *= r;
+        count *= g.out_shape[slot];
+    }
+    if (count == 0) return 0;
+    TSX_REQUIRE(lhs_dev && rhs_dev && out_dev, "add_broadcast: null pointer");
+    const int64_t blocks = (count + 255) / 256;
+    hipLaunchKernelGGL(add_broadcast_kernel, dim3(unsigned(blocks < 8192 ? blocks : 8192)), dim3(256), 0, tsx::as_stream(stream),
+                       lhs_dev, rhs_dev, g, count, out_dev);
+    TSX_LAUNCH_CHECK("add_broadcast_kernel");
+    return 0;
 }
 
 int tsx_mish_f32(const float *x_dev, int64_t count, float *out_dev, void *stream) {

@@ -47,7 +47,8 @@ def test_hot_path_operators_are_registered_for_hip():
     from tennis_amd import operators as ops
     for name in ops.SYMBOLS:
         assert hasattr(ops.lib(), name)
-    for op in ("quantize", "conv2d_quantized", "conv2d", "conv2d_winograd", "inner_prod", "add_bias", "relu", "leaky_relu"):
+    for op in ("quantize", "conv2d_quantized", "conv2d", "conv2d_winograd", "inner_prod", "add_bias", "relu", "leaky_relu",
+               "pooling2d", "global_pooling2d", "add", "depthwise_conv2d"):
         assert ops.is_registered("hip", op), op
     assert not ops.is_registered("hip", "softmax")
     assert not ops.is_registered("cpu", "conv2d")            # this library ships no host operators
@@ -93,3 +94,15 @@ def test_parameter_checking_follows_the_reference():
         ops.check_params("quantize", {})
     with pytest.raises(ops.OperatorError, match="scale"):
         ops.check_params("leaky_relu", {})
+    # pooling2d: ksize / stride / padding on the two image axes only (base_pooling2d.cpp:66-98)
+    pool = {"format": "NCHW", "type": np.array([0], np.int32), "padding": np.zeros((4, 2), np.int32),
+            "ksize": np.array([1, 1, 3, 3], np.int32), "stride": np.array([1, 1, 2, 2], np.int32)}
+    ops.check_params("pooling2d", pool)                       # padding_type is optional (BLACK)
+    with pytest.raises(ops.OperatorError, match="do not support ksize"):
+        ops.check_params("pooling2d", dict(pool, ksize=np.array([1, 2, 3, 3], np.int32)))
+    with pytest.raises(ops.OperatorError, match="do not support padding"):
+        ops.check_params("pooling2d", dict(pool, padding=np.array([[0, 0], [0, 1], [0, 0], [0, 0]], np.int32)))
+    with pytest.raises(ops.OperatorError, match="type"):
+        ops.check_params("global_pooling2d", {"format": "NCHW"})
+    ops.check_params("add", {})
+    ops.check_params("depthwise_conv2d", {k: v for k, v in good.items() if k != "dequantize_scales"})

@@ -90,6 +90,36 @@ def test_fp32_operators_in_tennis_workbench(ts):
     assert close(hip, cpu)
 
 
+def test_glue_operators_in_tennis_workbench(ts):
+    """pooling2d / global_pooling2d / add / depthwise_conv2d run by TenniS's Workbench with strict device
+    lookup, so the "hip" classes (not the host fallback) produce the result; bitwise against the host operators."""
+    rng = np.random.default_rng(902)
+    x = rng.standard_normal((2, 6, 14, 12)).astype(np.float32)
+
+    def strict_both(op, params, inputs, out_bytes):
+        cpu = ts.run_op_intree("cpu", op, params, inputs, out_bytes)
+        hip = ts.run_op_intree("hip", op, params, inputs, out_bytes, strict=True)
+        assert cpu.shape == hip.shape
+        assert np.array_equal(bits(cpu), bits(hip)), (op, params)
+
+    for kind, k, s, pads, white in ((0, (3, 3), (2, 2), (0, 1, 0, 1), False), (1, (2, 2), (2, 2), (0, 0, 0, 0), False),
+                                    (1, (3, 3), (1, 1), (1, 1, 1, 1), True), (0, (5, 5), (1, 1), (2, 2, 2, 2), False)):
+        p = {"format": "NCHW", "type": np.array([kind], np.int32),
+             "padding": np.array([[0, 0], [0, 0], [pads[0], pads[1]], [pads[2], pads[3]]], np.int32),
+             "padding_type": np.array([3 if white else 0], np.int32),
+             "ksize": np.array([1, 1, k[0], k[1]], np.int32), "stride": np.array([1, 1, s[0], s[1]], np.int32)}
+        strict_both("pooling2d", p, [x], x.nbytes + 4096)
+    for kind in (0, 1):
+        strict_both("global_pooling2d", {"format": "NCHW", "type": np.array([kind], np.int32)}, [x], 4 * 12)
+    for shape in ((2, 6, 14, 12), (1,), (1, 6, 1, 1), (2, 1, 14, 1), (14, 12)):
+        b = rng.standard_normal(shape).astype(np.float32)
+        strict_both("add", {}, [x, b], x.nbytes)
+        strict_both("add", {}, [b, x], x.nbytes)
+    w = rng.standard_normal((1, 6, 3, 3)).astype(np.float32)
+    for pads, strides, dil, pv in (((1, 1, 1, 1), (1, 1), (1, 1), 0.0), ((0, 2, 1, 0), (2, 1), (1, 2), 0.5)):
+        strict_both("depthwise_conv2d", conv_params(ts, pads, strides, dil, pv), [x, w], x.nbytes + 8192)
+
+
 def test_unregistered_operator_falls_back_to_cpu(ts):
     """An operator the backend does not register runs through TenniS's device -> cpu lookup order
     (src/global/operator_factory.cpp:60-81) on a "hip" Workbench, with the tensors copied by the

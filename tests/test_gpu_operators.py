@@ -133,6 +133,45 @@ def test_elementwise_operators(ops, port):
         ops.run_op("add_bias", {"dim": np.array([1], np.int32)}, [x, np.zeros(4, np.float32)])
 
 
+def _pool_params(kind, ksize, strides, pads, white=False):
+    return {"format": "NCHW", "type": np.array([{"max": 0, "avg": 1}[kind]], np.int32),
+            "padding": np.array([[0, 0], [0, 0], [pads[0], pads[1]], [pads[2], pads[3]]], np.int32),
+            "padding_type": np.array([3 if white else 0], np.int32),
+            "ksize": np.array([1, 1, ksize[0], ksize[1]], np.int32),
+            "stride": np.array([1, 1, strides[0], strides[1]], np.int32)}
+
+
+def test_glue_operators(ops, port):
+    """pooling2d, global_pooling2d, add (equal shapes, scalar, bias, general broadcast, either side)
+    and depthwise_conv2d created by name; bitwise against the oracle."""
+    rng = np.random.default_rng(505)
+    x = rng.standard_normal((2, 5, 13, 11)).astype(np.float32)
+    for kind, k, s, pads, white in (("max", (3, 3), (2, 2), (1, 1, 1, 1), False), ("avg", (2, 3), (2, 1), (1, 0, 1, 1), False),
+                                    ("avg", (3, 3), (1, 1), (1, 1, 1, 1), True), ("max", (5, 5), (1, 1), (2, 2, 2, 2), False)):
+        got = ops.run_op("pooling2d", _pool_params(kind, k, s, pads, white), [x])
+        want = port.pooling2d(x, kind, k, s, pads, white)
+        assert got.shape == want.shape and np.array_equal(bits(got), bits(want)), (kind, k, s, pads, white)
+    for kind in ("max", "avg"):
+        got = ops.run_op("global_pooling2d", {"format": "NCHW", "type": np.array([{"max": 0, "avg": 1}[kind]], np.int32)}, [x])
+        assert got.shape == (2, 5, 1, 1) and np.array_equal(bits(got), bits(port.global_pooling2d(x, kind)))
+    for shape in ((2, 5, 13, 11), (1,), (1, 5, 1, 1), (5, 1, 1), (2, 1, 13, 1), (13, 11), (1, 1, 1, 11)):
+        b = rng.standard_normal(shape).astype(np.float32)
+        for lhs, rhs in ((x, b), (b, x)):
+            got = ops.run_op("add", {}, [lhs, rhs])
+            want = lhs + rhs                                   # one IEEE addition per element
+            assert got.shape == want.shape and np.array_equal(bits(got), bits(want)), shape
+    with pytest.raises(ops.OperatorError, match="Can not reduce shape"):
+        ops.run_op("add", {}, [x, np.zeros((2, 4, 13, 11), np.float32)])
+    w = rng.standard_normal((1, 5, 3, 3)).astype(np.float32)
+    for pads, strides, dil, pv in (((1, 1, 1, 1), (1, 1), (1, 1), 0.0), ((0, 2, 1, 0), (2, 1), (1, 2), 0.5)):
+        params = ops.conv_params(pads, strides, dil, pv)
+        got = ops.run_op("depthwise_conv2d", params, [x, w])
+        want = port.depthwise_conv2d(x, w, pads, strides, dil, pv)
+        assert got.shape == want.shape and np.array_equal(bits(got), bits(want)), (pads, strides, dil)
+    with pytest.raises(ops.OperatorError):                     # multiplier > 1 is depthwise_conv2d_v2's business
+        ops.run_op("depthwise_conv2d", ops.conv_params((1, 1, 1, 1)), [x, np.zeros((2, 5, 3, 3), np.float32)])
+
+
 def test_operator_errors_at_run_time(ops):
     params = ops.conv_params((1, 1, 1, 1))
     params["dequantize_scales"] = np.ones(4, np.float32)
