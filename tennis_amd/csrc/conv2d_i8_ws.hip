@@ -6,7 +6,8 @@
 // cpu::Conv2DQuantizedCore, src/kernels/cpu/quantized/conv2d_quantized_core.cpp:18-147), but
 // a different data movement:
 //   * one workgroup (4 wavefronts) owns TH full output rows x 128 output channels; wavefront w
-//     owns channels [32w, 32w+32) and all positions of the tile.  Rows are counted across the
+//     owns channels [32w, 32w+32) and all positions of the tile (layers with at most 64 output
+//     channels: 64 channels, two wavefronts each on either half of the tile's positions).  Rows are counted across the
 //     whole batch (image n's rows follow image n-1's), so a tile may straddle two images: their
 //     staged rows are contiguous in memory, and a position in the second image just reads the
 //     window (KH-1)*dilation rows further down.  Tiles therefore need not divide the image
@@ -43,6 +44,7 @@ struct WsParams : EpiParams {
     const int8_t *wp;   // packed weights [ks_p][coutp/32][2 halves][64 lanes][16]
     int n, cout, coutp, ho, wo, hs, ws, cp, cblocks, kh, kw, dil_h, dil_w;
     int th, wr, wc, wpix, ksteps_p;
+    int wm;           // wavefronts along cout (4, or 2: the other factor of 4 splits the tile's positions)
     int stream_out;   // fp32 output written with streaming stores
 };
 
@@ -76,8 +78,13 @@ __global__ __launch_bounds__(256) void ws_pack_kernel(const int8_t *__restrict__
 
 // EXTRA = false compiles the residual input and the staged-layout output out of the epilogue (fewer
 // registers for the plain dequant + bias + activation case); STREAM selects streaming fp32 stores.
+//
+// Up to 4 position fragments the kernel is compiled for two wavefronts per SIMD (at most 256 registers): the
+// layers that take these tiles are bound by their epilogue's memory traffic (residual in, fp32 and staged int8
+// out), and a second resident workgroup per CU is worth more there than registers.
+// NT counts the position fragments of ONE wavefront; a tile holds (4 / wm) x NT of them.
 template <int NT, int FM, bool EXTRA, bool STREAM>
-__global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
+__global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <= 4 ? 2 : 1))) void conv_i8_ws_kernel(WsParams p_in) {
     WsParams p = p_in;
     if (!EXTRA) {
         p.residual = nullptr;
@@ -90,7 +97,9 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
     const int th0 = row0 - img * p.ho;       // ... and that row inside it
     const int rows_total = p.n * p.ho;
     const int wrap = p.hs - p.ho;            // staged rows between the last output row of an image and the next image's first
-    const int m0 = (blockIdx.y * 4 + wave) * (32 * FM);             // first cout of this wavefront
+    const int wave_m = p.wm == 4 ? wave : wave & 1;                  // position along cout
+    const int pos0 = p.wm == 4 ? 0 : (wave >> 1) * (NT * 32);        // first tile position of this wavefront
+    const int m0 = (blockIdx.y * p.wm + wave_m) * (32 * FM);         // first cout of this wavefront
     const int taps = p.kh * p.kw;
     const int win_bytes = p.wpix * PIX;
 
@@ -131,7 +140,7 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
     int b_base[NT];
     static_for<0, NT>([&](auto jc) {
         constexpr int j = decltype(jc)::value;
-        int pos = j * 32 + lane % 32;
+        int pos = pos0 + j * 32 + lane % 32;
         if (pos >= p.th * p.wo) pos = 0;       // padding positions: computed, never stored
         const int r = pos / p.wo, ow = pos - r * p.wo;
         const int wrow = r + (th0 + r >= p.ho ? wrap : 0);   // positions of the next image sit below its halo rows
@@ -253,7 +262,7 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
             const int64_t tile_base = (int64_t(img) * p.cout + cf) * howo;
             static_for<0, NT>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
-                const int pos = j * 32 + lane % 32;
+                const int pos = pos0 + j * 32 + lane % 32;
                 const int tr = pos / p.wo, ow = pos - tr * p.wo;
                 const bool wrapped = th0 + tr >= p.ho;
                 const int oh = th0 + tr - (wrapped ? p.ho : 0);
@@ -262,13 +271,13 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
                 static_for<0, 16>([&](auto rc) {
                     constexpr int r = decltype(rc)::value;
                     constexpr int dco = 8 * (r / 4) + (r % 4);
-                    res[j][r] = pos_ok ? __builtin_nontemporal_load(&(p.residual + tile_base + int64_t(dco) * howo)[lane_off]) : 0.f;
+                    res[j][r] = pos_ok ? (p.residual + tile_base + int64_t(dco) * howo)[lane_off] : 0.f;
                 });
             });
         }
         static_for<0, NT>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
-            const int pos = j * 32 + lane % 32;
+            const int pos = pos0 + j * 32 + lane % 32;
             const int tr = pos / p.wo, ow = pos - tr * p.wo;
             const bool wrapped = th0 + tr >= p.ho;                 // this position belongs to the next image
             const int oh = th0 + tr - (wrapped ? p.ho : 0);
@@ -336,16 +345,24 @@ __global__ __launch_bounds__(WS_THREADS) void conv_i8_ws_kernel(WsParams p_in) {
                             (p.out_i8 + tile_base + int64_t(dco) * howo)[lane_off] = int8_t(qv[r]);
                         });
                         if (EXTRA && p.st_out) {
-                            // consumer's staged layout: accumulator registers 4g..4g+3 of a lane are 4 consecutive
-                            // channels of one pixel -> one dword per group
-                            int8_t *dst = p.st_out + ((int64_t(img + (wrapped ? 1 : 0)) * p.st_hs + oh + p.st_pt) * p.st_ws + ow + p.st_pl) * p.st_cp +
-                                          cf + 4 * (lane / 32);
+                            // consumer's staged layout [pixel][channel].  Accumulator registers 4g..4g+3 of a lane are 4
+                            // consecutive channels of one pixel (one dword); the pixel's other 16 channels of this
+                            // fragment sit in lane +-32.  Two half-wave swaps leave every lane with 16 consecutive
+                            // channels -- lower half cf..cf+15, upper half cf+16..cf+31 -- for one 16-byte store
+                            // (4-byte stores at a pixel stride cost an L2 request each).
+                            uint32_t word[4];
                             static_for<0, 4>([&](auto gc) {
                                 constexpr int g4 = decltype(gc)::value;
-                                const uint32_t word = uint32_t(qv[4 * g4] & 0xff) | (uint32_t(qv[4 * g4 + 1] & 0xff) << 8) |
-                                                      (uint32_t(qv[4 * g4 + 2] & 0xff) << 16) | (uint32_t(qv[4 * g4 + 3] & 0xff) << 24);
-                                *reinterpret_cast<uint32_t *>(dst + 8 * g4) = word;
+                                word[g4] = uint32_t(qv[4 * g4] & 0xff) | (uint32_t(qv[4 * g4 + 1] & 0xff) << 8) |
+                                           (uint32_t(qv[4 * g4 + 2] & 0xff) << 16) | (uint32_t(qv[4 * g4 + 3] & 0xff) << 24);
                             });
+                            // swap(a, b): a's upper half-wave <-> b's lower half-wave
+                            const auto s02 = __builtin_amdgcn_permlane32_swap(word[0], word[2], false, false);
+                            const auto s13 = __builtin_amdgcn_permlane32_swap(word[1], word[3], false, false);
+                            int8_t *dst = p.st_out + ((int64_t(img + (wrapped ? 1 : 0)) * p.st_hs + oh + p.st_pt) * p.st_ws + ow + p.st_pl) * p.st_cp +
+                                          cf + 16 * (lane / 32);
+                            const v4i packed = {int(s02[0]), int(s02[1]), int(s13[0]), int(s13[1])};
+                            *reinterpret_cast<v4i *>(dst) = packed;
                         }
                     }
                 }
@@ -392,21 +409,24 @@ WsPlan ws_plan(const WsGeom &g) {
     // layers of a ResNet-50-shaped network, whose small maps want many small workgroups.  Ties go to the
     // fewest total fragments (least padding).
     constexpr int MAX_NT = 7;
-    if (g.wo < 1 || g.wo > 32 * MAX_NT) return pl;
+    // at most 64 output channels: two wavefronts along cout, two along the positions of a twice larger tile
+    const int wm = g.cout <= 64 ? 2 : 4, wn = 4 / wm;
+    if (g.wo < 1 || g.wo > 32 * MAX_NT * wn) return pl;
     const int wrap = g.hs - g.ho;
-    const int coutp = (g.cout + WS_BM - 1) / WS_BM * WS_BM;
+    const int bm = 32 * WS_FM * wm;
+    const int coutp = (g.cout + bm - 1) / bm * bm;
     const int ksteps_p = (g.cblocks * g.kh * g.kw + RING - 1) / RING * RING;
     double best_cost = -1;
     int64_t best_frags = 0;
-    for (int t = 1; t <= g.ho && t * g.wo <= 32 * MAX_NT; ++t) {
-        const int nt = (t * g.wo + 31) / 32;
+    for (int t = 1; t <= g.ho && t * g.wo <= 32 * MAX_NT * wn; ++t) {
+        const int nt = ((t * g.wo + 31) / 32 + wn - 1) / wn;   // fragments per wavefront
         const int64_t tiles = (int64_t(g.n) * g.ho + t - 1) / t;
         const bool straddle = g.ho % t != 0;
         const int wr = t + (g.kh - 1) * g.dil_h + (straddle ? wrap : 0);
         const int wp = wr * g.ws;
         if (wp > MAX_WP || size_t(2) * wp * PIX > 65536) continue;   // two windows must fit 64 KiB of LDS
-        const int64_t wgs = tiles * (coutp / WS_BM);
-        const int64_t frags = tiles * nt;
+        const int64_t wgs = tiles * (coutp / bm);
+        const int64_t frags = tiles * nt * wn;
         const double cost = double((wgs + 255) / 256) * (0.5 + nt * (nt > 4 ? 1.45 : 1.0));
         if (best_cost < 0 || cost < best_cost || (cost == best_cost && frags < best_frags)) {
             best_cost = cost;
@@ -420,6 +440,7 @@ WsPlan ws_plan(const WsGeom &g) {
     }
     if (best_cost < 0 || pl.tiles >= (int64_t(1) << 31)) return pl;
     pl.wc = g.ws;
+    pl.wm = wm;
     pl.ksteps_p = ksteps_p;
     pl.coutp = coutp;
     pl.packed_bytes = size_t(pl.ksteps_p) * pl.coutp * 64;
@@ -459,9 +480,10 @@ int ws_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t 
     p.wc = pl.wc;
     p.wpix = pl.wp;
     p.ksteps_p = pl.ksteps_p;
+    p.wm = pl.wm;
     // an output of L2 size or more that no fused consumer reads: stream it
     p.stream_out = (!ep.residual && !ep.st_out && ep.out_f32 && int64_t(g.n) * g.cout * g.ho * g.wo * 4 >= (int64_t(16) << 20)) ? 1 : 0;
-    const dim3 grid(unsigned(pl.tiles), unsigned(pl.coutp / WS_BM));
+    const dim3 grid(unsigned(pl.tiles), unsigned(pl.coutp / (32 * WS_FM * pl.wm)));
     const size_t lds_bytes = size_t(2) * pl.wp * PIX;
     switch (pl.nt) {
         case 1: return launch_nt<1>(p, grid, lds_bytes, stream);

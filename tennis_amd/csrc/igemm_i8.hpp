@@ -120,11 +120,12 @@ __device__ __forceinline__ void epilogue_rows16(const EpiParams &p, const v16i &
 
 struct WsPlan {
     bool ok;            // geometry supported
-    int th, nt;         // output rows per tile, 32-position fragments per tile
+    int th, nt;         // output rows per tile, 32-position fragments per wavefront
+    int wm;             // wavefronts along cout: 4, or 2 with the tile's positions split over the other factor
     int64_t tiles;      // tiles over the batch-wide row sequence
     int wr, wc, wp;     // window rows, cols, pixels
     int ksteps_p;       // K-steps padded to the A-ring size
-    int coutp;          // cout padded to the workgroup's 256
+    int coutp;          // cout padded to the workgroup's channels (32 x wm)
     size_t packed_bytes;
 };
 
