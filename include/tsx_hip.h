@@ -235,6 +235,24 @@ int tsx_pooling2d_f32(const float *x_dev, int64_t planes, int32_t h, int32_t w, 
                       int32_t pad_left, int32_t kh, int32_t kw, int32_t stride_h, int32_t stride_w, int32_t white_padding,
                       float *out_dev, int32_t out_h, int32_t out_w, void *stream);
 
+/* An h x w x c int8 map inside a pixel-major staged buffer [n][hs][ws][cp] (the layout
+ * tsx_conv2d_i8_staged_dims describes and tsx_epilogue.staged_out_dev is written in): the map's element
+ * (y, x, ch) of image i sits at ((i*hs + y + pad_top)*ws + x + pad_left)*cp + ch. */
+typedef struct tsx_staged_map {
+    void *data;
+    int32_t n, hs, ws, cp;
+    int32_t pad_top, pad_left;
+    int32_t h, w, c;
+} tsx_staged_map;
+
+/* cpu::Pooling2DCore MAX (src/kernels/cpu/pooling2d_core.cpp:48-93) applied between a quantized producer and a
+ * quantized consumer, on the producer's requantized int8 output: quantize (src/kernels/cpu/quantize.cpp:70-125) is
+ * monotone non-decreasing for a positive scale, so max-pooling the int8 values gives byte for byte what
+ * pooling2d(fp32) -> quantize gives.  Window clipped to the map as in the reference; dst->h, dst->w are the
+ * output size (tsx_pooling2d_out_size); dst's halo and channel padding beyond src->cp are left / zeroed. */
+int tsx_max_pooling2d_i8_staged(const tsx_staged_map *src, const tsx_staged_map *dst, int32_t kh, int32_t kw, int32_t pad_top,
+                                int32_t pad_left, int32_t stride_h, int32_t stride_w, void *stream);
+
 /* ---------------------------------------------------------------- Winograd F(6x6, 3x3) fp32 conv2d
  * Conv2dWinogradAlgorithm<float>::winograd_f63 (src/kernels/cpu/winograd_algorithm.cpp:846-947),
  * reached in the reference through base::Conv2DWinograd's two core calls

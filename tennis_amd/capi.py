@@ -75,6 +75,7 @@ SIGNATURES = {
     "tsx_add_bias_f32": (ctypes.c_int, [_vp, _i64, _i32, _i64, _vp, _vp, _vp]),
     "tsx_relu_f32": (ctypes.c_int, [_vp, _i64, _vp, _vp]),
     "tsx_leaky_relu_f32": (ctypes.c_int, [_vp, _i64, _f32, _vp, _vp]),
+    "tsx_max_pooling2d_i8_staged": (ctypes.c_int, [_vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
     "tsx_add_f32": (ctypes.c_int, [_vp, _vp, _i64, _i32, _f32, _vp, _vp]),
     "tsx_add_broadcast_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32, _vp, _vp]),
     "tsx_mish_f32": (ctypes.c_int, [_vp, _i64, _vp, _vp]),
@@ -188,6 +189,18 @@ class StagedInput:
         self.pad_top, self.pad_left = conv.pads[0], conv.pads[2]
         self.buf = torch.empty(max(ws_bytes, 16), dtype=torch.int8, device=conv.w.device)
         check(lib().tsx_conv2d_i8_stage_fill(ctypes.byref(geom), conv.padding_value, _ptr(self.buf), ws_bytes, _stream()))
+
+
+class StagedPlain:
+    """A staged int8 buffer without halo, [n][h][w][round_up(c, 64)], zero-initialised: a producer's requantized
+    output in the pixel-major layout when the consumer is not a convolution (a pooling pass in between)."""
+
+    def __init__(self, x_shape, device):
+        n, c, h, w = x_shape
+        self.x_shape = tuple(x_shape)
+        self.hs, self.ws, self.cp = h, w, (c + 63) // 64 * 64
+        self.pad_top = self.pad_left = 0
+        self.buf = torch.zeros(n * h * w * self.cp, dtype=torch.int8, device=device)
 
 
 class Conv2dI8:
@@ -439,6 +452,27 @@ def pooling2d(x, kind, ksize, strides, pads=(0, 0, 0, 0), white=False):
     check(lib().tsx_pooling2d_f32(_ptr(x), n * c, h, w, {"max": 0, "avg": 1}[kind], pads[0], pads[2], ksize[0], ksize[1],
                                   strides[0], strides[1], int(white), _ptr(out), ho, wo, _stream()))
     return out
+
+
+class StagedMap(ctypes.Structure):
+    """tsx_staged_map."""
+    _fields_ = [("data", ctypes.c_void_p), ("n", _i32), ("hs", _i32), ("ws", _i32), ("cp", _i32),
+                ("pad_top", _i32), ("pad_left", _i32), ("h", _i32), ("w", _i32), ("c", _i32)]
+
+
+def _staged_map(st):
+    n, c, h, w = st.x_shape
+    return StagedMap(_ptr(st.buf), n, st.hs, st.ws, st.cp, st.pad_top, st.pad_left, h, w, c)
+
+
+def max_pooling2d_staged(src, dst, ksize, strides, pads=(0, 0, 0, 0)):
+    """tsx_max_pooling2d_i8_staged between two StagedInput buffers (int8, pixel-major)."""
+    ho, wo = pool_out_size(src.x_shape[2], src.x_shape[3], ksize, pads, strides)
+    assert (ho, wo) == tuple(dst.x_shape[2:]), "destination map is not the pooled size"
+    a, b = _staged_map(src), _staged_map(dst)
+    check(lib().tsx_max_pooling2d_i8_staged(ctypes.byref(a), ctypes.byref(b), ksize[0], ksize[1], pads[0], pads[2],
+                                            strides[0], strides[1], _stream()))
+    return dst
 
 
 def global_pooling2d(x, kind):

@@ -344,6 +344,72 @@ __global__ __launch_bounds__(256) void stage_im2col_kernel(const void *__restric
     *reinterpret_cast<uint4 *>(xs + id * 16) = make_uint4(words[0], words[1], words[2], words[3]);
 }
 
+// The same staging with one workgroup per (image, output row).  Phase 1 quantizes the C x KH input rows
+// the output row reads once each into an LDS patch [c][kh][patch columns] (coalesced loads along W; the
+// lane-per-chunk kernel above quantizes every input element KH*KW/(SH*SW) times and gathers from global
+// memory); phase 2 assembles the 16-byte K chunks from patch bytes and stores them contiguously.
+template <bool QUANT>
+__global__ __launch_bounds__(256) void stage_im2col_rows_kernel(const void *__restrict__ src, Im2colGeom g, int wpatch,
+                                                               const float *__restrict__ scales, int n_scales,
+                                                               int64_t group_len, int64_t bulk8, int8_t *__restrict__ xs) {
+    extern __shared__ __attribute__((aligned(16))) int8_t patch[];   // [c * kh][wpatch]
+    const int tid = threadIdx.x;
+    const int oh = blockIdx.x % g.ho, ni = blockIdx.x / g.ho;
+    const bool uniform_scale = QUANT && (n_scales == 1 || group_len == int64_t(g.c) * g.h * g.w);
+    const float img_scale = uniform_scale ? scales[n_scales == 1 ? 0 : ni] : 0.f;
+    const int h0 = oh * g.sh - g.pad_top;
+    const int rows = g.c * g.kh;
+    for (int idx = tid; idx < rows * wpatch; idx += 256) {
+        const int row = idx / wpatch, col = idx - row * wpatch;
+        const int ci = row / g.kh, r = row - ci * g.kh;
+        const int hi = h0 + r * g.dh, wi = col - g.pad_left;
+        int q = g.pad_value;
+        if (hi >= 0 && hi < g.h && wi >= 0 && wi < g.w) {
+            const int64_t e = ((int64_t(ni) * g.c + ci) * g.h + hi) * g.w + wi;
+            if (QUANT) {
+                const float sc = uniform_scale ? img_scale : scales[e / group_len];
+                q = tsx::quantize_value(__fmul_rn(static_cast<const float *>(src)[e], sc), n_scales == 1 && e < bulk8);
+            } else {
+                q = static_cast<const int8_t *>(src)[e];
+            }
+        }
+        patch[idx] = int8_t(q);
+    }
+    __syncthreads();
+    const int chunks = g.cp / 16;
+    const int taps = g.kh * g.kw;
+    int8_t *dst = xs + (int64_t(ni) * g.ho + oh) * g.wo * g.cp;
+    for (int id = tid; id < g.wo * chunks; id += 256) {
+        const int ow = id / chunks, chunk = id - ow * chunks;
+        int k = chunk * 16;
+        int ci = k / taps;
+        int kh = (k - ci * taps) / g.kw;
+        int kw = k - ci * taps - kh * g.kw;
+        const int8_t *base = patch + ow * g.sw;
+        uint32_t words[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            uint32_t word = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                int q = 0;   // K padding: the packed weights are zero there as well
+                if (k < g.kk) q = base[(ci * g.kh + kh) * wpatch + kw * g.dw];
+                word |= uint32_t(q & 0xff) << (8 * j);
+                ++k;
+                if (++kw == g.kw) {
+                    kw = 0;
+                    if (++kh == g.kh) {
+                        kh = 0;
+                        ++ci;
+                    }
+                }
+            }
+            words[v] = word;
+        }
+        *reinterpret_cast<uint4 *>(dst + int64_t(id) * 16) = make_uint4(words[0], words[1], words[2], words[3]);
+    }
+}
+
 // Whole staged buffer = halo: T(padding_value) in the real channels, 0 in the channel padding.
 __global__ __launch_bounds__(256) void stage_fill_kernel(int8_t *__restrict__ xs, int64_t chunks, int cp, int c, int pad_value) {
     const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -820,13 +886,25 @@ int run_stage(const tsx_conv2d_geom *g, const Plan &pl, const void *x, bool x_is
                             g->dilation_w, g->pad_top, g->pad_left, pl.kk, pl.cp, int(int8_t(padding_value))};
         const int64_t threads = int64_t(pl.staged_bytes / 16);
         const dim3 grid(unsigned(tsx::ceil_div(threads, 256)));
+        // patch columns an output row touches; the row kernel needs the C x KH patch rows in LDS
+        const int wpatch = (pl.wo - 1) * g->stride_w + (g->kw - 1) * g->dilation_w + 1;
+        const size_t patch_bytes = size_t(g->c) * g->kh * wpatch;
+        const bool by_rows = patch_bytes <= 48 * 1024 && int64_t(g->n) * pl.ho < (int64_t(1) << 31);
+        const dim3 row_grid(unsigned(int64_t(g->n) * pl.ho));
         if (x_is_f32) {
             TSX_REQUIRE(x_scales && n_x_scales >= 1, "quantize_conv2d_i8: missing quantize scales");
             TSX_REQUIRE(n_x_scales == g->n, "quantize_conv2d_i8: n_x_scales (%d) must equal the batch (%d)", n_x_scales, g->n);
             const int64_t count = int64_t(g->n) * g->c * g->h * g->w;
             const int64_t group_len = int64_t(std::ceil(static_cast<float>(count) / static_cast<float>(n_x_scales)));
-            hipLaunchKernelGGL(stage_im2col_kernel<true>, grid, dim3(256), 0, stream, x, ig, x_scales, n_x_scales, group_len,
-                               (count >> 3) << 3, static_cast<int8_t *>(staged));
+            if (by_rows)
+                hipLaunchKernelGGL(stage_im2col_rows_kernel<true>, row_grid, dim3(256), patch_bytes, stream, x, ig, wpatch, x_scales,
+                                   n_x_scales, group_len, (count >> 3) << 3, static_cast<int8_t *>(staged));
+            else
+                hipLaunchKernelGGL(stage_im2col_kernel<true>, grid, dim3(256), 0, stream, x, ig, x_scales, n_x_scales, group_len,
+                                   (count >> 3) << 3, static_cast<int8_t *>(staged));
+        } else if (by_rows) {
+            hipLaunchKernelGGL(stage_im2col_rows_kernel<false>, row_grid, dim3(256), patch_bytes, stream, x, ig, wpatch,
+                               static_cast<const float *>(nullptr), 1, int64_t(1), int64_t(0), static_cast<int8_t *>(staged));
         } else {
             hipLaunchKernelGGL(stage_im2col_kernel<false>, grid, dim3(256), 0, stream, x, ig,
                                static_cast<const float *>(nullptr), 1, int64_t(1), int64_t(0), static_cast<int8_t *>(staged));

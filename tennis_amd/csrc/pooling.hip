@@ -57,6 +57,58 @@ __global__ __launch_bounds__(256) void pooling2d_kernel(const float *__restrict_
 // sequential order is kept and parallelism comes from the N*C planes (32 x 2048 at the end of a
 // ResNet-50-shaped network).
 
+// MAX pooling between two quantized convolutions, on int8 in the pixel-major staged layout
+// [n][hs][ws][cp] on both sides.  quantize is monotone non-decreasing for a positive scale, so
+// quantize(max(window)) == max(quantize(window)) element for element: pooling the producer's
+// requantized int8 output gives the bytes that pooling2d(fp32) -> quantize would, with a quarter of
+// the traffic and no layout pass in between.  One lane = 16 channels of one output pixel.
+typedef short s2v __attribute__((ext_vector_type(2)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t max_i8x4(uint32_t a, uint32_t b) {
+    // signed bytes compared as the high bytes of 16-bit lanes: odd bytes in place, even bytes shifted up
+    const uint32_t m = 0xff00ff00u;
+    const s2v hi = __builtin_elementwise_max(__builtin_bit_cast(s2v, a & m), __builtin_bit_cast(s2v, b & m));
+    const s2v lo = __builtin_elementwise_max(__builtin_bit_cast(s2v, (a << 8) & m), __builtin_bit_cast(s2v, (b << 8) & m));
+    return __builtin_bit_cast(uint32_t, hi) | (__builtin_bit_cast(uint32_t, lo) >> 8);
+}
+
+struct PoolStagedGeom {
+    int n, h, w, ho, wo, pad_top, pad_left, kh, kw, sh, sw;
+    int s_hs, s_ws, s_cp, s_pt, s_pl;   // source buffer
+    int d_hs, d_ws, d_cp, d_pt, d_pl;   // destination buffer
+};
+
+__global__ __launch_bounds__(256) void max_pooling2d_i8_staged_kernel(const int8_t *__restrict__ src, PoolStagedGeom g,
+                                                                     int8_t *__restrict__ dst) {
+    const int chunks = g.d_cp / 16;
+    const int64_t total = int64_t(g.n) * g.ho * g.wo * chunks;
+    const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id >= total) return;
+    const int chunk = int(id % chunks);
+    int64_t rest = id / chunks;
+    const int ow = int(rest % g.wo);
+    rest /= g.wo;
+    const int oh = int(rest % g.ho);
+    const int ni = int(rest / g.ho);
+    v4i r = {0, 0, 0, 0};   // channels the source does not have stay zero (channel padding)
+    if (chunk * 16 < g.s_cp) {
+        int hs = oh * g.sh - g.pad_top, ws = ow * g.sw - g.pad_left;
+        const int he = min(hs + g.kh, g.h), we = min(ws + g.kw, g.w);
+        hs = max(hs, 0);
+        ws = max(ws, 0);
+        const int8_t *base = src + ((int64_t(ni) * g.s_hs + g.s_pt) * g.s_ws + g.s_pl) * g.s_cp + chunk * 16;
+        r = *reinterpret_cast<const v4i *>(base + (int64_t(hs) * g.s_ws + ws) * g.s_cp);   // the first valid element
+        for (int ih = hs; ih < he; ++ih)
+            for (int iw = ws; iw < we; ++iw) {
+                const v4i v = *reinterpret_cast<const v4i *>(base + (int64_t(ih) * g.s_ws + iw) * g.s_cp);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) r[k] = int(max_i8x4(uint32_t(r[k]), uint32_t(v[k])));
+            }
+    }
+    *reinterpret_cast<v4i *>(dst + ((int64_t(ni) * g.d_hs + oh + g.d_pt) * g.d_ws + ow + g.d_pl) * g.d_cp + chunk * 16) = r;
+}
+
 }  // namespace
 
 extern "C" {
@@ -89,6 +141,33 @@ int tsx_pooling2d_f32(const float *x_dev, int64_t planes, int32_t h, int32_t w, 
     hipLaunchKernelGGL(pooling2d_kernel, dim3(unsigned(tsx::ceil_div(total, 256))), dim3(256), 0, tsx::as_stream(stream),
                        x_dev, g, out_dev);
     TSX_LAUNCH_CHECK("pooling2d_kernel");
+    return 0;
+}
+
+int tsx_max_pooling2d_i8_staged(const tsx_staged_map *src, const tsx_staged_map *dst, int32_t kh, int32_t kw, int32_t pad_top,
+                                int32_t pad_left, int32_t stride_h, int32_t stride_w, void *stream) {
+    TSX_REQUIRE(src && dst && src->data && dst->data, "max_pooling2d_i8_staged: null pointer");
+    for (const tsx_staged_map *m : {src, dst}) {
+        TSX_REQUIRE(m->n > 0 && m->h > 0 && m->w > 0 && m->c > 0 && m->cp >= m->c && m->cp % 64 == 0 && m->pad_top >= 0 &&
+                        m->pad_left >= 0 && m->h + m->pad_top <= m->hs && m->w + m->pad_left <= m->ws,
+                    "max_pooling2d_i8_staged: map %dx%dx%d does not fit [%d][%d][%d] at (%d,%d)", m->h, m->w, m->c, m->hs,
+                    m->ws, m->cp, m->pad_top, m->pad_left);
+        TSX_REQUIRE(reinterpret_cast<uintptr_t>(m->data) % 16 == 0, "max_pooling2d_i8_staged: buffers must be 16-byte aligned");
+    }
+    TSX_REQUIRE(src->n == dst->n && src->c == dst->c, "max_pooling2d_i8_staged: batch / channels differ");
+    // padding smaller than the window: together with the next check every window holds a valid element
+    TSX_REQUIRE(kh > 0 && kw > 0 && stride_h > 0 && stride_w > 0 && pad_top >= 0 && pad_left >= 0 && pad_top < kh && pad_left < kw,
+                "max_pooling2d_i8_staged: bad window");
+    TSX_REQUIRE((int64_t(dst->h) - 1) * stride_h - pad_top < src->h && (int64_t(dst->w) - 1) * stride_w - pad_left < src->w,
+                "max_pooling2d_i8_staged: output %dx%d has windows outside the %dx%d map", dst->h, dst->w, src->h, src->w);
+    PoolStagedGeom g{src->n, src->h, src->w, dst->h, dst->w, pad_top, pad_left, kh, kw, stride_h, stride_w,
+                     src->hs, src->ws, src->cp, src->pad_top, src->pad_left,
+                     dst->hs, dst->ws, dst->cp, dst->pad_top, dst->pad_left};
+    const int64_t total = int64_t(dst->n) * dst->h * dst->w * (dst->cp / 16);
+    TSX_REQUIRE(tsx::ceil_div(total, 256) < (int64_t(1) << 31), "max_pooling2d_i8_staged: tensor too large");
+    hipLaunchKernelGGL(max_pooling2d_i8_staged_kernel, dim3(unsigned(tsx::ceil_div(total, 256))), dim3(256), 0,
+                       tsx::as_stream(stream), static_cast<const int8_t *>(src->data), g, static_cast<int8_t *>(dst->data));
+    TSX_LAUNCH_CHECK("max_pooling2d_i8_staged_kernel");
     return 0;
 }
 

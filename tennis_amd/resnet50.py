@@ -175,12 +175,29 @@ class ResNet50Int8:
         sxs = self._batch_scales(n)
         relu = lambda spec: "relu" if spec.relu else None
 
-        y = self.conv[stem.name](x, dq=self._dq[stem.name], bias=self.bias[stem.name], act=relu(stem),
-                                 x_scales=sxs[stem.name])[0]
-        y = capi.pooling2d(y, "max", *self.POOL)
         c1 = net[0][0]
-        s_in = self._staged_input(c1, y.shape)
-        self.conv[c1.name].stage(y, s_in, x_scales=sxs[c1.name])     # the only staging pass after the stem
+        if net[0][3] is not None:
+            # Nothing reads the pooled tensor in fp32 (the first block's shortcut is a projection), and quantize
+            # commutes with max: the stem requantizes for layer 1 in its epilogue and the pooling runs on int8,
+            # from the stem's pixel-major output straight into layer 1's staged input.
+            h1 = (x.shape[2] + 2 * stem.pad - stem.k) // stem.stride + 1
+            w1 = (x.shape[3] + 2 * stem.pad - stem.k) // stem.stride + 1
+            key = ("stem_out", n, h1, w1)
+            if key not in self._staged:
+                self._staged[key] = capi.StagedPlain((n, stem.cout, h1, w1), self.dev)
+            s_stem = self._staged[key]
+            self.conv[stem.name](x, dq=self._dq[stem.name], bias=self.bias[stem.name], act=relu(stem),
+                                 x_scales=sxs[stem.name], q_scales=sxs[c1.name], want_f32=False, staged_out=s_stem)
+            hp, wp = capi.pool_out_size(h1, w1, self.POOL[0], self.POOL[2], self.POOL[1])
+            s_in = self._staged_input(c1, (n, stem.cout, hp, wp))
+            capi.max_pooling2d_staged(s_stem, s_in, *self.POOL)
+            y = None
+        else:
+            y = self.conv[stem.name](x, dq=self._dq[stem.name], bias=self.bias[stem.name], act=relu(stem),
+                                     x_scales=sxs[stem.name])[0]
+            y = capi.pooling2d(y, "max", *self.POOL)
+            s_in = self._staged_input(c1, y.shape)
+            self.conv[c1.name].stage(y, s_in, x_scales=sxs[c1.name])     # the only staging pass after the stem
         for bi, (c1, c2, c3, proj) in enumerate(net):
             conv1, conv2, conv3 = self.conv[c1.name], self.conv[c2.name], self.conv[c3.name]
             in_shape = s_in.x_shape

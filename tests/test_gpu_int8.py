@@ -214,6 +214,47 @@ def test_conv2d_i8_staged_hand_over(tsx, port, cmid, a_strides):
         A(_dev(xq), dq=_dev(dqa), q_scales=_dev(qs), staged_out=small)
 
 
+@pytest.mark.parametrize("geom", [((3, 3), (2, 2), (0, 1, 0, 1)), ((2, 2), (2, 2), (0, 0, 0, 0)), ((3, 3), (1, 1), (1, 1, 1, 1)),
+                                  ((5, 5), (1, 1), (2, 2, 2, 2))])
+@pytest.mark.parametrize("few_channels", [False, True])   # producer = window-stationary kernel / im2col-staged stem
+def test_max_pooling_on_staged_int8(tsx, port, geom, few_channels):
+    """producer (requantized, pixel-major int8) -> max pooling on int8 -> consumer convolution must equal the
+    operator chain conv -> bias -> relu -> pooling2d(fp32) -> quantize -> conv2d_quantized bit for bit."""
+    ksize, strides, pads = geom
+    rng = np.random.default_rng(206)
+    n, cin, h, w, cmid = (2, 3, 23, 21, 64) if few_channels else (2, 40, 13, 15, 70)
+    k = 7 if few_channels else 3
+    x = rng.standard_normal((n, cin, h, w)).astype(np.float32)
+    x_scales = np.full(n, 40.0, np.float32)
+    wa = rng.integers(-127, 128, (cmid, cin, k, k)).astype(np.int8)
+    dqa = rng.uniform(1e-4, 3e-4, cmid).astype(np.float32)
+    ba = rng.standard_normal(cmid).astype(np.float32)
+    qs = np.full(n, 5.0, np.float32)
+    a_strides = (2, 2) if few_channels else (1, 1)
+    A = tsx.Conv2dI8(_dev(wa), (k // 2,) * 4, a_strides)
+    xq = port.quantize(x, x_scales)
+    exp_f = port.conv2d_i8_fused(xq, wa, dqa, ba, "relu", 0.0, None, (k // 2,) * 4, a_strides)[0]
+    pooled = port.pooling2d(exp_f, "max", ksize, strides, pads)
+    pooled_q = port.quantize(pooled, qs)
+    wb = rng.integers(-127, 128, (48, cmid, 3, 3)).astype(np.int8)
+    dqb = rng.uniform(1e-4, 3e-4, 48).astype(np.float32)
+    B = tsx.Conv2dI8(_dev(wb), (1, 1, 1, 1))
+    s_mid = tsx.StagedPlain(tuple(exp_f.shape), "cuda")
+    f, q, _ = A(_dev(x), dq=_dev(dqa), bias=_dev(ba), act="relu", x_scales=_dev(x_scales), q_scales=_dev(qs), want_f32=False,
+                staged_out=s_mid)
+    assert f is None and q is None
+    s_b = tsx.StagedInput(B, tuple(pooled.shape))
+    tsx.max_pooling2d_staged(s_mid, s_b, ksize, strides, pads)
+    got = B.run_staged(s_b, _dev(dqb))[0].cpu().numpy()
+    assert np.array_equal(bits(got), bits(port.conv2d_quantized(pooled_q, wb, dqb, (1, 1, 1, 1))))
+    with pytest.raises(tsx.TsxError):                # windows that start outside the map
+        bad = tsx.StagedInput(B, (n, cmid, pooled.shape[2] + 3, pooled.shape[3]))
+        a, b = tsx._staged_map(s_mid), tsx._staged_map(bad)
+        import ctypes
+        tsx.check(tsx.lib().tsx_max_pooling2d_i8_staged(ctypes.byref(a), ctypes.byref(b), ksize[0], ksize[1], pads[0], pads[2],
+                                                        strides[0], strides[1], None))
+
+
 def test_quantize_conv2d_fused_input(tsx, port):
     rng = np.random.default_rng(203)
     for n in (1, 4):
