@@ -359,32 +359,56 @@ __global__ __launch_bounds__(256) void stage_im2col_rows_kernel(const void *__re
     const float img_scale = uniform_scale ? scales[n_scales == 1 ? 0 : ni] : 0.f;
     const int h0 = oh * g.sh - g.pad_top;
     const int rows = g.c * g.kh;
-    for (int idx = tid; idx < rows * wpatch; idx += 256) {
-        const int row = idx / wpatch, col = idx - row * wpatch;
+    // phase 1: wavefront per patch row, lanes along W (no per-element index arithmetic)
+    for (int row = tid >> 6; row < rows; row += 4) {
         const int ci = row / g.kh, r = row - ci * g.kh;
-        const int hi = h0 + r * g.dh, wi = col - g.pad_left;
-        int q = g.pad_value;
-        if (hi >= 0 && hi < g.h && wi >= 0 && wi < g.w) {
-            const int64_t e = ((int64_t(ni) * g.c + ci) * g.h + hi) * g.w + wi;
-            if (QUANT) {
-                const float sc = uniform_scale ? img_scale : scales[e / group_len];
-                q = tsx::quantize_value(__fmul_rn(static_cast<const float *>(src)[e], sc), n_scales == 1 && e < bulk8);
-            } else {
-                q = static_cast<const int8_t *>(src)[e];
+        const int hi = h0 + r * g.dh;
+        const bool row_in = hi >= 0 && hi < g.h;
+        const int64_t e0 = ((int64_t(ni) * g.c + ci) * g.h + hi) * g.w;
+        for (int col = tid & 63; col < wpatch; col += 64) {
+            const int wi = col - g.pad_left;
+            int q = g.pad_value;
+            if (row_in && wi >= 0 && wi < g.w) {
+                const int64_t e = e0 + wi;
+                if (QUANT) {
+                    const float sc = uniform_scale ? img_scale : scales[e / group_len];
+                    q = tsx::quantize_value(__fmul_rn(static_cast<const float *>(src)[e], sc), n_scales == 1 && e < bulk8);
+                } else {
+                    q = static_cast<const int8_t *>(src)[e];
+                }
             }
+            patch[row * wpatch + col] = int8_t(q);
         }
-        patch[idx] = int8_t(q);
     }
     __syncthreads();
-    const int chunks = g.cp / 16;
+    // phase 2: a lane keeps one K chunk for the whole row, so the patch offsets of its 16 bytes are
+    // computed once; per output pixel it reads 16 bytes at (pixel origin + offset) and stores 16 bytes.
+    const int chunks = g.cp / 16;          // <= 256 (K <= 4096)
+    const int ppi = 256 / chunks;          // pixels per pass over the workgroup
+    const int chunk = tid % chunks, p0 = tid / chunks;
+    if (p0 >= ppi) return;
     const int taps = g.kh * g.kw;
-    int8_t *dst = xs + (int64_t(ni) * g.ho + oh) * g.wo * g.cp;
-    for (int id = tid; id < g.wo * chunks; id += 256) {
-        const int ow = id / chunks, chunk = id - ow * chunks;
+    int off[16];
+    {
         int k = chunk * 16;
         int ci = k / taps;
         int kh = (k - ci * taps) / g.kw;
         int kw = k - ci * taps - kh * g.kw;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            off[j] = k < g.kk ? (ci * g.kh + kh) * wpatch + kw * g.dw : -1;   // K padding reads as zero
+            ++k;
+            if (++kw == g.kw) {
+                kw = 0;
+                if (++kh == g.kh) {
+                    kh = 0;
+                    ++ci;
+                }
+            }
+        }
+    }
+    int8_t *dst = xs + (int64_t(ni) * g.ho + oh) * g.wo * g.cp + chunk * 16;
+    for (int ow = p0; ow < g.wo; ow += ppi) {
         const int8_t *base = patch + ow * g.sw;
         uint32_t words[4];
 #pragma unroll
@@ -392,21 +416,14 @@ __global__ __launch_bounds__(256) void stage_im2col_rows_kernel(const void *__re
             uint32_t word = 0;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                int q = 0;   // K padding: the packed weights are zero there as well
-                if (k < g.kk) q = base[(ci * g.kh + kh) * wpatch + kw * g.dw];
+                const int o = off[v * 4 + j];
+                const int b = base[o >= 0 ? o : 0];
+                const int q = o >= 0 ? b : 0;
                 word |= uint32_t(q & 0xff) << (8 * j);
-                ++k;
-                if (++kw == g.kw) {
-                    kw = 0;
-                    if (++kh == g.kh) {
-                        kh = 0;
-                        ++ci;
-                    }
-                }
             }
             words[v] = word;
         }
-        *reinterpret_cast<uint4 *>(dst + int64_t(id) * 16) = make_uint4(words[0], words[1], words[2], words[3]);
+        *reinterpret_cast<uint4 *>(dst + int64_t(ow) * g.cp) = make_uint4(words[0], words[1], words[2], words[3]);
     }
 }
 
