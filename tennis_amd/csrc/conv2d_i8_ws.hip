@@ -359,7 +359,11 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
                             // swap(a, b): a's upper half-wave <-> b's lower half-wave
                             const auto s02 = __builtin_amdgcn_permlane32_swap(word[0], word[2], false, false);
                             const auto s13 = __builtin_amdgcn_permlane32_swap(word[1], word[3], false, false);
-                            int8_t *dst = p.st_out + ((int64_t(img + (wrapped ? 1 : 0)) * p.st_hs + oh + p.st_pt) * p.st_ws + ow + p.st_pl) * p.st_cp +
+                            // the consumer's buffer is addressed by the real row/column (this kernel's rows may be virtual)
+                            const int pix = oh * p.wo + ow;
+                            const int roh = p.wo == p.o_w ? oh : pix / p.o_w;
+                            const int row_ = p.wo == p.o_w ? ow : pix - roh * p.o_w;
+                            int8_t *dst = p.st_out + ((int64_t(img + (wrapped ? 1 : 0)) * p.st_hs + roh + p.st_pt) * p.st_ws + row_ + p.st_pl) * p.st_cp +
                                           cf + 16 * (lane / 32);
                             const v4i packed = {int(s02[0]), int(s02[1]), int(s13[0]), int(s13[1])};
                             *reinterpret_cast<v4i *>(dst) = packed;
@@ -396,9 +400,22 @@ int launch_nt(const WsParams &p, dim3 grid, size_t lds_bytes, hipStream_t stream
 
 }  // namespace
 
-WsPlan ws_plan(const WsGeom &g) {
+WsPlan ws_plan(const WsGeom &g_in) {
     WsPlan pl{};
     pl.ok = false;
+    // A 1x1 layer reading a buffer without halo is a plain [positions][channels] matrix: rows mean nothing,
+    // so it is tiled as rows of ONE pixel (ho*wo of them per image) -- a tile is then any number of
+    // consecutive pixels, chosen below as whole fragments whatever the map's width (3136 = 56x56 positions
+    // per image give 128-position tiles with no padding; a 608-wide map is no obstacle).
+    WsGeom g = g_in;
+    if (g.kh == 1 && g.kw == 1 && g.hs == g.ho && g.ws == g.wo && int64_t(g.n) * g.ho * g.wo < (int64_t(1) << 31)) {
+        g.ho = g.hs = g_in.ho * g_in.wo;
+        g.wo = g.ws = 1;
+    }
+    pl.ho = g.ho;
+    pl.wo = g.wo;
+    pl.hs = g.hs;
+    pl.ws = g.ws;
     // stride-1 only (the caller checks strides).  A tile is TH output rows of the batch-wide row
     // sequence, at most MAX_NT fragments of 32 positions.  Candidates are ranked by a model of the
     // busiest CU's time in units of one fragment's work,
@@ -465,10 +482,10 @@ int ws_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t 
     p.n = g.n;
     p.cout = g.cout;
     p.coutp = pl.coutp;
-    p.ho = g.ho;
-    p.wo = g.wo;
-    p.hs = g.hs;
-    p.ws = g.ws;
+    p.ho = pl.ho;   // the plan's view of the map (1-pixel rows for 1x1 layers)
+    p.wo = pl.wo;
+    p.hs = pl.hs;
+    p.ws = pl.ws;
     p.cp = g.cp;
     p.cblocks = g.cblocks;
     p.kh = g.kh;

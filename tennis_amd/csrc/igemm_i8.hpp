@@ -122,6 +122,7 @@ struct WsPlan {
     bool ok;            // geometry supported
     int th, nt;         // output rows per tile, 32-position fragments per wavefront
     int wm;             // wavefronts along cout: 4, or 2 with the tile's positions split over the other factor
+    int ho, wo, hs, ws; // the map as the kernel walks it: the real one, or rows of one pixel for 1x1 layers without halo
     int64_t tiles;      // tiles over the batch-wide row sequence
     int wr, wc, wp;     // window rows, cols, pixels
     int ksteps_p;       // K-steps padded to the A-ring size
