@@ -74,6 +74,8 @@ int tsx_conv2d_out_size(const tsx_conv2d_geom *g, int32_t *out_h, int32_t *out_w
  *                                           other branch of the block, same shape as the output)
  *   y = act(y)                              relu.cpp / leaky_relu.cpp (incl. their SIMD-body /
  *                                           scalar-tail difference in signed zero and NaN)
+ *   (residual_after_act != 0 swaps the last two: y = act(y) + residual[i], a shortcut that joins
+ *   behind the activation, as in darknet-style residual units)
  *   q = quantize(y)           if out_i8     quantize.cpp:70-125 with q_scales[n_qscales]
  * All pointers are device pointers; unused ones are NULL. */
 typedef struct tsx_epilogue {
@@ -93,6 +95,7 @@ typedef struct tsx_epilogue {
      * channel padding are written once by tsx_conv2d_i8_stage_fill.  NULL = not used. */
     int8_t *staged_out_dev;
     int32_t staged_hs, staged_ws, staged_cp, staged_pad_top, staged_pad_left;
+    int32_t residual_after_act; /* 0: act(y + residual); 1: act(y) + residual */
 } tsx_epilogue;
 
 /* ---------------------------------------------------------------- quantize

@@ -34,7 +34,7 @@ class Epilogue(ctypes.Structure):
     _fields_ = [("dq_dev", _vp), ("row_scale_dev", _vp), ("bias_dev", _vp), ("act", _i32), ("slope", _f32),
                 ("q_scales_dev", _vp), ("n_qscales", _i32), ("residual_dev", _vp), ("staged_out_dev", _vp),
                 ("staged_hs", _i32), ("staged_ws", _i32), ("staged_cp", _i32), ("staged_pad_top", _i32),
-                ("staged_pad_left", _i32)]
+                ("staged_pad_left", _i32), ("residual_after_act", _i32)]
 
 
 class TsxError(RuntimeError):
@@ -160,7 +160,8 @@ def quantize(x, scales):
 class _EpilogueArgs:
     """Keeps the device tensors of an epilogue alive next to the C struct."""
 
-    def __init__(self, dq, bias=None, act=None, slope=0.0, q_scales=None, row_scale=None, residual=None, staged_out=None):
+    def __init__(self, dq, bias=None, act=None, slope=0.0, q_scales=None, row_scale=None, residual=None, staged_out=None,
+                 residual_after_act=False):
         self.dq = _dev(dq, torch.float32)
         self.bias = _dev(bias, torch.float32)
         self.q_scales = _dev(q_scales, torch.float32)
@@ -169,6 +170,7 @@ class _EpilogueArgs:
         self.c = Epilogue(_ptr(self.dq), _ptr(self.row_scale), _ptr(self.bias), _ACT[act], float(slope),
                           _ptr(self.q_scales), 0 if self.q_scales is None else self.q_scales.numel(),
                           _ptr(self.residual))
+        self.c.residual_after_act = int(bool(residual_after_act))
         self.staged_out = staged_out     # StagedInput of the consuming convolution
         if staged_out is not None:
             self.c.staged_out_dev = staged_out.buf.data_ptr()
@@ -243,7 +245,7 @@ class Conv2dI8:
                                         _stream()))
 
     def run_staged(self, staged, dq, bias=None, act=None, slope=0.0, q_scales=None, want_f32=True, residual=None,
-                   staged_out=None):
+                   staged_out=None, residual_after_act=False):
         """The convolution on a StagedInput (its own, or another consumer's of the same tensor).  Returns
         (out_f32 or None, out_i8 or None); with staged_out the int8 output goes to that StagedInput instead."""
         geom, packed, _ = self._plan(staged.x_shape)
@@ -251,7 +253,8 @@ class Conv2dI8:
         shape = (staged.x_shape[0], self.w.shape[0], ho, wo)
         if residual is not None and tuple(residual.shape) != shape:
             raise TsxError("residual shape %s != output shape %s" % (tuple(residual.shape), shape))
-        ep = _EpilogueArgs(dq, bias, act, slope, q_scales, residual=residual, staged_out=staged_out)
+        ep = _EpilogueArgs(dq, bias, act, slope, q_scales, residual=residual, staged_out=staged_out,
+                           residual_after_act=residual_after_act)
         out_f32 = torch.empty(shape, dtype=torch.float32, device=self.w.device) if want_f32 else None
         out_i8 = (torch.empty(shape, dtype=torch.int8, device=self.w.device)
                   if (q_scales is not None and staged_out is None) else None)
@@ -260,7 +263,7 @@ class Conv2dI8:
         return out_f32, out_i8
 
     def __call__(self, x, dq=None, bias=None, act=None, slope=0.0, q_scales=None, x_scales=None,
-                 want_f32=True, want_acc=False, residual=None, staged_out=None):
+                 want_f32=True, want_acc=False, residual=None, staged_out=None, residual_after_act=False):
         """x: int8 NCHW device tensor, or fp32 NCHW with x_scales (fused quantize); residual: fp32 tensor of
         the output's shape added before the activation.
 
@@ -270,7 +273,8 @@ class Conv2dI8:
         geom, packed, ws_bytes = self._plan(tuple(x.shape))
         ho, wo = conv_out_size(geom)
         shape = (x.shape[0], self.w.shape[0], ho, wo)
-        ep = _EpilogueArgs(dq, bias, act, slope, q_scales, residual=residual, staged_out=staged_out) if dq is not None else None
+        ep = (_EpilogueArgs(dq, bias, act, slope, q_scales, residual=residual, staged_out=staged_out,
+                            residual_after_act=residual_after_act) if dq is not None else None)
         if residual is not None and tuple(residual.shape) != shape:
             raise TsxError("residual shape %s != output shape %s" % (tuple(residual.shape), shape))
         out_f32 = torch.empty(shape, dtype=torch.float32, device=x.device) if (want_f32 and ep) else None

@@ -865,6 +865,7 @@ void fill_epilogue(tsx::EpiParams &p, const tsx_epilogue *ep, int64_t count, flo
     p.bias = ep ? ep->bias_dev : nullptr;
     p.q_scales = ep ? ep->q_scales_dev : nullptr;
     p.residual = ep ? ep->residual_dev : nullptr;
+    p.res_after = (ep && ep->residual_dev && ep->residual_after_act) ? 1 : 0;
     p.act = ep ? ep->act : 0;
     p.slope = ep ? ep->slope : 0.f;
     p.n_qscales = ep ? ep->n_qscales : 0;

@@ -300,7 +300,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
                         constexpr int r = decltype(rc)::value;
                         v[r] = __fadd_rn(v[r], bias[r]);
                     });
-                    if (EXTRA && p.residual) static_for<0, 16>([&](auto rc) {
+                    if (EXTRA && p.residual && !p.res_after) static_for<0, 16>([&](auto rc) {
                         constexpr int r = decltype(rc)::value;
                         v[r] = __fadd_rn(v[r], res[j][r]);
                     });
@@ -320,6 +320,10 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
                             v[r] = apply_act(v[r], TSX_ACT_MISH, 0.f, true);
                         });
                     }
+                    if (EXTRA && p.residual && p.res_after) static_for<0, 16>([&](auto rc) {
+                        constexpr int r = decltype(rc)::value;
+                        v[r] = __fadd_rn(v[r], res[j][r]);
+                    });
                     if (p.out_f32) static_for<0, 16>([&](auto rc) {
                         constexpr int r = decltype(rc)::value;
                         constexpr int dco = 8 * (r / 4) + (r % 4);

@@ -22,6 +22,7 @@ struct EpiParams {
     int8_t *st_out;
     int st_hs, st_ws, st_cp, st_pt, st_pl;
     int o_c, o_h, o_w;   // NCHW extents of the output, to decode a linear index
+    int res_after;       // residual joins behind the activation instead of in front of it
 };
 
 // fp32 value of one accumulator after dequant -> row scale -> bias -> residual -> activation;
@@ -30,8 +31,10 @@ __device__ __forceinline__ float epi_value(const EpiParams &p, int acc, int64_t 
     float v = __fmul_rn(float(acc), dq);
     if (p.row_scale) v = __fmul_rn(v, row_scale);
     if (p.bias) v = __fadd_rn(v, bias);
-    if (p.residual) v = __fadd_rn(v, p.residual[idx]);
-    return apply_act(v, p.act, p.slope, idx < p.act_body);
+    if (p.residual && !p.res_after) v = __fadd_rn(v, p.residual[idx]);
+    v = apply_act(v, p.act, p.slope, idx < p.act_body);
+    if (p.residual && p.res_after) v = __fadd_rn(v, p.residual[idx]);
+    return v;
 }
 
 // Epilogue of one accumulator: every requested output of element idx.
@@ -72,10 +75,12 @@ __device__ __forceinline__ void epilogue_rows16(const EpiParams &p, const v16i &
 #pragma unroll
         for (int r = 0; r < 16; ++r) v[r] = __fadd_rn(v[r], bias[r]);
     }
+    float res[16];
     if (p.residual) {
-        float res[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) res[r] = p.residual[idx0 + int64_t(8 * (r / 4) + (r % 4)) * row_stride];
+    }
+    if (p.residual && !p.res_after) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) v[r] = __fadd_rn(v[r], res[r]);
     }
@@ -88,6 +93,10 @@ __device__ __forceinline__ void epilogue_rows16(const EpiParams &p, const v16i &
     } else if (p.act == TSX_ACT_MISH) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) v[r] = apply_act(v[r], TSX_ACT_MISH, 0.f, true);
+    }
+    if (p.residual && p.res_after) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) v[r] = __fadd_rn(v[r], res[r]);
     }
     if (p.out_f32) {
 #pragma unroll

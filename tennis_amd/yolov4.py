@@ -166,6 +166,7 @@ class YoloV4Int8:
             self.conv[i] = capi.Conv2dI8(torch.from_numpy(p["wq"]).to(self.dev), (l["size"] // 2,) * 4, (l["stride"],) * 2)
             self.bias[i] = torch.from_numpy(p["bias"]).to(self.dev)
         self.scales = None
+        self._shapes = {}
 
     def set_scales(self, scales, n):
         self.scales = dict(scales)
@@ -179,9 +180,141 @@ class YoloV4Int8:
         self.set_scales(self.scales, x.shape[0])
         return dict(self.scales)
 
-    def forward(self, x):
+    def forward(self, x, chained=True):
         assert self.scales is not None
-        return self._run(x, calibrating=False)
+        return self._run_chained(x) if chained else self._run(x, calibrating=False)
+
+    # ---------------------------------------------------------------- chained inference
+    def _chain_plan(self):
+        """Who reads what, with single-source routes looked through and `conv -> shortcut` pairs folded into the
+        convolution's epilogue (darknet's shortcut adds behind the activation).  Returns per layer: the resolved
+        sources, the consumers of each tensor, and for folded shortcuts the convolution that absorbs them."""
+        L = self.L
+
+        def root(j):
+            while j >= 0 and L[j]["type"] == "route" and len(self.srcs[j]) == 1:
+                j = self.srcs[j][0]
+            return j
+
+        rsrcs = [[root(j) for j in s] for s in self.srcs]
+        identity = [l["type"] == "route" and len(self.srcs[i]) == 1 for i, l in enumerate(L)]
+        consumers = {i: [] for i in range(-1, len(L))}
+        for i, s in enumerate(rsrcs):
+            if not identity[i]:
+                for j in s:
+                    consumers[j].append(i)
+        heads = {root(h) for h in self.heads}
+        folded = {}      # shortcut layer -> the convolution whose epilogue performs it
+        for i, l in enumerate(L):
+            if l["type"] == "shortcut":
+                a, b = rsrcs[i]
+                if L[a]["type"] == "conv" and consumers[a] == [i] and a not in heads and a != b:
+                    folded[i] = a
+        return rsrcs, consumers, heads, folded
+
+    def _run_chained(self, x):
+        """Inference with int8 hand-over: a convolution whose output feeds convolutions writes it requantized
+        straight into their staged input (one buffer per consumer geometry; consumers of one tensor share its
+        calibrated scale), keeps an fp32 copy only if something else reads it (route, shortcut, pooling,
+        upsample, a head), and performs a following shortcut in its epilogue.  Values equal the
+        operator-by-operator path (_run)."""
+        n = x.shape[0]
+        if not hasattr(self, "_plan"):
+            self._plan = self._chain_plan()
+            self._staged = {}
+        rsrcs, consumers, heads, folded = self._plan
+        absorbed = {a: s for s, a in folded.items()}
+        L = self.L
+        outs = [None] * len(L)            # fp32 tensors
+        staged_for = {}                   # consumer conv -> StagedInput holding its input (written by the producer)
+        last_use = {}
+        for i, s in enumerate(rsrcs):
+            for j in s:
+                last_use[j] = i
+        get = lambda j: x if j < 0 else outs[j]
+
+        def staged_input(k, shape):
+            key = (k, tuple(shape))
+            if key not in self._staged:
+                self._staged[key] = capi.StagedInput(self.conv[k], shape)
+            return self._staged[key]
+
+        for i, l in enumerate(L):
+            t = l["type"]
+            if t == "conv":
+                out_id = absorbed.get(i, i)                     # the tensor this kernel produces
+                conv = self.conv[i]
+                src = rsrcs[i][0]
+                in_shape = tuple(x.shape) if src < 0 else self._shapes[src]
+                ho = (in_shape[2] + 2 * (l["size"] // 2) - l["size"]) // l["stride"] + 1
+                wo = (in_shape[3] + 2 * (l["size"] // 2) - l["size"]) // l["stride"] + 1
+                shape = (n, l["filters"], ho, wo)
+                self._shapes[out_id] = shape
+                self._shapes[i] = shape
+                # consumers of the produced tensor
+                conv_cons = [k for k in consumers[out_id] if L[k]["type"] == "conv"]
+                others = [k for k in consumers[out_id] if L[k]["type"] != "conv"]
+                target, served = None, []
+                for k in conv_cons:
+                    if self._stageable(k):
+                        st = staged_input(k, shape)
+                        if target is None:
+                            target, served = st, [k]
+                        elif (st.hs, st.ws, st.cp, st.pad_top, st.pad_left) == (target.hs, target.ws, target.cp, target.pad_top, target.pad_left):
+                            served.append(k)
+                for k in served:
+                    assert self.scales[k] == self.scales[served[0]]   # calibrated on the same tensor
+                    staged_for[k] = target
+                want_f32 = bool(others) or out_id in heads or any(k not in served for k in conv_cons)
+                kw = dict(dq=self.dq[i], bias=self.bias[i], act=l["act"], slope=0.1, want_f32=want_f32)
+                if target is not None:
+                    kw.update(q_scales=self.sx[served[0]], staged_out=target)
+                if i in absorbed:
+                    kw.update(residual=outs[rsrcs[absorbed[i]][1]], residual_after_act=True)
+                if i in staged_for:
+                    y = conv.run_staged(staged_for[i], **kw)[0]
+                else:
+                    y = conv(get(src), x_scales=self.sx[i], **kw)[0]
+                outs[out_id] = y
+                if out_id != i:
+                    outs[i] = None
+            elif t == "shortcut":
+                if i not in folded:
+                    a, b = rsrcs[i]
+                    outs[i] = capi.add(outs[a], outs[b])
+                    self._shapes[i] = self._shapes[a]
+            elif t == "route":
+                s = rsrcs[i]
+                if len(self.srcs[i]) == 1:
+                    outs[i] = None                                 # looked through
+                    self._shapes[i] = self._shapes[s[0]]
+                else:
+                    outs[i] = capi.concat_channels([outs[j] for j in s])
+                    self._shapes[i] = tuple(outs[i].shape)
+            elif t == "maxpool":
+                k = l["size"]
+                outs[i] = capi.pooling2d(outs[rsrcs[i][0]], "max", (k, k), (1, 1), (k // 2,) * 4)
+                self._shapes[i] = tuple(outs[i].shape)
+            elif t == "upsample":
+                src = outs[rsrcs[i][0]]
+                outs[i] = capi.resize_nearest(src, src.shape[2] * 2, src.shape[3] * 2)
+                self._shapes[i] = tuple(outs[i].shape)
+            for j in rsrcs[i]:                                     # free activations nothing reads any more
+                if j >= 0 and last_use.get(j) == i and j not in heads:
+                    outs[j] = None
+        res = []
+        for h in self.heads:
+            j = h
+            while L[j]["type"] == "route" and len(self.srcs[j]) == 1:
+                j = self.srcs[j][0]
+            res.append(outs[j])
+        return res
+
+    def _stageable(self, k):
+        """True when convolution k can read a staged buffer a producer wrote (not an im2col-staged layer)."""
+        l = self.L[k]
+        cin = self.host[k]["wq"].shape[1]
+        return not (l["size"] > 1 and cin <= 8 and cin * l["size"] ** 2 <= 512)
 
     def _run(self, x, calibrating):
         n = x.shape[0]

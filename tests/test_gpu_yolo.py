@@ -55,7 +55,10 @@ def test_yolov4_shaped_network(port, mish):
     x = np.random.default_rng(6).uniform(0, 1, (2, 3, 64, 64)).astype(np.float32)
     xd = torch.from_numpy(x).cuda()
     scales = net.calibrate(xd)
-    got = [t.cpu().numpy() for t in net.forward(xd)]
+    got = [t.cpu().numpy() for t in net.forward(xd)]                      # chained: int8 hand-over, folded shortcuts
+    plain = [t.cpu().numpy() for t in net.forward(xd, chained=False)]      # one operator per layer, fp32 in between
+    for g, q in zip(got, plain):
+        assert np.array_equal(bits(g), bits(q))
     srcs, _ = yolov4.resolve(L)
     exp = oracle_forward(port, L, heads, srcs, params, scales, x)
     assert [g.shape for g in got] == [(2, 24, 8, 8), (2, 24, 4, 4), (2, 24, 2, 2)]
