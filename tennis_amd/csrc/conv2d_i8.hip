@@ -779,7 +779,7 @@ struct Plan {
     // few input channels x large kernel: K packed by explicit im2col, the layer runs as a 1x1 convolution
     bool im2col;
     int kk;   // C*KH*KW
-    // stride-1 layers whose tap window fits LDS take the window-stationary kernel
+    // layers whose tap window fits LDS take the window-stationary kernel
     bool use_ws;
     tsx::WsGeom wsg;
     tsx::WsPlan wsp;
@@ -818,10 +818,11 @@ int make_plan(const tsx_conv2d_geom *g, Plan *pl) {
     pl->staged_bytes = size_t(g->n) * pl->hs * pl->ws * pl->cp;
     pl->packed_bytes = size_t(pl->taps) * pl->cblocks * pl->coutp * KSTEP;
     pl->use_ws = false;
-    if (pl->im2col || (g->stride_h == 1 && g->stride_w == 1)) {
+    {
         pl->wsg = tsx::WsGeom{g->n, g->cout, pl->ho, pl->wo, pl->hs, pl->ws, pl->cp, pl->cblocks,
                               pl->im2col ? 1 : g->kh, pl->im2col ? 1 : g->kw,
-                              pl->im2col ? 1 : g->dilation_h, pl->im2col ? 1 : g->dilation_w};
+                              pl->im2col ? 1 : g->dilation_h, pl->im2col ? 1 : g->dilation_w,
+                              pl->im2col ? 1 : g->stride_h, pl->im2col ? 1 : g->stride_w};
         pl->wsp = tsx::ws_plan(pl->wsg);
         if (pl->wsp.ok) {
             pl->use_ws = true;

@@ -1,5 +1,5 @@
-// Window-stationary int8 convolution for stride-1 layers (the 3x3 body of ResNet-like nets
-// and BASELINE config 2) on v_mfma_i32_32x32x32_i8
+// Window-stationary int8 convolution (the 3x3 body of ResNet-like nets and BASELINE config 2; any
+// stride, maps of any width through column tiles) on v_mfma_i32_32x32x32_i8
 // (the 16x16x64 form runs at half the rate on this part).
 //
 // Same arithmetic as the generic implicit GEMM in conv2d_i8.hip (exact int32 sums of
@@ -44,7 +44,9 @@ struct WsParams : EpiParams {
     const int8_t *wp;   // packed weights [ks_p][coutp/32][2 halves][64 lanes][16]
     int n, cout, coutp, ho, wo, hs, ws, cp, cblocks, kh, kw, dil_h, dil_w;
     int th, wr, wc, wpix, ksteps_p;
-    int wm;           // wavefronts along cout (4, or 2: the other factor of 4 splits the tile's positions)
+    int wm;           // wavefronts along cout (4, 2 or 1: the other factor of 4 splits the tile's positions)
+    int tw, ctiles;   // tile width in output columns, column tiles per row (1: whole rows)
+    int sh, sw;       // strides
     int stream_out;   // fp32 output written with streaming stores
 };
 
@@ -92,13 +94,16 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
     }
     extern __shared__ __attribute__((aligned(16))) int8_t lds[];   // 2 x wpix x PIX
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
-    const int row0 = blockIdx.x * p.th;      // first output row of the tile, counted over the whole batch
+    const int rtile = blockIdx.x / p.ctiles;
+    const int col0 = (blockIdx.x - rtile * p.ctiles) * p.tw;   // first output column of the tile
+    const int row0 = rtile * p.th;           // first output row of the tile, counted over the whole batch
     const int img = row0 / p.ho;             // image of the tile's first row
     const int th0 = row0 - img * p.ho;       // ... and that row inside it
     const int rows_total = p.n * p.ho;
-    const int wrap = p.hs - p.ho;            // staged rows between the last output row of an image and the next image's first
-    const int wave_m = p.wm == 4 ? wave : wave & 1;                  // position along cout
-    const int pos0 = p.wm == 4 ? 0 : (wave >> 1) * (NT * 32);        // first tile position of this wavefront
+    // staged rows from where output row `ho` of an image would start to the next image's first row
+    const int wrap = p.hs - p.ho * p.sh;
+    const int wave_m = wave & (p.wm - 1);                            // position along cout
+    const int pos0 = (p.wm == 4 ? 0 : p.wm == 2 ? wave >> 1 : wave) * (NT * 32);   // first tile position of this wavefront
     const int m0 = (blockIdx.y * p.wm + wave_m) * (32 * FM);         // first cout of this wavefront
     const int taps = p.kh * p.kw;
     const int win_bytes = p.wpix * PIX;
@@ -114,10 +119,12 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
         if (pix >= p.wpix) pix = p.wpix - 1;   // duplicates rewrite the same bytes
         int wrow = pix / p.wc;
         const int wcol = pix - wrow * p.wc;
-        // stride 1: window row r is staged row (img * hs + th0) + r of the batch-wide staged row sequence
-        int64_t row = int64_t(img) * p.hs + th0 + wrow;
+        // window row r is staged row (img * hs + th0 * stride) + r of the batch-wide staged row sequence
+        int64_t row = int64_t(img) * p.hs + th0 * p.sh + wrow;
         if (row >= int64_t(p.n) * p.hs) row = int64_t(p.n) * p.hs - 1;   // last tile: rows no stored output uses
-        fill_src[i] = p.xs + (row * p.ws + wcol) * p.cp + chunk * 16;
+        int col = col0 * p.sw + wcol;
+        if (col >= p.ws) col = p.ws - 1;                                 // last column tile: columns no stored output uses
+        fill_src[i] = p.xs + (row * p.ws + col) * p.cp + chunk * 16;
         fill_dst[i] = pix * PIX + chunk * 16;
     });
     const int n_fill = (p.wpix * 4 + WS_THREADS - 1) / WS_THREADS;   // <= MAX_FILL, uniform
@@ -141,10 +148,10 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
     static_for<0, NT>([&](auto jc) {
         constexpr int j = decltype(jc)::value;
         int pos = pos0 + j * 32 + lane % 32;
-        if (pos >= p.th * p.wo) pos = 0;       // padding positions: computed, never stored
-        const int r = pos / p.wo, ow = pos - r * p.wo;
-        const int wrow = r + (th0 + r >= p.ho ? wrap : 0);   // positions of the next image sit below its halo rows
-        b_base[j] = (wrow * p.wc + ow) * PIX + (lane / 32) * 16;
+        if (pos >= p.th * p.tw) pos = 0;       // padding positions: computed, never stored
+        const int r = pos / p.tw, tc = pos - r * p.tw;
+        const int wrow = r * p.sh + (th0 + r >= p.ho ? wrap : 0);   // positions of the next image sit below its halo rows
+        b_base[j] = (wrow * p.wc + tc * p.sw) * PIX + (lane / 32) * 16;
     });
 
     // ---- A ring: the wavefront's FM fragments (32 cout each) x 2 halves of K-step ks, 1 KiB each
@@ -231,7 +238,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
     }
 
     // ---- epilogue: accumulator register r of lane l = cout 8*(r/4) + 4*(l/32) + r%4, position l%32
-    const int tile_pos = p.th * p.wo;
+    const int tile_pos = p.th * p.tw;
     const int howo = p.ho * p.wo;
     const int64_t count = int64_t(p.n) * p.cout * howo;
     // hot case: no raw accumulators wanted, every element inside the activation's SIMD-body range,
@@ -263,10 +270,10 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
             static_for<0, NT>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
                 const int pos = pos0 + j * 32 + lane % 32;
-                const int tr = pos / p.wo, ow = pos - tr * p.wo;
+                const int tr = pos / p.tw, ow = col0 + pos - tr * p.tw;
                 const bool wrapped = th0 + tr >= p.ho;
                 const int oh = th0 + tr - (wrapped ? p.ho : 0);
-                const bool pos_ok = pos < tile_pos && row0 + tr < rows_total;
+                const bool pos_ok = pos < tile_pos && row0 + tr < rows_total && ow < p.wo;
                 const unsigned lane_off = unsigned((wrapped ? p.cout * howo : 0) + (4 * (lane / 32)) * howo + oh * p.wo + ow);
                 static_for<0, 16>([&](auto rc) {
                     constexpr int r = decltype(rc)::value;
@@ -278,10 +285,10 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
         static_for<0, NT>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
             const int pos = pos0 + j * 32 + lane % 32;
-            const int tr = pos / p.wo, ow = pos - tr * p.wo;
+            const int tr = pos / p.tw, ow = col0 + pos - tr * p.tw;
             const bool wrapped = th0 + tr >= p.ho;                 // this position belongs to the next image
             const int oh = th0 + tr - (wrapped ? p.ho : 0);
-            const bool pos_ok = pos < tile_pos && row0 + tr < rows_total;
+            const bool pos_ok = pos < tile_pos && row0 + tr < rows_total && ow < p.wo;
             const float q_scale = wrapped ? q_scale_b : q_scale_a;
             if (fast && cf + 32 <= p.cout) {
                 // uniform base in scalar registers + one 32-bit lane offset: no per-store address math
@@ -420,9 +427,9 @@ WsPlan ws_plan(const WsGeom &g_in) {
     pl.wo = g.wo;
     pl.hs = g.hs;
     pl.ws = g.ws;
-    // stride-1 only (the caller checks strides).  A tile is TH output rows of the batch-wide row
-    // sequence, at most MAX_NT fragments of 32 positions.  Candidates are ranked by a model of the
-    // busiest CU's time in units of one fragment's work,
+    // A tile is TH output rows of the batch-wide row sequence x TW output columns (whole rows when they fit),
+    // at most MAX_NT fragments of 32 positions per wavefront.  Candidates are ranked by a model of the busiest
+    // CU's time in units of one fragment's work,
     //     (workgroups per CU) x (0.5 + fragments x slow),
     // where 0.5 is the per-workgroup fixed cost and slow = 1.45 for tiles of more than 4 fragments
     // (one workgroup per CU, so one wavefront per SIMD with nothing to hide its LDS/L2 waits).  The two
@@ -430,37 +437,49 @@ WsPlan ws_plan(const WsGeom &g_in) {
     // layers of a ResNet-50-shaped network, whose small maps want many small workgroups.  Ties go to the
     // fewest total fragments (least padding).
     constexpr int MAX_NT = 7;
-    // at most 64 output channels: two wavefronts along cout, two along the positions of a twice larger tile
-    const int wm = g.cout <= 64 ? 2 : 4, wn = 4 / wm;
-    if (g.wo < 1 || g.wo > 32 * MAX_NT * wn) return pl;
-    const int wrap = g.hs - g.ho;
+    // few output channels: fewer wavefronts along cout, the others take more positions of a larger tile
+    const int wm = g.cout <= 32 ? 1 : g.cout <= 64 ? 2 : 4, wn = 4 / wm;
+    const int cap = 32 * MAX_NT * wn;
+    if (g.wo < 1 || g.sh < 1 || g.sw < 1) return pl;
+    const int wrap = g.hs - g.ho * g.sh;
     const int bm = 32 * WS_FM * wm;
     const int coutp = (g.cout + bm - 1) / bm * bm;
     const int ksteps_p = (g.cblocks * g.kh * g.kw + RING - 1) / RING * RING;
     double best_cost = -1;
     int64_t best_frags = 0;
-    for (int t = 1; t <= g.ho && t * g.wo <= 32 * MAX_NT * wn; ++t) {
-        const int nt = ((t * g.wo + 31) / 32 + wn - 1) / wn;   // fragments per wavefront
-        const int64_t tiles = (int64_t(g.n) * g.ho + t - 1) / t;
-        const bool straddle = g.ho % t != 0;
-        const int wr = t + (g.kh - 1) * g.dil_h + (straddle ? wrap : 0);
-        const int wp = wr * g.ws;
-        if (wp > MAX_WP || size_t(2) * wp * PIX > 65536) continue;   // two windows must fit 64 KiB of LDS
-        const int64_t wgs = tiles * (coutp / bm);
-        const int64_t frags = tiles * nt * wn;
-        const double cost = double((wgs + 255) / 256) * (0.5 + nt * (nt > 4 ? 1.45 : 1.0));
-        if (best_cost < 0 || cost < best_cost || (cost == best_cost && frags < best_frags)) {
-            best_cost = cost;
-            best_frags = frags;
-            pl.th = t;
-            pl.nt = nt;
-            pl.tiles = tiles;
-            pl.wr = wr;
-            pl.wp = wp;
+    // tile widths: the whole row where it (and its window) fits, else multiples of 32 columns (a fragment is
+    // then one run of a row)
+    auto consider = [&](int tw) {
+        const int ctiles = (g.wo + tw - 1) / tw;
+        const int wc = (tw - 1) * g.sw + (g.kw - 1) * g.dil_w + 1;
+        for (int t = 1; t <= g.ho && t * tw <= cap; ++t) {
+            const int nt = ((t * tw + 31) / 32 + wn - 1) / wn;   // fragments per wavefront
+            const int64_t tiles = (int64_t(g.n) * g.ho + t - 1) / t * ctiles;
+            const bool straddle = g.ho % t != 0;
+            const int wr = (t - 1) * g.sh + (g.kh - 1) * g.dil_h + 1 + (straddle && wrap > 0 ? wrap : 0);
+            const int wp = wr * wc;
+            if (wp > MAX_WP || size_t(2) * wp * PIX > 65536) continue;   // two windows must fit 64 KiB of LDS
+            const int64_t wgs = tiles * (coutp / bm);
+            const int64_t frags = tiles * nt * wn;
+            const double cost = double((wgs + 255) / 256) * (0.5 + nt * (nt > 4 ? 1.45 : 1.0));
+            if (best_cost < 0 || cost < best_cost || (cost == best_cost && frags < best_frags)) {
+                best_cost = cost;
+                best_frags = frags;
+                pl.th = t;
+                pl.tw = tw;
+                pl.ctiles = ctiles;
+                pl.nt = nt;
+                pl.tiles = tiles;
+                pl.wr = wr;
+                pl.wc = wc;
+                pl.wp = wp;
+            }
         }
-    }
+    };
+    if (g.wo <= cap) consider(g.wo);
+    if (best_cost < 0)
+        for (int tw = 32; tw <= cap && tw < g.wo; tw += 32) consider(tw);
     if (best_cost < 0 || pl.tiles >= (int64_t(1) << 31)) return pl;
-    pl.wc = g.ws;
     pl.wm = wm;
     pl.ksteps_p = ksteps_p;
     pl.coutp = coutp;
@@ -502,6 +521,10 @@ int ws_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t 
     p.wpix = pl.wp;
     p.ksteps_p = pl.ksteps_p;
     p.wm = pl.wm;
+    p.tw = pl.tw;
+    p.ctiles = pl.ctiles;
+    p.sh = g.sh;
+    p.sw = g.sw;
     // an output of L2 size or more that no fused consumer reads: stream it
     p.stream_out = (!ep.residual && !ep.st_out && ep.out_f32 && int64_t(g.n) * g.cout * g.ho * g.wo * 4 >= (int64_t(16) << 20)) ? 1 : 0;
     const dim3 grid(unsigned(pl.tiles), unsigned(pl.coutp / (32 * WS_FM * pl.wm)));

@@ -130,7 +130,8 @@ __device__ __forceinline__ void epilogue_rows16(const EpiParams &p, const v16i &
 struct WsPlan {
     bool ok;            // geometry supported
     int th, nt;         // output rows per tile, 32-position fragments per wavefront
-    int wm;             // wavefronts along cout: 4, or 2 with the tile's positions split over the other factor
+    int tw, ctiles;     // output columns per tile, column tiles per row
+    int wm;             // wavefronts along cout: 4, 2 or 1, with the tile's positions split over the other factor of 4
     int ho, wo, hs, ws; // the map as the kernel walks it: the real one, or rows of one pixel for 1x1 layers without halo
     int64_t tiles;      // tiles over the batch-wide row sequence
     int wr, wc, wp;     // window rows, cols, pixels
@@ -140,7 +141,7 @@ struct WsPlan {
 };
 
 struct WsGeom {
-    int n, cout, ho, wo, hs, ws, cp, cblocks, kh, kw, dil_h, dil_w;
+    int n, cout, ho, wo, hs, ws, cp, cblocks, kh, kw, dil_h, dil_w, sh, sw;
 };
 
 WsPlan ws_plan(const WsGeom &g);

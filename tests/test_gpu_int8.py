@@ -71,6 +71,12 @@ CONV_CASES = [
     (1, 130, 9, 9, 200, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),     # ragged channels / cout > one tile
     (5, 96, 7, 7, 129, 1, 1, (0, 0, 0, 0), (1, 1), (1, 1)),
     (2, 256, 28, 28, 256, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),   # two images of BASELINE config 2
+    (1, 16, 5, 300, 40, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),     # rows wider than a tile: column tiles
+    (2, 16, 7, 301, 72, 3, 3, (1, 1, 1, 1), (2, 2), (1, 1)),     # ... with stride 2
+    (2, 16, 9, 50, 24, 3, 3, (1, 0, 2, 1), (1, 1), (1, 1)),      # at most 32 output channels: one wavefront along cout
+    (3, 70, 15, 13, 96, 3, 3, (1, 1, 1, 1), (2, 2), (1, 1)),     # stride 2, tiles straddling images
+    (3, 40, 14, 14, 130, 1, 1, (0, 0, 0, 0), (2, 2), (1, 1)),    # 1x1 stride 2 (a projection shortcut)
+    (2, 24, 11, 12, 33, 3, 3, (2, 2, 2, 2), (2, 1), (2, 2)),     # mixed strides with dilation
 ]
 
 
