@@ -824,7 +824,10 @@ int make_plan(const tsx_conv2d_geom *g, Plan *pl) {
                               pl->im2col ? 1 : g->dilation_h, pl->im2col ? 1 : g->dilation_w,
                               pl->im2col ? 1 : g->stride_h, pl->im2col ? 1 : g->stride_w};
         pl->wsp = tsx::ws_plan(pl->wsg);
-        if (pl->wsp.ok) {
+        // a strided 1x1 layer would fill its window with pixels it skips (3 of 4 at stride 2): the generic
+        // kernel, which gathers only the pixels it multiplies, is the faster one there
+        const bool strided_1x1 = !pl->im2col && pl->taps == 1 && (g->stride_h > 1 || g->stride_w > 1);
+        if (pl->wsp.ok && !strided_1x1) {
             pl->use_ws = true;
             pl->packed_bytes = pl->wsp.packed_bytes;
         }
