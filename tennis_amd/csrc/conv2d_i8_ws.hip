@@ -17,6 +17,9 @@
 //     one block ahead, 80-byte pixel stride = bank-conflict-free 16-byte reads); every tap is
 //     then a shifted read of the same LDS data, so activations cross L2 -> CU once, not
 //     KH*KW times, and the K loop needs one barrier per channel block, not per K-step;
+//     A 1x1 layer has one K-step per channel block, too short to cover the window's L2 latency one block
+//     ahead: its windows hold up to 4 channel blocks per pixel (pixel stride 64*blocks + 16) and the blocks
+//     of a window are walked like taps;
 //   * weights never touch LDS: each wavefront streams its own rows from the packed
 //     buffer (1 KiB contiguous per MFMA operand) into a 4-deep register ring, three
 //     K-steps ahead of use.
@@ -32,7 +35,7 @@ namespace tsx {
 namespace {
 
 constexpr int RING = 4;         // A register ring depth (K-steps)
-constexpr int PIX = 80;         // LDS bytes per window pixel (64 + 16 pad)
+constexpr int PIX = 80;         // LDS bytes per window pixel (64 + 16 pad) when a window holds one channel block
 constexpr int WS_THREADS = 256;
 constexpr int WS_FM = 1;        // 32-cout fragments per wavefront
 constexpr int WS_BM = 4 * 32 * WS_FM;   // output channels per workgroup
@@ -47,6 +50,10 @@ struct WsParams : EpiParams {
     int wm;           // wavefronts along cout (4, 2 or 1: the other factor of 4 splits the tile's positions)
     int tw, ctiles;   // tile width in output columns, column tiles per row (1: whole rows)
     int sh, sw;       // strides
+    // a window holds `cbs` channel blocks per pixel: pix = 64*cbs + 16 bytes, 4*cbs = 1 << chunk_shift chunks;
+    // a tap is tap_row/tap_col bytes further into the window per kernel row / column (for cbs > 1 the "taps"
+    // are the window's channel blocks: kh = 1, kw = cbs, tap_col = 64)
+    int pix, chunk_shift, stage_bytes, tap_row, tap_col;
     int stream_out;   // fp32 output written with streaming stores
 };
 
@@ -106,16 +113,16 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
     const int pos0 = (p.wm == 4 ? 0 : p.wm == 2 ? wave >> 1 : wave) * (NT * 32);   // first tile position of this wavefront
     const int m0 = (blockIdx.y * p.wm + wave_m) * (32 * FM);         // first cout of this wavefront
     const int taps = p.kh * p.kw;
-    const int win_bytes = p.wpix * PIX;
+    const int win_bytes = p.wpix * p.pix;
 
-    // ---- window fill bookkeeping: chunk q = tid + i*256 -> pixel q/4, 16-byte chunk q%4
+    // ---- window fill bookkeeping: chunk q = tid + i*256 -> pixel q / chunks-per-pixel, 16-byte chunk q % ...
     const int8_t *fill_src[MAX_FILL];
     int fill_dst[MAX_FILL];
     static_for<0, MAX_FILL>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
         const int q = tid + i * WS_THREADS;
-        int pix = q >> 2;
-        const int chunk = q & 3;
+        int pix = q >> p.chunk_shift;
+        const int chunk = q & ((1 << p.chunk_shift) - 1);
         if (pix >= p.wpix) pix = p.wpix - 1;   // duplicates rewrite the same bytes
         int wrow = pix / p.wc;
         const int wcol = pix - wrow * p.wc;
@@ -125,15 +132,15 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
         int col = col0 * p.sw + wcol;
         if (col >= p.ws) col = p.ws - 1;                                 // last column tile: columns no stored output uses
         fill_src[i] = p.xs + (row * p.ws + col) * p.cp + chunk * 16;
-        fill_dst[i] = pix * PIX + chunk * 16;
+        fill_dst[i] = pix * p.pix + chunk * 16;
     });
-    const int n_fill = (p.wpix * 4 + WS_THREADS - 1) / WS_THREADS;   // <= MAX_FILL, uniform
+    const int n_fill = ((p.wpix << p.chunk_shift) + WS_THREADS - 1) / WS_THREADS;   // <= MAX_FILL, uniform
     v4i wreg[MAX_FILL];   // native vectors: arrays of HIP's uint4 struct do not stay in registers
 
     auto window_load = [&](int cb) __attribute__((always_inline)) {
         static_for<0, MAX_FILL>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
-            if (i < n_fill) wreg[i] = *reinterpret_cast<const v4i *>(fill_src[i] + cb * 64);
+            if (i < n_fill) wreg[i] = *reinterpret_cast<const v4i *>(fill_src[i] + cb * p.stage_bytes);
         });
     };
     auto window_store = [&](int buf) __attribute__((always_inline)) {
@@ -151,7 +158,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
         if (pos >= p.th * p.tw) pos = 0;       // padding positions: computed, never stored
         const int r = pos / p.tw, tc = pos - r * p.tw;
         const int wrow = r * p.sh + (th0 + r >= p.ho ? wrap : 0);   // positions of the next image sit below its halo rows
-        b_base[j] = (wrow * p.wc + tc * p.sw) * PIX + (lane / 32) * 16;
+        b_base[j] = (wrow * p.wc + tc * p.sw) * p.pix + (lane / 32) * 16;
     });
 
     // ---- A ring: the wavefront's FM fragments (32 cout each) x 2 halves of K-step ks, 1 KiB each
@@ -225,7 +232,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
                 const int next = cb + 1 < p.cblocks ? cb + 1 : p.cblocks - 1;
                 window_load(next);
             }
-            toff = buf * win_bytes + (kr * p.dil_h * p.wc + kc * p.dil_w) * PIX;
+            toff = buf * win_bytes + kr * p.tap_row + kc * p.tap_col;
             b_read(b0, toff);                            // first half of the next K-step
             static_for<0, FM>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
@@ -481,6 +488,14 @@ WsPlan ws_plan(const WsGeom &g_in) {
         for (int tw = 32; tw <= cap && tw < g.wo; tw += 32) consider(tw);
     if (best_cost < 0 || pl.tiles >= (int64_t(1) << 31)) return pl;
     pl.wm = wm;
+    // 1x1 layers: as many channel blocks per window as divide the layer's, fit the fill registers and LDS
+    pl.cbs = 1;
+    if (g.kh == 1 && g.kw == 1)
+        for (int c = 4; c > 1; c >>= 1)
+            if (g.cblocks % c == 0 && pl.wp * 4 * c <= MAX_FILL * WS_THREADS && size_t(2) * pl.wp * (64 * c + 16) <= 65536) {
+                pl.cbs = c;
+                break;
+            }
     pl.ksteps_p = ksteps_p;
     pl.coutp = coutp;
     pl.packed_bytes = size_t(pl.ksteps_p) * pl.coutp * 64;
@@ -525,10 +540,22 @@ int ws_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t 
     p.ctiles = pl.ctiles;
     p.sh = g.sh;
     p.sw = g.sw;
+    p.pix = 64 * pl.cbs + 16;
+    p.chunk_shift = pl.cbs == 4 ? 4 : pl.cbs == 2 ? 3 : 2;
+    p.stage_bytes = 64 * pl.cbs;
+    p.tap_row = g.dil_h * pl.wc * p.pix;
+    p.tap_col = g.dil_w * p.pix;
+    if (pl.cbs > 1) {          // the blocks of a window take the place of taps
+        p.cblocks = g.cblocks / pl.cbs;
+        p.kh = 1;
+        p.kw = pl.cbs;
+        p.tap_row = 0;
+        p.tap_col = 64;
+    }
     // an output of L2 size or more that no fused consumer reads: stream it
     p.stream_out = (!ep.residual && !ep.st_out && ep.out_f32 && int64_t(g.n) * g.cout * g.ho * g.wo * 4 >= (int64_t(16) << 20)) ? 1 : 0;
     const dim3 grid(unsigned(pl.tiles), unsigned(pl.coutp / (32 * WS_FM * pl.wm)));
-    const size_t lds_bytes = size_t(2) * pl.wp * PIX;
+    const size_t lds_bytes = size_t(2) * pl.wp * (64 * pl.cbs + 16);
     switch (pl.nt) {
         case 1: return launch_nt<1>(p, grid, lds_bytes, stream);
         case 2: return launch_nt<2>(p, grid, lds_bytes, stream);

@@ -131,6 +131,7 @@ struct WsPlan {
     bool ok;            // geometry supported
     int th, nt;         // output rows per tile, 32-position fragments per wavefront
     int tw, ctiles;     // output columns per tile, column tiles per row
+    int cbs;            // channel blocks per window (1x1 layers: up to 4)
     int wm;             // wavefronts along cout: 4, 2 or 1, with the tile's positions split over the other factor of 4
     int ho, wo, hs, ws; // the map as the kernel walks it: the real one, or rows of one pixel for 1x1 layers without halo
     int64_t tiles;      // tiles over the batch-wide row sequence
