@@ -33,7 +33,7 @@ CFG = dict(n=32, c=256, h=28, w=28, cout=256, k=3, pad=1)
 
 # HBM bytes per launch of the two kernels on this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a
 # known-size copy (profiles/conv2d_i8_config2_hbm_traffic.txt); a profiler figure, not measured by this script.
-TRAFFIC_CONV_BYTES = 45.13e6
+TRAFFIC_CONV_BYTES = 45.19e6
 TRAFFIC_STAGE_BYTES = 33.62e6
 
 
@@ -90,7 +90,7 @@ def cpu_baseline(x, x_scales, wq, dq, bias, pad, images):
 
 def resnet_leg(steps=20):
     """ResNet-50-shaped int8 network, batch 32 at 3x224x224 (BASELINE config 4): img/s of the whole forward pass,
-    replayed from a captured HIP graph (the pass is ~130 short kernels; capture removes the host launch cost)."""
+    replayed from a captured HIP graph (the pass is 58 short kernels; capture removes the host launch cost)."""
     import torch
     from tennis_amd import resnet50
     n, size = 32, 224
@@ -168,6 +168,8 @@ def main():
                     help="for runs under a profiler: skip the int8-output variant (same kernel name as the roofline "
                          "kernel), the MFMA-rate probe and the CPU baseline, so per-kernel statistics cover the timed "
                          "kernels only")
+    ap.add_argument("--network", choices=("resnet", "yolo"),
+                    help="run only that network leg and print its figures (for per-kernel profiles of a network)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
@@ -182,6 +184,9 @@ def main():
         sys.exit(3)
     L = capi.lib()
     dev = torch.device("cuda:0")
+    if args.network:
+        print(json.dumps(resnet_leg() if args.network == "resnet" else yolo_leg()))
+        return
     cfg = CFG
     x, x_scales, wq, dq, bias = make_inputs(cfg)
     pad = cfg["pad"]
