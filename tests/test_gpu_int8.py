@@ -149,7 +149,45 @@ def test_conv2d_i8_epilogue_signed_zero_and_tail(tsx, port):
     assert np.signbit(exp.ravel()[-1])        # 27 elements: the last three are the scalar tail
 
 
-@pytest.mark.parametrize("strides", [(1, 1), (2, 2)])     # window-stationary kernel / generic implicit GEMM
+@pytest.mark.parametrize("case", [
+    # n, cin, h, w, cout, k, pad, consumer kernel (its halo decides whether the producer's rows are flat pixel lists)
+    (3, 768, 7, 9, 130, 1, 0, 3),      # 12 channel blocks -> windows of 4; consumer with halo
+    (2, 384, 5, 6, 64, 1, 0, 1),       # 6 blocks -> windows of 2; 64 output channels; flat consumer
+    (2, 192, 6, 5, 24, 1, 0, 3),       # 3 blocks -> single-block windows; one wavefront along cout
+    (1, 40, 4, 300, 72, 3, 1, 3),      # column tiles
+    (2, 24, 9, 37, 20, 3, 1, 1),       # <= 32 output channels, 3x3
+])
+@pytest.mark.parametrize("after", [False, True])      # residual in front of / behind the activation
+def test_conv2d_i8_all_epilogue_terms_on_every_tiling(tsx, port, case, after):
+    """Residual join + fp32 output + requantized staged output together, on the tilings the plan picks for
+    1x1 layers (flat pixel lists, multi-block windows), few output channels and column tiles; the staged
+    output is checked through a consumer convolution."""
+    n, cin, h, w, cout, k, pad, ck = case
+    rng = np.random.default_rng(207)
+    xq = rng.integers(-128, 128, (n, cin, h, w)).astype(np.int8)
+    wa = rng.integers(-127, 128, (cout, cin, k, k)).astype(np.int8)
+    dqa = rng.uniform(1e-5, 3e-5, cout).astype(np.float32)
+    ba = rng.standard_normal(cout).astype(np.float32)
+    qs = np.full(n, 7.0, np.float32)
+    A = tsx.Conv2dI8(_dev(wa), (pad,) * 4)
+    plain = port.conv2d_i8_fused(xq, wa, dqa, ba, None, pads=(pad,) * 4)[0]
+    res = (rng.standard_normal(plain.shape) * np.abs(plain).mean()).astype(np.float32)
+    exp = port.add(port.leaky_relu(plain, 0.1), res) if after else port.leaky_relu(port.add(plain, res), 0.1)
+    exp_q = port.quantize(exp, qs)
+    wb = rng.integers(-127, 128, (40, cout, ck, ck)).astype(np.int8)
+    dqb = rng.uniform(1e-4, 3e-4, 40).astype(np.float32)
+    B = tsx.Conv2dI8(_dev(wb), (ck // 2,) * 4)
+    sb = tsx.StagedInput(B, tuple(plain.shape))
+    sa = tsx.StagedInput(A, tuple(xq.shape))
+    A.stage(_dev(xq), sa)
+    f = A.run_staged(sa, _dev(dqa), _dev(ba), "leaky_relu", 0.1, q_scales=_dev(qs), residual=_dev(res), staged_out=sb,
+                     residual_after_act=after)[0]
+    assert np.array_equal(bits(f.cpu().numpy()), bits(exp))
+    got = B.run_staged(sb, _dev(dqb))[0].cpu().numpy()
+    assert np.array_equal(bits(got), bits(port.conv2d_quantized(exp_q, wb, dqb, (ck // 2,) * 4)))
+
+
+@pytest.mark.parametrize("strides", [(1, 1), (2, 2)])
 def test_conv2d_i8_residual_join_in_epilogue(tsx, port, strides):
     """conv -> add_bias -> add(residual) -> relu (-> quantize) fused, against the separate operators."""
     rng = np.random.default_rng(204)
