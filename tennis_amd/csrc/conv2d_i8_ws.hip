@@ -5,21 +5,23 @@
 // Same arithmetic as the generic implicit GEMM in conv2d_i8.hip (exact int32 sums of
 // cpu::Conv2DQuantizedCore, src/kernels/cpu/quantized/conv2d_quantized_core.cpp:18-147), but
 // a different data movement:
-//   * one workgroup (4 wavefronts) owns TH full output rows x 128 output channels; wavefront w
-//     owns channels [32w, 32w+32) and all positions of the tile (layers with at most 64 output
-//     channels: 64 channels, two wavefronts each on either half of the tile's positions).  Rows are counted across the
-//     whole batch (image n's rows follow image n-1's), so a tile may straddle two images: their
-//     staged rows are contiguous in memory, and a position in the second image just reads the
-//     window (KH-1)*dilation rows further down.  Tiles therefore need not divide the image
-//     height (28 rows = 3.5 tiles of 8 rows = 7 position fragments with no padding);
+//   * one workgroup (4 wavefronts) owns a tile of TH output rows x TW output columns x 128 output
+//     channels; wavefront w owns channels [32w, 32w+32) and all positions of the tile (layers with
+//     at most 64 / 32 output channels: 64 / 32 channels, the other wavefronts taking further
+//     positions of a 2x / 4x larger tile).  Rows are counted across the whole batch (image n's rows
+//     follow image n-1's), so a tile may straddle two images: their staged rows are contiguous in
+//     memory, and a position in the second image just reads the window hs - ho*stride rows further
+//     down.  Tiles therefore need not divide the image height.  TW is the whole row where the row
+//     and its window fit, else a multiple of 32 columns.  A 1x1 layer reading a buffer without halo
+//     is tiled as rows of one pixel (the plan's view of the map): any run of consecutive pixels;
 //   * per 64-channel block the input *window* that all KH*KW taps of the tile read
-//     ((TH + (KH-1)*dil) rows x staged width) is copied once into LDS (double buffered,
-//     one block ahead, 80-byte pixel stride = bank-conflict-free 16-byte reads); every tap is
-//     then a shifted read of the same LDS data, so activations cross L2 -> CU once, not
-//     KH*KW times, and the K loop needs one barrier per channel block, not per K-step;
-//     A 1x1 layer has one K-step per channel block, too short to cover the window's L2 latency one block
-//     ahead: its windows hold up to 4 channel blocks per pixel (pixel stride 64*blocks + 16) and the blocks
-//     of a window are walked like taps;
+//     (((TH-1)*stride + (KH-1)*dil + 1) rows x ((TW-1)*stride + (KW-1)*dil + 1) columns) is copied
+//     once into LDS (double buffered, one block ahead, 80-byte pixel stride = bank-conflict-free
+//     16-byte reads); every tap is then a shifted read of the same LDS data, so activations cross
+//     L2 -> CU once, not KH*KW times, and the K loop needs one barrier per channel block, not per
+//     K-step.  A 1x1 layer has one K-step per channel block, too short to cover the window's L2
+//     latency one block ahead: its windows hold up to 4 channel blocks per pixel (pixel stride
+//     64*blocks + 16) and the blocks of a window are walked like taps;
 //   * weights never touch LDS: each wavefront streams its own rows from the packed
 //     buffer (1 KiB contiguous per MFMA operand) into a 4-deep register ring, three
 //     K-steps ahead of use.
@@ -38,7 +40,6 @@ constexpr int RING = 4;         // A register ring depth (K-steps)
 constexpr int PIX = 80;         // LDS bytes per window pixel (64 + 16 pad) when a window holds one channel block
 constexpr int WS_THREADS = 256;
 constexpr int WS_FM = 1;        // 32-cout fragments per wavefront
-constexpr int WS_BM = 4 * 32 * WS_FM;   // output channels per workgroup
 constexpr int MAX_FILL = 7;     // window chunks per thread per channel block
 constexpr int MAX_WP = MAX_FILL * WS_THREADS / 4;   // 448 window pixels
 
@@ -404,8 +405,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
 
 template <int NT>
 int launch_nt(const WsParams &p, dim3 grid, size_t lds_bytes, hipStream_t stream) {
-    // 32 cout per wavefront (128 per workgroup): two workgroups share a CU, so one
-    // wavefront's LDS/L2 waits are covered by the other on the same SIMD.
+    // EXTRA: residual input and/or staged int8 output; STREAM: a large fp32 output nothing reads back soon
     if (p.residual || p.st_out)
         hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, true, false>), grid, dim3(WS_THREADS), lds_bytes, stream, p);
     else if (p.stream_out)

@@ -125,7 +125,7 @@ __device__ __forceinline__ void epilogue_rows16(const EpiParams &p, const v16i &
     }
 }
 
-// ---- window-stationary stride-1 convolution kernel (conv2d_i8_ws.hip) ----
+// ---- window-stationary convolution kernel (conv2d_i8_ws.hip) ----
 
 struct WsPlan {
     bool ok;            // geometry supported
