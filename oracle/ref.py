@@ -120,6 +120,25 @@ def run_op(op, params, inputs, out_bytes, threads=1):
     return buf[:out.bytes].view(_TS2NP[out.dtype]).reshape(shape).copy()
 
 
+def save_tensor(path, value):
+    """Write ``value`` (numpy array or str) as a TenniS `.t` file with the reference's own serializer."""
+    keep = []
+    t = _pack("", value, keep)
+    _check(lib().ref_save_tensor(str(path).encode(), ctypes.byref(t)))
+
+
+def load_tensor(path, max_bytes=1 << 24):
+    """Read a `.t` file with the reference's own reader; returns (dtype code, numpy array of raw dtype)."""
+    buf = np.empty(max_bytes, dtype=np.uint8)
+    out = _Output()
+    out.data = buf.ctypes.data
+    out.capacity = max_bytes
+    _check(lib().ref_load_tensor(str(path).encode(), ctypes.byref(out)))
+    shape = tuple(out.shape[k] for k in range(out.ndim))
+    np_type = _TS2NP.get(out.dtype, np.uint8)
+    return out.dtype, buf[:out.bytes].view(np_type).reshape(shape).copy()
+
+
 def _conv_params(pads, strides, dilations, padding_value=0.0):
     return {
         "format": "NCHW",

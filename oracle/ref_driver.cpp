@@ -161,6 +161,26 @@ int ref_run_op_on(const char *device, int strict, const char *op, int nparams, c
     });
 }
 
+// The reference's own tensor file format (`.t`: Tensor::serialize / externalize, src/core/tensor.cpp:314-389,
+// through tensor::save / tensor::load, include/core/tensor_builder.h:153-159): written and read by the compiled
+// library itself, to make fixtures for and cross-check an independent reader / writer of the format.
+int ref_save_tensor(const char *path, const ref_tensor *t) {
+    return guarded([&] { ts::tensor::save(path, make_tensor(*t)); });
+}
+
+int ref_load_tensor(const char *path, ref_output *out) {
+    return guarded([&] {
+        ts::Tensor y = ts::tensor::load(path);
+        if (y.fields_count() != 1) throw std::runtime_error("packed tensors are not supported by this driver");
+        out->dtype = int32_t(y.dtype());
+        out->ndim = int32_t(y.dims());
+        for (int i = 0; i < out->ndim && i < 8; ++i) out->shape[i] = y.size(i);
+        out->bytes = int64_t(y.count()) * ts::type_bytes(y.dtype());
+        if (out->bytes > out->capacity) throw std::runtime_error("output buffer too small");
+        std::memcpy(out->data, y.data(), size_t(out->bytes));
+    });
+}
+
 // Conv2dWinogradAlgorithm<float>::winograd_f63 / winograd_f23 on raw weights
 // (kernel_transformed=false).  pad = {top, bottom, left, right}.
 int ref_winograd(int f63, const float *x, int n, int c, int h, int w, const float *k, int cout,

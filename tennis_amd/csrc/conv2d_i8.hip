@@ -822,7 +822,7 @@ int make_plan(const tsx_conv2d_geom *g, Plan *pl) {
         pl->wsg = tsx::WsGeom{g->n, g->cout, pl->ho, pl->wo, pl->hs, pl->ws, pl->cp, pl->cblocks,
                               pl->im2col ? 1 : g->kh, pl->im2col ? 1 : g->kw,
                               pl->im2col ? 1 : g->dilation_h, pl->im2col ? 1 : g->dilation_w,
-                              pl->im2col ? 1 : g->stride_h, pl->im2col ? 1 : g->stride_w};
+                              pl->im2col ? 1 : g->stride_h, pl->im2col ? 1 : g->stride_w, 0};
         pl->wsp = tsx::ws_plan(pl->wsg);
         // a strided 1x1 layer would fill its window with pixels it skips (3 of 4 at stride 2): the generic
         // kernel, which gathers only the pixels it multiplies, is the faster one there
@@ -1140,16 +1140,20 @@ int tsx_conv2d_i8_staged_at(const tsx_conv2d_geom *g, const void *staged_dev, in
 
 // ---- GEMM: a [m][k] is a batch of m "images" with k channels and 1x1 extent.
 
+// K-steps of the packed GEMM weights: padded with zero steps to the window-stationary kernel's ring of 4
+// (the tiled and the skinny kernel walk only the first round_up(k, 64) / 64 of them).
+static int gemm_packed_ksteps(int32_t k) { return int(tsx::round_up(tsx::round_up(k, KSTEP) / KSTEP, 4)); }
+
 size_t tsx_gemm_i8_packed_weight_bytes(int32_t k, int32_t n) {
     if (k <= 0 || n <= 0) return 0;
-    return size_t(tsx::round_up(k, KSTEP)) * size_t(tsx::round_up(n, BM));
+    return size_t(gemm_packed_ksteps(k)) * KSTEP * size_t(tsx::round_up(n, BM));
 }
 
 int tsx_gemm_i8_pack_weights(int32_t k, int32_t n, int32_t transposed, const int8_t *w_dev, void *packed_dev,
                              void *stream) {
     TSX_REQUIRE(k > 0 && n > 0 && w_dev && packed_dev, "gemm_i8_pack_weights: bad argument");
     TSX_REQUIRE(reinterpret_cast<uintptr_t>(packed_dev) % 16 == 0, "gemm_i8_pack_weights: packed buffer must be 16-byte aligned");
-    const int cblocks = int(tsx::round_up(k, KSTEP) / KSTEP), coutp = int(tsx::round_up(n, BM));
+    const int cblocks = gemm_packed_ksteps(k), coutp = int(tsx::round_up(n, BM));
     const int64_t threads = int64_t(cblocks) * coutp * KSTEP / 16;
     // element (k, n): [k][n] row-major -> k*n_ + n ; transposed [n][k] -> n*k_ + k
     const int64_t ld_cout = transposed ? k : 1, ld_c = transposed ? 1 : n;
@@ -1207,6 +1211,14 @@ int tsx_gemm_i8(int32_t m, int32_t n, int32_t k, const int8_t *a_dev, const void
         hipLaunchKernelGGL(gemm_i8_skinny_kernel, dim3(unsigned(tsx::ceil_div(n, 32))), dim3(SK_WAVES * 64), 0, stream, p);
         TSX_LAUNCH_CHECK("gemm_i8_skinny_kernel");
         return 0;
+    }
+    // Enough rows to fill MFMA fragments: the window-stationary kernel in its GEMM form (a 1x1 layer over m
+    // one-pixel rows, row-major output).  Residual terms stay on the tiled kernel.
+    if (!p.residual && !p.st_out) {
+        const tsx::WsGeom wg{1, n, m, 1, m, 1, kp, kp / KSTEP, 1, 1, 1, 1, 1, 1, 1};
+        const tsx::WsPlan wpl = tsx::ws_plan(wg);
+        if (wpl.ok && wpl.ksteps_p == gemm_packed_ksteps(k) && wpl.coutp == p.coutp)
+            return tsx::ws_launch(wg, wpl, p.xs, p.wp, static_cast<const tsx::EpiParams &>(p), stream);
     }
     return launch_igemm<true>(p, stream);
 }

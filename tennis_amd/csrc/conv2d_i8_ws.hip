@@ -31,32 +31,10 @@
 // MFMA operand layout (v_mfma_i32_32x32x32_i8): lane l supplies row/column l%32 and the 16
 // K bytes of group l/32 (two MFMAs, "halves", cover a 64-byte K-step); accumulator register r
 // of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32.  Rows = cout, columns = positions.
-#include "igemm_i8.hpp"
+#include "conv2d_i8_ws_kernel.hpp"
 
 namespace tsx {
 namespace {
-
-constexpr int RING = 4;         // A register ring depth (K-steps)
-constexpr int PIX = 80;         // LDS bytes per window pixel (64 + 16 pad) when a window holds one channel block
-constexpr int WS_THREADS = 256;
-constexpr int WS_FM = 1;        // 32-cout fragments per wavefront
-constexpr int MAX_FILL = 7;     // window chunks per thread per channel block
-constexpr int MAX_WP = MAX_FILL * WS_THREADS / 4;   // 448 window pixels
-
-struct WsParams : EpiParams {
-    const int8_t *xs;   // staged activations [n][hs][ws][cp]
-    const int8_t *wp;   // packed weights [ks_p][coutp/32][2 halves][64 lanes][16]
-    int n, cout, coutp, ho, wo, hs, ws, cp, cblocks, kh, kw, dil_h, dil_w;
-    int th, wr, wc, wpix, ksteps_p;
-    int wm;           // wavefronts along cout (4, 2 or 1: the other factor of 4 splits the tile's positions)
-    int tw, ctiles;   // tile width in output columns, column tiles per row (1: whole rows)
-    int sh, sw;       // strides
-    // a window holds `cbs` channel blocks per pixel: pix = 64*cbs + 16 bytes, 4*cbs = 1 << chunk_shift chunks;
-    // a tap is tap_row/tap_col bytes further into the window per kernel row / column (for cbs > 1 the "taps"
-    // are the window's channel blocks: kh = 1, kw = cbs, tap_col = 64)
-    int pix, chunk_shift, stage_bytes, tap_row, tap_col;
-    int stream_out;   // fp32 output written with streaming stores
-};
 
 // packed[ks][frag][half][lane][16]: ks = cb*taps + tap; frag = cout/32; lane l: cout frag*32 + l%32,
 // channels cb*64 + half*32 + (l/32)*16 + 0..15.  K-steps >= cblocks*taps, rows >= cout, channels >= c: zero.
@@ -86,335 +64,6 @@ __global__ __launch_bounds__(256) void ws_pack_kernel(const int8_t *__restrict__
     *reinterpret_cast<uint4 *>(packed + id * 16) = make_uint4(words[0], words[1], words[2], words[3]);
 }
 
-// EXTRA = false compiles the residual input and the staged-layout output out of the epilogue (fewer
-// registers for the plain dequant + bias + activation case); STREAM selects streaming fp32 stores.
-//
-// Up to 4 position fragments the kernel is compiled for two wavefronts per SIMD (at most 256 registers): the
-// layers that take these tiles are bound by their epilogue's memory traffic (residual in, fp32 and staged int8
-// out), and a second resident workgroup per CU is worth more there than registers.
-// NT counts the position fragments of ONE wavefront; a tile holds (4 / wm) x NT of them.
-template <int NT, int FM, bool EXTRA, bool STREAM>
-__global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <= 4 ? 2 : 1))) void conv_i8_ws_kernel(WsParams p_in) {
-    WsParams p = p_in;
-    if (!EXTRA) {
-        p.residual = nullptr;
-        p.st_out = nullptr;
-    }
-    extern __shared__ __attribute__((aligned(16))) int8_t lds[];   // 2 x wpix x PIX
-    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
-    const int rtile = blockIdx.x / p.ctiles;
-    const int col0 = (blockIdx.x - rtile * p.ctiles) * p.tw;   // first output column of the tile
-    const int row0 = rtile * p.th;           // first output row of the tile, counted over the whole batch
-    const int img = row0 / p.ho;             // image of the tile's first row
-    const int th0 = row0 - img * p.ho;       // ... and that row inside it
-    const int rows_total = p.n * p.ho;
-    // staged rows from where output row `ho` of an image would start to the next image's first row
-    const int wrap = p.hs - p.ho * p.sh;
-    const int wave_m = wave & (p.wm - 1);                            // position along cout
-    const int pos0 = (p.wm == 4 ? 0 : p.wm == 2 ? wave >> 1 : wave) * (NT * 32);   // first tile position of this wavefront
-    const int m0 = (blockIdx.y * p.wm + wave_m) * (32 * FM);         // first cout of this wavefront
-    const int taps = p.kh * p.kw;
-    const int win_bytes = p.wpix * p.pix;
-
-    // ---- window fill bookkeeping: chunk q = tid + i*256 -> pixel q / chunks-per-pixel, 16-byte chunk q % ...
-    const int8_t *fill_src[MAX_FILL];
-    int fill_dst[MAX_FILL];
-    static_for<0, MAX_FILL>([&](auto ic) {
-        constexpr int i = decltype(ic)::value;
-        const int q = tid + i * WS_THREADS;
-        int pix = q >> p.chunk_shift;
-        const int chunk = q & ((1 << p.chunk_shift) - 1);
-        if (pix >= p.wpix) pix = p.wpix - 1;   // duplicates rewrite the same bytes
-        int wrow = pix / p.wc;
-        const int wcol = pix - wrow * p.wc;
-        // window row r is staged row (img * hs + th0 * stride) + r of the batch-wide staged row sequence
-        int64_t row = int64_t(img) * p.hs + th0 * p.sh + wrow;
-        if (row >= int64_t(p.n) * p.hs) row = int64_t(p.n) * p.hs - 1;   // last tile: rows no stored output uses
-        int col = col0 * p.sw + wcol;
-        if (col >= p.ws) col = p.ws - 1;                                 // last column tile: columns no stored output uses
-        fill_src[i] = p.xs + (row * p.ws + col) * p.cp + chunk * 16;
-        fill_dst[i] = pix * p.pix + chunk * 16;
-    });
-    const int n_fill = ((p.wpix << p.chunk_shift) + WS_THREADS - 1) / WS_THREADS;   // <= MAX_FILL, uniform
-    v4i wreg[MAX_FILL];   // native vectors: arrays of HIP's uint4 struct do not stay in registers
-
-    auto window_load = [&](int cb) __attribute__((always_inline)) {
-        static_for<0, MAX_FILL>([&](auto ic) {
-            constexpr int i = decltype(ic)::value;
-            if (i < n_fill) wreg[i] = *reinterpret_cast<const v4i *>(fill_src[i] + cb * p.stage_bytes);
-        });
-    };
-    auto window_store = [&](int buf) __attribute__((always_inline)) {
-        static_for<0, MAX_FILL>([&](auto ic) {
-            constexpr int i = decltype(ic)::value;
-            if (i < n_fill) *reinterpret_cast<v4i *>(&lds[buf * win_bytes + fill_dst[i]]) = wreg[i];
-        });
-    };
-
-    // ---- B operand addresses: fragment j, lane l -> tile position j*32 + l%32, K group l/32
-    int b_base[NT];
-    static_for<0, NT>([&](auto jc) {
-        constexpr int j = decltype(jc)::value;
-        int pos = pos0 + j * 32 + lane % 32;
-        if (pos >= p.th * p.tw) pos = 0;       // padding positions: computed, never stored
-        const int r = pos / p.tw, tc = pos - r * p.tw;
-        const int wrow = r * p.sh + (th0 + r >= p.ho ? wrap : 0);   // positions of the next image sit below its halo rows
-        b_base[j] = (wrow * p.wc + tc * p.sw) * p.pix + (lane / 32) * 16;
-    });
-
-    // ---- A ring: the wavefront's FM fragments (32 cout each) x 2 halves of K-step ks, 1 KiB each
-    const int8_t *a_ptr = p.wp + (int64_t(m0 / 32) * 128 + lane) * 16;
-    const int64_t a_kstride = int64_t(p.coutp / 32) * 128 * 16;
-    v4i areg[RING][2 * FM];
-    auto a_load = [&](auto slot, int ks) __attribute__((always_inline)) {
-        constexpr int s = decltype(slot)::value;
-        if (ks >= p.ksteps_p) ks = p.ksteps_p - 1;
-        const int8_t *src = a_ptr + ks * a_kstride;
-        static_for<0, 2 * FM>([&](auto fc) {
-            constexpr int f = decltype(fc)::value;
-            areg[s][f] = *reinterpret_cast<const v4i *>(src + f * 1024);
-        });
-    };
-
-    v16i acc[FM][NT];
-    static_for<0, FM>([&](auto ic) {
-        static_for<0, NT>([&](auto jc) {
-            static_for<0, 16>([&](auto rc) { acc[decltype(ic)::value][decltype(jc)::value][decltype(rc)::value] = 0; });
-        });
-    });
-
-    // ---- prologue
-    window_load(0);
-    static_for<0, RING - 1>([&](auto sc) { a_load(sc, decltype(sc)::value); });
-    window_store(0);
-    __syncthreads();
-    int cb = 0, tap = 0, kr = 0, kc = 0, buf = 0;
-    window_load(p.cblocks > 1 ? 1 : 0);   // block cb+1, in flight during block cb's taps
-
-    // B fragments are read one half-step ahead of the MFMAs that use them (one wavefront per
-    // SIMD: nothing else hides the LDS latency).
-    v4i b0[NT], b1[NT];
-    auto b_read = [&](v4i(&dst)[NT], int off) __attribute__((always_inline)) {
-        static_for<0, NT>([&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-            dst[j] = *reinterpret_cast<const v4i *>(&lds[b_base[j] + off]);
-        });
-    };
-    int toff = 0;   // buf * win_bytes + tap shift
-    b_read(b0, toff);
-
-    for (int ks0 = 0; ks0 < p.ksteps_p; ks0 += RING) {
-        static_for<0, RING>([&](auto uc) {
-            constexpr int u = decltype(uc)::value;
-            // prefetch weights of K-step ks0+u+RING-1 into the slot freed by the previous step
-            a_load(std::integral_constant<int, (u + RING - 1) % RING>{}, ks0 + u + RING - 1);
-            b_read(b1, toff + 32);                       // second half of this K-step
-            static_for<0, FM>([&](auto ic) {
-                constexpr int i = decltype(ic)::value;
-                static_for<0, NT>([&](auto jc) {
-                    constexpr int j = decltype(jc)::value;
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[u][i * 2], b0[j], acc[i][j], 0, 0, 0);
-                });
-            });
-            // advance (cb, tap); on a channel-block boundary swap in the next window
-            ++tap;
-            if (++kc == p.kw) {
-                kc = 0;
-                ++kr;
-            }
-            if (tap == taps) {
-                tap = 0;
-                kr = 0;
-                kc = 0;
-                ++cb;
-                window_store(buf ^ 1);
-                __syncthreads();
-                buf ^= 1;
-                const int next = cb + 1 < p.cblocks ? cb + 1 : p.cblocks - 1;
-                window_load(next);
-            }
-            toff = buf * win_bytes + kr * p.tap_row + kc * p.tap_col;
-            b_read(b0, toff);                            // first half of the next K-step
-            static_for<0, FM>([&](auto ic) {
-                constexpr int i = decltype(ic)::value;
-                static_for<0, NT>([&](auto jc) {
-                    constexpr int j = decltype(jc)::value;
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[u][i * 2 + 1], b1[j], acc[i][j], 0, 0, 0);
-                });
-            });
-        });
-    }
-
-    // ---- epilogue: accumulator register r of lane l = cout 8*(r/4) + 4*(l/32) + r%4, position l%32
-    const int tile_pos = p.th * p.tw;
-    const int howo = p.ho * p.wo;
-    const int64_t count = int64_t(p.n) * p.cout * howo;
-    // hot case: no raw accumulators wanted, every element inside the activation's SIMD-body range,
-    // a tensor small enough for 32-bit lane offsets, and -- for the requantized output -- one
-    // quantize group per image (or a single scale whose round-half-even bulk covers everything),
-    // so the consumer's scale is uniform for this tile and needs no per-element division
-    const bool want_q = p.out_i8 || p.st_out;
-    const bool q_uniform = !want_q || (p.n_qscales == 1 ? p.q_bulk8 == count : p.q_group_len == int64_t(p.cout) * howo);
-    const bool fast = (p.out_f32 || want_q) && !p.out_acc && p.act_body == count && count < (int64_t(1) << 30) && q_uniform;
-    // a tile may end in the next image: one consumer scale per image, selected per lane
-    const float q_scale_a = (fast && want_q) ? p.q_scales[p.n_qscales == 1 ? 0 : img] : 0.f;
-    const float q_scale_b = (fast && want_q) ? p.q_scales[p.n_qscales == 1 ? 0 : min(img + 1, p.n - 1)] : 0.f;
-    const bool q_even = p.n_qscales == 1;   // single-scale quantize rounds half to even in its bulk
-    static_for<0, FM>([&](auto fc) {
-        constexpr int f = decltype(fc)::value;
-        const int cf = m0 + f * 32;   // first cout of this fragment (uniform)
-        float dq[16], bias[16];
-        static_for<0, 16>([&](auto rc) {
-            constexpr int r = decltype(rc)::value;
-            const int co = cf + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
-            const bool in = co < p.cout;
-            dq[r] = (in && p.dq) ? p.dq[co] : 0.f;
-            bias[r] = (in && p.bias) ? p.bias[co] : 0.f;
-        });
-        // the other branch of a residual join: the loads of every fragment are in flight before the first use
-        float res[NT][16];
-        if (fast && cf + 32 <= p.cout && p.residual) {
-            const int64_t tile_base = (int64_t(img) * p.cout + cf) * howo;
-            static_for<0, NT>([&](auto jc) {
-                constexpr int j = decltype(jc)::value;
-                const int pos = pos0 + j * 32 + lane % 32;
-                const int tr = pos / p.tw, ow = col0 + pos - tr * p.tw;
-                const bool wrapped = th0 + tr >= p.ho;
-                const int oh = th0 + tr - (wrapped ? p.ho : 0);
-                const bool pos_ok = pos < tile_pos && row0 + tr < rows_total && ow < p.wo;
-                const unsigned lane_off = unsigned((wrapped ? p.cout * howo : 0) + (4 * (lane / 32)) * howo + oh * p.wo + ow);
-                static_for<0, 16>([&](auto rc) {
-                    constexpr int r = decltype(rc)::value;
-                    constexpr int dco = 8 * (r / 4) + (r % 4);
-                    res[j][r] = pos_ok ? (p.residual + tile_base + int64_t(dco) * howo)[lane_off] : 0.f;
-                });
-            });
-        }
-        static_for<0, NT>([&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-            const int pos = pos0 + j * 32 + lane % 32;
-            const int tr = pos / p.tw, ow = col0 + pos - tr * p.tw;
-            const bool wrapped = th0 + tr >= p.ho;                 // this position belongs to the next image
-            const int oh = th0 + tr - (wrapped ? p.ho : 0);
-            const bool pos_ok = pos < tile_pos && row0 + tr < rows_total && ow < p.wo;
-            const float q_scale = wrapped ? q_scale_b : q_scale_a;
-            if (fast && cf + 32 <= p.cout) {
-                // uniform base in scalar registers + one 32-bit lane offset: no per-store address math
-                const int64_t tile_base = (int64_t(img) * p.cout + cf) * howo;
-                const unsigned lane_off = unsigned((wrapped ? p.cout * howo : 0) + (4 * (lane / 32)) * howo + oh * p.wo + ow);
-                if (pos_ok) {
-                    // One pass per epilogue term over the fragment's 16 accumulators, each behind a single
-                    // uniform branch: testing the (uniform) options per element costs more instructions than
-                    // the arithmetic itself.
-                    float v[16];
-                    static_for<0, 16>([&](auto rc) {
-                        constexpr int r = decltype(rc)::value;
-                        v[r] = __fmul_rn(float(acc[f][j][r]), dq[r]);
-                    });
-                    if (p.bias) static_for<0, 16>([&](auto rc) {
-                        constexpr int r = decltype(rc)::value;
-                        v[r] = __fadd_rn(v[r], bias[r]);
-                    });
-                    if (EXTRA && p.residual && !p.res_after) static_for<0, 16>([&](auto rc) {
-                        constexpr int r = decltype(rc)::value;
-                        v[r] = __fadd_rn(v[r], res[j][r]);
-                    });
-                    if (p.act == TSX_ACT_RELU) {
-                        static_for<0, 16>([&](auto rc) {
-                            constexpr int r = decltype(rc)::value;
-                            v[r] = v[r] > 0.f ? v[r] : 0.f;
-                        });
-                    } else if (p.act == TSX_ACT_LEAKY_RELU) {
-                        static_for<0, 16>([&](auto rc) {
-                            constexpr int r = decltype(rc)::value;
-                            v[r] = apply_act(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
-                        });
-                    } else if (p.act == TSX_ACT_MISH) {
-                        static_for<0, 16>([&](auto rc) {
-                            constexpr int r = decltype(rc)::value;
-                            v[r] = apply_act(v[r], TSX_ACT_MISH, 0.f, true);
-                        });
-                    }
-                    if (EXTRA && p.residual && p.res_after) static_for<0, 16>([&](auto rc) {
-                        constexpr int r = decltype(rc)::value;
-                        v[r] = __fadd_rn(v[r], res[j][r]);
-                    });
-                    if (p.out_f32) static_for<0, 16>([&](auto rc) {
-                        constexpr int r = decltype(rc)::value;
-                        constexpr int dco = 8 * (r / 4) + (r % 4);
-                        // streaming store for large plain outputs: lines that never become dirty in L2 need no
-                        // write-back burst when the kernel ends; outputs a following kernel reads stay cached
-                        float *o = &(p.out_f32 + tile_base + int64_t(dco) * howo)[lane_off];
-                        if (STREAM) __builtin_nontemporal_store(v[r], o);
-                        else *o = v[r];
-                    });
-                    if (want_q) {
-                        int qv[16];
-                        if (q_even) static_for<0, 16>([&](auto rc) {
-                            constexpr int r = decltype(rc)::value;
-                            qv[r] = quantize_value(__fmul_rn(v[r], q_scale), true);
-                        });
-                        else static_for<0, 16>([&](auto rc) {
-                            constexpr int r = decltype(rc)::value;
-                            qv[r] = quantize_value(__fmul_rn(v[r], q_scale), false);
-                        });
-                        if (p.out_i8) static_for<0, 16>([&](auto rc) {
-                            constexpr int r = decltype(rc)::value;
-                            constexpr int dco = 8 * (r / 4) + (r % 4);
-                            (p.out_i8 + tile_base + int64_t(dco) * howo)[lane_off] = int8_t(qv[r]);
-                        });
-                        if (EXTRA && p.st_out) {
-                            // consumer's staged layout [pixel][channel].  Accumulator registers 4g..4g+3 of a lane are 4
-                            // consecutive channels of one pixel (one dword); the pixel's other 16 channels of this
-                            // fragment sit in lane +-32.  Two half-wave swaps leave every lane with 16 consecutive
-                            // channels -- lower half cf..cf+15, upper half cf+16..cf+31 -- for one 16-byte store
-                            // (4-byte stores at a pixel stride cost an L2 request each).
-                            uint32_t word[4];
-                            static_for<0, 4>([&](auto gc) {
-                                constexpr int g4 = decltype(gc)::value;
-                                word[g4] = uint32_t(qv[4 * g4] & 0xff) | (uint32_t(qv[4 * g4 + 1] & 0xff) << 8) |
-                                           (uint32_t(qv[4 * g4 + 2] & 0xff) << 16) | (uint32_t(qv[4 * g4 + 3] & 0xff) << 24);
-                            });
-                            // swap(a, b): a's upper half-wave <-> b's lower half-wave
-                            const auto s02 = __builtin_amdgcn_permlane32_swap(word[0], word[2], false, false);
-                            const auto s13 = __builtin_amdgcn_permlane32_swap(word[1], word[3], false, false);
-                            // the consumer's buffer is addressed by the real row/column (this kernel's rows may be virtual)
-                            const int pix = oh * p.wo + ow;
-                            const int roh = p.wo == p.o_w ? oh : pix / p.o_w;
-                            const int row_ = p.wo == p.o_w ? ow : pix - roh * p.o_w;
-                            int8_t *dst = p.st_out + ((int64_t(img + (wrapped ? 1 : 0)) * p.st_hs + roh + p.st_pt) * p.st_ws + row_ + p.st_pl) * p.st_cp +
-                                          cf + 16 * (lane / 32);
-                            const v4i packed = {int(s02[0]), int(s02[1]), int(s13[0]), int(s13[1])};
-                            *reinterpret_cast<v4i *>(dst) = packed;
-                        }
-                    }
-                }
-            } else {
-                const int co0 = cf + 4 * (lane / 32);
-                const int64_t base = (int64_t(img + (wrapped ? 1 : 0)) * p.cout + co0) * howo + oh * p.wo + ow;
-                static_for<0, 16>([&](auto rc) {
-                    constexpr int r = decltype(rc)::value;
-                    constexpr int dco = 8 * (r / 4) + (r % 4);
-                    if (pos_ok && co0 + dco < p.cout)
-                        emit(p, acc[f][j][r], base + int64_t(dco) * howo, dq[r], bias[r], 0.f);
-                });
-            }
-        });
-    });
-}
-
-template <int NT>
-int launch_nt(const WsParams &p, dim3 grid, size_t lds_bytes, hipStream_t stream) {
-    // EXTRA: residual input and/or staged int8 output; STREAM: a large fp32 output nothing reads back soon
-    if (p.residual || p.st_out)
-        hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, true, false>), grid, dim3(WS_THREADS), lds_bytes, stream, p);
-    else if (p.stream_out)
-        hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, false, true>), grid, dim3(WS_THREADS), lds_bytes, stream, p);
-    else
-        hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, false, false>), grid, dim3(WS_THREADS), lds_bytes, stream, p);
-    TSX_LAUNCH_CHECK("conv_i8_ws_kernel");
-    return 0;
-}
 
 }  // namespace
 
@@ -450,7 +99,8 @@ WsPlan ws_plan(const WsGeom &g_in) {
     if (g.wo < 1 || g.sh < 1 || g.sw < 1) return pl;
     const int wrap = g.hs - g.ho * g.sh;
     const int bm = 32 * WS_FM * wm;
-    const int coutp = (g.cout + bm - 1) / bm * bm;
+    // GEMM weights are packed once for every kernel that may read them: rows padded to 128
+    const int coutp = g.gemm ? (g.cout + 127) / 128 * 128 : (g.cout + bm - 1) / bm * bm;
     const int ksteps_p = (g.cblocks * g.kh * g.kw + RING - 1) / RING * RING;
     double best_cost = -1;
     int64_t best_frags = 0;
@@ -554,16 +204,19 @@ int ws_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t 
     }
     // an output of L2 size or more that no fused consumer reads: stream it
     p.stream_out = (!ep.residual && !ep.st_out && ep.out_f32 && int64_t(g.n) * g.cout * g.ho * g.wo * 4 >= (int64_t(16) << 20)) ? 1 : 0;
-    const dim3 grid(unsigned(pl.tiles), unsigned(pl.coutp / (32 * WS_FM * pl.wm)));
+    p.rowmajor = g.gemm ? 1 : 0;
+    if (g.gemm) p.stream_out = 0;
+    const int bm = 32 * WS_FM * pl.wm;
+    const dim3 grid(unsigned(pl.tiles), unsigned((g.cout + bm - 1) / bm));
     const size_t lds_bytes = size_t(2) * pl.wp * (64 * pl.cbs + 16);
     switch (pl.nt) {
-        case 1: return launch_nt<1>(p, grid, lds_bytes, stream);
-        case 2: return launch_nt<2>(p, grid, lds_bytes, stream);
-        case 3: return launch_nt<3>(p, grid, lds_bytes, stream);
-        case 4: return launch_nt<4>(p, grid, lds_bytes, stream);
-        case 5: return launch_nt<5>(p, grid, lds_bytes, stream);
-        case 6: return launch_nt<6>(p, grid, lds_bytes, stream);
-        case 7: return launch_nt<7>(p, grid, lds_bytes, stream);
+        case 1: return ws_launch_nt<1>(p, grid, lds_bytes, stream);
+        case 2: return ws_launch_nt<2>(p, grid, lds_bytes, stream);
+        case 3: return ws_launch_nt<3>(p, grid, lds_bytes, stream);
+        case 4: return ws_launch_nt<4>(p, grid, lds_bytes, stream);
+        case 5: return ws_launch_nt<5>(p, grid, lds_bytes, stream);
+        case 6: return ws_launch_nt<6>(p, grid, lds_bytes, stream);
+        case 7: return ws_launch_nt<7>(p, grid, lds_bytes, stream);
     }
     return fail(TSX_E_INVALID, "conv_i8_ws: unsupported fragment count %d", pl.nt);
 }

@@ -143,6 +143,9 @@ struct WsPlan {
 
 struct WsGeom {
     int n, cout, ho, wo, hs, ws, cp, cblocks, kh, kw, dil_h, dil_w, sh, sw;
+    // GEMM form: n = 1 image of ho = m one-pixel rows with k channels; the output is [m][cout] row-major, the
+    // epilogue's row_scale applies, and the weights are packed with rows padded to 128 and K-steps to 4
+    int gemm;
 };
 
 WsPlan ws_plan(const WsGeom &g);

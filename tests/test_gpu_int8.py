@@ -366,6 +366,42 @@ def test_gemm_i8(tsx, port, m, k, n, transpose):
     assert np.array_equal(bits(out.cpu().numpy()), bits(exp))
 
 
+@pytest.mark.parametrize("m,k,n", [(33, 64, 128), (256, 1024, 1024), (130, 200, 260), (257, 320, 96), (100, 512, 30),
+                                   (64, 128, 64), (500, 192, 1000)])
+@pytest.mark.parametrize("act", [None, "relu"])
+def test_gemm_i8_f32_output_only(tsx, port, m, k, n, act):
+    """More than 32 rows and only the fp32 output wanted: the window-stationary kernel's row-major epilogue
+    (16-byte stores; scalar stores when n is not a multiple of 4), with and without the per-row scale."""
+    rng = np.random.default_rng(310 + m)
+    a = rng.integers(-128, 128, (m, k)).astype(np.int8)
+    b = rng.integers(-128, 128, (k, n)).astype(np.int8)
+    dqw = rng.uniform(1e-3, 1e-2, n).astype(np.float32)
+    dqa = rng.uniform(1e-3, 1e-2, m).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    g = tsx.GemmI8(_dev(b))
+    for row_scale in (dqa, None):
+        out, _, _ = g(_dev(a), dq=_dev(dqw), row_scale=None if row_scale is None else _dev(row_scale), bias=_dev(bias), act=act)
+        exp = port.gemm_i8_dequant(a, b, dqw, np.ones(m, np.float32) if row_scale is None else row_scale, bias)
+        if act == "relu":
+            exp = port.relu(exp)
+        assert np.array_equal(bits(out.cpu().numpy()), bits(exp)), (m, k, n, act, row_scale is None)
+
+
+def test_gemm_i8_requantized_rows(tsx, port):
+    """int8 output with one consumer scale per row (base_quantize.cpp:26 groups by the first extent)."""
+    rng = np.random.default_rng(320)
+    m, k, n = 70, 256, 136
+    a = rng.integers(-128, 128, (m, k)).astype(np.int8)
+    b = rng.integers(-128, 128, (k, n)).astype(np.int8)
+    dqw = rng.uniform(1e-4, 1e-3, n).astype(np.float32)
+    qs = rng.uniform(5, 20, m).astype(np.float32)
+    g = tsx.GemmI8(_dev(b))
+    out, q, _ = g(_dev(a), dq=_dev(dqw), q_scales=_dev(qs))
+    exp = port.gemm_i8_dequant(a, b, dqw, np.ones(m, np.float32), np.zeros(n, np.float32))
+    assert np.array_equal(bits(out.cpu().numpy()), bits(exp))
+    assert np.array_equal(q.cpu().numpy(), port.quantize(exp, qs))
+
+
 def test_gemm_i8_largest_sweep_shape_by_rows(tsx, port):
     """M=4096, K=N=4096 (largest shape of the GEMM sweep): rows are independent, so a random
     subset of rows is checked against the oracle, all columns."""
