@@ -156,6 +156,50 @@ def yolo_leg(steps=5):
             "steps": steps, "outputs_finite": bool(all(torch.isfinite(o).all().item() for o in outs))}
 
 
+def gemm_leg(reps=20):
+    """int8 GEMM sweep (BASELINE config 3): M in {1, 32, 256, 4096}, K = N in {1024, 2048, 4096}; one launch of
+    tsx_gemm_i8 with per-row and per-output-channel dequantize scales and bias, fp32 output; GPU time per launch
+    from a HIP-graph replay of `reps` launches."""
+    import torch
+    from tennis_amd import capi
+    rows = []
+    for k in (1024, 2048, 4096):
+        n = k
+        gemm = capi.GemmI8(torch.randint(-128, 128, (k, n), dtype=torch.int8, device="cuda"))
+        dq = torch.rand(n, device="cuda") * 1e-2
+        bias = torch.randn(n, device="cuda")
+        for m in (1, 32, 256, 4096):
+            a = torch.randint(-128, 128, (m, k), dtype=torch.int8, device="cuda")
+            rs = torch.rand(m, device="cuda") * 1e-2
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                gemm(a, dq=dq, row_scale=rs, bias=bias)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for _ in range(reps):
+                    gemm(a, dq=dq, row_scale=rs, bias=bias)
+            graph.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(3):
+                graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            t = e0.elapsed_time(e1) * 1e-3 / (3 * reps)
+            ops = 2.0 * m * n * k
+            nbytes = m * k + k * n + 4.0 * m * n + 4.0 * n
+            # M <= 32 streams the weights once: HBM-bound; larger M is MFMA-bound
+            rows.append({"m": m, "k": k, "n": n, "us": t * 1e6, "TOPS": ops / t / 1e12, "GBps": nbytes / t / 1e9,
+                         "bound": "hbm" if m <= 32 else "mfma",
+                         "frac": (nbytes / t / 1e9 / PEAK_HBM_GBS) if m <= 32 else (ops / t / 1e12 / PEAK_INT8_TOPS)})
+    return {"workload": "BASELINE config 3: int8 GEMM sweep, per-row x per-output-channel dequantize + bias, fp32 out",
+            "launches_per_figure": 3 * reps, "shapes": rows}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -164,6 +208,7 @@ def main():
     ap.add_argument("--cpu-images", type=int, default=32, help="images of the batch timed on the CPU (0 = skip)")
     ap.add_argument("--no-resnet", action="store_true", help="skip the ResNet-50-shaped network leg")
     ap.add_argument("--no-yolo", action="store_true", help="skip the YOLOv4-shaped network leg")
+    ap.add_argument("--no-gemm", action="store_true", help="skip the int8 GEMM sweep leg")
     ap.add_argument("--profile", action="store_true",
                     help="for runs under a profiler: skip the int8-output variant (same kernel name as the roofline "
                          "kernel), the MFMA-rate probe and the CPU baseline, so per-kernel statistics cover the timed "
@@ -341,6 +386,8 @@ def main():
         result["resnet50_int8_bs32"] = resnet_leg()
     if not args.no_yolo and not args.profile:
         result["yolov4_int8_bs8"] = yolo_leg()
+    if not args.no_gemm and not args.profile:
+        result["gemm_i8_sweep"] = gemm_leg()
     if args.cpu_images > 0 and not args.profile:
         result["cpu_baseline"] = cpu_baseline(x, x_scales, wq, dq, bias, pad, min(args.cpu_images, cfg["n"]))
     print(json.dumps(result))

@@ -76,6 +76,8 @@ def build(verbose=True, jobs=8):
                 continue
             if "remark:" in l:
                 skip = 2      # the remark's source excerpt and caret line follow it
+                while keep and keep[-1].startswith("In file included from"):
+                    keep.pop()   # the include trail that led to the remark
                 continue
             if skip and (" | " in l or l.strip().startswith("|")):
                 skip -= 1
@@ -102,7 +104,7 @@ def build(verbose=True, jobs=8):
 
 BACKEND_DIR = os.path.join(HERE, "backend")
 BACKEND_LIB = os.path.join(LIB_DIR, "libtsx_backend.so")
-BACKEND_SOURCES = ["ts/ts_api.cpp", "ts/base_ops.cpp", "hip/hip_device.cpp", "hip/hip_ops_quantized.cpp", "hip/hip_ops_float.cpp", "hip/hip_ops_glue.cpp", "capi_ops.cpp"]
+BACKEND_SOURCES = ["ts/ts_api.cpp", "ts/base_ops.cpp", "hip/hip_device.cpp", "hip/hip_ops_quantized.cpp", "hip/hip_ops_float.cpp", "hip/hip_ops_glue.cpp", "hip/hip_ops_v2.cpp", "capi_ops.cpp"]
 
 
 def build_backend(verbose=True):

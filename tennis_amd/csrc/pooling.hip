@@ -30,8 +30,8 @@ __global__ __launch_bounds__(256) void pooling2d_kernel(const float *__restrict_
     ws = max(ws, 0);
     float r;
     if (g.type == 0) {
-        // the reference reads the first element unconditionally; a window with no valid element
-        // cannot occur for a shape its own size rule produces, and is reported as 0 here
+        // the reference reads the first element unconditionally; the launcher admits no MAX window
+        // without a valid element
         float m = (hs < he && ws < we) ? in[hs * g.w + ws] : 0.f;
         for (int ih = hs; ih < he; ++ih)
             for (int iw = ws; iw < we; ++iw) {
@@ -131,10 +131,12 @@ int tsx_pooling2d_f32(const float *x_dev, int64_t planes, int32_t h, int32_t w, 
                 "pooling2d: non-positive extent");
     TSX_REQUIRE(type == 0 || type == 1, "pooling2d: type must be 0 (max) or 1 (avg)");
     TSX_REQUIRE(pad_top >= 0 && pad_left >= 0, "pooling2d: negative padding");
-    // every window must hold at least one element's row/column start inside the map (the reference
-    // reads in[hs][ws] unconditionally for MAX)
-    TSX_REQUIRE((int64_t(out_h) - 1) * stride_h - pad_top < h && (int64_t(out_w) - 1) * stride_w - pad_left < w,
-                "pooling2d: output %dx%d has windows outside the %dx%d map", out_h, out_w, h, w);
+    // The ceil-mode size rule can give a last window that starts behind the map (9 rows, pads 1+2, 3 rows at
+    // stride 2: the sixth window starts at row 9).  The reference's average of no element is 0
+    // (src/kernels/cpu/pooling2d_core.cpp:131-134, 179), which the kernel reproduces; its MAX reads
+    // in[hs][ws] unconditionally (:69), i.e. behind the plane -- there is no value to match, so that is refused.
+    TSX_REQUIRE(type == 1 || ((int64_t(out_h) - 1) * stride_h - pad_top < h && (int64_t(out_w) - 1) * stride_w - pad_left < w),
+                "pooling2d: max pooling output %dx%d has windows outside the %dx%d map", out_h, out_w, h, w);
     PoolGeom g{planes, h, w, out_h, out_w, type, pad_top, pad_left, kh, kw, stride_h, stride_w, white_padding ? 1 : 0};
     const int64_t total = planes * out_h * out_w;
     TSX_REQUIRE(tsx::ceil_div(total, 256) < (int64_t(1) << 31), "pooling2d: tensor too large");

@@ -86,6 +86,15 @@ def main():
     save_case("global_pooling2d/avg", "global_pooling2d", {"format": "NCHW", "type": np.array([1], np.int32)}, [x])
     save_case("add/broadcast", "add", {}, [x, f32(1, 6, 1, 1)])
     save_case("depthwise_conv2d/3x3", "depthwise_conv2d", conv_params((1, 1, 1, 1)), [x, f32(1, 6, 3, 3)])
+    # the "_v2" operators: padding (pooling: also ksize and stride) arrive as inputs
+    pad42 = conv_params((1, 2, 0, 1))["padding"]
+    v2 = {k: v for k, v in conv_params((0, 0, 0, 0), (2, 1)).items() if k != "padding"}
+    save_case("conv2d_v2/3x3_s2x1", "conv2d_v2", v2, [x, pad42, f32(5, 6, 3, 3) * 0.2])
+    save_case("depthwise_conv2d_v2/3x3_s2x1", "depthwise_conv2d_v2", v2, [x, pad42, f32(1, 6, 3, 3)])
+    save_case("conv2d_winograd_v2/auto_mode", "conv2d_winograd_v2", {"format": "NCHW"},
+              [f32(1, 6, 14, 13), conv_params((1, 1, 1, 1))["padding"], f32(5, 6, 3, 3) * 0.2])
+    save_case("pooling2d_v2/avg_3x2", "pooling2d_v2", {"format": "NCHW", "type": np.array([1], np.int32)},
+              [x, pad42, np.array([1, 1, 3, 2], np.int32), np.array([1, 1, 2, 1], np.int32)])
     # an operator the "hip" device does not register: the runner reports SKIP, as TenniS's does
     save_case("softmax/not_on_device", "softmax", {"dim": np.array([1], np.int32)}, [f32(3, 5)])
 

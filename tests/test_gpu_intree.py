@@ -130,3 +130,22 @@ def test_unregistered_operator_falls_back_to_cpu(ts):
     cpu = ts.run_op_intree("cpu", "sigmoid", {}, [x], x.nbytes)
     hip = ts.run_op_intree("hip", "sigmoid", {}, [x], x.nbytes, strict=False)
     assert np.array_equal(bits(cpu), bits(hip))
+
+
+def test_v2_wrappers_in_tennis_workbench(ts):
+    """The dynamic-padding wrappers registered for "hip" against TenniS's own (cpu) ones, both inside its Workbench."""
+    rng = np.random.default_rng(905)
+    x = rng.standard_normal((2, 6, 12, 10)).astype(np.float32)
+    w = (rng.standard_normal((7, 6, 3, 3)) * 0.2).astype(np.float32)
+    full = conv_params(ts, (0, 2, 1, 0), (2, 1), (1, 1), 0.5)
+    v2 = {k: v for k, v in full.items() if k != "padding"}
+    cpu, hip = both(ts, "conv2d_v2", v2, [x, full["padding"], w], 1 << 20)
+    assert close(hip, cpu)
+    cpu, hip = both(ts, "depthwise_conv2d_v2", v2, [x, full["padding"], w[:1].copy()], 1 << 20)
+    assert close(hip, cpu)
+    cpu, hip = both(ts, "pooling2d_v2", {"format": "NCHW", "type": np.array([1], np.int32)},
+                    [x, conv_params(ts, (0, 1, 1, 0))["padding"], np.array([1, 1, 3, 2], np.int32), np.array([1, 1, 2, 1], np.int32)],
+                    1 << 20)
+    assert np.array_equal(bits(cpu), bits(hip))
+    cpu, hip = both(ts, "conv2d_winograd_v2", {"format": "NCHW"}, [x, conv_params(ts, (1, 1, 1, 1))["padding"], w], 1 << 20)
+    assert np.array_equal(bits(cpu), bits(hip))

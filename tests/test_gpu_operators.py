@@ -147,7 +147,9 @@ def test_glue_operators(ops, port):
     rng = np.random.default_rng(505)
     x = rng.standard_normal((2, 5, 13, 11)).astype(np.float32)
     for kind, k, s, pads, white in (("max", (3, 3), (2, 2), (1, 1, 1, 1), False), ("avg", (2, 3), (2, 1), (1, 0, 1, 1), False),
-                                    ("avg", (3, 3), (1, 1), (1, 1, 1, 1), True), ("max", (5, 5), (1, 1), (2, 2, 2, 2), False)):
+                                    ("avg", (3, 3), (1, 1), (1, 1, 1, 1), True), ("max", (5, 5), (1, 1), (2, 2, 2, 2), False),
+                                    # ceil mode puts the last row of windows behind the map: the average of nothing is 0
+                                    ("avg", (3, 2), (2, 1), (1, 2, 0, 1), False), ("avg", (3, 2), (2, 1), (1, 2, 0, 1), True)):
         got = ops.run_op("pooling2d", _pool_params(kind, k, s, pads, white), [x])
         want = port.pooling2d(x, kind, k, s, pads, white)
         assert got.shape == want.shape and np.array_equal(bits(got), bits(want)), (kind, k, s, pads, white)
@@ -160,6 +162,8 @@ def test_glue_operators(ops, port):
             got = ops.run_op("add", {}, [lhs, rhs])
             want = lhs + rhs                                   # one IEEE addition per element
             assert got.shape == want.shape and np.array_equal(bits(got), bits(want)), shape
+    with pytest.raises(ops.OperatorError, match="windows outside"):      # the reference's MAX reads behind the plane there
+        ops.run_op("pooling2d", _pool_params("max", (3, 2), (2, 1), (1, 2, 0, 1)), [x])
     with pytest.raises(ops.OperatorError, match="Can not reduce shape"):
         ops.run_op("add", {}, [x, np.zeros((2, 4, 13, 11), np.float32)])
     w = rng.standard_normal((1, 5, 3, 3)).astype(np.float32)
@@ -184,3 +188,31 @@ def test_operator_errors_at_run_time(ops):
         ops.run_op("conv2d_quantized", params, [x.astype(np.float32), np.zeros((4, 8, 3, 3), np.float32)])
     with pytest.raises(ops.OperatorNotFound):
         ops.run_op("softmax", {}, [np.zeros((2, 2), np.float32)])
+
+
+def test_v2_operators_equal_their_plain_twins(ops):
+    """conv2d_v2 / depthwise_conv2d_v2 / conv2d_winograd_v2 / pooling2d_v2 take padding (ksize, stride) as
+    inputs (src/kernels/cpu/conv2d_v2.cpp:60-92) and must give what the plain operator gives for the same values."""
+    rng = np.random.default_rng(507)
+    x = rng.standard_normal((2, 6, 12, 10)).astype(np.float32)
+    w = (rng.standard_normal((7, 6, 3, 3)) * 0.2).astype(np.float32)
+    for pads in ((1, 1, 1, 1), (0, 2, 1, 0)):
+        full = ops.conv_params(pads, (2, 1), (1, 1), 0.5)
+        v2 = {k: v for k, v in full.items() if k != "padding"}
+        got = ops.run_op("conv2d_v2", v2, [x, full["padding"], w])
+        assert np.array_equal(bits(got), bits(ops.run_op("conv2d", full, [x, w])))
+        assert ops.run_op("conv2d_v2", v2, [x, full["padding"], w], infer_only=True)[1] == got.shape
+        wd = w[:1].copy()
+        got = ops.run_op("depthwise_conv2d_v2", v2, [x, full["padding"].astype(np.int64), wd])   # cast to INT32 inside
+        assert np.array_equal(bits(got), bits(ops.run_op("depthwise_conv2d", full, [x, wd])))
+        wino = {k: full[k] for k in ("format", "padding_value")}
+        got = ops.run_op("conv2d_winograd_v2", wino, [x, full["padding"], w])
+        assert np.array_equal(bits(got), bits(ops.run_op("conv2d_winograd", dict(wino, padding=full["padding"]), [x, w])))
+        pool = _pool_params("avg", (3, 2), (2, 1), (pads[0], 1, pads[2], pads[3]), True)   # every window touches the map
+        got = ops.run_op("pooling2d_v2", {k: pool[k] for k in ("format", "type", "padding_type")},
+                         [x, pool["padding"], pool["ksize"], pool["stride"]])
+        assert np.array_equal(bits(got), bits(ops.run_op("pooling2d", pool, [x])))
+    with pytest.raises(ops.OperatorError, match="expects 3 inputs"):
+        ops.run_op("conv2d_v2", v2, [x, w])
+    with pytest.raises(ops.OperatorError):      # stride is required (conv2d_v2.cpp:17)
+        ops.run_op("conv2d_v2", {"format": "NCHW"}, [x, full["padding"], w])
