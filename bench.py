@@ -200,6 +200,81 @@ def gemm_leg(reps=20):
             "launches_per_figure": 3 * reps, "shapes": rows}
 
 
+PEAK_FP32_TFLOPS = 157.3   # MI355X dense fp32 MFMA
+
+
+def kernels_leg(reps=20):
+    """Every other kernel of the path on its own (for per-kernel counters under rocprofv3 and the figures next
+    to BASELINE config 2): each is launched `reps` times back to back after 3 warm-up launches and timed with
+    events on the launch stream.  `work` is algorithmic: ops for the MFMA-bound kernels, bytes for the HBM-bound."""
+    import torch
+    from tennis_amd import capi
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cuda").manual_seed(7)
+    rnd = lambda *s: torch.randn(s, device=dev, generator=g)
+    ri8 = lambda *s: torch.randint(-128, 128, s, dtype=torch.int8, device=dev, generator=g)
+    rows = []
+
+    def timed(name, bound, work, fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        t = e0.elapsed_time(e1) * 1e-3 / reps
+        peak = {"hbm": PEAK_HBM_GBS * 1e9, "mfma_i8": PEAK_INT8_TOPS * 1e12, "mfma_f32": PEAK_FP32_TFLOPS * 1e12}[bound]
+        rows.append({"kernel": name, "bound": bound, "us": t * 1e6, "work": work, "achieved": work / t,
+                     "unit": "B/s" if bound == "hbm" else "op/s", "frac": work / t / peak})
+
+    # fp32 BASELINE config 1 (1x64x56x56 * 64x64x3x3, bias + ReLU): implicit GEMM and both Winograd modes
+    x1, w1, b1 = torch.rand((1, 64, 56, 56), device=dev) * 2 - 1, rnd(64, 64, 3, 3) * 0.06, rnd(64) * 0.01
+    flops1 = 2.0 * 64 * 56 * 56 * 64 * 9
+    timed("conv2d_f32 config 1 (gemm_f32_kernel)", "mfma_f32", flops1, lambda: capi.conv2d_f32(x1, w1, (1, 1, 1, 1), bias=b1, act="relu"))
+    w63, w23 = capi.WinogradF63(w1, (1, 1, 1, 1)), capi.WinogradF23(w1, (1, 1, 1, 1))
+    timed("winograd F(6,3) config 1 (direct-conv flops)", "mfma_f32", flops1, lambda: w63(x1, bias=b1, act="relu"))
+    timed("winograd F(2,3) config 1 (direct-conv flops)", "mfma_f32", flops1, lambda: w23(x1, bias=b1, act="relu"))
+    # int8 GEMM: largest and a mid shape of BASELINE config 3, and the weight-streaming single row
+    k = n = 4096
+    gemm = capi.GemmI8(ri8(k, n))
+    dq, bias = torch.rand(n, device=dev) * 1e-2, rnd(n)
+    for m in (4096, 256, 1):
+        a, rs = ri8(m, k), torch.rand(m, device=dev) * 1e-2
+        if m > 32:
+            timed("gemm_i8 M=%d K=N=4096 (conv_i8_ws_kernel, row-major)" % m, "mfma_i8", 2.0 * m * n * k,
+                  lambda a=a, rs=rs: gemm(a, dq=dq, row_scale=rs, bias=bias))
+        else:
+            timed("gemm_i8 M=%d K=N=4096 (gemm_i8_skinny_kernel)" % m, "hbm", m * k + k * n + 4.0 * m * n + 4.0 * n,
+                  lambda a=a, rs=rs: gemm(a, dq=dq, row_scale=rs, bias=bias))
+    # memory-bound 1x1 int8 layer (ResNet stage 1 expansion, 64 -> 256 channels at 56x56, batch 32), staged int8 in, fp32 out
+    xq = ri8(32, 64, 56, 56)
+    c11 = capi.Conv2dI8(ri8(256, 64, 1, 1))
+    dq11, b11 = torch.rand(256, device=dev) * 1e-3, rnd(256)
+    st = capi.StagedInput(c11, xq.shape)
+    c11.stage(xq, st)
+    ws_bytes = c11._plan(tuple(xq.shape))[2]
+    timed("conv2d_i8 1x1 64->256 @56x56 bs32, fp32 out (conv_i8_ws_kernel)", "hbm", float(ws_bytes) + 4.0 * 32 * 256 * 56 * 56,
+          lambda: c11.run_staged(st, dq11, b11, "relu"))
+    # HBM-bound glue on a 32x256x56x56 fp32 tensor (103 MB)
+    x = rnd(32, 256, 56, 56)
+    nb = 4.0 * x.numel()
+    wd = rnd(1, 256, 3, 3)
+    timed("depthwise_conv2d 3x3 s1 p1", "hbm", 2 * nb, lambda: capi.depthwise_conv2d(x, wd, (1, 1, 1, 1)))
+    timed("relu", "hbm", 2 * nb, lambda: capi.relu(x))
+    bb = rnd(256)
+    timed("add_bias", "hbm", 2 * nb, lambda: capi.add_bias(x, bb))
+    x2 = rnd(32, 256, 56, 56)
+    timed("add + relu (residual join)", "hbm", 3 * nb, lambda: capi.add(x, x2, act="relu"))
+    qs = torch.full((32,), 20.0, device=dev)
+    timed("quantize", "hbm", 1.25 * nb, lambda: capi.quantize(x, qs))
+    timed("pooling2d max 3x3 s2 p1", "hbm", 1.25 * nb, lambda: capi.pooling2d(x, "max", (3, 3), (2, 2), (1, 1, 1, 1)))
+    return {"workload": "kernels of the path one by one; time per launch includes the wrapper's output allocation from "
+                        "torch's caching allocator (no device allocation in steady state)", "reps": reps, "kernels": rows}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -215,6 +290,9 @@ def main():
                          "kernels only")
     ap.add_argument("--network", choices=("resnet", "yolo"),
                     help="run only that network leg and print its figures (for per-kernel profiles of a network)")
+    ap.add_argument("--kernels", action="store_true",
+                    help="run only the one-by-one kernel leg (GEMM, fp32, Winograd, 1x1, depthwise, elementwise, pooling) "
+                         "and print its figures (for per-kernel counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)", file=sys.stderr)
@@ -231,6 +309,9 @@ def main():
     dev = torch.device("cuda:0")
     if args.network:
         print(json.dumps(resnet_leg() if args.network == "resnet" else yolo_leg()))
+        return
+    if args.kernels:
+        print(json.dumps(kernels_leg()))
         return
     cfg = CFG
     x, x_scales, wq, dq, bias = make_inputs(cfg)

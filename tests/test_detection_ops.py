@@ -18,6 +18,9 @@ DW_CASES = [
     ((5, 3), (2, 1, 0, 1), (1, 2), (1, 1), 0.5),
     ((3, 3), (2, 2, 2, 2), (1, 1), (2, 2), 0.0),
     ((1, 1), (0, 0, 0, 0), (1, 1), (1, 1), 0.0),
+    # 3x3 / stride 1 / column padding 1 on rows whose length is a multiple of 4: the vector-load path
+    ((3, 3), (1, 1, 1, 1), (1, 1), (1, 1), 0.75),
+    ((3, 3), (0, 2, 1, 1), (1, 1), (1, 1), -1.5),
 ]
 
 
@@ -85,7 +88,7 @@ def _dev(a):
 @pytest.mark.parametrize("case", DW_CASES)
 def test_hip_depthwise(tsx, port, case):
     k, pads, st, dl, pv = case
-    for shape in ((2, 6, 11, 9), (3, 70, 28, 28)):
+    for shape in ((2, 6, 11, 9), (3, 70, 28, 28), (1, 3, 40, 64)):
         x = _x(21, shape)
         w = np.random.default_rng(22).standard_normal((1, shape[1], k[0], k[1])).astype(np.float32)
         bias = np.random.default_rng(23).standard_normal(shape[1]).astype(np.float32)
