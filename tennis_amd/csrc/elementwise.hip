@@ -36,11 +36,19 @@ __global__ __launch_bounds__(256) void elementwise_kernel(const float *__restric
             if (MODE == 3)
                 for (int j = 0; j < 4; ++j) u[j] = base + j < count ? bias[base + j] : 0.f;
         }
+        // add_bias: a lane's four elements share their channel when the inner extent is a multiple of 4 (one
+        // division instead of four; 32-bit where the tensor allows it)
+        const bool one_channel = MODE == 0 && full && (inner & 3) == 0;
+        float lane_bias = 0.f;
+        if (one_channel)
+            lane_bias = bias[count < (int64_t(1) << 32) ? int((unsigned(base) / unsigned(inner)) % unsigned(channels))
+                                                        : int((base / inner) % channels)];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int64_t i = base + j;
             if (MODE == 0) {
-                if (i < count) v[j] = __fadd_rn(v[j], bias[(i / inner) % channels]);
+                if (one_channel) v[j] = __fadd_rn(v[j], lane_bias);
+                else if (i < count) v[j] = __fadd_rn(v[j], bias[(i / inner) % channels]);
             } else if (MODE == 3) {
                 v[j] = tsx::apply_act(__fadd_rn(v[j], u[j]), act, slope, i < body);
             } else if (MODE == 4) {

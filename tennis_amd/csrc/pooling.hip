@@ -16,20 +16,59 @@ struct PoolGeom {
     int h, w, ho, wo, type, pad_top, pad_left, kh, kw, sh, sw, white;
 };
 
+// KH, KW > 0: a window of that size, unrolled -- every element is loaded from a clamped address before the
+// first comparison or addition, so a lane's loads are in flight together (the runtime-sized loop below waits
+// for each element in turn: one memory round trip per window element).  KH == 0: any window size.
+template <int KH, int KW>
 __global__ __launch_bounds__(256) void pooling2d_kernel(const float *__restrict__ x, PoolGeom g, float *__restrict__ out) {
     const int64_t total = g.planes * g.ho * g.wo;
     const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
     if (id >= total) return;
-    const int ow = int(id % g.wo);
-    const int oh = int((id / g.wo) % g.ho);
-    const int64_t pc = id / g.wo / g.ho;
+    int ow, oh;
+    int64_t pc;
+    if (total < (int64_t(1) << 32)) {   // 32-bit divisions: a 64-bit one costs more than the window's loads
+        const unsigned u = unsigned(id), row = u / unsigned(g.wo);
+        ow = int(u - row * unsigned(g.wo));
+        pc = row / unsigned(g.ho);
+        oh = int(row - unsigned(pc) * unsigned(g.ho));
+    } else {
+        ow = int(id % g.wo);
+        oh = int((id / g.wo) % g.ho);
+        pc = id / g.wo / g.ho;
+    }
     const float *in = x + pc * g.h * g.w;
     int hs = oh * g.sh - g.pad_top, ws = ow * g.sw - g.pad_left;
     const int he = min(hs + g.kh, g.h), we = min(ws + g.kw, g.w);
     hs = max(hs, 0);
     ws = max(ws, 0);
     float r;
-    if (g.type == 0) {
+    if (KH > 0) {
+        const int h0 = oh * g.sh - g.pad_top, w0 = ow * g.sw - g.pad_left;
+        float v[KH > 0 ? KH * KW : 1];
+#pragma unroll
+        for (int i = 0; i < KH; ++i)
+#pragma unroll
+            for (int j = 0; j < KW; ++j)
+                v[i * KW + j] = in[min(max(h0 + i, 0), g.h - 1) * g.w + min(max(w0 + j, 0), g.w - 1)];
+        // the valid elements in row-major order, as the reference walks them
+        float m = 0.f, sum = 0.f;
+        int count = 0;
+#pragma unroll
+        for (int i = 0; i < KH; ++i)
+#pragma unroll
+            for (int j = 0; j < KW; ++j) {
+                const bool ok = h0 + i >= 0 && h0 + i < g.h && w0 + j >= 0 && w0 + j < g.w;
+                const float e = v[i * KW + j];
+                if (ok) {
+                    if (count == 0 || e > m) m = e;    // MAX starts from the first valid element, replaces on `>`
+                    sum = __fadd_rn(sum, e);
+                    ++count;
+                }
+            }
+        if (g.type == 0) r = m;
+        else if (g.white) r = __fdiv_rn(sum, float(KH * KW));
+        else r = count == 0 ? 0.f : __fdiv_rn(sum, float(count));
+    } else if (g.type == 0) {
         // the reference reads the first element unconditionally; the launcher admits no MAX window
         // without a valid element
         float m = (hs < he && ws < we) ? in[hs * g.w + ws] : 0.f;
@@ -140,8 +179,15 @@ int tsx_pooling2d_f32(const float *x_dev, int64_t planes, int32_t h, int32_t w, 
     PoolGeom g{planes, h, w, out_h, out_w, type, pad_top, pad_left, kh, kw, stride_h, stride_w, white_padding ? 1 : 0};
     const int64_t total = planes * out_h * out_w;
     TSX_REQUIRE(tsx::ceil_div(total, 256) < (int64_t(1) << 31), "pooling2d: tensor too large");
-    hipLaunchKernelGGL(pooling2d_kernel, dim3(unsigned(tsx::ceil_div(total, 256))), dim3(256), 0, tsx::as_stream(stream),
-                       x_dev, g, out_dev);
+    const dim3 grid(unsigned(tsx::ceil_div(total, 256)));
+    if (kh == 3 && kw == 3)
+        hipLaunchKernelGGL((pooling2d_kernel<3, 3>), grid, dim3(256), 0, tsx::as_stream(stream), x_dev, g, out_dev);
+    else if (kh == 2 && kw == 2)
+        hipLaunchKernelGGL((pooling2d_kernel<2, 2>), grid, dim3(256), 0, tsx::as_stream(stream), x_dev, g, out_dev);
+    else if (kh == 5 && kw == 5)
+        hipLaunchKernelGGL((pooling2d_kernel<5, 5>), grid, dim3(256), 0, tsx::as_stream(stream), x_dev, g, out_dev);
+    else
+        hipLaunchKernelGGL((pooling2d_kernel<0, 0>), grid, dim3(256), 0, tsx::as_stream(stream), x_dev, g, out_dev);
     TSX_LAUNCH_CHECK("pooling2d_kernel");
     return 0;
 }
