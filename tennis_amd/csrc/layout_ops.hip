@@ -12,10 +12,10 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 __global__ __launch_bounds__(256) void concat_channels_kernel(const float *__restrict__ src, int64_t n, int64_t row,
                                                              float *__restrict__ dst, int64_t dst_row, int64_t dst_off,
                                                              bool vec) {
+    // blockIdx.y walks the batch, blockIdx.x one image's row: no division per element
     const int64_t per = vec ? row / 4 : row;
-    const int64_t total = n * per;
-    for (int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; id < total; id += int64_t(gridDim.x) * blockDim.x) {
-        const int64_t ni = id / per, e = id - ni * per;
+    for (int64_t ni = blockIdx.y; ni < n; ni += gridDim.y)
+    for (int64_t e = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; e < per; e += int64_t(gridDim.x) * blockDim.x) {
         if (vec)
             *reinterpret_cast<v4f *>(dst + ni * dst_row + dst_off + e * 4) = *reinterpret_cast<const v4f *>(src + ni * row + e * 4);
         else
@@ -175,9 +175,10 @@ int tsx_concat_channels_f32(const float *src_dev, int64_t n, int32_t c_src, int6
     const int64_t row = int64_t(c_src) * inner, dst_row = int64_t(c_dst) * inner, dst_off = int64_t(c_offset) * inner;
     const bool vec = row % 4 == 0 && dst_row % 4 == 0 && dst_off % 4 == 0 && reinterpret_cast<uintptr_t>(src_dev) % 16 == 0 &&
                      reinterpret_cast<uintptr_t>(dst_dev) % 16 == 0;
-    int64_t blocks = tsx::ceil_div(n * (vec ? row / 4 : row), 256);
+    int64_t blocks = tsx::ceil_div(vec ? row / 4 : row, 256);
     if (blocks > 256 * 16) blocks = 256 * 16;
-    hipLaunchKernelGGL(concat_channels_kernel, dim3(unsigned(blocks)), dim3(256), 0, tsx::as_stream(stream), src_dev, n, row,
+    const unsigned batch_blocks = unsigned(n < 65535 ? n : 65535);
+    hipLaunchKernelGGL(concat_channels_kernel, dim3(unsigned(blocks), batch_blocks), dim3(256), 0, tsx::as_stream(stream), src_dev, n, row,
                        dst_dev, dst_row, dst_off, vec);
     TSX_LAUNCH_CHECK("concat_channels_kernel");
     return 0;
