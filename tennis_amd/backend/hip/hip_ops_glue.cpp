@@ -90,6 +90,44 @@ public:
     }
 };
 
+// concat along any axis: every input is one strided copy [outer][extent_i * inner] into its slot of the
+// output rows (src/kernels/cpu/concat.cpp copies the same blocks with memcpy).  Elements of 4 bytes.
+class Concat : public OperatorOnHip<base::Concat> {
+public:
+    void concat(const std::vector<Tensor> &x, int dim, Tensor &out) override {
+        if (type_bytes(out.dtype()) != 4)
+            TS_LOG_ERROR << "[hip] concat not support data type(" << out.dtype() << "): " << type_str(out.dtype()) << eject;
+        int64_t outer = 1, inner = 1;
+        for (int i = 0; i < dim; ++i) outer *= out.size(size_t(i));
+        for (size_t i = size_t(dim) + 1; i < out.dims(); ++i) inner *= out.size(i);
+        int32_t offset = 0;
+        for (auto &t : x) {
+            const int32_t extent = t.size(size_t(dim));
+            if (extent > 0 && outer > 0 && inner > 0)
+                check(tsx_concat_channels_f32(t.data<float>(), outer, extent, inner, out.data<float>(), out.size(size_t(dim)), offset,
+                                              current_stream()),
+                      "tsx_concat_channels_f32");
+            offset += extent;
+        }
+    }
+};
+
+// _resize2d: the nearest-neighbour mode on the two innermost axes (NCHW maps, the upsampling of detection necks).
+class Resize2D : public OperatorOnHip<base::Resize2D> {
+public:
+    void resize2d(const Tensor &x, int dim, Resize2DType type, Tensor &out) override {
+        if (type != Resize2DType::NEAREST)
+            TS_LOG_ERROR << "[hip] _resize2d supports type NEAREST (2) only, got " << int(type) << eject;
+        if (x.dtype() != FLOAT32) TS_LOG_ERROR << "[hip] _resize2d not support data type(" << x.dtype() << "): " << type_str(x.dtype()) << eject;
+        if (size_t(dim) + 2 != x.dims()) TS_LOG_ERROR << "[hip] _resize2d resizes the two innermost axes only (NCHW)" << eject;
+        int64_t planes = 1;
+        for (int i = 0; i < dim; ++i) planes *= x.size(size_t(i));
+        check(tsx_resize_nearest_f32(x.data<float>(), planes, x.size(size_t(dim)), x.size(size_t(dim) + 1), out.data<float>(),
+                                     out.size(size_t(dim)), out.size(size_t(dim) + 1), current_stream()),
+              "tsx_resize_nearest_f32");
+    }
+};
+
 }  // namespace hip
 }  // namespace ts
 
@@ -99,3 +137,5 @@ TS_REGISTER_OPERATOR(Pooling2D, ts::hip::DEVICE, name::layer::pooling2d())
 TS_REGISTER_OPERATOR(GlobalPooling2D, ts::hip::DEVICE, name::layer::global_pooling2d())
 TS_REGISTER_OPERATOR(Add, ts::hip::DEVICE, name::layer::add())
 TS_REGISTER_OPERATOR(DepthwiseConv2D, ts::hip::DEVICE, name::layer::depthwise_conv2d())
+TS_REGISTER_OPERATOR(Concat, ts::hip::DEVICE, name::layer::concat())
+TS_REGISTER_OPERATOR(Resize2D, ts::hip::DEVICE, name::layer::resize2d())

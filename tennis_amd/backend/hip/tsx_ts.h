@@ -19,6 +19,8 @@
 #endif
 #ifdef TSX_TS_GLUE_OPS
 #include <backend/base/base_add.h>
+#include <backend/base/base_concat.h>
+#include <backend/base/base_resize2d.h>
 #include <backend/base/base_depthwise_conv2d.h>
 #include <backend/base/base_global_pooling2d.h>
 #include <backend/base/base_pooling2d.h>

@@ -2,6 +2,8 @@
 // graph which TenniS rejects at init()/infer() is rejected here for the same reason.
 #include "base_ops.h"
 
+#include <sstream>
+
 namespace ts {
 namespace base {
 
@@ -516,6 +518,129 @@ int LeakyReLU::run(Stack &stack) {
     auto x = stack[0].view(memory_device);
     auto &out = *stack.push(x.proto(), memory_device);
     leaky_relu(x, m_scale, out);
+    return 1;
+}
+
+// ---------------------------------------------------------------- concat
+Concat::Concat() { field(name::dim, REQUIRED); }
+
+void Concat::init() {
+    supper::init();
+    m_dim = tensor::to_int(get(name::dim));
+}
+
+namespace {
+[[noreturn]] void concat_mismatch(Stack &stack, int dim) {
+    std::ostringstream oss;
+    for (size_t j = 0; j < stack.size(); ++j)
+        oss << (j ? ", " : "") << type_str(stack[j].dtype()) << ":" << to_string(stack[j].sizes());
+    TS_LOG_ERROR << "Can not concat {" << oss.str() << "} at dim=" << dim << eject;
+    throw Exception("unreachable");
+}
+}  // namespace
+
+int Concat::infer(Stack &stack, std::vector<Tensor::Prototype> &output) {
+    const size_t inputs = stack.size();
+    if (inputs == 0) TS_LOG_ERROR << "concat needs at least one input" << eject;
+    output.resize(1);
+    if (inputs == 1) {
+        output[0] = stack[0].proto();
+        return 1;
+    }
+    const DTYPE dtype = stack[0].dtype();
+    Shape shape = stack[0].sizes();
+    const int dims = int(shape.size());
+    const int dim = m_dim >= 0 ? m_dim : dims + m_dim;
+    if (dim < 0 || dim >= dims) TS_LOG_ERROR << "Concat dim must in [-" << dims << ", " << dims << ")" << eject;
+    for (size_t i = 1; i < inputs; ++i) {
+        const Tensor &t = stack[i];
+        if (t.dtype() != dtype || int(t.dims()) != dims) concat_mismatch(stack, m_dim);
+        for (int j = 0; j < dims; ++j)
+            if (j != dim && t.size(size_t(j)) != shape[size_t(j)]) concat_mismatch(stack, m_dim);
+        shape[size_t(dim)] += t.size(size_t(dim));
+    }
+    output[0] = Tensor::Prototype(dtype, shape);
+    return 1;
+}
+
+int Concat::run(Stack &stack) {
+    std::vector<Tensor::Prototype> protos;
+    infer(stack, protos);
+    const size_t inputs = stack.size();
+    auto memory_device = running_memory_device();
+    std::vector<Tensor> x;
+    for (size_t i = 0; i < inputs; ++i) x.push_back(stack[i].view(memory_device));
+    Tensor out = *stack.push(protos[0], memory_device);
+    const int dims = int(x[0].dims());
+    concat(x, m_dim >= 0 ? m_dim : dims + m_dim, out);
+    return 1;
+}
+
+// ---------------------------------------------------------------- _resize2d
+Resize2D::Resize2D() { field(name::type, OPTIONAL, tensor::from(int(Resize2DType::LINEAR))); }
+
+void Resize2D::init() { m_type = Resize2DType(tensor::to_int(get(name::type))); }
+
+namespace {
+// The axis that becomes the new height (base_resize2d.cpp:27-63): the first positive entry of `size` that is
+// not merely a copy of the extent with an unchanged tail behind the pair; -1 when the request is not a 2-D resize.
+int resized_height_dim(const Shape &shape, const int32_t *size, int n) {
+    int found = -1;
+    for (int i = 0; i < n; ++i) {
+        if (size[i] == 0) return -1;
+        if (size[i] < 0) continue;
+        if (shape[size_t(i)] == size[i]) {
+            bool tail_kept = true;
+            for (int j = i + 2; j < n && tail_kept; ++j) tail_kept = shape[size_t(j)] == size[j] || size[j] < 0;
+            if (!tail_kept) continue;
+        }
+        found = i;
+        break;
+    }
+    if (found < 0 || found >= n - 1 || size[found + 1] <= 0) return -1;
+    for (int i = found + 2; i < n; ++i)
+        if (size[i] == 0 || !(shape[size_t(i)] == size[i] || size[i] < 0)) return -1;
+    return found;
+}
+
+Tensor::Prototype resized_proto(Stack &stack, int &dim, bool &same) {
+    if (stack.size() != 2) TS_LOG_ERROR << "_resize2d expects 2 inputs (x, size), got " << stack.size() << eject;
+    const Tensor &x = stack[0];
+    Tensor size = tensor::cast(INT32, stack[1].view(MemoryDevice(CPU)));
+    if (!(size.dims() == 1 && int(x.dims()) == size.size(0) && size.size(0) >= 2))
+        TS_LOG_ERROR << "_resize2d: size must hold one entry per axis of x (at least 2)" << eject;
+    const int n = size.size(0);
+    const int32_t *data = size.data<int32_t>();
+    dim = resized_height_dim(x.sizes(), data, n);
+    if (dim < 0) TS_LOG_ERROR << "Can not resize " << to_string(x.sizes()) << " to " << to_string(Shape(std::vector<int32_t>(data, data + n))) << eject;
+    Shape out = x.sizes();
+    same = out[size_t(dim)] == data[dim] && out[size_t(dim) + 1] == data[dim + 1];
+    out[size_t(dim)] = data[dim];
+    out[size_t(dim) + 1] = data[dim + 1];
+    return Tensor::Prototype(x.dtype(), out);
+}
+}  // namespace
+
+int Resize2D::infer(Stack &stack, std::vector<Tensor::Prototype> &output) {
+    int dim;
+    bool same;
+    output.assign(1, resized_proto(stack, dim, same));
+    return 1;
+}
+
+int Resize2D::run(Stack &stack) {
+    int dim;
+    bool same;
+    const Tensor::Prototype proto = resized_proto(stack, dim, same);
+    if (same) {   // nothing to resize: the input is the output
+        const Tensor x = stack[0];
+        stack.push(x);
+        return 1;
+    }
+    auto memory_device = running_memory_device();
+    Tensor x = stack[0].view(memory_device);
+    Tensor out = *stack.push(proto, memory_device);
+    resize2d(x, dim, m_type, out);
     return 1;
 }
 

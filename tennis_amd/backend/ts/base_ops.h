@@ -193,6 +193,38 @@ private:
     float m_scale = 0;
 };
 
+// concat (src/backend/base/base_concat.cpp:13-130): inputs of one dtype and equal shape except along `dim`
+// (negative counts from the end) joined along it.
+class Concat : public OperatorOnDevice {
+public:
+    using supper = OperatorOnDevice;
+    Concat();
+    void init() override;
+    int run(Stack &stack) override;
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override;
+    virtual void concat(const std::vector<Tensor> &x, int dim, Tensor &out) = 0;
+
+private:
+    int m_dim = 0;
+};
+
+// _resize2d (src/backend/base/base_resize2d.cpp:12-121): inputs x and an INT32 size vector with one entry per
+// axis of x; the two neighbouring positive entries that differ from x's extents (or, all equal, the first
+// positive pair) are the new height and width, -1 keeps an axis.
+class Resize2D : public OperatorOnDevice {
+public:
+    using supper = OperatorOnDevice;
+    Resize2D();
+    void init() override;
+    int run(Stack &stack) override;
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override;
+    // axes dim and dim + 1 of x are resized to those of out
+    virtual void resize2d(const Tensor &x, int dim, Resize2DType type, Tensor &out) = 0;
+
+private:
+    Resize2DType m_type = Resize2DType::LINEAR;
+};
+
 }  // namespace base
 
 // ts::ElementWiseReduce (include/backend/base/element_wise_reduce.h:12-118; src/backend/base/

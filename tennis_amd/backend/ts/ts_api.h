@@ -451,6 +451,7 @@ enum WinogradConv2DMode { F6X6_3X3 = 0, F2X2_3X3 = 1 };
 // include/backend/common_structure.h:84-94
 enum class Pooling2DType : int { MAX = 0, AVG = 1 };
 enum class Padding2DType : int { BLACK = 0, COPY = 1, LOOP = 2, WHITE = 3 };
+enum class Resize2DType : int { LINEAR = 0, CUBIC = 1, NEAREST = 2, HARD = 3 };   // include/backend/common_structure.h:96-101
 // include/backend/common_function.h:14-20 (ceil of an fp32 quotient)
 Size2D pooling2d_forward(const Size2D &x, const Padding2D &padding, const KSize2D &ksize, const Stride2D &stride);
 Size2D conv2d_forward(const Size2D &x, const Padding2D &padding, const KSize2D &ksize, const Stride2D &stride,
@@ -489,6 +490,8 @@ inline const char *add() { return "add"; }
 inline const char *pooling2d() { return "pooling2d"; }
 inline const char *global_pooling2d() { return "global_pooling2d"; }
 inline const char *depthwise_conv2d() { return "depthwise_conv2d"; }
+inline const char *concat() { return "concat"; }
+inline const char *resize2d() { return "_resize2d"; }
 }  // namespace layer
 }  // namespace name
 

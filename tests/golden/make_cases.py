@@ -95,6 +95,11 @@ def main():
               [f32(1, 6, 14, 13), conv_params((1, 1, 1, 1))["padding"], f32(5, 6, 3, 3) * 0.2])
     save_case("pooling2d_v2/avg_3x2", "pooling2d_v2", {"format": "NCHW", "type": np.array([1], np.int32)},
               [x, pad42, np.array([1, 1, 3, 2], np.int32), np.array([1, 1, 2, 1], np.int32)])
+    # layout operators of detection necks
+    save_case("concat/channels", "concat", {"dim": np.array([1], np.int32)}, [x, f32(2, 3, 9, 8), f32(2, 1, 9, 8)])
+    save_case("concat/last_axis", "concat", {"dim": np.array([-1], np.int32)}, [f32(3, 5, 2), f32(3, 5, 7)])
+    save_case("_resize2d/nearest_up", "_resize2d", {"type": np.array([2], np.int32)}, [x, np.array([-1, -1, 18, 16], np.int32)])
+    save_case("_resize2d/nearest_odd", "_resize2d", {"type": np.array([2], np.int32)}, [x, np.array([-1, -1, 13, 5], np.int32)])
     # an operator the "hip" device does not register: the runner reports SKIP, as TenniS's does
     save_case("softmax/not_on_device", "softmax", {"dim": np.array([1], np.int32)}, [f32(3, 5)])
 

@@ -149,3 +149,12 @@ def test_v2_wrappers_in_tennis_workbench(ts):
     assert np.array_equal(bits(cpu), bits(hip))
     cpu, hip = both(ts, "conv2d_winograd_v2", {"format": "NCHW"}, [x, conv_params(ts, (1, 1, 1, 1))["padding"], w], 1 << 20)
     assert np.array_equal(bits(cpu), bits(hip))
+
+
+def test_concat_and_resize2d_in_tennis_workbench(ts):
+    rng = np.random.default_rng(906)
+    a, b = rng.standard_normal((2, 5, 7, 6)).astype(np.float32), rng.standard_normal((2, 3, 7, 6)).astype(np.float32)
+    cpu, hip = both(ts, "concat", {"dim": np.array([1], np.int32)}, [a, b], 1 << 20)
+    assert np.array_equal(bits(cpu), bits(hip))
+    cpu, hip = both(ts, "_resize2d", {"type": np.array([2], np.int32)}, [a, np.array([-1, -1, 14, 12], np.int32)], 1 << 20)
+    assert np.array_equal(bits(cpu), bits(hip))

@@ -216,3 +216,33 @@ def test_v2_operators_equal_their_plain_twins(ops):
         ops.run_op("conv2d_v2", v2, [x, w])
     with pytest.raises(ops.OperatorError):      # stride is required (conv2d_v2.cpp:17)
         ops.run_op("conv2d_v2", {"format": "NCHW"}, [x, full["padding"], w])
+
+
+def test_concat_and_resize2d_operators(ops, port):
+    """concat (any axis, 4-byte elements) and _resize2d (nearest) created by name: exact copies."""
+    rng = np.random.default_rng(508)
+    a, b, c = (rng.standard_normal(s).astype(np.float32) for s in ((2, 5, 7, 6), (2, 3, 7, 6), (2, 1, 7, 6)))
+    got = ops.run_op("concat", {"dim": np.array([1], np.int32)}, [a, b, c])
+    assert np.array_equal(bits(got), bits(np.concatenate([a, b, c], axis=1)))
+    got = ops.run_op("concat", {"dim": np.array([-4], np.int32)}, [a, a])
+    assert np.array_equal(bits(got), bits(np.concatenate([a, a], axis=0)))
+    i1, i2 = rng.integers(-9, 9, (3, 4, 5)).astype(np.int32), rng.integers(-9, 9, (3, 4, 2)).astype(np.int32)
+    got = ops.run_op("concat", {"dim": np.array([2], np.int32)}, [i1, i2])
+    assert got.dtype == np.int32 and np.array_equal(got, np.concatenate([i1, i2], axis=2))
+    assert np.array_equal(ops.run_op("concat", {"dim": np.array([0], np.int32)}, [a]), a)      # one input: itself
+    with pytest.raises(ops.OperatorError, match="Can not concat"):
+        ops.run_op("concat", {"dim": np.array([1], np.int32)}, [a, np.zeros((2, 3, 7, 5), np.float32)])
+    with pytest.raises(ops.OperatorError, match="Can not concat"):
+        ops.run_op("concat", {"dim": np.array([1], np.int32)}, [a, b.astype(np.float64)])
+    with pytest.raises(ops.OperatorError, match="Concat dim must in"):
+        ops.run_op("concat", {"dim": np.array([4], np.int32)}, [a, b])
+    nearest = {"type": np.array([2], np.int32)}
+    for ho, wo in ((14, 12), (9, 11), (7, 6), (3, 13)):
+        size = np.array([-1, -1, ho, wo], np.int32)
+        assert ops.run_op("_resize2d", nearest, [a, size], infer_only=True)[1] == (2, 5, ho, wo)
+        got = ops.run_op("_resize2d", nearest, [a, size])
+        assert np.array_equal(bits(got), bits(port.resize_nearest(a, ho, wo))), (ho, wo)
+    with pytest.raises(ops.OperatorError, match="NEAREST"):
+        ops.run_op("_resize2d", {}, [a, np.array([-1, -1, 14, 12], np.int32)])               # default type is LINEAR
+    with pytest.raises(ops.OperatorError, match="Can not resize"):
+        ops.run_op("_resize2d", nearest, [a, np.array([-1, 4, 0, 12], np.int32)])
