@@ -225,6 +225,17 @@ int tsx_add_broadcast_f32(const float *lhs_dev, const int32_t *lhs_shape, const 
  *                      [1][C][KH][KW] (base_depthwise_conv2d.cpp:11-24), geometry as tsx_conv2d_geom with cout == c;
  *                      optional add_bias + activation fused behind it; same fused-multiply-add order as the reference */
 int tsx_mish_f32(const float *x_dev, int64_t count, float *out_dev, void *stream);
+/* The nodes TenniS graphs compose Mish from, one by one:
+ *   tsx_softplus_f32   cpu::Softplus (src/kernels/cpu/softplus.cpp:30-39): float(log(double(expf(x)) + 1.0))
+ *   tsx_tanh_f32       cpu::Tanh (src/kernels/cpu/tanh.cpp:14-23): 2 * (1 / (1 + expf(-2x))) - 1 in float
+ *   tsx_mul_f32 / tsx_mul_broadcast_f32   cpu::Mul (src/kernels/cpu/mul.cpp) on equal shapes / with the shape
+ *                      alignment of tsx_add_broadcast_f32 above; one IEEE multiplication per element (bit-exact)
+ * expf / log are the device's library routines: softplus and tanh agree with the host's to a few ulp. */
+int tsx_softplus_f32(const float *x_dev, int64_t count, float *out_dev, void *stream);
+int tsx_tanh_f32(const float *x_dev, int64_t count, float *out_dev, void *stream);
+int tsx_mul_f32(const float *a_dev, const float *b_dev, int64_t count, float *out_dev, void *stream);
+int tsx_mul_broadcast_f32(const float *lhs_dev, const int32_t *lhs_shape, const float *rhs_dev, const int32_t *rhs_shape,
+                          int32_t dims, float *out_dev, void *stream);
 int tsx_concat_channels_f32(const float *src_dev, int64_t n, int32_t c_src, int64_t inner, float *dst_dev, int32_t c_dst,
                             int32_t c_offset, void *stream);
 int tsx_resize_nearest_f32(const float *x_dev, int64_t planes, int32_t h, int32_t w, float *out_dev, int32_t out_h,

@@ -73,6 +73,49 @@ private:
     }
 };
 
+// mul: as add, one IEEE multiplication per element.
+class Mul : public OperatorOnHip<base::Mul> {
+public:
+    void reduce_with_same_shape(const Tensor &lhs, const Tensor &rhs, Tensor &out) override {
+        check_type(out);
+        check(tsx_mul_f32(lhs.data<float>(), rhs.data<float>(), out.count(), out.data<float>(), current_stream()), "tsx_mul_f32");
+    }
+
+    void reduce_with_broadcast(const Tensor &lhs, const Tensor &rhs, Tensor &out) override {
+        check_type(out);
+        const Shape &ls = lhs.sizes(), &rs = rhs.sizes();
+        if (ls.size() != rs.size() || ls.size() > 8)
+            TS_LOG_ERROR << "[hip] mul: can not broadcast " << to_string(ls) << " with " << to_string(rs) << eject;
+        const std::vector<int32_t> l(ls.begin(), ls.end()), r(rs.begin(), rs.end());
+        check(tsx_mul_broadcast_f32(lhs.data<float>(), l.data(), rhs.data<float>(), r.data(), int32_t(l.size()), out.data<float>(),
+                                    current_stream()),
+              "tsx_mul_broadcast_f32");
+    }
+
+private:
+    static void check_type(const Tensor &out) {
+        if (out.dtype() != FLOAT32) TS_LOG_ERROR << "[hip] mul not support data type(" << out.dtype() << "): " << type_str(out.dtype()) << eject;
+    }
+};
+
+// softplus and tanh: the two activations (with mul) that TenniS graphs compose Mish from
+// (src/kernels/cpu/softplus.cpp:30-39, tanh.cpp:14-23).
+class Softplus : public OperatorOnHip<base::Activation> {
+public:
+    void active(const Tensor &x, Tensor &out) override {
+        if (x.dtype() != FLOAT32) TS_LOG_ERROR << "[hip] softplus not support data type: " << type_str(x.dtype()) << eject;
+        check(tsx_softplus_f32(x.data<float>(), x.count(), out.data<float>(), current_stream()), "tsx_softplus_f32");
+    }
+};
+
+class Tanh : public OperatorOnHip<base::Activation> {
+public:
+    void active(const Tensor &x, Tensor &out) override {
+        if (x.dtype() != FLOAT32) TS_LOG_ERROR << "[hip] tanh not support data type: " << type_str(x.dtype()) << eject;
+        check(tsx_tanh_f32(x.data<float>(), x.count(), out.data<float>(), current_stream()), "tsx_tanh_f32");
+    }
+};
+
 // depthwise_conv2d: weights [1, C, KH, KW]; the core signature is base::Conv2D's.
 class DepthwiseConv2D : public OperatorOnHip<base::DepthwiseConv2D> {
 public:
@@ -136,6 +179,9 @@ using namespace ts::hip;
 TS_REGISTER_OPERATOR(Pooling2D, ts::hip::DEVICE, name::layer::pooling2d())
 TS_REGISTER_OPERATOR(GlobalPooling2D, ts::hip::DEVICE, name::layer::global_pooling2d())
 TS_REGISTER_OPERATOR(Add, ts::hip::DEVICE, name::layer::add())
+TS_REGISTER_OPERATOR(Mul, ts::hip::DEVICE, name::layer::mul())
+TS_REGISTER_OPERATOR(Softplus, ts::hip::DEVICE, "softplus")
+TS_REGISTER_OPERATOR(Tanh, ts::hip::DEVICE, "tanh")
 TS_REGISTER_OPERATOR(DepthwiseConv2D, ts::hip::DEVICE, name::layer::depthwise_conv2d())
 TS_REGISTER_OPERATOR(Concat, ts::hip::DEVICE, name::layer::concat())
 TS_REGISTER_OPERATOR(Resize2D, ts::hip::DEVICE, name::layer::resize2d())

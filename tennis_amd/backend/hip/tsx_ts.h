@@ -19,6 +19,8 @@
 #endif
 #ifdef TSX_TS_GLUE_OPS
 #include <backend/base/base_add.h>
+#include <backend/base/base_mul.h>
+#include <backend/base/base_activation.h>
 #include <backend/base/base_concat.h>
 #include <backend/base/base_resize2d.h>
 #include <backend/base/base_depthwise_conv2d.h>

@@ -250,5 +250,6 @@ public:
 
 namespace base {
 using Add = ElementWiseReduce;   // include/backend/base/base_add.h:12
+using Mul = ElementWiseReduce;   // include/backend/base/base_mul.h
 }
 }  // namespace ts

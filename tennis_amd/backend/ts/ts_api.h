@@ -491,6 +491,9 @@ inline const char *pooling2d() { return "pooling2d"; }
 inline const char *global_pooling2d() { return "global_pooling2d"; }
 inline const char *depthwise_conv2d() { return "depthwise_conv2d"; }
 inline const char *concat() { return "concat"; }
+inline const char *mul() { return "mul"; }
+inline const char *softplus() { return "softplus"; }
+inline const char *tanh() { return "tanh"; }
 inline const char *resize2d() { return "_resize2d"; }
 }  // namespace layer
 }  // namespace name

@@ -79,6 +79,10 @@ SIGNATURES = {
     "tsx_add_f32": (ctypes.c_int, [_vp, _vp, _i64, _i32, _f32, _vp, _vp]),
     "tsx_add_broadcast_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32, _vp, _vp]),
     "tsx_mish_f32": (ctypes.c_int, [_vp, _i64, _vp, _vp]),
+    "tsx_softplus_f32": (ctypes.c_int, [_vp, _i64, _vp, _vp]),
+    "tsx_tanh_f32": (ctypes.c_int, [_vp, _i64, _vp, _vp]),
+    "tsx_mul_f32": (ctypes.c_int, [_vp, _vp, _i64, _vp, _vp]),
+    "tsx_mul_broadcast_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32, _vp, _vp]),
     "tsx_concat_channels_f32": (ctypes.c_int, [_vp, _i64, _i32, _i64, _vp, _i32, _i32, _vp]),
     "tsx_resize_nearest_f32": (ctypes.c_int, [_vp, _i64, _i32, _i32, _vp, _i32, _i32, _vp]),
     "tsx_depthwise_conv2d_f32": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, _f32, _vp, _i32, _f32, _vp, _vp]),
@@ -487,6 +491,30 @@ def mish(x):
     x = _dev(x, torch.float32)
     out = torch.empty_like(x)
     check(lib().tsx_mish_f32(_ptr(x), x.numel(), _ptr(out), _stream()))
+    return out
+
+
+def softplus(x):
+    x = _dev(x, torch.float32)
+    out = torch.empty_like(x)
+    check(lib().tsx_softplus_f32(_ptr(x), x.numel(), _ptr(out), _stream()))
+    return out
+
+
+def tanh(x):
+    x = _dev(x, torch.float32)
+    out = torch.empty_like(x)
+    check(lib().tsx_tanh_f32(_ptr(x), x.numel(), _ptr(out), _stream()))
+    return out
+
+
+def mul(a, b):
+    """tsx_mul_f32: a * b on equal shapes."""
+    a, b = _dev(a, torch.float32), _dev(b, torch.float32)
+    if a.shape != b.shape:
+        raise TsxError("mul: shapes %s and %s differ" % (tuple(a.shape), tuple(b.shape)))
+    out = torch.empty_like(a)
+    check(lib().tsx_mul_f32(_ptr(a), _ptr(b), a.numel(), _ptr(out), _stream()))
     return out
 
 

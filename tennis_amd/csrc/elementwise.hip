@@ -5,6 +5,11 @@
 //   cpu::LeakyReLU  src/kernels/cpu/leaky_relu.cpp:41-66    body fma(scale, min(x,0), max(x,0)), tail x>0?x:x*scale
 //   cpu::Add        src/kernels/cpu/add.cpp                 y = a + b on equal shapes (a residual join), optionally
 //                                                           followed by the activation operator in the same pass
+//   cpu::Mul        src/kernels/cpu/mul.cpp                 y = a * b, equal shapes or broadcast
+//   cpu::Softplus   src/kernels/cpu/softplus.cpp:30-39      y = float(log(double(expf(x)) + 1.0))
+//   cpu::Tanh       src/kernels/cpu/tanh.cpp:14-23          y = 2 * (1 / (1 + expf(-2x))) - 1 in float
+// (softplus, tanh and mul are the nodes TenniS graphs compose Mish from; expf / log are this device's library
+// routines, so those two agree with the host's to a few ulp, not bit for bit)
 // Each lane handles 4 consecutive elements (16-byte accesses) in a grid-stride loop.
 #include "tsx_common.hpp"
 
@@ -13,7 +18,7 @@ namespace {
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 // MODE 0: add_bias (layout [pre][channels][inner]); 1: relu; 2: leaky_relu; 3: add (second operand in `bias`) + act;
-// 4: mish
+// 4: mish; 5: softplus; 6: tanh; 7: mul (second operand in `bias`)
 template <int MODE>
 __global__ __launch_bounds__(256) void elementwise_kernel(const float *__restrict__ x, int64_t count,
                                                          const float *__restrict__ bias, int channels, int64_t inner,
@@ -27,13 +32,13 @@ __global__ __launch_bounds__(256) void elementwise_kernel(const float *__restric
         if (full) {
             const v4f in = *reinterpret_cast<const v4f *>(x + base);
             v[0] = in[0]; v[1] = in[1]; v[2] = in[2]; v[3] = in[3];
-            if (MODE == 3) {
+            if (MODE == 3 || MODE == 7) {
                 const v4f in2 = *reinterpret_cast<const v4f *>(bias + base);
                 u[0] = in2[0]; u[1] = in2[1]; u[2] = in2[2]; u[3] = in2[3];
             }
         } else {
             for (int j = 0; j < 4; ++j) v[j] = base + j < count ? x[base + j] : 0.f;
-            if (MODE == 3)
+            if (MODE == 3 || MODE == 7)
                 for (int j = 0; j < 4; ++j) u[j] = base + j < count ? bias[base + j] : 0.f;
         }
         // add_bias: a lane's four elements share their channel when the inner extent is a multiple of 4 (one
@@ -53,6 +58,12 @@ __global__ __launch_bounds__(256) void elementwise_kernel(const float *__restric
                 v[j] = tsx::apply_act(__fadd_rn(v[j], u[j]), act, slope, i < body);
             } else if (MODE == 4) {
                 v[j] = tsx::apply_act(v[j], TSX_ACT_MISH, 0.f, true);
+            } else if (MODE == 5) {
+                v[j] = float(log(double(expf(v[j])) + 1.0));
+            } else if (MODE == 6) {
+                v[j] = __fsub_rn(__fmul_rn(2.f, __fdiv_rn(1.f, __fadd_rn(1.f, expf(-__fmul_rn(2.f, v[j]))))), 1.f);
+            } else if (MODE == 7) {
+                v[j] = __fmul_rn(v[j], u[j]);
             } else {
                 v[j] = tsx::apply_act(v[j], MODE == 1 ? TSX_ACT_RELU : TSX_ACT_LEAKY_RELU, slope, i < body);
             }
@@ -73,7 +84,7 @@ int launch(const float *x, int64_t count, const float *bias, int channels, int64
     if (count == 0) return 0;
     TSX_REQUIRE(x && out, "elementwise: null pointer");
     const bool vec = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
-                     (MODE != 3 || reinterpret_cast<uintptr_t>(bias) % 16 == 0);
+                     ((MODE != 3 && MODE != 7) || reinterpret_cast<uintptr_t>(bias) % 16 == 0);
     int64_t blocks = tsx::ceil_div(tsx::ceil_div(count, 4), 256);
     if (blocks > 256 * 8) blocks = 256 * 8;
     hipLaunchKernelGGL(elementwise_kernel<MODE>, dim3(unsigned(blocks)), dim3(256), 0, tsx::as_stream(stream), x, count,
@@ -82,14 +93,15 @@ int launch(const float *x, int64_t count, const float *bias, int channels, int64
     return 0;
 }
 
-// out = lhs + rhs with numpy-style broadcasting over up to 8 aligned axes (an extent of 1 repeats).
+// out = lhs + rhs (MUL: lhs * rhs) with numpy-style broadcasting over up to 8 aligned axes (an extent of 1 repeats).
 // One lane per output element; an operand's stride is 0 on the axes it is broadcast along.
 struct BroadcastGeom {
     int out_shape[8];   // right-aligned; leading unused axes have extent 1
     int64_t lhs_stride[8], rhs_stride[8];
 };
 
-__global__ __launch_bounds__(256) void add_broadcast_kernel(const float *__restrict__ lhs, const float *__restrict__ rhs,
+template <bool MUL>
+__global__ __launch_bounds__(256) void broadcast_kernel(const float *__restrict__ lhs, const float *__restrict__ rhs,
                                                            BroadcastGeom g, int64_t count, float *__restrict__ out) {
     const int64_t stride = int64_t(gridDim.x) * blockDim.x;
     for (int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += stride) {
@@ -102,8 +114,35 @@ __global__ __launch_bounds__(256) void add_broadcast_kernel(const float *__restr
             lo += c * g.lhs_stride[d];
             ro += c * g.rhs_stride[d];
         }
-        out[i] = __fadd_rn(lhs[lo], rhs[ro]);
+        out[i] = MUL ? __fmul_rn(lhs[lo], rhs[ro]) : __fadd_rn(lhs[lo], rhs[ro]);
     }
+}
+
+template <bool MUL>
+int launch_broadcast(const char *who, const float *lhs_dev, const int32_t *lhs_shape, const float *rhs_dev, const int32_t *rhs_shape,
+                     int32_t dims, float *out_dev, void *stream) {
+    TSX_REQUIRE(dims >= 1 && dims <= 8 && lhs_shape && rhs_shape, "%s: 1..8 axes, got %d", who, dims);
+    BroadcastGeom g{};
+    for (int d = 0; d < 8; ++d) g.out_shape[d] = 1;
+    int64_t count = 1, ls = 1, rs = 1;
+    for (int d = dims - 1; d >= 0; --d) {
+        const int l = lhs_shape[d], r = rhs_shape[d];
+        TSX_REQUIRE(l >= 0 && r >= 0 && (l == r || l == 1 || r == 1), "%s: axis %d: %d vs %d", who, d, l, r);
+        const int slot = d + 8 - dims;
+        g.out_shape[slot] = l == 1 ? r : l;
+        g.lhs_stride[slot] = l == 1 ? 0 : ls;
+        g.rhs_stride[slot] = r == 1 ? 0 : rs;
+        ls *= l;
+        rs *= r;
+        count *= g.out_shape[slot];
+    }
+    if (count == 0) return 0;
+    TSX_REQUIRE(lhs_dev && rhs_dev && out_dev, "%s: null pointer", who);
+    const int64_t blocks = (count + 255) / 256;
+    hipLaunchKernelGGL(broadcast_kernel<MUL>, dim3(unsigned(blocks < 8192 ? blocks : 8192)), dim3(256), 0, tsx::as_stream(stream),
+                       lhs_dev, rhs_dev, g, count, out_dev);
+    TSX_LAUNCH_CHECK("broadcast_kernel");
+    return 0;
 }
 
 }  // namespace
@@ -135,28 +174,27 @@ int tsx_add_f32(const float *a_dev, const float *b_dev, int64_t count, int32_t a
 
 int tsx_add_broadcast_f32(const float *lhs_dev, const int32_t *lhs_shape, const float *rhs_dev, const int32_t *rhs_shape,
                           int32_t dims, float *out_dev, void *stream) {
-    TSX_REQUIRE(dims >= 1 && dims <= 8 && lhs_shape && rhs_shape, "add_broadcast: 1..8 axes, got %d", dims);
-    BroadcastGeom g{};
-    for (int d = 0; d < 8; ++d) g.out_shape[d] = 1;
-    int64_t count = 1, ls = 1, rs = 1;
-    for (int d = dims - 1; d >= 0; --d) {
-        const int l = lhs_shape[d], r = rhs_shape[d];
-        TSX_REQUIRE(l >= 0 && r >= 0 && (l == r || l == 1 || r == 1), "add_broadcast: axis %d: %d vs %d", d, l, r);
-        const int slot = d + 8 - dims;
-        g.out_shape[slot] = l == 1 ? r : l;
-        g.lhs_stride[slot] = l == 1 ? 0 : ls;
-        g.rhs_stride[slot] = r == 1 ? 0 : rs;
-        ls *= l;
-        rs *= r;
-        count *= g.out_shape[slot];
-    }
-    if (count == 0) return 0;
-    TSX_REQUIRE(lhs_dev && rhs_dev && out_dev, "add_broadcast: null pointer");
-    const int64_t blocks = (count + 255) / 256;
-    hipLaunchKernelGGL(add_broadcast_kernel, dim3(unsigned(blocks < 8192 ? blocks : 8192)), dim3(256), 0, tsx::as_stream(stream),
-                       lhs_dev, rhs_dev, g, count, out_dev);
-    TSX_LAUNCH_CHECK("add_broadcast_kernel");
-    return 0;
+    return launch_broadcast<false>("add_broadcast", lhs_dev, lhs_shape, rhs_dev, rhs_shape, dims, out_dev, stream);
+}
+
+int tsx_mul_f32(const float *a_dev, const float *b_dev, int64_t count, float *out_dev, void *stream) {
+    TSX_REQUIRE(count >= 0 && (count == 0 || b_dev), "mul: bad argument");
+    return launch<7>(a_dev, count, b_dev, 1, 1, 0.f, out_dev, stream);
+}
+
+int tsx_mul_broadcast_f32(const float *lhs_dev, const int32_t *lhs_shape, const float *rhs_dev, const int32_t *rhs_shape,
+                          int32_t dims, float *out_dev, void *stream) {
+    return launch_broadcast<true>("mul_broadcast", lhs_dev, lhs_shape, rhs_dev, rhs_shape, dims, out_dev, stream);
+}
+
+int tsx_softplus_f32(const float *x_dev, int64_t count, float *out_dev, void *stream) {
+    TSX_REQUIRE(count >= 0, "softplus: negative count");
+    return launch<5>(x_dev, count, nullptr, 1, 1, 0.f, out_dev, stream);
+}
+
+int tsx_tanh_f32(const float *x_dev, int64_t count, float *out_dev, void *stream) {
+    TSX_REQUIRE(count >= 0, "tanh: negative count");
+    return launch<6>(x_dev, count, nullptr, 1, 1, 0.f, out_dev, stream);
 }
 
 int tsx_mish_f32(const float *x_dev, int64_t count, float *out_dev, void *stream) {

@@ -100,6 +100,11 @@ def main():
     save_case("concat/last_axis", "concat", {"dim": np.array([-1], np.int32)}, [f32(3, 5, 2), f32(3, 5, 7)])
     save_case("_resize2d/nearest_up", "_resize2d", {"type": np.array([2], np.int32)}, [x, np.array([-1, -1, 18, 16], np.int32)])
     save_case("_resize2d/nearest_odd", "_resize2d", {"type": np.array([2], np.int32)}, [x, np.array([-1, -1, 13, 5], np.int32)])
+    # the nodes graphs compose Mish from
+    save_case("softplus/4d", "softplus", {}, [x * 3])
+    save_case("tanh/4d", "tanh", {}, [x * 2])
+    save_case("mul/broadcast", "mul", {}, [x, f32(1, 6, 1, 1)])
+    save_case("mul/same_shape", "mul", {}, [x, f32(2, 6, 9, 8)])
     # an operator the "hip" device does not register: the runner reports SKIP, as TenniS's does
     save_case("softmax/not_on_device", "softmax", {"dim": np.array([1], np.int32)}, [f32(3, 5)])
 

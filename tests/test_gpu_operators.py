@@ -246,3 +246,27 @@ def test_concat_and_resize2d_operators(ops, port):
         ops.run_op("_resize2d", {}, [a, np.array([-1, -1, 14, 12], np.int32)])               # default type is LINEAR
     with pytest.raises(ops.OperatorError, match="Can not resize"):
         ops.run_op("_resize2d", nearest, [a, np.array([-1, 4, 0, 12], np.int32)])
+
+
+def test_mish_composition_operators(ops, port):
+    """softplus, tanh and mul -- the nodes TenniS graphs compose Mish from.  mul is one IEEE multiplication per
+    element (bitwise); softplus and tanh use the device's expf / log: a few ulp from the host's, checked to
+    1e-6 relative + 1e-6 absolute against the oracle, and the composition equals the fused Mish kernel bit for bit."""
+    from tennis_amd import capi
+    rng = np.random.default_rng(509)
+    x = (rng.standard_normal((2, 5, 13, 11)) * 4).astype(np.float32)
+    x.flat[:6] = [0.0, -0.0, 30.0, -30.0, 88.0, -88.0]
+    sp = ops.run_op("softplus", {}, [x])
+    assert np.allclose(sp, port.softplus(x), rtol=1e-6, atol=1e-6)
+    th = ops.run_op("tanh", {}, [x])
+    assert np.allclose(th, port.tanh(x), rtol=1e-6, atol=1e-6)
+    b = rng.standard_normal((1, 5, 1, 1)).astype(np.float32)
+    for lhs, rhs in ((x, x[::-1].copy()), (x, b), (b, x), (x, np.float32([2.5]))):
+        got = ops.run_op("mul", {}, [lhs, rhs])
+        assert np.array_equal(bits(got), bits(lhs * rhs))
+    mish = ops.run_op("mul", {}, [x, ops.run_op("tanh", {}, [sp])])
+    import torch
+    fused = capi.mish(torch.from_numpy(x).cuda()).cpu().numpy()
+    assert np.array_equal(bits(mish), bits(fused))
+    with pytest.raises(ops.OperatorError):
+        ops.run_op("softplus", {}, [x.astype(np.float64)])
