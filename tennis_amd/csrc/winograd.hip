@@ -158,15 +158,19 @@ __global__ __launch_bounds__(256) void wino_input_transform_kernel(const float *
 
 // C[b][m][n] = A[b % a_batches][m][k] * B[b][k][n] in the reference's accumulation order
 // (math_cpu.cpp:386-700 as restated by the CPU oracle): m8/n8 = extents rounded down to 8.
+// Columns below n8 are one fused-multiply-add chain in ascending k per output; the columns from n8 on sum four
+// interleaved partial chains first.  Two kernels: the tiled one for the columns below n8, this one (one lane per
+// output, columns j0..n) for the rest.
 __global__ __launch_bounds__(256) void gemm_f32_seq_kernel(const float *__restrict__ a, const float *__restrict__ b,
                                                           float *__restrict__ c, int m, int n, int k, int batches,
-                                                          int a_batches) {
-    const int64_t total = int64_t(batches) * m * n;
+                                                          int a_batches, int j0) {
+    const int cols = n - j0;
+    const int64_t total = int64_t(batches) * m * cols;
     const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
     if (id >= total) return;
-    const int j = int(id % n);
-    const int i = int((id / n) % m);
-    const int bt = int(id / n / m);
+    const int j = j0 + int(id % cols);
+    const int i = int((id / cols) % m);
+    const int bt = int(id / cols / m);
     const float *ar = a + (int64_t(bt % a_batches) * m + i) * k;
     const float *bc = b + int64_t(bt) * k * n + j;
     const int m8 = m / 8 * 8, n8 = n / 8 * 8, k4 = k / 4 * 4;
@@ -194,7 +198,98 @@ __global__ __launch_bounds__(256) void gemm_f32_seq_kernel(const float *__restri
         for (int kk = k4; kk < k; ++kk) acc = fmaf(ar[kk], bc[int64_t(kk) * n], acc);
         r = acc;
     }
-    c[id] = r;
+    c[(int64_t(bt) * m + i) * n + j] = r;
+}
+
+// The columns below n8: every output is the same chain acc = fma(B[k][j], A[i][k], acc) over ascending k, so a
+// lane can hold a 4 x 4 block of outputs and feed 16 chains from 4 values of A and 4 of B per k -- an eighth of
+// the loads of one lane per output, the same bits.  VEC: k and n multiples of 4 and 16-byte aligned operands, so
+// A is read four k at a time and B four columns at a time as 16-byte loads.  Lanes run along the column blocks.
+template <bool VEC>
+__global__ __launch_bounds__(256) void gemm_f32_seq_tiled_kernel(const float *__restrict__ a, const float *__restrict__ b,
+                                                                float *__restrict__ c, int m, int n, int k, int batches,
+                                                                int a_batches, int n8) {
+    const int jb = n8 / 4, ib = (m + 3) / 4;
+    const int64_t total = int64_t(batches) * ib * jb;
+    const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id >= total) return;
+    const int j = int(id % jb) * 4;
+    const int i = int((id / jb) % ib) * 4;
+    const int bt = int(id / jb / ib);
+    const float *ab = a + int64_t(bt % a_batches) * m * k;
+    const float *bc = b + int64_t(bt) * k * n + j;
+    const float *ar[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) ar[r] = ab + int64_t(min(i + r, m - 1)) * k;   // rows past m: computed, not stored
+    float acc[4][4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[r][q] = 0.f;
+    int kk = 0;
+    if (VEC) {
+        for (; kk + 4 <= k; kk += 4) {
+            float4 av[4], bv[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) av[r] = *reinterpret_cast<const float4 *>(ar[r] + kk);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) bv[t] = *reinterpret_cast<const float4 *>(bc + int64_t(kk + t) * n);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float av_t = t == 0 ? av[r].x : t == 1 ? av[r].y : t == 2 ? av[r].z : av[r].w;
+                    acc[r][0] = fmaf(bv[t].x, av_t, acc[r][0]);
+                    acc[r][1] = fmaf(bv[t].y, av_t, acc[r][1]);
+                    acc[r][2] = fmaf(bv[t].z, av_t, acc[r][2]);
+                    acc[r][3] = fmaf(bv[t].w, av_t, acc[r][3]);
+                }
+            }
+        }
+    }
+    for (; kk < k; ++kk) {
+        float bv[4], av[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) bv[q] = bc[int64_t(kk) * n + q];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) av[r] = ar[r][kk];
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc[r][q] = fmaf(bv[q], av[r], acc[r][q]);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        if (i + r >= m) break;
+        float *dst = c + (int64_t(bt) * m + i + r) * n + j;
+        if (VEC) *reinterpret_cast<float4 *>(dst) = make_float4(acc[r][0], acc[r][1], acc[r][2], acc[r][3]);
+        else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) dst[q] = acc[r][q];
+        }
+    }
+}
+
+// Both parts of the sequential-order GEMM on `stream`.
+int launch_gemm_f32_seq(const float *a, const float *b, float *c, int m, int n, int k, int batches, int a_batches,
+                        hipStream_t stream) {
+    const int n8 = n / 8 * 8;
+    if (n8 > 0) {
+        const int64_t threads = int64_t(batches) * ((m + 3) / 4) * (n8 / 4);
+        const bool vec = k % 4 == 0 && n % 4 == 0 && reinterpret_cast<uintptr_t>(a) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(b) % 16 == 0 && reinterpret_cast<uintptr_t>(c) % 16 == 0;
+        const dim3 grid(unsigned(ceil_div(threads, 256)));
+        if (vec) hipLaunchKernelGGL(gemm_f32_seq_tiled_kernel<true>, grid, dim3(256), 0, stream, a, b, c, m, n, k, batches, a_batches, n8);
+        else hipLaunchKernelGGL(gemm_f32_seq_tiled_kernel<false>, grid, dim3(256), 0, stream, a, b, c, m, n, k, batches, a_batches, n8);
+        TSX_LAUNCH_CHECK("gemm_f32_seq_tiled_kernel");
+    }
+    if (n8 < n) {
+        const int64_t threads = int64_t(batches) * m * (n - n8);
+        hipLaunchKernelGGL(gemm_f32_seq_kernel, dim3(unsigned(ceil_div(threads, 256))), dim3(256), 0, stream, a, b, c, m, n, k,
+                           batches, a_batches, n8);
+        TSX_LAUNCH_CHECK("gemm_f32_seq_kernel");
+    }
+    return 0;
 }
 
 // One thread per (image, cout, tile): Y = A^T M A, cut to the true output, then the optional
@@ -422,10 +517,7 @@ int tsx_conv2d_winograd_f63_nchw(const tsx_conv2d_geom *q, const float *x_dev, c
     TSX_LAUNCH_CHECK("wino_input_transform_kernel");
 
     const int batches = g.n * 64;
-    const int64_t gemm_threads = int64_t(batches) * g.cout * g.tiles;
-    hipLaunchKernelGGL(tsx::gemm_f32_seq_kernel, dim3(unsigned(tsx::ceil_div(gemm_threads, 256))), dim3(256), 0, stream,
-                       u_dev, v, mm, g.cout, g.tiles, g.c, batches, 64);
-    TSX_LAUNCH_CHECK("gemm_f32_seq_kernel");
+    if (int rc = tsx::launch_gemm_f32_seq(u_dev, v, mm, g.cout, g.tiles, g.c, batches, 64, stream)) return rc;
 
     const int64_t out_threads = int64_t(g.n) * g.cout * g.tiles;
     const int64_t count = int64_t(g.n) * g.cout * g.ho * g.wo;
@@ -476,10 +568,7 @@ int tsx_conv2d_winograd_f23_nchw(const tsx_conv2d_geom *q, const float *x_dev, c
     TSX_LAUNCH_CHECK("wino23_input_transform_kernel");
 
     const int batches = g.n * 16;
-    const int64_t gemm_threads = int64_t(batches) * g.cout * g.tiles;
-    hipLaunchKernelGGL(tsx::gemm_f32_seq_kernel, dim3(unsigned(tsx::ceil_div(gemm_threads, 256))), dim3(256), 0, stream,
-                       u_dev, v, mm, g.cout, g.tiles, g.c, batches, 16);
-    TSX_LAUNCH_CHECK("gemm_f32_seq_kernel");
+    if (int rc = tsx::launch_gemm_f32_seq(u_dev, v, mm, g.cout, g.tiles, g.c, batches, 16, stream)) return rc;
 
     const int64_t out_threads = int64_t(g.n) * g.cout * g.tiles;
     const int64_t count = int64_t(g.n) * g.cout * g.ho * g.wo;
