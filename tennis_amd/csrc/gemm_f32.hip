@@ -27,6 +27,8 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 constexpr int KC = 32;          // K per staged chunk
 constexpr int THREADS = 256;
 
+constexpr int MAX_SLOTS = 8;    // B elements a thread fetches per chunk (KC * BN / THREADS at BN = 64)
+
 // B operand = implicit im2col of an NCHW tensor (src/kernels/cpu/im2col.cpp:37-111).
 struct ConvLoader {
     const float *x;
@@ -46,15 +48,33 @@ struct ConvLoader {
         h0 = ho * stride_h - pad_top;
         w0 = wo_ * stride_w - pad_left;
     }
-    __device__ __forceinline__ float load(int k, int kdim) const {
-        if (!col_ok || k >= kdim) return 0.f;
+    // A thread fetches the same few rows k of every staged chunk, KC further each time: row k is kept as
+    // (input channel, tap) and stepped, so the K loop has no division (tap -> kernel row / column is a
+    // multiply-shift, exact for the tap counts of any real kernel).
+    int slot_ci[MAX_SLOTS], slot_tap[MAX_SLOTS], slot_k[MAX_SLOTS];
+    __device__ __forceinline__ void init_slot(int i, int k) {
         const int khw = kh * kw;
-        const int ci = k / khw;
-        const int rem = k - ci * khw;
-        const int r = rem / kw, s = rem - r * kw;
+        slot_k[i] = k;
+        slot_ci[i] = k / khw;
+        slot_tap[i] = k - slot_ci[i] * khw;
+    }
+    __device__ __forceinline__ void advance_slot(int i, int step) {
+        const int khw = kh * kw;
+        slot_k[i] += step;
+        slot_ci[i] += step / khw;
+        slot_tap[i] += step % khw;
+        if (slot_tap[i] >= khw) {
+            slot_tap[i] -= khw;
+            ++slot_ci[i];
+        }
+    }
+    __device__ __forceinline__ float load_slot(int i, int kdim) const {
+        if (!col_ok || slot_k[i] >= kdim) return 0.f;
+        const int inv_kw = (65536 + kw - 1) / kw;
+        const int r = (slot_tap[i] * inv_kw) >> 16, s = slot_tap[i] - r * kw;
         const int hh = h0 + r * dil_h, ww = w0 + s * dil_w;
         if (hh < 0 || hh >= h || ww < 0 || ww >= w) return padding_value;
-        return img[(int64_t(ci) * h + hh) * w + ww];
+        return img[(int64_t(slot_ci[i]) * h + hh) * w + ww];
     }
 };
 
@@ -68,9 +88,12 @@ struct MatLoader {
         col_ok = col < ncols;
         colp = b + int64_t(col_ok ? col : 0) * ld_n;
     }
-    __device__ __forceinline__ float load(int k, int kdim) const {
-        if (!col_ok || k >= kdim) return 0.f;
-        return colp[int64_t(k) * ld_k];
+    int slot_k[MAX_SLOTS];
+    __device__ __forceinline__ void init_slot(int i, int k) { slot_k[i] = k; }
+    __device__ __forceinline__ void advance_slot(int i, int step) { slot_k[i] += step; }
+    __device__ __forceinline__ float load_slot(int i, int kdim) const {
+        if (!col_ok || slot_k[i] >= kdim) return 0.f;
+        return colp[int64_t(slot_k[i]) * ld_k];
     }
 };
 
@@ -104,8 +127,13 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmArgs g, Loader ld
     const float *a = g.a + batch * g.a_batch;
     if constexpr (std::is_same<Loader, MatLoader>::value) ld.b += batch * g.b_batch;
 
+    static_assert(B_PER <= MAX_SLOTS, "more B elements per thread than loader slots");
     ld.set_column(n0 + tid % BN, g.n);
     const int b_krow = tid / BN;                    // this thread's first k row of the B tile
+    static_for<0, B_PER>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        ld.init_slot(i, b_krow + i * (THREADS / BN));
+    });
 
     v16f acc;
     static_for<0, 16>([&](auto rc) { acc[decltype(rc)::value] = 0.f; });
@@ -119,9 +147,10 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmArgs g, Loader ld
             const bool ok = m0 + mm < g.m && k0 + kk < g.k;
             a_reg[i] = ok ? a[int64_t(m0 + mm) * g.k + k0 + kk] : 0.f;
         });
-        static_for<0, B_PER>([&](auto ic) {
+        static_for<0, B_PER>([&](auto ic) {      // chunks are fetched in ascending order: the slots step with them
             constexpr int i = decltype(ic)::value;
-            b_reg[i] = ld.load(k0 + b_krow + i * (THREADS / BN), g.k);
+            b_reg[i] = ld.load_slot(i, g.k);
+            ld.advance_slot(i, KC);
         });
     };
     auto store_chunk = [&]() __attribute__((always_inline)) {
