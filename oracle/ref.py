@@ -139,6 +139,19 @@ def load_tensor(path, max_bytes=1 << 24):
     return out.dtype, buf[:out.bytes].view(np_type).reshape(shape).copy()
 
 
+def run_module(path, inputs, out_bytes=1 << 24, device="cpu", threads=1):
+    """Load a `.tsm` file with the reference's own Module::Load, run it in a Workbench; returns output 0."""
+    keep = []
+    i = (_Tensor * max(len(inputs), 1))(*[_pack("", v, keep) for v in inputs])
+    buf = np.empty(out_bytes, dtype=np.uint8)
+    out = _Output()
+    out.data = buf.ctypes.data
+    out.capacity = out_bytes
+    _check(lib().ref_run_module(str(path).encode(), device.encode(), len(inputs), i, int(threads), ctypes.byref(out)))
+    shape = tuple(out.shape[k] for k in range(out.ndim))
+    return buf[:out.bytes].view(_TS2NP[out.dtype]).reshape(shape).copy()
+
+
 def _conv_params(pads, strides, dilations, padding_value=0.0):
     return {
         "format": "NCHW",

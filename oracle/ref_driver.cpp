@@ -22,6 +22,7 @@
 
 #include "runtime/workbench.h"
 #include "module/bubble.h"
+#include "module/module.h"
 #include "core/tensor.h"
 #include "core/tensor_builder.h"
 #include "backend/common_structure.h"
@@ -172,6 +173,26 @@ int ref_load_tensor(const char *path, ref_output *out) {
     return guarded([&] {
         ts::Tensor y = ts::tensor::load(path);
         if (y.fields_count() != 1) throw std::runtime_error("packed tensors are not supported by this driver");
+        out->dtype = int32_t(y.dtype());
+        out->ndim = int32_t(y.dims());
+        for (int i = 0; i < out->ndim && i < 8; ++i) out->shape[i] = y.size(i);
+        out->bytes = int64_t(y.count()) * ts::type_bytes(y.dtype());
+        if (out->bytes > out->capacity) throw std::runtime_error("output buffer too small");
+        std::memcpy(out->data, y.data(), size_t(out->bytes));
+    });
+}
+
+// A module file (`.tsm`, Module::Load, src/module/module.cpp:295-330) loaded into a Workbench of the named
+// computing device and run once: the reference's own reader, graph compiler and runtime, to cross-check an
+// independent reader / writer / runner of the format.  Copies output slot 0 back.
+int ref_run_module(const char *path, const char *device, int ninputs, const ref_tensor *inputs, int threads, ref_output *out) {
+    return guarded([&] {
+        auto module = ts::Module::Load(path);
+        auto bench = ts::Workbench::Load(module, ts::ComputingDevice(device, 0));
+        bench->runtime().set_computing_thread_number(threads);
+        for (int i = 0; i < ninputs; ++i) bench->input(i, make_tensor(inputs[i]));
+        bench->run();
+        ts::Tensor y = bench->output(0).view(ts::MemoryDevice(ts::CPU));
         out->dtype = int32_t(y.dtype());
         out->ndim = int32_t(y.dims());
         for (int i = 0; i < out->ndim && i < 8; ++i) out->shape[i] = y.size(i);

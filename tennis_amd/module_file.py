@@ -1,0 +1,179 @@
+"""TenniS module files (`.tsm`): reader, writer and an operator-by-operator runner on device "hip".
+
+Format (doc/zh_CN/module.md section 4; Module::Save / Module::Load, src/module/module.cpp:236-320; nodes
+src/module/menu.cpp:88-122; parameters src/module/bubble.cpp:140-189), all little-endian:
+
+    header   uint32 fake, uint32 code = 0x19910929, 120 reserved bytes
+    inputs   uint32 n, uint32 node index * n
+    outputs  uint32 n, uint32 node index * n
+    graph    uint32 n, then per node:
+               bubble   uint32 params, per parameter: uint32 name length, name, a packed tensor (tensor_file)
+               inputs   uint32 n, uint32 node index * n
+
+A node's operator and name are the retention parameters "#op" and "#name"; "<param>" nodes are the module's
+inputs, "<const>" nodes carry their tensor in parameter "value".
+
+`run_module` evaluates the graph in dependency order, one `operators.run_op` per node, on the device's own
+operator classes: it is the counterpart of loading the module into a Workbench of ComputingDevice("hip"), without
+TenniS's graph compiler (no operator fusion, no constant folding; every node must be an operator the device
+registers -- there is no host fallback).
+"""
+import struct
+
+import numpy as np
+
+from . import operators, tensor_file
+
+MODULE_CODE_V1 = 0x19910929
+PARAMETER, CONST = "<param>", "<const>"
+
+
+class ModuleFileError(ValueError):
+    pass
+
+
+class Node:
+    def __init__(self, op, name, params=None, inputs=()):
+        self.op, self.name = op, name
+        self.params = dict(params or {})   # without the "#op" / "#name" retention parameters
+        self.inputs = list(inputs)         # node indices
+
+    def __repr__(self):
+        return "Node(%r, %r, inputs=%r)" % (self.op, self.name, self.inputs)
+
+
+class Module:
+    def __init__(self, nodes, inputs, outputs):
+        self.nodes, self.inputs, self.outputs = list(nodes), list(inputs), list(outputs)
+
+
+def _u32(buf, pos, what):
+    if pos + 4 > len(buf):
+        raise ModuleFileError("truncated module file: %s at offset %d" % (what, pos))
+    return struct.unpack_from("<I", buf, pos)[0], pos + 4
+
+
+def _index_list(buf, pos, what, limit=None):
+    n, pos = _u32(buf, pos, what)
+    out = []
+    for _ in range(n):
+        v, pos = _u32(buf, pos, what)
+        if limit is not None and v >= limit:
+            raise ModuleFileError("%s: node index %d out of range (%d nodes)" % (what, v, limit))
+        out.append(v)
+    return out, pos
+
+
+def _packed_tensor(buf, pos):
+    """One serialized (packed) tensor starting at pos; returns (value, end)."""
+    fields, p = _u32(buf, pos, "tensor field count")
+    for _ in range(fields):
+        if p + 5 > len(buf):
+            raise ModuleFileError("truncated module file: tensor prototype at offset %d" % p)
+        code, ndims = struct.unpack_from("<BI", buf, p)
+        p += 5
+        if p + 4 * ndims > len(buf):
+            raise ModuleFileError("truncated module file: tensor sizes at offset %d" % p)
+        shape = struct.unpack_from("<%dI" % ndims, buf, p)
+        p += 4 * ndims
+        if code not in tensor_file._TS2NP:
+            raise ModuleFileError("tensor dtype code %d has no fixed-size element" % code)
+        p += int(np.prod(shape, dtype=np.int64)) * np.dtype(tensor_file._TS2NP[code]).itemsize
+    if p > len(buf):
+        raise ModuleFileError("truncated module file: tensor data runs past the end")
+    vals = [tensor_file._value(c, a) for c, a in tensor_file.parse_fields(bytes(buf[pos:p]))]
+    return (vals[0] if len(vals) == 1 else vals), p
+
+
+def parse_module(buf):
+    if len(buf) < 128:
+        raise ModuleFileError("truncated module file: no header")
+    _, code = struct.unpack_from("<II", buf, 0)
+    if code != MODULE_CODE_V1:
+        raise ModuleFileError("module code 0x%08x is not format V1 (0x%08x)" % (code, MODULE_CODE_V1))
+    pos = 128
+    inputs, pos = _index_list(buf, pos, "module inputs")
+    outputs, pos = _index_list(buf, pos, "module outputs")
+    count, pos = _u32(buf, pos, "node count")
+    nodes = []
+    for i in range(count):
+        nparams, pos = _u32(buf, pos, "parameter count of node %d" % i)
+        params = {}
+        for _ in range(nparams):
+            n, pos = _u32(buf, pos, "parameter name length")
+            if pos + n > len(buf):
+                raise ModuleFileError("truncated module file: parameter name at offset %d" % pos)
+            name = bytes(buf[pos:pos + n]).decode()
+            pos += n
+            params[name], pos = _packed_tensor(buf, pos)
+        node_inputs, pos = _index_list(buf, pos, "inputs of node %d" % i, count)
+        if "#op" not in params or "#name" not in params:
+            raise ModuleFileError("node %d has no #op / #name" % i)
+        nodes.append(Node(params.pop("#op"), params.pop("#name"), params, node_inputs))
+    for what, idx in (("input", inputs), ("output", outputs)):
+        for v in idx:
+            if v >= count:
+                raise ModuleFileError("module %s index %d out of range (%d nodes)" % (what, v, count))
+    if pos != len(buf):
+        raise ModuleFileError("%d bytes behind the graph" % (len(buf) - pos))
+    return Module(nodes, inputs, outputs)
+
+
+def read_module(path):
+    with open(path, "rb") as fh:
+        return parse_module(fh.read())
+
+
+def serialize_module(module):
+    out = [struct.pack("<II", 0, MODULE_CODE_V1), bytes(120)]
+    for idx in (module.inputs, module.outputs):
+        out.append(struct.pack("<I%dI" % len(idx), len(idx), *idx))
+    out.append(struct.pack("<I", len(module.nodes)))
+    for node in module.nodes:
+        params = dict(node.params)
+        params["#op"], params["#name"] = node.op, node.name
+        out.append(struct.pack("<I", len(params)))
+        for name in sorted(params):          # TenniS keeps parameters in an ordered map
+            raw = name.encode()
+            out.append(struct.pack("<I", len(raw)) + raw + tensor_file.serialize(params[name]))
+        out.append(struct.pack("<I%dI" % len(node.inputs), len(node.inputs), *node.inputs))
+    return b"".join(out)
+
+
+def write_module(path, module):
+    with open(path, "wb") as fh:
+        fh.write(serialize_module(module))
+
+
+def run_module(module, feeds, device="hip", device_id=0):
+    """Outputs of ``module`` for ``feeds`` (one array per module input, in the module's input order)."""
+    if len(feeds) != len(module.inputs):
+        raise ModuleFileError("module has %d inputs, %d fed" % (len(module.inputs), len(feeds)))
+    values = {i: np.asarray(v) for i, v in zip(module.inputs, feeds)}
+    entered = set()              # nodes whose inputs are being evaluated (cycle detection)
+    stack = list(reversed(module.outputs))
+    while stack:                 # depth-first without recursion: graphs are hundreds of nodes deep
+        i = stack[-1]
+        if i in values:
+            stack.pop()
+            continue
+        node = module.nodes[i]
+        if node.op == PARAMETER:
+            raise ModuleFileError("input node %r (%d) is not among the module's inputs" % (node.name, i))
+        if node.op == CONST:
+            if "value" not in node.params:
+                raise ModuleFileError("<const> node %r has no value" % node.name)
+            values[i] = np.asarray(node.params["value"])
+            stack.pop()
+            continue
+        missing = [j for j in node.inputs if j not in values]
+        if missing:
+            if i in entered:
+                raise ModuleFileError("the graph has a cycle through node %d" % i)
+            entered.add(i)
+            stack.extend(reversed(missing))
+            continue
+        params = {k: v for k, v in node.params.items() if not k.startswith("#")}
+        values[i] = operators.run_op(node.op, params, [values[j] for j in node.inputs], device=device, device_id=device_id)
+        stack.pop()
+    return [values[i] for i in module.outputs]
