@@ -1,0 +1,149 @@
+// conv2d_quantized_fused: the operator chain of the int8 hot path as ONE node of device "hip",
+//     quantize -> conv2d_quantized -> add_bias -> relu / leaky_relu
+// (src/kernels/cpu/quantize.cpp, quantized/conv2d_quantized_core.cpp, add_bias.cpp, relu.cpp, leaky_relu.cpp),
+// run as the two kernels of tsx_quantize_conv2d_i8_nchw (staging with the quantize fused in, MFMA kernel with the
+// dequantize + bias + activation epilogue) instead of four operators exchanging fp32 tensors.  TenniS has no such
+// node: it is what a graph rewrite for this device puts in the chain's place (TenniS's own rewrites of this kind
+// are its zipper options, src/compiler/option/winograd_zipper_option.cpp:16-96); tennis_amd/module_file.py holds
+// that rewrite for module graphs.  Values are those of the chain, bit for bit.
+//
+// Inputs: x fp32 NCHW, w int8 OIHW[, bias fp32 [cout]].  Parameters: those of conv2d_quantized (format, padding
+// [4,2], padding_value, stride [4], dilation [4], dequantize_scales [cout]) plus quantize_scale [n] (the
+// quantize node's) and, optionally, activation ("relu" or "leaky_relu") with scale (leaky_relu's slope).
+#define TSX_TS_QUANTIZED_OPS   // Padding2D / Stride2D / Dilation2D come with the quantized skeleton
+#include "hip_ops_common.h"
+
+#include <string>
+#include <vector>
+
+namespace ts {
+namespace hip {
+
+class Conv2DQuantizedFused : public Operator {
+public:
+    using self = Conv2DQuantizedFused;
+    using supper = Operator;
+
+    Conv2DQuantizedFused() {
+        field(name::format, REQUIRED);
+        field(name::padding, REQUIRED);
+        field(name::padding_value, OPTIONAL, tensor::from(0.0f));
+        field(name::stride, REQUIRED);
+        field(name::dilation, OPTIONAL);
+        field(name::typo::dialations, OPTIONAL);
+        field(name::dequantize_scales, REQUIRED);
+        field(name::quantize_scale, REQUIRED);
+        field("activation", OPTIONAL, tensor::from("none"));
+        field(name::scale, OPTIONAL, tensor::from(0.0f));
+    }
+
+    void init() override {
+        supper::init();
+        if (tensor::to_string(get(name::format)) != "NCHW") TS_LOG_ERROR << "conv2d_quantized_fused only support NCHW" << eject;
+        const std::vector<int32_t> pad = ints(name::padding, 8), stride = ints(name::stride, 4);
+        if (!has(name::dilation) && !has(name::typo::dialations))
+            TS_LOG_ERROR << "conv2d_quantized_fused: dilation must be set" << eject;
+        const std::vector<int32_t> dil = ints(has(name::dilation) ? std::string(name::dilation) : std::string(name::typo::dialations), 4);
+        if (pad[0] || pad[1] || pad[2] || pad[3] || stride[0] != 1 || stride[1] != 1 || dil[0] != 1 || dil[1] != 1)
+            TS_LOG_ERROR << "conv2d_quantized_fused: padding / stride / dilation of the batch and channel axes must be 0 / 1 / 1" << eject;
+        m_pad = {pad[4], pad[5], pad[6], pad[7]};
+        m_stride = {stride[2], stride[3]};
+        m_dil = {dil[2], dil[3]};
+        m_padding_value = tensor::to_float(get(name::padding_value));
+        m_dq = tensor::array::to_float(get(name::dequantize_scales));
+        m_q = tensor::array::to_float(get(name::quantize_scale));
+        const std::string act = tensor::to_string(get("activation"));
+        if (act == "none") m_act = TSX_ACT_NONE;
+        else if (act == "relu") m_act = TSX_ACT_RELU;
+        else if (act == "leaky_relu") m_act = TSX_ACT_LEAKY_RELU;
+        else TS_LOG_ERROR << "conv2d_quantized_fused: activation must be none, relu or leaky_relu, got " << act << eject;
+        m_slope = tensor::to_float(get(name::scale));
+    }
+
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override {
+        tsx_conv2d_geom g;
+        output.assign(1, out_proto(stack, g));
+        return 1;
+    }
+
+    int run(Stack &stack) override {
+        tsx_conv2d_geom g;
+        const Tensor::Prototype proto = out_proto(stack, g);
+        auto &context = ctx::ref<DeviceContext>();
+        const MemoryDevice device = context.memory_device;
+        Tensor x = stack[0].view(device), w = stack[1].view(device);
+        Tensor bias;
+        const bool with_bias = stack.size() == 3;
+        if (with_bias) bias = stack[2].view(device);
+        Tensor out = *stack.push(proto, device);
+        void *stream = current_stream();
+        const size_t packed_bytes = tsx_conv2d_i8_packed_weight_bytes(&g);
+        if (packed_bytes == 0) TS_LOG_ERROR << "[hip] conv2d_quantized_fused: " << tsx_last_error() << eject;
+        if (m_packed.empty() || m_packed_from != w.data() || size_t(m_packed.count()) != packed_bytes || m_packed_cin != g.c) {
+            m_packed = Tensor(device, INT8, Shape({int32_t(packed_bytes)}));
+            check(tsx_conv2d_i8_pack_weights(&g, w.data<int8_t>(), m_packed.data(), stream), "tsx_conv2d_i8_pack_weights");
+            m_packed_from = w.data();
+            m_packed_cin = g.c;
+        }
+        const size_t ws_bytes = tsx_conv2d_i8_workspace_bytes(&g);
+        if (m_workspace.empty() || size_t(m_workspace.count()) < ws_bytes || m_workspace.device() != device)
+            m_workspace = Tensor(device, INT8, Shape({int32_t(ws_bytes ? ws_bytes : 16)}));
+        tsx_epilogue ep{};
+        ep.dq_dev = m_dq_dev.get(m_dq, device);
+        ep.bias_dev = with_bias ? bias.data<float>() : nullptr;
+        ep.act = m_act;
+        ep.slope = m_slope;
+        check(tsx_quantize_conv2d_i8_nchw(&g, x.data<float>(), m_q_dev.get(m_q, device), int32_t(m_q.size()), m_packed.data(),
+                                          m_padding_value, &ep, out.data<float>(), nullptr, nullptr, m_workspace.data(), ws_bytes,
+                                          stream),
+              "tsx_quantize_conv2d_i8_nchw");
+        return 1;
+    }
+
+private:
+    std::vector<int32_t> ints(const std::string &param, size_t count) {
+        const std::vector<int32_t> v = tensor::array::to_int(get(param));
+        if (v.size() != count) TS_LOG_ERROR << "conv2d_quantized_fused: " << param << " must hold " << count << " integers" << eject;
+        return v;
+    }
+
+    // checks the inputs against the parameters; fills the geometry; returns the output prototype
+    Tensor::Prototype out_proto(Stack &stack, tsx_conv2d_geom &g) {
+        if (stack.size() != 2 && stack.size() != 3)
+            TS_LOG_ERROR << "conv2d_quantized_fused expects 2 or 3 inputs (x, w[, bias]), got " << stack.size() << eject;
+        const Tensor &x = stack[0], &w = stack[1];
+        if (x.dims() != 4 || w.dims() != 4 || x.dtype() != FLOAT32 || w.dtype() != INT8)
+            TS_LOG_ERROR << "conv2d_quantized_fused: x must be float32 NCHW and w int8 OIHW" << eject;
+        if (x.size(1) != w.size(1))
+            TS_LOG_ERROR << "conv2d_quantized_fused: x has " << x.size(1) << " channels, w " << w.size(1) << eject;
+        if (int32_t(m_dq.size()) != w.size(0))
+            TS_LOG_ERROR << "conv2d_quantized_fused: " << m_dq.size() << " dequantize scales for " << w.size(0) << " output channels" << eject;
+        if (int32_t(m_q.size()) != x.size(0))      // base_quantize.cpp:26
+            TS_LOG_ERROR << "conv2d_quantized_fused: " << m_q.size() << " quantize scales for a batch of " << x.size(0) << eject;
+        if (stack.size() == 3 && !(stack[2].dtype() == FLOAT32 && stack[2].count() == w.size(0)))
+            TS_LOG_ERROR << "conv2d_quantized_fused: bias must hold one float32 per output channel" << eject;
+        g = make_geom(x, w, Padding2D(m_pad[0], m_pad[1], m_pad[2], m_pad[3]), Stride2D(m_stride[0], m_stride[1]),
+                      Dilation2D(m_dil[0], m_dil[1]));
+        // include/backend/common_function.h:30-40
+        const int ho = (g.h + g.pad_top + g.pad_bottom - (g.dilation_h * (g.kh - 1) + 1)) / g.stride_h + 1;
+        const int wo = (g.w + g.pad_left + g.pad_right - (g.dilation_w * (g.kw - 1) + 1)) / g.stride_w + 1;
+        if (ho <= 0 || wo <= 0) TS_LOG_ERROR << "conv2d_quantized_fused: empty output " << ho << "x" << wo << eject;
+        return Tensor::Prototype(FLOAT32, Shape({x.size(0), w.size(0), ho, wo}));
+    }
+
+    std::vector<int32_t> m_pad, m_stride, m_dil;
+    float m_padding_value = 0.f, m_slope = 0.f;
+    int m_act = TSX_ACT_NONE;
+    std::vector<float> m_dq, m_q;
+    DeviceFloats m_dq_dev, m_q_dev;
+    Tensor m_packed, m_workspace;
+    const void *m_packed_from = nullptr;
+    int m_packed_cin = 0;
+};
+
+}  // namespace hip
+}  // namespace ts
+
+using namespace ts;
+using namespace ts::hip;
+TS_REGISTER_OPERATOR(Conv2DQuantizedFused, ts::hip::DEVICE, "conv2d_quantized_fused")

@@ -104,7 +104,7 @@ def build(verbose=True, jobs=8):
 
 BACKEND_DIR = os.path.join(HERE, "backend")
 BACKEND_LIB = os.path.join(LIB_DIR, "libtsx_backend.so")
-BACKEND_SOURCES = ["ts/ts_api.cpp", "ts/base_ops.cpp", "hip/hip_device.cpp", "hip/hip_ops_quantized.cpp", "hip/hip_ops_float.cpp", "hip/hip_ops_glue.cpp", "hip/hip_ops_v2.cpp", "capi_ops.cpp"]
+BACKEND_SOURCES = ["ts/ts_api.cpp", "ts/base_ops.cpp", "hip/hip_device.cpp", "hip/hip_ops_quantized.cpp", "hip/hip_ops_float.cpp", "hip/hip_ops_glue.cpp", "hip/hip_ops_v2.cpp", "hip/hip_ops_fused.cpp", "capi_ops.cpp"]
 
 
 def build_backend(verbose=True):

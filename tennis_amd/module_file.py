@@ -177,3 +177,70 @@ def run_module(module, feeds, device="hip", device_id=0):
         values[i] = operators.run_op(node.op, params, [values[j] for j in node.inputs], device=device, device_id=device_id)
         stack.pop()
     return [values[i] for i in module.outputs]
+
+
+FUSED = "conv2d_quantized_fused"
+
+
+def fuse_quantized_chains(module):
+    """The graph rewrite for device "hip": every chain
+
+        quantize -> conv2d_quantized [-> add_bias (channel axis, constant bias)] [-> relu | leaky_relu]
+
+    whose intermediate tensors have no other consumer becomes one `conv2d_quantized_fused` node (two kernels
+    instead of up to four operators exchanging fp32 / int8 tensors; same values bit for bit).  A quantize node that
+    feeds several convolutions is folded into each of them.  Returns a new Module without the dead nodes; TenniS's
+    counterpart of such a pass is a zipper option of its graph compiler
+    (src/compiler/option/winograd_zipper_option.cpp:16-96)."""
+    nodes = [Node(n.op, n.name, n.params, n.inputs) for n in module.nodes]
+    users = {}
+    for i, n in enumerate(nodes):
+        for j in n.inputs:
+            users.setdefault(j, []).append(i)
+    for j in module.outputs:
+        users.setdefault(j, []).append(-1)
+
+    def only_user(i, op):
+        u = users.get(i, [])
+        return u[0] if len(u) == 1 and u[0] >= 0 and nodes[u[0]].op == op and nodes[u[0]].inputs[0] == i else None
+
+    for ci, conv in enumerate(list(nodes)):
+        if conv.op != "conv2d_quantized" or len(conv.inputs) != 2:
+            continue
+        q = nodes[conv.inputs[0]]
+        if q.op != "quantize" or len(q.inputs) != 1 or nodes[conv.inputs[1]].op != CONST:
+            continue
+        params = dict(conv.params)
+        params["quantize_scale"] = q.params["quantize_scale"]
+        inputs = [q.inputs[0], conv.inputs[1]]
+        last = ci
+        bi = only_user(last, "add_bias")
+        if bi is not None:
+            b = nodes[bi]
+            on_channels = b.params.get("format") == "NCHW" or int(np.asarray(b.params.get("dim", -99)).ravel()[0]) == 1
+            if len(b.inputs) == 2 and nodes[b.inputs[1]].op == CONST and on_channels:
+                inputs.append(b.inputs[1])
+                last = bi
+        ai = only_user(last, "relu")
+        if ai is not None:
+            params["activation"] = "relu"
+            last = ai
+        else:
+            ai = only_user(last, "leaky_relu")
+            if ai is not None and "scale" in nodes[ai].params:
+                params["activation"] = "leaky_relu"
+                params["scale"] = nodes[ai].params["scale"]
+                last = ai
+        # the fused node takes the place of the chain's last node, so its consumers keep their links
+        nodes[last] = Node(FUSED, nodes[last].name, params, inputs)
+    # drop what no output reaches any more, renumber
+    keep, stack = set(), list(module.outputs) + list(module.inputs)
+    while stack:
+        i = stack.pop()
+        if i not in keep:
+            keep.add(i)
+            stack.extend(nodes[i].inputs)
+    order = sorted(keep)
+    new_index = {old: new for new, old in enumerate(order)}
+    out_nodes = [Node(nodes[i].op, nodes[i].name, nodes[i].params, [new_index[j] for j in nodes[i].inputs]) for i in order]
+    return Module(out_nodes, [new_index[i] for i in module.inputs], [new_index[i] for i in module.outputs])

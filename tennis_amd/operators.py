@@ -44,6 +44,13 @@ def lib():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise OperatorError("libtsx_backend.so is not built: run `python -m tennis_amd.build`")
+        try:
+            # torch ships a HIP runtime of its own: where it is used in the same process it has to come up before
+            # the library's (loaded from /opt/rocm), or torch no longer finds the device afterwards
+            import torch
+            torch.cuda.is_available()
+        except ImportError:
+            pass
         L = ctypes.CDLL(LIB_PATH)
         L.tsxop_last_error.restype = ctypes.c_char_p
         _lib = L

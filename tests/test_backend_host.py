@@ -49,7 +49,8 @@ def test_hot_path_operators_are_registered_for_hip():
         assert hasattr(ops.lib(), name)
     for op in ("quantize", "conv2d_quantized", "conv2d", "conv2d_winograd", "inner_prod", "add_bias", "relu", "leaky_relu",
                "pooling2d", "global_pooling2d", "add", "depthwise_conv2d", "conv2d_v2", "conv2d_winograd_v2",
-               "depthwise_conv2d_v2", "pooling2d_v2", "concat", "_resize2d", "mul", "softplus", "tanh"):
+               "depthwise_conv2d_v2", "pooling2d_v2", "concat", "_resize2d", "mul", "softplus", "tanh",
+               "conv2d_quantized_fused"):
         assert ops.is_registered("hip", op), op
     assert not ops.is_registered("hip", "softmax")
     assert not ops.is_registered("cpu", "conv2d")            # this library ships no host operators

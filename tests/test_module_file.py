@@ -88,11 +88,81 @@ def test_reference_loads_and_runs_a_freshly_written_module(ref, tmp_path):
     assert np.array_equal(y, np.maximum(x + b.reshape(1, 6, 1, 1), 0))
 
 
+@pytest.fixture(scope="module")
+def hip_device():
+    """torch initialises its HIP runtime before the operator library loads its own, as in the other GPU tests."""
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return "hip"
+
+
 @pytest.mark.gpu
-def test_module_runs_on_hip_like_in_the_reference():
+def test_module_runs_on_hip_like_in_the_reference(hip_device):
     m = mf.read_module(BLOCK)
     x = tensor_file.read_tensor(os.path.join(MODULES, "quantized_block.input_0.t"))
     want = tensor_file.read_tensor(os.path.join(MODULES, "quantized_block.output_0.t"))
     (got,) = mf.run_module(m, [x])
     assert got.dtype == want.dtype and got.shape == want.shape
     assert np.array_equal(bits(got), bits(want))       # int8 chain and exact glue operators: bit for bit
+
+
+def test_fusing_rewrite_structure():
+    """quantize -> conv2d_quantized -> add_bias -> relu becomes one node; the quantize node shared with the shortcut
+    convolution is folded into both; dead nodes go and links are renumbered."""
+    m = mf.read_module(BLOCK)
+    f = mf.fuse_quantized_chains(m)
+    ops = [n.op for n in f.nodes]
+    assert ops.count(mf.FUSED) == 2 and not {"quantize", "conv2d_quantized", "add_bias", "relu"} & set(ops)
+    assert len(f.nodes) == 8 and f.inputs == [0]
+    main = next(n for n in f.nodes if n.op == mf.FUSED and len(n.inputs) == 3)
+    assert main.params["activation"] == "relu" and [f.nodes[i].op for i in main.inputs] == ["<param>", "<const>", "<const>"]
+    assert np.array_equal(main.params["quantize_scale"], m.nodes[1].params["quantize_scale"])
+    short = next(n for n in f.nodes if n.op == mf.FUSED and len(n.inputs) == 2)
+    assert "activation" not in short.params
+    assert f.nodes[f.outputs[0]].op == "concat"
+    mf.parse_module(mf.serialize_module(f))                  # still a well-formed module
+    # a convolution whose output has a second consumer keeps its add_bias outside the fused node
+    N = mf.Node
+    w = np.zeros((4, 8, 1, 1), np.int8)
+    conv = dict(m.nodes[9].params, dequantize_scales=np.ones(4, np.float32))
+    g = mf.Module([N("<param>", "x"), N("quantize", "q", {"quantize_scale": np.ones(1, np.float32)}, [0]), N("<const>", "w", {"value": w}),
+                   N("conv2d_quantized", "c", conv, [1, 2]), N("<const>", "b", {"value": np.zeros(4, np.float32)}),
+                   N("add_bias", "ab", {"format": "NCHW"}, [3, 4]), N("add", "sum", {}, [3, 5])], [0], [6])
+    fg = mf.fuse_quantized_chains(g)
+    assert [n.op for n in fg.nodes].count("add_bias") == 1 and [n.op for n in fg.nodes].count(mf.FUSED) == 1
+
+
+@pytest.mark.gpu
+def test_fused_module_equals_the_unfused_one(hip_device):
+    m = mf.read_module(BLOCK)
+    x = tensor_file.read_tensor(os.path.join(MODULES, "quantized_block.input_0.t"))
+    want = tensor_file.read_tensor(os.path.join(MODULES, "quantized_block.output_0.t"))
+    (got,) = mf.run_module(mf.fuse_quantized_chains(m), [x])
+    assert np.array_equal(bits(got), bits(want))
+
+
+@pytest.mark.gpu
+def test_fused_operator_against_the_operator_chain(hip_device):
+    from tennis_amd import operators as ops
+    rng = np.random.default_rng(41)
+    x = (rng.standard_normal((3, 20, 9, 11)) * 6).astype(np.float32)
+    w = rng.integers(-127, 128, (10, 20, 3, 3)).astype(np.int8)
+    bias = rng.standard_normal(10).astype(np.float32)
+    qs = np.array([7.0, 9.5, 12.25], np.float32)
+    for pads, strides, dil, pv, act in (((1, 1, 1, 1), (1, 1), (1, 1), 0.0, "relu"), ((0, 2, 1, 0), (2, 1), (1, 2), 3.0, "leaky_relu"),
+                                        ((1, 0, 0, 1), (1, 2), (1, 1), 0.0, "none")):
+        conv = dict(ops.conv_params(pads, strides, dil, pv), dequantize_scales=rng.uniform(1e-4, 1e-3, 10).astype(np.float32))
+        y = ops.run_op("conv2d_quantized", conv, [ops.run_op("quantize", {"quantize_scale": qs}, [x]), w])
+        y = ops.run_op("add_bias", {"format": "NCHW"}, [y, bias])
+        if act == "relu":
+            y = ops.run_op("relu", {}, [y])
+        elif act == "leaky_relu":
+            y = ops.run_op("leaky_relu", {"scale": np.array([0.1], np.float32)}, [y])
+        fused = dict(conv, quantize_scale=qs, activation=act, scale=np.array([0.1], np.float32))
+        assert ops.run_op(mf.FUSED, fused, [x, w, bias], infer_only=True)[1] == y.shape
+        got = ops.run_op(mf.FUSED, fused, [x, w, bias])
+        assert np.array_equal(bits(got), bits(y)), (pads, strides, dil, act)
+    with pytest.raises(ops.OperatorError, match="quantize scales for a batch"):
+        ops.run_op(mf.FUSED, dict(fused, quantize_scale=qs[:2]), [x, w, bias])
+    with pytest.raises(ops.OperatorError, match="activation must be"):
+        ops.run_op(mf.FUSED, dict(fused, activation="gelu"), [x, w, bias])

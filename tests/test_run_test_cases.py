@@ -95,8 +95,16 @@ def test_unregistered_operator_is_skipped():
     assert tc.run("hip") == run_test.SKIP and "Not supported operator" in tc.log[0]
 
 
+@pytest.fixture(scope="module")
+def hip_device():
+    """torch initialises its HIP runtime before the operator library loads its own, as in the other GPU tests."""
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return "hip"
+
+
 @pytest.mark.gpu
-def test_reference_cases_pass_on_hip():
+def test_reference_cases_pass_on_hip(hip_device):
     out = io.StringIO()
     results = run_test.run_tree(CASES, "hip", 0, out=out)
     text = out.getvalue()
@@ -107,7 +115,7 @@ def test_reference_cases_pass_on_hip():
 
 
 @pytest.mark.gpu
-def test_integer_and_bit_exact_cases_match_exactly():
+def test_integer_and_bit_exact_cases_match_exactly(hip_device):
     """The runner's tolerance is the reference's; the operators that are exact by construction are held to 0."""
     from tennis_amd import operators
     for sub in ("quantize/per_image", "quantize/single_scale", "conv2d_quantized/3x3_pad1", "conv2d_quantized/1x1_s2",
@@ -121,7 +129,7 @@ def test_integer_and_bit_exact_cases_match_exactly():
 
 
 @pytest.mark.gpu
-def test_wrong_expected_output_fails(tmp_path):
+def test_wrong_expected_output_fails(tmp_path, hip_device):
     src = os.path.join(CASES, "relu", "4d")
     for name in os.listdir(src):
         (tmp_path / name).write_bytes(open(os.path.join(src, name), "rb").read())
