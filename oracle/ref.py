@@ -91,6 +91,23 @@ def run_op_intree(device, op, params, inputs, out_bytes, threads=1, strict=True)
     return buf[:out.bytes].view(_TS2NP[out.dtype]).reshape(shape).copy()
 
 
+def run_module_intree(device, path, inputs, out_bytes=1 << 24, threads=1):
+    """Load a `.tsm` file into a TenniS Workbench on ``device`` ("cpu" or "hip") of the in-tree build: TenniS's own
+    module loader, graph compiler and runtime, with this repository's backend serving device "hip"."""
+    L = intree_lib()
+    keep = []
+    i = (_Tensor * max(len(inputs), 1))(*[_pack("", v, keep) for v in inputs])
+    buf = np.empty(out_bytes, dtype=np.uint8)
+    out = _Output()
+    out.data = buf.ctypes.data
+    out.capacity = out_bytes
+    rc = L.ref_run_module(str(path).encode(), device.encode(), len(inputs), i, int(threads), ctypes.byref(out))
+    if rc != 0:
+        raise RuntimeError("TenniS raised: " + L.ref_last_error().decode(errors="replace"))
+    shape = tuple(out.shape[k] for k in range(out.ndim))
+    return buf[:out.bytes].view(_TS2NP[out.dtype]).reshape(shape).copy()
+
+
 def _pack(name, value, keep):
     """Turn a python value into a _Tensor; ``keep`` holds the buffers alive."""
     if isinstance(value, str):

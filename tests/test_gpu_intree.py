@@ -158,3 +158,19 @@ def test_concat_and_resize2d_in_tennis_workbench(ts):
     assert np.array_equal(bits(cpu), bits(hip))
     cpu, hip = both(ts, "_resize2d", {"type": np.array([2], np.int32)}, [a, np.array([-1, -1, 14, 12], np.int32)], 1 << 20)
     assert np.array_equal(bits(cpu), bits(hip))
+
+
+def test_module_file_in_tennis_workbench_on_hip(ts):
+    """A `.tsm` module loaded by TenniS's own Module::Load, compiled by its graph compiler and run by its Workbench on
+    ComputingDevice("hip"): the whole drop-in path (quantize, conv2d_quantized x2, add_bias, relu, pooling2d, concat
+    served by this backend).  Same values as on TenniS's CPU device and as the committed expected output."""
+    import os
+    from tennis_amd import tensor_file
+    root = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "modules")
+    path = os.path.join(root, "quantized_block.tsm")
+    x = tensor_file.read_tensor(os.path.join(root, "quantized_block.input_0.t"))
+    want = tensor_file.read_tensor(os.path.join(root, "quantized_block.output_0.t"))
+    cpu = ts.run_module_intree("cpu", path, [x])
+    hip = ts.run_module_intree("hip", path, [x])
+    assert np.array_equal(bits(cpu), bits(want))
+    assert hip.shape == want.shape and np.array_equal(bits(hip), bits(want))
