@@ -274,3 +274,52 @@ class ResNet50Int8:
             sx, dq = self._batch_scales(n)["fc"], self._dq["fc"]
         p8 = capi.quantize(pooled, sx)
         return self.fc(p8, dq=dq, bias=self.bias["fc"])[0]
+
+
+def to_module(desc, params, batch, act_scale=16.0):
+    """The network as a TenniS module graph (tennis_amd.module_file.Module) for a fixed batch size: per convolution
+    quantize -> conv2d_quantized -> add_bias [-> relu], max pooling behind the stem, `add` + relu at every residual
+    join, global average pooling and an fp32 inner_prod + add_bias classifier (TenniS has no quantized inner_prod).
+    Every activation is quantized with the same multiplier `act_scale` (a module for exercising runtimes, not a
+    calibrated model).  The graph a TenniS front end would hand to Workbench::Load."""
+    from . import module_file as mf
+    stem, net, fc = desc
+    nodes = []
+
+    def add(op, name, p=None, inputs=()):
+        nodes.append(mf.Node(op, name, p or {}, list(inputs)))
+        return len(nodes) - 1
+
+    def conv(spec, x, relu):
+        p = params[spec.name]
+        scales = np.full(batch, act_scale, np.float32)
+        q = add("quantize", spec.name + ".q", {"quantize_scale": scales}, [x])
+        w = add(mf.CONST, spec.name + ".w", {"value": p["wq"]})
+        cp = {"format": "NCHW",
+              "padding": np.array([[0, 0], [0, 0], [spec.pad, spec.pad], [spec.pad, spec.pad]], np.int32),
+              "padding_value": np.array([0.0], np.float32),
+              "stride": np.array([1, 1, spec.stride, spec.stride], np.int32),
+              "dilation": np.array([1, 1, 1, 1], np.int32),
+              "dequantize_scales": (np.float32(1.0) / (np.float32(act_scale) * p["sw"])).astype(np.float32)}
+        c = add("conv2d_quantized", spec.name, cp, [q, w])
+        b = add(mf.CONST, spec.name + ".b", {"value": p["bias"]})
+        y = add("add_bias", spec.name + ".bias", {"format": "NCHW"}, [c, b])
+        return add("relu", spec.name + ".relu", {}, [y]) if relu else y
+
+    x = add(mf.PARAMETER, "x")
+    y = conv(stem, x, True)
+    (kh, kw), (sh, sw_), pads = ResNet50Int8.POOL
+    y = add("pooling2d", "pool", {"format": "NCHW", "type": np.array([0], np.int32),
+                                  "padding": np.array([[0, 0], [0, 0], [pads[0], pads[1]], [pads[2], pads[3]]], np.int32),
+                                  "padding_type": np.array([0], np.int32), "ksize": np.array([1, 1, kh, kw], np.int32),
+                                  "stride": np.array([1, 1, sh, sw_], np.int32)}, [y])
+    for c1, c2, c3, proj in net:
+        sc = y if proj is None else conv(proj, y, False)
+        z = conv(c3, conv(c2, conv(c1, y, True), True), False)
+        y = add("relu", c3.name + ".out", {}, [add("add", c3.name + ".join", {}, [z, sc])])
+    y = add("global_pooling2d", "gap", {"format": "NCHW", "type": np.array([1], np.int32)}, [y])
+    wf = add(mf.CONST, "fc.w", {"value": (params["fc"]["wq"].astype(np.float32) / params["fc"]["sw"][None, :]).astype(np.float32)})
+    y = add("inner_prod", "fc", {}, [y, wf])
+    bf = add(mf.CONST, "fc.b", {"value": params["fc"]["bias"]})
+    y = add("add_bias", "fc.bias", {"dim": np.array([1], np.int32)}, [y, bf])
+    return mf.Module(nodes, [x], [y])

@@ -174,3 +174,26 @@ def test_module_file_in_tennis_workbench_on_hip(ts):
     hip = ts.run_module_intree("hip", path, [x])
     assert np.array_equal(bits(cpu), bits(want))
     assert hip.shape == want.shape and np.array_equal(bits(hip), bits(want))
+
+
+def test_resnet_shaped_module_in_tennis_workbench_on_hip(ts, tmp_path):
+    """A ResNet-50-shaped int8 network (quarter width, one bottleneck per stage: 17 quantized convolutions, 4
+    residual joins, pooling, global pooling, classifier) written as a `.tsm` module and run (a) by TenniS's own
+    runtime on its CPU device, (b) by TenniS's own runtime on ComputingDevice("hip"), (c) by this repository's
+    operator-by-operator module runner, plain and with the chain-fusing rewrite.  Everything up to the fp32
+    classifier is exact arithmetic shared by all four; the classifier's MFMA summation order differs from the
+    host's, hence the fp32 tolerance of 1e-4 relative + 1e-5 absolute on the logits."""
+    from tennis_amd import module_file as mf, resnet50
+    desc, params = resnet50.make_parameters(seed=3, width=0.25, blocks=(1, 1, 1, 1), classes=10)
+    module = resnet50.to_module(desc, params, batch=2)
+    path = str(tmp_path / "resnet_shaped.tsm")
+    mf.write_module(path, module)
+    x = np.random.default_rng(1).random((2, 3, 64, 64), dtype=np.float32)
+    cpu = ts.run_module_intree("cpu", path, [x])
+    hip = ts.run_module_intree("hip", path, [x])
+    assert cpu.shape == (2, 10) and hip.shape == (2, 10) and np.abs(cpu).max() > 0.1
+    assert close(hip, cpu)
+    (own,) = mf.run_module(module, [x])
+    (fused,) = mf.run_module(mf.fuse_quantized_chains(module), [x])
+    assert np.array_equal(bits(own), bits(hip))          # the same device operators, with or without TenniS around them
+    assert np.array_equal(bits(fused), bits(own))
