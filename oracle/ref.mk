@@ -50,7 +50,7 @@ $(OUT)/libref_driver.so: $(HERE)ref_driver.cpp $(OUT)/libtennis_ref.so
 HIPCC   ?= /opt/rocm/bin/hipcc
 REPO    := $(abspath $(HERE)..)
 HIPDIR  := $(REPO)/tennis_amd/backend/hip
-HIPOBJS := $(OBJ)/hip/hip_device.o $(OBJ)/hip/hip_ops_quantized.o $(OBJ)/hip/hip_ops_float.o $(OBJ)/hip/hip_ops_glue.o $(OBJ)/hip/hip_ops_v2.o $(OBJ)/hip/hip_ops_fused.o
+HIPOBJS := $(OBJ)/hip/hip_device.o $(OBJ)/hip/hip_ops_quantized.o $(OBJ)/hip/hip_ops_float.o $(OBJ)/hip/hip_ops_glue.o $(OBJ)/hip/hip_ops_v2.o $(OBJ)/hip/hip_ops_fused.o $(OBJ)/hip/hip_zipper_option.o
 intree: $(OUT)/libtennis_hip.so $(OUT)/libref_driver_hip.so
 
 $(OBJ)/hip/%.o: $(HIPDIR)/%.cpp $(wildcard $(HIPDIR)/*.h) $(REPO)/include/tsx_hip.h

@@ -91,6 +91,13 @@ def run_op_intree(device, op, params, inputs, out_bytes, threads=1, strict=True)
     return buf[:out.bytes].view(_TS2NP[out.dtype]).reshape(shape).copy()
 
 
+def fused_chain_count_intree():
+    """Chains the "hip" device's zipper option has replaced so far in the in-tree library."""
+    L = intree_lib()
+    L.ref_hip_fused_chain_count.restype = ctypes.c_long
+    return int(L.ref_hip_fused_chain_count())
+
+
 def run_module_intree(device, path, inputs, out_bytes=1 << 24, threads=1):
     """Load a `.tsm` file into a TenniS Workbench on ``device`` ("cpu" or "hip") of the in-tree build: TenniS's own
     module loader, graph compiler and runtime, with this repository's backend serving device "hip"."""

@@ -170,8 +170,13 @@ def test_module_file_in_tennis_workbench_on_hip(ts):
     path = os.path.join(root, "quantized_block.tsm")
     x = tensor_file.read_tensor(os.path.join(root, "quantized_block.input_0.t"))
     want = tensor_file.read_tensor(os.path.join(root, "quantized_block.output_0.t"))
+    fused0 = ts.fused_chain_count_intree()
     cpu = ts.run_module_intree("cpu", path, [x])
+    assert ts.fused_chain_count_intree() == fused0        # the zipper option is for device "hip" only
     hip = ts.run_module_intree("hip", path, [x])
+    # TenniS's compiler, walking the graph with this backend's zipper option, has replaced both chains of the
+    # module (quantize -> conv -> add_bias -> relu and quantize -> conv) by conv2d_quantized_fused nodes
+    assert ts.fused_chain_count_intree() == fused0 + 2
     assert np.array_equal(bits(cpu), bits(want))
     assert hip.shape == want.shape and np.array_equal(bits(hip), bits(want))
 
@@ -190,7 +195,9 @@ def test_resnet_shaped_module_in_tennis_workbench_on_hip(ts, tmp_path):
     mf.write_module(path, module)
     x = np.random.default_rng(1).random((2, 3, 64, 64), dtype=np.float32)
     cpu = ts.run_module_intree("cpu", path, [x])
+    fused0 = ts.fused_chain_count_intree()
     hip = ts.run_module_intree("hip", path, [x])
+    assert ts.fused_chain_count_intree() == fused0 + 17   # every quantized convolution of the network, fused by TenniS's compiler
     assert cpu.shape == (2, 10) and hip.shape == (2, 10) and np.abs(cpu).max() > 0.1
     assert close(hip, cpu)
     (own,) = mf.run_module(module, [x])
