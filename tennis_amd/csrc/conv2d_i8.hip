@@ -115,7 +115,9 @@ struct StageRow {
 // per channel, coalesced along W across lanes), packs the 4 quantized bytes of each pixel into one
 // dword and writes VW dwords to the tile -- no byte-granular LDS traffic.  WL = power of two >= W/VW
 // keeps the mapping division-free; loads are issued in batches of NB quads before any is consumed.
-template <bool QUANT, int VW>
+// RMODE says how the row's elements round: 0 = all half away from zero (the reference's scalar loop),
+// 1 = all half to even (its AVX body), 2 = per element (the one row that holds the body/tail border).
+template <bool QUANT, int VW, int RMODE>
 __device__ __forceinline__ void stage_quads(const StageGeom &g, const StageRow &r, int8_t *tile, int tid) {
     typedef float vf __attribute__((ext_vector_type(VW == 1 ? 2 : VW)));   // VW == 1 uses scalars
     constexpr int NB = VW == 4 ? 2 : 4;
@@ -174,23 +176,31 @@ __device__ __forceinline__ void stage_quads(const StageGeom &g, const StageRow &
         for (int u = 0; u < NB; ++u) {
             const int c = (qb + u * qstep + q_lane) * 4;
             if (!(lane_ok && c < r.creal)) continue;
+            // bytes of the quad that are real channels (the last quad of a ragged channel count keeps zeros above)
+            const uint32_t keep = c + 3 < r.creal ? 0xffffffffu : 0xffffffffu >> (8 * (c + 4 - r.creal));
 #pragma unroll
             for (int v = 0; v < VW; ++v) {
-                uint32_t word = 0;
+                int q[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    int q = 0;
-                    if (c + j < r.creal) {
-                        if (QUANT) {
+                    if (QUANT) {
+                        float sc = r.row_scale;
+                        bool half_even = RMODE == 1;
+                        if (RMODE == 2 || !r.uniform_scale) {   // the element's linear index is only needed here
                             const int64_t e = row_base + int64_t(c + j) * plane + v;
-                            const float sc = r.uniform_scale ? r.row_scale : r.scales[e / r.group_len];
-                            q = tsx::quantize_value(__fmul_rn(fv[u][j][v], sc), r.n_scales == 1 && e < r.bulk8);
-                        } else {
-                            q = bv[u][j][v];
+                            if (!r.uniform_scale) sc = c + j < r.creal ? r.scales[e / r.group_len] : 0.f;
+                            if (RMODE == 2) half_even = e < r.bulk8;
                         }
+                        q[j] = tsx::quantize_value(__fmul_rn(fv[u][j][v], sc), half_even);
+                    } else {
+                        q[j] = bv[u][j][v];
                     }
-                    word |= uint32_t(q & 0xff) << (8 * j);
                 }
+                // low bytes of q[0..3] into one dword: three byte permutes (selector 0-3 = bytes of the second
+                // operand, 4-7 = bytes of the first, 0x0c = zero)
+                const uint32_t lo = __builtin_amdgcn_perm(uint32_t(q[1]), uint32_t(q[0]), 0x0c0c0400u);
+                const uint32_t hi = __builtin_amdgcn_perm(uint32_t(q[3]), uint32_t(q[2]), 0x0c0c0400u);
+                const uint32_t word = __builtin_amdgcn_perm(hi, lo, 0x05040100u) & keep;
                 *reinterpret_cast<uint32_t *>(&tile[(wi + v + g.pad_left) * STAGE_LROW + c]) = word;
             }
         }
@@ -221,9 +231,24 @@ __global__ __launch_bounds__(256) void stage_rows_kernel(const void *__restrict_
     for (int c0 = 0; c0 < g.cp; c0 += STAGE_CG) {
         const int cg = min(STAGE_CG, g.cp - c0);        // multiple of 64
         const int creal = max(0, min(cg, g.c - c0));    // channels that exist in the source
+        // Lane = (run of VW pixels along W, channel quad): see stage_quads.  The widest run the row
+        // length and the source alignment allow keeps the number of load instructions down.
+        const uintptr_t addr = reinterpret_cast<uintptr_t>(src);
+        const int esz = QUANT ? 4 : 1;
+        int vw = 1;
+        if (g.w % 4 == 0 && addr % (4 * esz) == 0) vw = 4;
+        else if (g.w % 2 == 0 && addr % (2 * esz) == 0) vw = 2;
+        int wl = 1;
+        while (wl * vw < g.w) wl <<= 1;
+        // stage_quads writes every dword of the interior pixels up to the last real channel quad, so
+        // on that path the pre-fill only has to cover the halo pixels and the channel padding: the
+        // two write disjoint dwords and need no barrier between them.
+        const bool quad_path = row_inside && wl <= 64;
+        const int real_words = (creal + 3) / 4;
         // pre-fill: halo value for real channels, zero for channel padding
         for (int idx = tid; idx < g.ws * (cg / 4); idx += 256) {
             const int pix = idx / (cg / 4), cw = idx - pix * (cg / 4);
+            if (quad_path && cw < real_words && pix >= g.pad_left && pix < g.pad_left + g.w) continue;
             uint32_t v = pad4;
             if (cw * 4 + 4 > creal) {
                 v = 0;
@@ -232,22 +257,30 @@ __global__ __launch_bounds__(256) void stage_rows_kernel(const void *__restrict_
             }
             *reinterpret_cast<uint32_t *>(&tile[pix * STAGE_LROW + cw * 4]) = v;
         }
-        __syncthreads();
+        if (!quad_path) __syncthreads();
         if (row_inside) {
-            // Lane = (run of VW pixels along W, channel quad): see stage_quads.  The widest run the
-            // row length and the source alignment allow keeps the number of load instructions down.
-            const uintptr_t addr = reinterpret_cast<uintptr_t>(src);
-            const int esz = QUANT ? 4 : 1;
-            int vw = 1;
-            if (g.w % 4 == 0 && addr % (4 * esz) == 0) vw = 4;
-            else if (g.w % 2 == 0 && addr % (2 * esz) == 0) vw = 2;
-            int wl = 1;
-            while (wl * vw < g.w) wl <<= 1;
-            if (wl <= 64) {
+            if (quad_path) {
                 const StageRow r{src, scales, n_scales, group_len, bulk8, uniform_scale, row_scale, ni, hi, c0, creal};
-                if (vw == 4) stage_quads<QUANT, 4>(g, r, tile, tid);
-                else if (vw == 2) stage_quads<QUANT, 2>(g, r, tile, tid);
-                else stage_quads<QUANT, 1>(g, r, tile, tid);
+                // how this row's elements round: linear indices run from lo to hi_e, the AVX body ends at bulk8
+                int rmode = 0;
+                if (QUANT && n_scales == 1) {
+                    const int64_t lo = ((int64_t(ni) * g.c + c0) * g.h + hi) * g.w;
+                    const int64_t hi_e = lo + int64_t(creal - 1) * g.h * g.w + g.w - 1;
+                    rmode = hi_e < bulk8 ? 1 : lo >= bulk8 ? 0 : 2;
+                }
+                if (vw == 4) {
+                    if (rmode == 0) stage_quads<QUANT, 4, 0>(g, r, tile, tid);
+                    else if (rmode == 1) stage_quads<QUANT, 4, 1>(g, r, tile, tid);
+                    else stage_quads<QUANT, 4, 2>(g, r, tile, tid);
+                } else if (vw == 2) {
+                    if (rmode == 0) stage_quads<QUANT, 2, 0>(g, r, tile, tid);
+                    else if (rmode == 1) stage_quads<QUANT, 2, 1>(g, r, tile, tid);
+                    else stage_quads<QUANT, 2, 2>(g, r, tile, tid);
+                } else {
+                    if (rmode == 0) stage_quads<QUANT, 1, 0>(g, r, tile, tid);
+                    else if (rmode == 1) stage_quads<QUANT, 1, 1>(g, r, tile, tid);
+                    else stage_quads<QUANT, 1, 2>(g, r, tile, tid);
+                }
             } else {
                 for (int idx = tid; idx < creal * g.w; idx += 256) {
                     const int c = idx / g.w, wi = idx - c * g.w;
@@ -271,7 +304,7 @@ __global__ __launch_bounds__(256) void stage_rows_kernel(const void *__restrict_
             *reinterpret_cast<v4i *>(dst + int64_t(pix) * g.cp + ch * 16) =
                 *reinterpret_cast<const v4i *>(&tile[pix * STAGE_LROW + ch * 16]);
         }
-        __syncthreads();
+        if (c0 + STAGE_CG < g.cp) __syncthreads();     // the next pass refills the tile
     }
 }
 

@@ -64,10 +64,15 @@ __device__ __forceinline__ void static_for(F &&f) {
 // NaN and |v| >= 2^31 convert to INT_MIN, i.e. -128 after the clamp
 // (src/kernels/cpu/quantize.cpp:15-29,83-96).
 __device__ __forceinline__ int quantize_value(float v, bool half_even) {
-    // rintf = round half to even (_mm256_cvtps_epi32); roundf = half away from zero (round()).
-    const float r = half_even ? __builtin_rintf(v) : __builtin_roundf(v);
+    // rintf = round half to even (_mm256_cvtps_epi32).  round() = half away from zero, computed as
+    // trunc(v + copysign(0.5 - 2^-25, v)): the addend is the float below 0.5, so 0.49999997 stays 0 while
+    // every x.5 still reaches the next integer (the sum rounds up to it); equal to roundf(v) for
+    // |v| < 2^23 and, like it, far outside the clamp beyond (three instructions instead of roundf's six;
+    // this runs once per element in the staging kernel, which is bound by its arithmetic).
+    const float away = __builtin_truncf(v + __builtin_copysignf(0.49999997f, v));
+    const float r = half_even ? __builtin_rintf(v) : away;
     // selects, not branches: this runs once per output element in the epilogues
-    const float c = __builtin_fminf(__builtin_fmaxf(r, -128.f), 127.f);
+    const float c = __builtin_amdgcn_fmed3f(r, -128.f, 127.f);   // the clamp as one instruction; NaN is overridden below
     const bool in_range = __builtin_fabsf(v) < 2147483648.0f;   // false for NaN as well
     return in_range ? int(c) : -128;
 }
