@@ -47,6 +47,44 @@ def test_quantize_known_answers(tsx):
     assert two.tolist() == [[1, 2, 3, -1, -2, 4, 5, 6, 1, 2, 3]] * 2
 
 
+def _tie_neighbourhood():
+    """Every x.5 from -131.5 to 131.5 with the float just below and just above it, the float below 0.5 (which
+    v + 0.5 would round up to 1), and values around 2^23 where a float has no fraction bits left."""
+    half = np.arange(-132, 132, dtype=np.float32) + np.float32(0.5)
+    vals = [half, np.nextafter(half, np.float32(np.inf)), np.nextafter(half, np.float32(-np.inf)),
+            np.array([0.49999997, -0.49999997, 0.0, -0.0, 8388607.5, -8388607.5, 8388609.0, -8388609.0,
+                      4194303.5, -4194303.5, 126.99999, -127.99999, 1e-30, -1e-30], np.float32)]
+    return np.concatenate(vals).astype(np.float32)
+
+
+@pytest.mark.parametrize("ns", [1, 2])
+def test_quantize_tie_neighbourhood(tsx, port, ns):
+    """Round-half-away (several scales, and the tail of the single-scale case) and round-half-even (its body) on the
+    values where the two differ from each other and from truncation of v + 0.5."""
+    v = _tie_neighbourhood()
+    x = np.stack([np.resize(v, 811)] * ns)                   # 811 = 8 * 101 + 3: a body and a tail
+    s = np.ones(ns, np.float32)
+    got = tsx.quantize(_dev(x), _dev(s)).cpu().numpy()
+    assert np.array_equal(got, port.quantize(x, s))
+    if ns == 2:   # half away from zero, stated without the oracle: sign(v) * floor(|v| + 0.5) in exact arithmetic
+        want = np.clip(np.sign(x) * np.floor(np.abs(x).astype(np.float64) + 0.5), -128, 127).astype(np.int8)
+        assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("n", [1, 2])
+def test_staged_quantize_tie_neighbourhood(tsx, port, n):
+    """The same values through the quantize fused into the staging kernel: a 1x1 convolution with identity weights
+    and unit scales hands the quantized input back as fp32."""
+    v = _tie_neighbourhood()
+    c, h, w = 8, 9, 12                                          # 864 elements per image
+    x = np.stack([np.resize(np.roll(v, 5 * i), c * h * w).reshape(c, h, w) for i in range(n)])
+    wq = np.eye(c, dtype=np.int8).reshape(c, c, 1, 1)
+    s = np.ones(n, np.float32)
+    conv = tsx.Conv2dI8(_dev(wq), (0, 0, 0, 0))
+    out, _, _ = conv(_dev(x), dq=_dev(np.ones(c, np.float32)), x_scales=_dev(s))
+    assert np.array_equal(out.cpu().numpy(), port.quantize(x, s).astype(np.float32))
+
+
 def test_quantize_unaligned_view(tsx, port):
     import torch
     rng = np.random.default_rng(101)
