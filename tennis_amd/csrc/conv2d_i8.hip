@@ -53,14 +53,27 @@ __global__ __launch_bounds__(256) void stage_nchw_kernel(const void *__restrict_
     const int64_t total = int64_t(g.n) * g.hs * chunks * g.ws;
     const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
     if (id >= total) return;
-    const int wsi = int(id % g.ws);
-    int64_t rest = id / g.ws;
-    const int chunk = int(rest % chunks);
-    rest /= chunks;
-    const int hsi = int(rest % g.hs);
-    const int ni = int(rest / g.hs);
+    int wsi, chunk, hsi, ni;
+    if (total <= 0xffffffffll) {   // the usual case: three 32-bit divisions instead of three 64-bit ones per lane
+        const uint32_t id32 = uint32_t(id);
+        uint32_t rest = id32 / uint32_t(g.ws);
+        wsi = int(id32 - rest * uint32_t(g.ws));
+        const uint32_t r2 = rest / uint32_t(chunks);
+        chunk = int(rest - r2 * uint32_t(chunks));
+        ni = int(r2 / uint32_t(g.hs));
+        hsi = int(r2 - uint32_t(ni) * uint32_t(g.hs));
+    } else {
+        wsi = int(id % g.ws);
+        int64_t rest = id / g.ws;
+        chunk = int(rest % chunks);
+        rest /= chunks;
+        hsi = int(rest % g.hs);
+        ni = int(rest / g.hs);
+    }
     const int hi = hsi - g.pad_top, wi = wsi - g.pad_left;
     const bool inside = hi >= 0 && hi < g.h && wi >= 0 && wi < g.w;
+    // one scale group per image (the usual case when there are several): no division per element
+    const bool per_image = group_len == int64_t(g.c) * g.h * g.w;
     uint32_t words[4];
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
@@ -74,7 +87,7 @@ __global__ __launch_bounds__(256) void stage_nchw_kernel(const void *__restrict_
                 if (inside) {
                     const int64_t idx = ((int64_t(ni) * g.c + ci) * g.h + hi) * g.w + wi;
                     if (QUANT) {
-                        const float s = n_scales == 1 ? scales[0] : scales[idx / group_len];
+                        const float s = n_scales == 1 ? scales[0] : per_image ? scales[ni] : scales[idx / group_len];
                         q = tsx::quantize_value(__fmul_rn(static_cast<const float *>(src)[idx], s),
                                                 n_scales == 1 && idx < bulk8);
                     } else {
