@@ -28,9 +28,18 @@ __global__ __launch_bounds__(256) void resize_nearest_kernel(const float *__rest
     const int64_t total = planes * ho * wo;
     const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
     if (id >= total) return;
-    const int xd = int(id % wo);
-    const int yd = int((id / wo) % ho);
-    const int64_t p = id / wo / ho;
+    int xd, yd;
+    int64_t p;
+    if (total <= 0xffffffffll) {   // 32-bit divisions where the element count allows: this kernel is bound by its arithmetic
+        const uint32_t id32 = uint32_t(id), r = id32 / uint32_t(wo), p32 = r / uint32_t(ho);
+        xd = int(id32 - r * uint32_t(wo));
+        yd = int(r - p32 * uint32_t(ho));
+        p = p32;
+    } else {
+        xd = int(id % wo);
+        yd = int((id / wo) % ho);
+        p = id / wo / ho;
+    }
     int xs = xd, ys = yd;
     if (!(h == ho && w == wo)) {
         const double sx = double(w) / wo, sy = double(h) / ho;

@@ -124,12 +124,21 @@ __global__ __launch_bounds__(256) void max_pooling2d_i8_staged_kernel(const int8
     const int64_t total = int64_t(g.n) * g.ho * g.wo * chunks;
     const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
     if (id >= total) return;
-    const int chunk = int(id % chunks);
-    int64_t rest = id / chunks;
-    const int ow = int(rest % g.wo);
-    rest /= g.wo;
-    const int oh = int(rest % g.ho);
-    const int ni = int(rest / g.ho);
+    int chunk, ow, oh, ni;
+    if (total <= 0xffffffffll) {   // 32-bit divisions where the lane count allows
+        const uint32_t id32 = uint32_t(id), r1 = id32 / uint32_t(chunks), r2 = r1 / uint32_t(g.wo), r3 = r2 / uint32_t(g.ho);
+        chunk = int(id32 - r1 * uint32_t(chunks));
+        ow = int(r1 - r2 * uint32_t(g.wo));
+        oh = int(r2 - r3 * uint32_t(g.ho));
+        ni = int(r3);
+    } else {
+        chunk = int(id % chunks);
+        int64_t rest = id / chunks;
+        ow = int(rest % g.wo);
+        rest /= g.wo;
+        oh = int(rest % g.ho);
+        ni = int(rest / g.ho);
+    }
     v4i r = {0, 0, 0, 0};   // channels the source does not have stay zero (channel padding)
     if (chunk * 16 < g.s_cp) {
         int hs = oh * g.sh - g.pad_top, ws = ow * g.sw - g.pad_left;
