@@ -411,19 +411,40 @@ __global__ __launch_bounds__(256) void stage_im2col_rows_kernel(const void *__re
         const int hi = h0 + r * g.dh;
         const bool row_in = hi >= 0 && hi < g.h;
         const int64_t e0 = ((int64_t(ni) * g.c + ci) * g.h + hi) * g.w;
-        for (int col = tid & 63; col < wpatch; col += 64) {
-            const int wi = col - g.pad_left;
-            int q = g.pad_value;
-            if (row_in && wi >= 0 && wi < g.w) {
-                const int64_t e = e0 + wi;
-                if (QUANT) {
-                    const float sc = uniform_scale ? img_scale : scales[e / group_len];
-                    q = tsx::quantize_value(__fmul_rn(static_cast<const float *>(src)[e], sc), n_scales == 1 && e < bulk8);
-                } else {
-                    q = static_cast<const int8_t *>(src)[e];
-                }
+        // four column steps at a time with their loads issued together: a loop that loads, converts and stores
+        // one step at a time pays one memory round trip per step, and this phase was most of the kernel's time
+        for (int cb = 0; cb < wpatch; cb += 256) {
+            float fv[4];
+            int bv[4];
+            bool in[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int wi = cb + u * 64 + (tid & 63) - g.pad_left;
+                in[u] = row_in && wi >= 0 && wi < g.w && cb + u * 64 + (tid & 63) < wpatch;
+                // unconditional loads (element 0 where the patch cell is halo): a load behind a branch is waited
+                // for before the next one is issued
+                const int64_t a = in[u] ? e0 + wi : 0;
+                fv[u] = 0.f;
+                bv[u] = 0;
+                if (QUANT) fv[u] = static_cast<const float *>(src)[a];
+                else bv[u] = static_cast<const int8_t *>(src)[a];
             }
-            patch[row * wpatch + col] = int8_t(q);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int col = cb + u * 64 + (tid & 63);
+                if (col >= wpatch) continue;
+                int q = g.pad_value;
+                if (in[u]) {
+                    if (QUANT) {
+                        const int64_t e = e0 + (col - g.pad_left);
+                        const float sc = uniform_scale ? img_scale : scales[e / group_len];
+                        q = tsx::quantize_value(__fmul_rn(fv[u], sc), n_scales == 1 && e < bulk8);
+                    } else {
+                        q = bv[u];
+                    }
+                }
+                patch[row * wpatch + col] = int8_t(q);
+            }
         }
     }
     __syncthreads();
