@@ -204,3 +204,47 @@ def test_resnet_shaped_module_in_tennis_workbench_on_hip(ts, tmp_path):
     (fused,) = mf.run_module(mf.fuse_quantized_chains(module), [x])
     assert np.array_equal(bits(own), bits(hip))          # the same device operators, with or without TenniS around them
     assert np.array_equal(bits(fused), bits(own))
+
+
+def test_zipper_option_leaky_relu_and_shared_convolution(ts, tmp_path):
+    """The graph compiler's rewrite on the cases the fixtures do not hold: a chain that ends in leaky_relu behind an
+    add_bias given by `dim`, and a convolution whose output has two readers (a relu and an add_bias), where only
+    quantize + convolution may fold and both readers must stay.  Two chains fused; values as on TenniS's CPU device."""
+    import sys, os
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"))
+    from make_modules import conv_params
+    from tennis_amd import module_file as mf
+    rng = np.random.default_rng(77)
+    n, c, h, w, ca, cb = 2, 16, 9, 11, 12, 20
+    wa = rng.integers(-127, 128, (ca, c, 3, 3)).astype(np.int8)
+    wb = rng.integers(-127, 128, (cb, c, 1, 1)).astype(np.int8)
+    N = mf.Node
+    nodes = [
+        N(mf.PARAMETER, "x"),                                                                                   # 0
+        N("quantize", "q", {"quantize_scale": np.array([7.5, 12.0], np.float32)}, [0]),                          # 1
+        N(mf.CONST, "wa", {"value": wa}),                                                                       # 2
+        N("conv2d_quantized", "conv_a", dict(conv_params((1, 1, 1, 1)),
+                                             dequantize_scales=rng.uniform(1e-4, 1e-3, ca).astype(np.float32)), [1, 2]),   # 3
+        N(mf.CONST, "ba", {"value": rng.standard_normal(ca).astype(np.float32)}),                               # 4
+        N("add_bias", "bias_a", {"dim": np.array([1], np.int32)}, [3, 4]),                                      # 5
+        N("leaky_relu", "act_a", {"scale": np.array([0.1], np.float32)}, [5]),                                  # 6
+        N(mf.CONST, "wb", {"value": wb}),                                                                       # 7
+        N("conv2d_quantized", "conv_b", dict(conv_params((0, 0, 0, 0)),
+                                             dequantize_scales=rng.uniform(1e-3, 1e-2, cb).astype(np.float32)), [1, 7]),   # 8
+        N("relu", "relu_b", {}, [8]),                                                                           # 9
+        N(mf.CONST, "bb", {"value": rng.standard_normal(cb).astype(np.float32)}),                               # 10
+        N("add_bias", "bias_b", {"format": "NCHW"}, [8, 10]),                                                   # 11
+        N("concat", "join", {"dim": np.array([1], np.int32)}, [6, 9, 11]),                                      # 12
+    ]
+    module = mf.Module(nodes, [0], [12])
+    path = str(tmp_path / "zipper_cases.tsm")
+    mf.write_module(path, module)
+    x = (rng.standard_normal((n, c, h, w)) * 6).astype(np.float32)
+    cpu = ts.run_module_intree("cpu", path, [x])
+    fused0 = ts.fused_chain_count_intree()
+    hip = ts.run_module_intree("hip", path, [x])
+    assert ts.fused_chain_count_intree() == fused0 + 2
+    assert cpu.shape == (n, ca + 2 * cb, h, w)
+    assert np.array_equal(bits(hip), bits(cpu))
+    (own,) = mf.run_module(mf.fuse_quantized_chains(module), [x])     # the same rewrite outside TenniS
+    assert np.array_equal(bits(own), bits(cpu))
