@@ -259,9 +259,8 @@ __global__ __launch_bounds__(256) void stage_rows_kernel(const void *__restrict_
         const bool quad_path = row_inside && wl <= 64;
         const int real_words = (creal + 3) / 4;
         // pre-fill: halo value for real channels, zero for channel padding
-        for (int idx = tid; idx < g.ws * (cg / 4); idx += 256) {
-            const int pix = idx / (cg / 4), cw = idx - pix * (cg / 4);
-            if (quad_path && cw < real_words && pix >= g.pad_left && pix < g.pad_left + g.w) continue;
+        const int wpr = cg / 4;   // dwords per pixel
+        auto fill_word = [&](int pix, int cw) {
             uint32_t v = pad4;
             if (cw * 4 + 4 > creal) {
                 v = 0;
@@ -269,8 +268,28 @@ __global__ __launch_bounds__(256) void stage_rows_kernel(const void *__restrict_
                     if (cw * 4 + j < creal) v |= uint32_t(g.pad_value & 0xff) << (8 * j);
             }
             *reinterpret_cast<uint32_t *>(&tile[pix * STAGE_LROW + cw * 4]) = v;
+        };
+        if (quad_path) {
+            // only the halo pixels (left and right of the row) and the channel padding of the interior pixels:
+            // a loop over the whole tile costs a division per dword, as much arithmetic as the row itself
+            const int halo_px = g.ws - g.w;
+            for (int idx = tid; idx < halo_px * wpr; idx += 256) {
+                const int hp = idx / wpr, cw = idx - hp * wpr;
+                fill_word(hp < g.pad_left ? hp : hp + g.w, cw);
+            }
+            const int pad_words = wpr - real_words;
+            if (pad_words > 0)
+                for (int idx = tid; idx < g.w * pad_words; idx += 256) {
+                    const int ip = idx / pad_words;
+                    fill_word(g.pad_left + ip, real_words + idx - ip * pad_words);
+                }
+        } else {
+            for (int idx = tid; idx < g.ws * wpr; idx += 256) {
+                const int pix = idx / wpr;
+                fill_word(pix, idx - pix * wpr);
+            }
+            __syncthreads();
         }
-        if (!quad_path) __syncthreads();
         if (row_inside) {
             if (quad_path) {
                 const StageRow r{src, scales, n_scales, group_len, bulk8, uniform_scale, row_scale, ni, hi, c0, creal};
