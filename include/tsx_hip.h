@@ -130,6 +130,21 @@ int tsx_quantize_conv2d_i8_nchw(const tsx_conv2d_geom *g, const float *x_f32_dev
                                 const tsx_epilogue *ep, float *out_f32_dev, int8_t *out_i8_dev,
                                 int32_t *out_acc_dev, void *workspace_dev, size_t workspace_bytes, void *stream);
 
+/* tsx_quantize_conv2d_i8_nchw for callers that cannot allocate device memory or pass a workspace (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same arguments, kernels and results as tsx_quantize_conv2d_i8_nchw, minus the workspace: the staged copy of
+ * the activations lives in a device array built into the library, TSX_NOALLOC_SCRATCH_BYTES per GPU (held until
+ * the process ends).  A layer whose tsx_conv2d_i8_workspace_bytes() exceeds that is rejected with
+ * TSX_E_WORKSPACE.  The call allocates and frees nothing; its first call on a device looks the array's address
+ * up once.  All calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams, two
+ * threads) race -- serialise them. */
+#define TSX_NOALLOC_SCRATCH_BYTES (8u << 20)
+size_t tsx_noalloc_scratch_bytes(void);
+int tsx_quantize_conv2d_i8_nchw_noalloc(const tsx_conv2d_geom *g, const float *x_f32_dev, const float *x_scales_dev,
+                                        int32_t n_x_scales, const void *packed_w_dev, float padding_value,
+                                        const tsx_epilogue *ep, float *out_f32_dev, int8_t *out_i8_dev,
+                                        int32_t *out_acc_dev, void *stream);
+
 /* The two halves of the calls above, for callers that keep the staged activations around
  * (several convolutions reading one tensor, or timing the MFMA kernel by itself):
  *   stage  : NCHW int8 (x_is_f32 == 0) or NCHW fp32 + quantize (x_is_f32 != 0) -> channel-blocked

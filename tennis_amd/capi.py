@@ -58,6 +58,9 @@ SIGNATURES = {
                                           _vp, _vp, _sz, _vp]),
     "tsx_quantize_conv2d_i8_nchw": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, _i32, _vp, _f32,
                                                    ctypes.POINTER(Epilogue), _vp, _vp, _vp, _vp, _sz, _vp]),
+    "tsx_noalloc_scratch_bytes": (_sz, []),
+    "tsx_quantize_conv2d_i8_nchw_noalloc": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, _i32, _vp, _f32,
+                                                           ctypes.POINTER(Epilogue), _vp, _vp, _vp, _vp]),
     "tsx_conv2d_i8_stage": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _i32, _vp, _i32, _f32, _vp, _sz, _vp]),
     "tsx_conv2d_i8_staged": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, ctypes.POINTER(Epilogue), _vp, _vp,
                                             _vp, _vp]),

@@ -23,6 +23,7 @@
 #include "igemm_i8.hpp"
 
 #include <cmath>
+#include <mutex>
 
 namespace {
 
@@ -1150,6 +1151,58 @@ int tsx_quantize_conv2d_i8_nchw(const tsx_conv2d_geom *g, const float *x_f32_dev
                                 void *workspace_dev, size_t workspace_bytes, void *stream) {
     return run_conv(g, x_f32_dev, true, x_scales_dev, n_x_scales, packed_w_dev, padding_value, ep, out_f32_dev,
                     out_i8_dev, out_acc_dev, workspace_dev, workspace_bytes, stream);
+}
+
+// ---- the allocation-free variant: the staging workspace is a file-scope device array
+//
+// Every device the library runs on holds its own copy of `scratch` at its own address until the process
+// ends.  In host code the array's name is only a handle for hipGetSymbolAddress: the address kernels and
+// copies may use is looked up once per device, with that device current, and kept in scratch_ptr[].
+static __device__ __align__(256) unsigned char scratch[TSX_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_mutex;
+void *scratch_ptr[MAX_DEVICES] = {nullptr};
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int scratch_on_current_device(void **out) {
+    int dev = -1;
+    TSX_HIP(hipGetDevice(&dev));
+    TSX_REQUIRE(dev >= 0 && dev < MAX_DEVICES, "noalloc: device ordinal %d out of range", dev);
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        TSX_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        TSX_REQUIRE(ptr && reinterpret_cast<uintptr_t>(ptr) % 256 == 0, "noalloc: bad scratch address");
+        scratch_ptr[dev] = ptr;
+    }
+    *out = scratch_ptr[dev];
+    return 0;
+}
+}  // namespace
+
+size_t tsx_noalloc_scratch_bytes(void) { return TSX_NOALLOC_SCRATCH_BYTES; }
+
+int tsx_quantize_conv2d_i8_nchw_noalloc(const tsx_conv2d_geom *g, const float *x_f32_dev, const float *x_scales_dev,
+                                        int32_t n_x_scales, const void *packed_w_dev, float padding_value,
+                                        const tsx_epilogue *ep, float *out_f32_dev, int8_t *out_i8_dev,
+                                        int32_t *out_acc_dev, void *stream) {
+    Plan pl;
+    int rc = make_plan(g, &pl);
+    if (rc) return rc;
+    if (pl.staged_bytes > size_t(TSX_NOALLOC_SCRATCH_BYTES))
+        return tsx::fail(TSX_E_WORKSPACE,
+                         "quantize_conv2d_i8_noalloc: this layer stages %zu bytes, the built-in scratch holds %zu; "
+                         "use tsx_quantize_conv2d_i8_nchw with a caller workspace",
+                         pl.staged_bytes, size_t(TSX_NOALLOC_SCRATCH_BYTES));
+    void *ws = nullptr;
+    rc = scratch_on_current_device(&ws);
+    if (rc) return rc;
+    // The staging kernel writes every byte of the staged extent the MFMA kernel reads (halo and channel
+    // padding included), so nothing of the previous call's contents has to be cleared.
+    return run_conv(g, x_f32_dev, true, x_scales_dev, n_x_scales, packed_w_dev, padding_value, ep, out_f32_dev,
+                    out_i8_dev, out_acc_dev, ws, size_t(TSX_NOALLOC_SCRATCH_BYTES), stream);
 }
 
 int tsx_conv2d_i8_stage(const tsx_conv2d_geom *g, const void *x_dev, int32_t x_is_f32, const float *x_scales_dev,
