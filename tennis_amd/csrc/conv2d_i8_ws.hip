@@ -150,6 +150,7 @@ WsPlan ws_plan(const WsGeom &g_in) {
     pl.coutp = coutp;
     pl.packed_bytes = size_t(pl.ksteps_p) * pl.coutp * 64;
     pl.ok = true;
+    fl_plan(g_in, &pl);   // layers the flat-tile kernel suits better (same packed weights)
     return pl;
 }
 
@@ -163,6 +164,7 @@ int ws_pack_weights(const WsGeom &g, const WsPlan &pl, const int8_t *w_oihw, int
 
 int ws_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t *packed, const EpiParams &ep,
               hipStream_t stream) {
+    if (pl.flat) return fl_launch(g, pl, xs, packed, ep, stream);
     WsParams p{};
     static_cast<EpiParams &>(p) = ep;
     p.xs = xs;

@@ -139,6 +139,11 @@ struct WsPlan {
     int ksteps_p;       // K-steps padded to the A-ring size
     int coutp;          // cout padded to the workgroup's channels (32 x wm)
     size_t packed_bytes;
+    // flat-tile kernel (conv2d_i8_fl.hip) instead: a tile is fl_nta + fl_ntb consecutive fragments of the
+    // batch-wide flat position list; same packed weights
+    bool flat, fl_resident;
+    int fl_nta, fl_ntb, fl_wr, fl_wc, fl_wp, fl_rowp;
+    int64_t fl_tiles;
 };
 
 struct WsGeom {
@@ -151,6 +156,10 @@ struct WsGeom {
 WsPlan ws_plan(const WsGeom &g);
 int ws_pack_weights(const WsGeom &g, const WsPlan &pl, const int8_t *w_oihw, int c, int8_t *packed, hipStream_t stream);
 int ws_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t *packed, const EpiParams &ep,
+              hipStream_t stream);
+// flat-tile kernel: fills the fl_* fields of a valid plan when the layer suits it; launch
+void fl_plan(const WsGeom &g, WsPlan *pl);
+int fl_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t *packed, const EpiParams &ep,
               hipStream_t stream);
 
 }  // namespace tsx
