@@ -30,7 +30,14 @@ void *hip_allocator(int id, size_t new_size, void *mem, size_t mem_size) {
         return nullptr;
     }
     void *fresh = nullptr;
-    hip_check(hipMalloc(&fresh, new_size), "hipMalloc");
+    const hipError_t err = hipMalloc(&fresh, new_size);
+    if (err == hipErrorOutOfMemory || (err == hipSuccess && fresh == nullptr)) {
+        (void)hipGetLastError();   // the failed allocation must not show up at the next launch check
+        // what the reference's allocators throw (src/kernels/gpu/memory_gpu.cpp:54), so that callers that
+        // catch it (and Workbench's memory-pressure handling) see the same type from this device
+        throw OutOfMemoryException(MemoryDevice(DEVICE, id), new_size);
+    }
+    hip_check(err, "hipMalloc");
     if (mem) {
         const size_t keep = mem_size < new_size ? mem_size : new_size;
         if (keep) hip_check(hipMemcpy(fresh, mem, keep, hipMemcpyDeviceToDevice), "hipMemcpy");
@@ -52,6 +59,29 @@ void copy(void *dst, const void *src, size_t size, hipMemcpyKind kind, int devic
 void hip_from_cpu(int dst_id, void *dst, int, const void *src, size_t size) { copy(dst, src, size, hipMemcpyHostToDevice, dst_id); }
 void cpu_from_hip(int, void *dst, int src_id, const void *src, size_t size) { copy(dst, src, size, hipMemcpyDeviceToHost, src_id); }
 void hip_from_hip(int dst_id, void *dst, int, const void *src, size_t size) { copy(dst, src, size, hipMemcpyDeviceToDevice, dst_id); }
+
+}  // namespace
+
+int HostDelegate::run(Operator &self, Stack &stack) {
+    if (!m_host) {
+        Operator::shared host;
+        try {
+            host = OperatorCreator::Create(CPU, self.op(), true);
+        } catch (const Exception &) {
+            host = nullptr;
+        }
+        if (!host)
+            TS_LOG_ERROR << "[hip] " << self.op() << ": these inputs need the host operator, and no \"cpu\" operator "
+                         << "of that name is registered in this build" << eject;
+        // as OperatorInstruction::clone does (src/runtime/instruction.cpp:91-103): same parameters, then init()
+        for (auto &param : self.params()) host->set(param.first, param.second);
+        host->init();
+        m_host = host;
+    }
+    return m_host->run(stack);
+}
+
+namespace {
 
 void hip_admin(DeviceHandle **handle, int device_id, DeviceAdmin::Action action) {
     auto **h = reinterpret_cast<HipContextHandle **>(handle);

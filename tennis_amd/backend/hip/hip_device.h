@@ -21,11 +21,36 @@ void *current_stream();
 // (include/kernels/gpu/gpu_kernel.h:13-19).
 void check(int tsx_rc, const char *what);
 
+// The host operator of the same name, created on first use with the same parameters.  TenniS falls back to
+// the host only for operators a device does not register at all (src/global/operator_factory.cpp:60-81); a
+// registered "hip" class that meets a data type, format or mode its kernel does not cover hands the call to
+// this delegate instead of failing, so a graph that ran on the host keeps running on the device: inputs
+// reach the host through Tensor::view, the result is a host tensor the next operator views back.
+class HostDelegate {
+public:
+    int run(Operator &self, Stack &stack);
+
+private:
+    Operator::shared m_host;
+};
+
 template <typename OP>
 class OperatorOnHip : public OP {
 public:
     MemoryDevice running_memory_device() override { return MemoryDevice(DEVICE, current_device_id()); }
     static int current_device_id();
+
+    int run(Stack &stack) override {
+        if (!covers(stack)) return m_delegate.run(*this, stack);
+        return OP::run(stack);
+    }
+
+protected:
+    // false: the inputs on the stack need the host operator (see HostDelegate)
+    virtual bool covers(Stack &) { return true; }
+
+private:
+    HostDelegate m_delegate;
 };
 
 int context_device_id();

@@ -30,6 +30,18 @@ inline tsx_conv2d_geom make_geom(const Tensor &x, const Tensor &w, const Padding
     return g;
 }
 
+// Predicates for OperatorOnHip::covers: what the kernels behind a "hip" class take.
+inline bool inputs_are(Stack &stack, size_t count, DTYPE dtype) {
+    if (stack.size() < count) return true;   // let the skeleton report the wrong input count
+    for (size_t i = 0; i < count; ++i)
+        if (stack[int(i)].dtype() != dtype) return false;
+    return true;
+}
+
+inline bool format_is_nchw(const Operator &op) {
+    return !op.has(name::format) || tensor::to_string(op.get(name::format)) == name::NCHW;
+}
+
 // Host vector -> device tensor, cached while the host values stay the same (parameters such as
 // quantize_scale / dequantize_scales are fixed at init(); the reference hands them to the core by
 // value on every run).

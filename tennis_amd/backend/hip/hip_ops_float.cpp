@@ -28,6 +28,11 @@ public:
                                   out.data<float>(), current_stream()),
               "tsx_conv2d_f32_nchw");
     }
+
+protected:
+    // fp32 NCHW on the MFMA kernel; fp64 and NHWC graphs (the reference's device classes take both,
+    // src/kernels/gpu/conv2d_core.cu) run the host operator
+    bool covers(Stack &stack) override { return format_is_nchw(*this) && inputs_are(stack, 2, FLOAT32); }
 };
 
 // ---------------------------------------------------------------- conv2d_winograd (fp32, F(6,3) and F(2,3))
@@ -91,6 +96,9 @@ public:
                   "tsx_conv2d_winograd_f63_nchw");
     }
 
+protected:
+    bool covers(Stack &stack) override { return format_is_nchw(*this) && inputs_are(stack, 2, FLOAT32); }
+
 private:
     Tensor m_u;          // transformed kernel, [64 or 16][cout][cin], device memory
     Tensor m_workspace;
@@ -108,6 +116,9 @@ public:
                                  out.data<float>(), current_stream()),
               "tsx_inner_prod_f32");
     }
+
+protected:
+    bool covers(Stack &stack) override { return inputs_are(stack, 2, FLOAT32); }
 };
 
 // ---------------------------------------------------------------- add_bias / relu / leaky_relu
@@ -122,6 +133,9 @@ public:
                                current_stream()),
               "tsx_add_bias_f32");
     }
+
+protected:
+    bool covers(Stack &stack) override { return inputs_are(stack, 2, FLOAT32); }
 };
 
 class ReLU : public OperatorOnHip<base::Activation> {
@@ -130,6 +144,9 @@ public:
         if (x.dtype() != FLOAT32) TS_LOG_ERROR << this->op() << " not support data type: " << type_str(x.dtype()) << eject;
         check(tsx_relu_f32(x.data<float>(), x.count(), out.data<float>(), current_stream()), "tsx_relu_f32");
     }
+
+protected:
+    bool covers(Stack &stack) override { return inputs_are(stack, 1, FLOAT32); }
 };
 
 class LeakyReLU : public OperatorOnHip<base::LeakyReLU> {
@@ -138,6 +155,9 @@ public:
         if (x.dtype() != FLOAT32) TS_LOG_ERROR << this->op() << " not support data type: " << type_str(x.dtype()) << eject;
         check(tsx_leaky_relu_f32(x.data<float>(), x.count(), scale, out.data<float>(), current_stream()), "tsx_leaky_relu_f32");
     }
+
+protected:
+    bool covers(Stack &stack) override { return inputs_are(stack, 1, FLOAT32); }
 };
 
 }  // namespace hip

@@ -35,6 +35,10 @@ public:
                    const Size2D &ksize, const Stride2D &stride, Conv2DFormat format, Tensor &out) override {
         pool_nchw("Pooling2D", x, type, padding, padding_type, ksize, stride, format, out);
     }
+
+protected:
+    // the kernel pools fp32 [planes][h][w] maps: NHWC graphs and other element types run the host operator
+    bool covers(Stack &stack) override { return format_is_nchw(*this) && inputs_are(stack, 1, FLOAT32); }
 };
 
 class GlobalPooling2D : public OperatorOnHip<base::GlobalPooling2D> {
@@ -43,6 +47,9 @@ public:
                    const Size2D &ksize, const Stride2D &stride, Conv2DFormat format, Tensor &out) override {
         pool_nchw("GlobalPooling2D", x, type, padding, padding_type, ksize, stride, format, out);
     }
+
+protected:
+    bool covers(Stack &stack) override { return format_is_nchw(*this) && inputs_are(stack, 1, FLOAT32); }
 };
 
 // add: equal shapes take the vectorised pass; every other case of ElementWiseReduce::run (scalar,
@@ -66,6 +73,11 @@ public:
                                     current_stream()),
               "tsx_add_broadcast_f32");
     }
+
+protected:
+    // the reference's device classes take every numeric type (src/kernels/gpu/add.cu:211-214); the kernels
+    // here are fp32, anything else (an int32 index sum, fp64) runs the host operator
+    bool covers(Stack &stack) override { return inputs_are(stack, 2, FLOAT32); }
 
 private:
     static void check_type(const Tensor &out) {
@@ -92,6 +104,9 @@ public:
               "tsx_mul_broadcast_f32");
     }
 
+protected:
+    bool covers(Stack &stack) override { return inputs_are(stack, 2, FLOAT32); }
+
 private:
     static void check_type(const Tensor &out) {
         if (out.dtype() != FLOAT32) TS_LOG_ERROR << "[hip] mul not support data type(" << out.dtype() << "): " << type_str(out.dtype()) << eject;
@@ -106,6 +121,9 @@ public:
         if (x.dtype() != FLOAT32) TS_LOG_ERROR << "[hip] softplus not support data type: " << type_str(x.dtype()) << eject;
         check(tsx_softplus_f32(x.data<float>(), x.count(), out.data<float>(), current_stream()), "tsx_softplus_f32");
     }
+
+protected:
+    bool covers(Stack &stack) override { return inputs_are(stack, 1, FLOAT32); }
 };
 
 class Tanh : public OperatorOnHip<base::Activation> {
@@ -114,6 +132,9 @@ public:
         if (x.dtype() != FLOAT32) TS_LOG_ERROR << "[hip] tanh not support data type: " << type_str(x.dtype()) << eject;
         check(tsx_tanh_f32(x.data<float>(), x.count(), out.data<float>(), current_stream()), "tsx_tanh_f32");
     }
+
+protected:
+    bool covers(Stack &stack) override { return inputs_are(stack, 1, FLOAT32); }
 };
 
 // depthwise_conv2d: weights [1, C, KH, KW]; the core signature is base::Conv2D's.
@@ -131,6 +152,9 @@ public:
                                        out.data<float>(), current_stream()),
               "tsx_depthwise_conv2d_f32");
     }
+
+protected:
+    bool covers(Stack &stack) override { return format_is_nchw(*this) && inputs_are(stack, 2, FLOAT32); }
 };
 
 // concat along any axis: every input is one strided copy [outer][extent_i * inner] into its slot of the
@@ -153,6 +177,14 @@ public:
             offset += extent;
         }
     }
+
+protected:
+    // blocks of 4-byte elements; other element sizes (int8 maps, fp64) are concatenated by the host operator
+    bool covers(Stack &stack) override {
+        for (size_t i = 1; i < stack.size(); ++i)
+            if (stack[int(i)].dtype() != stack[0].dtype()) return true;   // the skeleton rejects mixed types
+        return stack.size() == 0 || type_bytes(stack[0].dtype()) == 4;
+    }
 };
 
 // _resize2d: the nearest-neighbour mode on the two innermost axes (NCHW maps, the upsampling of detection necks).
@@ -168,6 +200,21 @@ public:
         check(tsx_resize_nearest_f32(x.data<float>(), planes, x.size(size_t(dim)), x.size(size_t(dim) + 1), out.data<float>(),
                                      out.size(size_t(dim)), out.size(size_t(dim) + 1), current_stream()),
               "tsx_resize_nearest_f32");
+    }
+
+protected:
+    // nearest-neighbour resizing of the two innermost axes of an fp32 tensor; the interpolating modes
+    // (LINEAR, CUBIC, HARD) and other layouts run the host operator (src/kernels/cpu/resize2d.cpp)
+    bool covers(Stack &stack) override {
+        if (Resize2DType(tensor::to_int(get(name::type))) != Resize2DType::NEAREST) return false;
+        if (stack.size() != 2 || stack[0].dtype() != FLOAT32) return false;
+        std::vector<Tensor::Prototype> out;
+        infer(stack, out);
+        const Shape &from = stack[0].sizes(), &to = out[0].sizes();
+        if (from.size() < 2 || from.size() != to.size()) return false;
+        for (size_t i = 0; i + 2 < from.size(); ++i)
+            if (from[i] != to[i]) return false;
+        return true;
     }
 };
 

@@ -25,6 +25,10 @@ public:
               "tsx_quantize_f32_i8");
     }
 
+protected:
+    // cpu::Quantize also takes fp64 input (src/kernels/cpu/quantize.cpp:109-125): that runs the host operator
+    bool covers(Stack &stack) override { return inputs_are(stack, 1, FLOAT32); }
+
 private:
     DeviceFloats m_scales;
 };

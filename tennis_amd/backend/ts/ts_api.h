@@ -228,6 +228,23 @@ private:
 };
 std::string to_string(const Shape &shape);
 
+// Thrown by a HardAllocator that cannot serve a request (include/global/hard_allocator.h:20-44).
+class OutOfMemoryException : public Exception {
+public:
+    explicit OutOfMemoryException(const MemoryDevice &device, size_t failed_size)
+        : Exception(OutOfMemoryMessage(device, failed_size)), m_device(device), m_failed_size(failed_size) {}
+    static std::string OutOfMemoryMessage(const MemoryDevice &device, size_t failed_size) {
+        return "No enough memory on " + std::string(device.type().c_str()) + ":" + std::to_string(device.id()) + ", " +
+               std::to_string(failed_size) + "B needed.";
+    }
+    const Device &device() const { return m_device; }
+    size_t failed_size() const { return m_failed_size; }
+
+private:
+    MemoryDevice m_device;
+    size_t m_failed_size;
+};
+
 // One allocation on one device, released through the device's HardAllocator.
 class Memory {
 public:

@@ -212,6 +212,15 @@ class StagedPlain:
         self.buf = torch.zeros(n * h * w * self.cp, dtype=torch.int8, device=device)
 
 
+def staged_interior(staged, images):
+    """The map inside a staged buffer (StagedInput / StagedPlain) as an int8 NCHW tensor of the given images:
+    a copy, for checkers that compare a producer's requantized hand-over with the operator chain's values."""
+    n, c, h, w = staged.x_shape
+    t = staged.buf[: n * staged.hs * staged.ws * staged.cp].view(n, staged.hs, staged.ws, staged.cp)
+    t = t[list(images), staged.pad_top:staged.pad_top + h, staged.pad_left:staged.pad_left + w, :c]
+    return t.permute(0, 3, 1, 2).contiguous()
+
+
 class Conv2dI8:
     """int8 conv2d with packed weights: the state a `conv2d_quantized` operator instance keeps.
 

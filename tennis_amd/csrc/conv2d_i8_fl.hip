@@ -30,10 +30,16 @@ void fl_plan(const WsGeom &g, WsPlan *pl) {
     if (disabled) return;
     const int64_t positions = int64_t(g.n) * g.ho * g.wo;
     if (positions >= (int64_t(1) << 31) - 256) return;
+    if (pl->packed_bytes >= (size_t(1) << 31)) return;   // the kernel addresses the weights with 32-bit offsets
     const int wrap = g.hs - g.ho * g.sh;
     const int wc = (g.wo - 1) * g.sw + (g.kw - 1) * g.dil_w + 1;
     if (wc > g.ws) return;
-    static const int splits[7][2] = {{1, 1}, {2, 1}, {2, 2}, {3, 2}, {3, 3}, {4, 3}, {4, 4}};
+    // Measured against the window-stationary kernel, the flat tiles pay on large layers that fill most of the
+    // chip with tiles of 6 to 8 fragments in one round (BASELINE config 2: 24.9 -> 23.4 us; the large 3x3
+    // layers of the YOLOv4-shaped network); small maps (ResNet's 14x14 and 7x7 layers, under 200 workgroups of
+    // short tiles) run 1-20 % slower on it and stay where they were.  The smaller splits remain instantiated
+    // for the planner to use once that changes.
+    static const int splits[3][2] = {{3, 3}, {4, 3}, {4, 4}};
     // One workgroup per CU: the busiest CU's time, in units of one fragment x 32 channels on one SIMD, is
     //     rounds x (fixed + F)
     // -- the same form as the window-stationary plan's model, whose workgroups pair up on a CU.
@@ -55,6 +61,7 @@ void fl_plan(const WsGeom &g, WsPlan *pl) {
         if (wp > FL_MAX_WP || size_t(2) * wr * rowp > size_t(FL_MAX_LDS)) continue;
         const int64_t tiles = (positions + f * 32 - 1) / (f * 32);
         const int64_t wgs = tiles * (pl->coutp / 128);
+        if (wgs < 160) continue;
         const double cost = double((wgs + 255) / 256) * (0.75 + f);
         if (best < 0 || cost < best) {
             best = cost;

@@ -109,16 +109,22 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
         b_base[j] = wrow * p.rowp + ow * p.sw * FL_PIX + (lane / 32) * 16;
     });
 
-    // ---- A ring: 2 halves of K-step ks for the wavefront's 32 output channels, 1 KiB each
-    const int8_t *a_ptr = p.wp + (int64_t(m0 / 32) * 128 + lane) * 16;
-    const int64_t a_kstride = int64_t(p.coutp / 32) * 128 * 16;
+    // ---- A ring: 2 halves of K-step ks for the wavefront's 32 output channels, 1 KiB each.  Buffer loads:
+    // descriptor and K-step offset stay in scalar registers, the lane supplies one constant 32-bit offset
+    // (per-lane 64-bit addresses cost a 64-bit multiply-add per load and measurably more time and power).
+    const int frag_u = __builtin_amdgcn_readfirstlane(m0 / 32);
+    const __amdgpu_buffer_rsrc_t a_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(p.wp), 0, 0x7fffffff, 0x00020000);
+    const int a_lane = lane * 16;
+    const int a_frag = frag_u * 2048;
+    const int a_kstride = (p.coutp / 32) * 2048;   // packed weights are below 2 GiB (checked by the launcher)
     v4i areg[FL_RING][2];
     auto a_load = [&](auto slot, int ks) __attribute__((always_inline)) {
         constexpr int s = decltype(slot)::value;
         if (ks >= p.ksteps_p) ks = p.ksteps_p - 1;
-        const int8_t *src = a_ptr + ks * a_kstride;
-        areg[s][0] = *reinterpret_cast<const v4i *>(src);
-        areg[s][1] = *reinterpret_cast<const v4i *>(src + 1024);
+        const int so = a_frag + ks * a_kstride;
+        areg[s][0] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_lane, so, 0));
+        areg[s][1] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_lane, so + 1024, 0));
     };
 
     v16i acc[NT];

@@ -126,6 +126,21 @@ class ResNet50Int8:
         self.scales = None      # name -> python float (multiplier applied before rounding)
         self._dq, self._sx = {}, {}
         self._staged = {}      # (conv name, input shape) -> StagedInput
+        # set to (images, list) to record, per convolution of the chained pass, the tensors it read and wrote for
+        # those images of the batch (copies; for per-layer checks against the operator chain)
+        self.trace = None
+
+    def _rec(self, spec, s_in=None, x=None, residual=None, out_f32=None, s_out=None, q_name=None):
+        if self.trace is None:
+            return
+        imgs, rows = self.trace
+        idx = list(imgs)
+        rows.append({"spec": spec, "in_q": None if s_in is None else capi.staged_interior(s_in, idx).cpu().numpy(),
+                     "in_f32": None if x is None else x[idx].cpu().numpy(),
+                     "residual": None if residual is None else residual[idx].cpu().numpy(),
+                     "out_f32": None if out_f32 is None else out_f32[idx].cpu().numpy(),
+                     "out_q": None if s_out is None else capi.staged_interior(s_out, idx).cpu().numpy(),
+                     "q_name": q_name})
 
     # ---- calibration: per-tensor scale = 127 / max|input of the layer| on this batch, measured on the
     # activations of the quantized network itself, layer by layer
@@ -191,6 +206,9 @@ class ResNet50Int8:
             hp, wp = capi.pool_out_size(h1, w1, self.POOL[0], self.POOL[2], self.POOL[1])
             s_in = self._staged_input(c1, (n, stem.cout, hp, wp))
             capi.max_pooling2d_staged(s_stem, s_in, *self.POOL)
+            self._rec(stem, x=x, s_out=s_stem, q_name=c1.name)
+            if self.trace is not None:
+                self.trace[1].append({"spec": "pool", "out_q": capi.staged_interior(s_in, list(self.trace[0])).cpu().numpy()})
             y = None
         else:
             y = self.conv[stem.name](x, dq=self._dq[stem.name], bias=self.bias[stem.name], act=relu(stem),
@@ -202,22 +220,28 @@ class ResNet50Int8:
             conv1, conv2, conv3 = self.conv[c1.name], self.conv[c2.name], self.conv[c3.name]
             in_shape = s_in.x_shape
             sc = y if proj is None else self.conv[proj.name].run_staged(s_in, self._dq[proj.name], self.bias[proj.name])[0]
+            if proj is not None:
+                self._rec(proj, s_in=s_in, out_f32=sc)
             s2 = self._staged_input(c2, (n, c1.cout, in_shape[2], in_shape[3]))
             conv1.run_staged(s_in, self._dq[c1.name], self.bias[c1.name], relu(c1), q_scales=sxs[c2.name], want_f32=False,
                              staged_out=s2)
+            self._rec(c1, s_in=s_in, s_out=s2, q_name=c2.name)
             h2 = (in_shape[2] + 2 * c2.pad - c2.k) // c2.stride + 1
             w2 = (in_shape[3] + 2 * c2.pad - c2.k) // c2.stride + 1
             s3 = self._staged_input(c3, (n, c2.cout, h2, w2))
             conv2.run_staged(s2, self._dq[c2.name], self.bias[c2.name], relu(c2), q_scales=sxs[c3.name], want_f32=False,
                              staged_out=s3)
+            self._rec(c2, s_in=s2, s_out=s3, q_name=c3.name)
             if bi + 1 < len(net):
                 nxt = net[bi + 1][0]
                 s_next = self._staged_input(nxt, (n, c3.cout, h2, w2))
                 y = conv3.run_staged(s3, self._dq[c3.name], self.bias[c3.name], "relu", q_scales=sxs[nxt.name],
                                      residual=sc, staged_out=s_next)[0]
+                self._rec(c3, s_in=s3, residual=sc, out_f32=y, s_out=s_next, q_name=nxt.name)
                 s_in = s_next
             else:
                 y = conv3.run_staged(s3, self._dq[c3.name], self.bias[c3.name], "relu", residual=sc)[0]
+                self._rec(c3, s_in=s3, residual=sc, out_f32=y)
         pooled = capi.global_pooling2d(y, "avg").reshape(n, fc[0])
         p8 = capi.quantize(pooled, sxs["fc"])
         return self.fc(p8, dq=self._dq["fc"], bias=self.bias["fc"])[0]

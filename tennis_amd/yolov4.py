@@ -167,6 +167,9 @@ class YoloV4Int8:
             self.bias[i] = torch.from_numpy(p["bias"]).to(self.dev)
         self.scales = None
         self._shapes = {}
+        # set to (images, list) to record, per convolution of the chained pass, the tensors it read and wrote for
+        # those images of the batch (copies; for per-layer checks against the operator chain)
+        self.trace = None
 
     def set_scales(self, scales, n):
         self.scales = dict(scales)
@@ -275,6 +278,16 @@ class YoloV4Int8:
                     y = conv.run_staged(staged_for[i], **kw)[0]
                 else:
                     y = conv(get(src), x_scales=self.sx[i], **kw)[0]
+                if self.trace is not None:
+                    idx = list(self.trace[0])
+                    res = kw.get("residual")
+                    self.trace[1].append({
+                        "layer": i, "in_q": capi.staged_interior(staged_for[i], idx).cpu().numpy() if i in staged_for else None,
+                        "in_f32": None if i in staged_for else get(src)[idx].cpu().numpy(),
+                        "residual": None if res is None else res[idx].cpu().numpy(),
+                        "out_f32": None if y is None else y[idx].cpu().numpy(),
+                        "out_q": None if target is None else capi.staged_interior(target, idx).cpu().numpy(),
+                        "q_layer": served[0] if served else None})
                 outs[out_id] = y
                 if out_id != i:
                     outs[i] = None

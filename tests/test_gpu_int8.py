@@ -459,3 +459,30 @@ def test_gemm_i8_largest_sweep_shape_by_rows(tsx, port):
     # checksum of checksums over the whole product: column sums of acc = (sum of rows of a) . b
     colsum = acc.cpu().numpy().astype(np.int64).sum(axis=0)
     assert np.array_equal(colsum, a.astype(np.int64).sum(axis=0) @ b.astype(np.int64))
+
+
+@pytest.mark.parametrize("k", [1024, 2048, 4096])
+@pytest.mark.parametrize("m", [1, 32, 256, 4096])
+def test_gemm_i8_whole_sweep(tsx, port, m, k):
+    """Every shape of the GEMM sweep (M in {1, 32, 256, 4096}, K = N in {1024, 2048, 4096}) as the bench calls
+    it: per-row and per-channel dequantize scales, bias, fp32 output only (the kernel each shape takes is the
+    one it takes there).  All rows up to 256; above, 64 random rows against the oracle plus a checksum of the
+    whole output against the rows' sum in float64 (rows are independent)."""
+    n = k
+    rng = np.random.default_rng(400 + m + k)
+    a = rng.integers(-128, 128, (m, k)).astype(np.int8)
+    b = rng.integers(-128, 128, (k, n)).astype(np.int8)
+    dqw = rng.uniform(1e-3, 1e-2, n).astype(np.float32)
+    dqa = rng.uniform(1e-3, 1e-2, m).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    g = tsx.GemmI8(_dev(b))
+    out, _, _ = g(_dev(a), dq=_dev(dqw), row_scale=_dev(dqa), bias=_dev(bias))
+    got = out.cpu().numpy()
+    rows = np.arange(m) if m <= 256 else np.sort(rng.choice(m, 64, replace=False))
+    exp = port.gemm_i8_dequant(a[rows], b, dqw, dqa[rows], bias)
+    assert np.array_equal(bits(got[rows]), bits(exp))
+    if m > 256:
+        # every row: the exact integer products through numpy, then the same three roundings
+        acc = a.astype(np.float64) @ b.astype(np.float64)          # exact: |acc| < 2^53
+        ref = ((acc.astype(np.float32) * dqw[None, :]) * dqa[:, None] + bias[None, :]).astype(np.float32)
+        assert np.array_equal(bits(got), bits(ref))

@@ -248,3 +248,56 @@ def test_zipper_option_leaky_relu_and_shared_convolution(ts, tmp_path):
     assert np.array_equal(bits(hip), bits(cpu))
     (own,) = mf.run_module(mf.fuse_quantized_chains(module), [x])     # the same rewrite outside TenniS
     assert np.array_equal(bits(own), bits(cpu))
+
+
+def test_inputs_a_hip_class_does_not_cover_run_the_host_operator(ts):
+    """A registered "hip" class that meets a data type or mode its kernel does not take hands the call to the
+    host operator of the same name (TenniS itself falls back only for operators a device does not register):
+    graphs that ran on "cpu" keep running on "hip", with the host's results bit for bit.  Strict device
+    lookup, so it is the "hip" class that is created and delegates."""
+    rng = np.random.default_rng(905)
+
+    def same(op, params, inputs, out_bytes):
+        cpu = ts.run_op_intree("cpu", op, params, inputs, out_bytes)
+        hip = ts.run_op_intree("hip", op, params, inputs, out_bytes, strict=True)
+        assert cpu.shape == hip.shape and cpu.dtype == hip.dtype, (op, cpu.dtype, hip.dtype)
+        assert np.array_equal(cpu.view(np.uint8), hip.view(np.uint8)), op
+        return cpu
+
+    a = rng.integers(-1000, 1000, (2, 3, 5, 7)).astype(np.int32)
+    b = rng.integers(-1000, 1000, (1, 3, 1, 1)).astype(np.int32)
+    assert same("add", {}, [a, b], a.nbytes).dtype == np.int32
+    assert same("mul", {}, [a, a], a.nbytes).dtype == np.int32
+    d = rng.standard_normal((2, 3, 5, 7))
+    assert same("add", {}, [d, d[::-1].copy()], d.nbytes).dtype == np.float64
+    # interpolating resize (type 0 = LINEAR, 1 = CUBIC): the device kernel is nearest-neighbour only
+    x = rng.standard_normal((2, 3, 9, 8)).astype(np.float32)
+    size = np.array([-1, -1, 17, 13], np.int32)
+    for kind in (0, 1, 2):
+        out = same("_resize2d", {"type": np.array([kind], np.int32)}, [x, size], 4 * 2 * 3 * 17 * 13)
+        assert out.shape == (2, 3, 17, 13)
+    # fp64 convolution and inner product
+    xd = rng.uniform(-1, 1, (2, 5, 9, 8))
+    wd = rng.standard_normal((7, 5, 3, 3)) * 0.1
+    out = same("conv2d", conv_params(ts, (1, 1, 1, 1)), [xd, wd], 8 * 2 * 7 * 9 * 8)
+    assert out.dtype == np.float64 and out.shape == (2, 7, 9, 8)
+    # (no fp64 inner_prod here: the reference's own leaves parts of its output unwritten on any device)
+    bd = rng.standard_normal(7)
+    assert same("add_bias", {"dim": np.array([1], np.int32)}, [out, bd], out.nbytes).dtype == np.float64
+    # int8 concat (1-byte elements)
+    q1 = rng.integers(-128, 128, (2, 3, 4, 5)).astype(np.int8)
+    q2 = rng.integers(-128, 128, (2, 6, 4, 5)).astype(np.int8)
+    assert same("concat", {"dim": np.array([1], np.int32)}, [q1, q2], 2 * 9 * 4 * 5).shape == (2, 9, 4, 5)
+    # fp64 activations
+    assert same("relu", {}, [d], d.nbytes).dtype == np.float64
+    # a case neither side supports fails the same way on both: NHWC pooling (pooling2d_core.cpp:234)
+    p = {"format": "NHWC", "type": np.array([0], np.int32),
+         "padding": np.array([[0, 0], [0, 0], [0, 0], [0, 0]], np.int32), "padding_type": np.array([0], np.int32),
+         "ksize": np.array([1, 2, 2, 1], np.int32), "stride": np.array([1, 2, 2, 1], np.int32)}
+    xn = rng.standard_normal((1, 8, 8, 3)).astype(np.float32)
+    errors = []
+    for device in ("cpu", "hip"):
+        with pytest.raises(RuntimeError) as e:
+            ts.run_op_intree(device, "pooling2d", p, [xn], xn.nbytes)
+        errors.append(str(e.value).split("only support")[-1])
+    assert errors[0] == errors[1] and "NCHW" in errors[0]

@@ -82,6 +82,52 @@ def test_resnet_shaped_network_bit_exact(port):
         torch.cuda.synchronize()
 
 
+def test_full_size_network_every_layer(port):
+    """BASELINE config 4 at its real size (batch 32, 3x224x224, full width and depth): the tile plans the
+    kernels pick here differ from the small network's.  Every convolution of the chained pass is checked by
+    itself for the first and the last image of the batch: the oracle runs the operator chain on the very
+    tensor the device kernel read (its staged int8 input), so one layer's result does not depend on another's.
+    Bar: bit-exact fp32 outputs and int8 hand-overs."""
+    import torch
+    from tennis_amd import resnet50
+    n = 32
+    desc, params = resnet50.make_parameters(seed=0)
+    net = resnet50.ResNet50Int8(desc, params)
+    x = torch.rand((n, 3, 224, 224), device="cuda", generator=torch.Generator(device="cuda").manual_seed(11))
+    scales = net.calibrate(x)
+    net.set_scales(scales, n)
+    imgs = (0, n - 1)
+    net.trace = (imgs, [])
+    logits = net.forward(x)
+    torch.cuda.synchronize()
+    rows, net.trace = net.trace[1], None
+    assert torch.isfinite(logits).all()
+    checked, prev_q = 0, None
+    for row in rows:
+        spec = row["spec"]
+        if spec == "pool":
+            pooled = port.pooling2d(prev_q.astype(np.float32), "max", (3, 3), (2, 2), (0, 1, 0, 1)).astype(np.int8)
+            assert np.array_equal(row["out_q"], pooled), "max pooling on int8"
+            continue
+        p = params[spec.name]
+        s = np.float32(scales[spec.name])
+        xq = row["in_q"] if row["in_q"] is not None else port.quantize(row["in_f32"], np.full(len(imgs), s, np.float32))
+        dq = (np.float32(1.0) / (s * p["sw"])).astype(np.float32)
+        y = port.add_bias(port.conv2d_quantized(xq, p["wq"], dq, (spec.pad,) * 4, (spec.stride, spec.stride)), p["bias"])
+        if row["residual"] is not None:
+            y = port.relu(port.add(y, row["residual"]))
+        elif spec.relu:
+            y = port.relu(y)
+        if row["out_f32"] is not None:
+            assert np.array_equal(bits(row["out_f32"]), bits(y)), spec.name
+        if row["out_q"] is not None:
+            q = port.quantize(y, np.full(len(imgs), np.float32(scales[row["q_name"]]), np.float32))
+            assert np.array_equal(row["out_q"], q), spec.name
+            prev_q = row["out_q"]
+        checked += 1
+    assert checked == 53      # 1 stem + 16 blocks x 3 + 4 projections
+
+
 def test_mac_count_of_the_full_network():
     from tennis_amd import resnet50
     desc = resnet50.layers()
