@@ -62,6 +62,25 @@ void hip_from_hip(int dst_id, void *dst, int, const void *src, size_t size) { co
 
 }  // namespace
 
+Tensor byte_tensor(const MemoryDevice &device, size_t bytes) {
+    const size_t rows = (bytes + 15) / 16;
+    if (rows > size_t(0x7fffffff)) TS_LOG_ERROR << "[hip] buffer of " << bytes << " bytes exceeds a tensor's extents" << eject;
+    return Tensor(device, INT8, Shape({int32_t(rows ? rows : 1), 16}));
+}
+
+void *context_scratch(size_t bytes, const MemoryDevice &device, Tensor &own) {
+    auto *context = ctx::get<DeviceContext>();
+    Tensor &slot = (context && context->handle && context->memory_device == device)
+                       ? reinterpret_cast<HipContextHandle *>(context->handle)->scratch
+                       : own;
+    if (slot.empty() || size_t(slot.count()) < bytes || slot.device() != device) {
+        // kernels already queued on the context's stream may still use the old buffer: drain it before the free
+        hip_check(hipStreamSynchronize(stream_of_context()), "hipStreamSynchronize");
+        slot = byte_tensor(device, bytes);
+    }
+    return slot.data();
+}
+
 int HostDelegate::run(Operator &self, Stack &stack) {
     if (!m_host) {
         Operator::shared host;

@@ -11,7 +11,19 @@ static const char *const DEVICE = "hip";   // DeviceType holds at most 7 charact
 struct HipContextHandle {
     void *stream = nullptr;   // hipStream_t of this DeviceContext
     int device_id = 0;
+    Tensor scratch;           // kernel scratch shared by the operators of this context (see context_scratch)
 };
+
+// Device tensor of `bytes` bytes (any size: shaped [ceil(bytes / 16), 16], so sizes of 2 GiB and more do not
+// overflow an int32 extent).
+Tensor byte_tensor(const MemoryDevice &device, size_t bytes);
+
+// Scratch of at least `bytes` bytes in the memory of the DeviceContext bound to the calling thread, for kernels
+// that need a workspace for the duration of one operator call (the staged activations of a quantized
+// convolution).  One buffer per context, grown to the largest request and reused by every operator of the
+// context: its stream orders the kernels that write and read it, the way the reference's operators share
+// the stack's scratch frame.  `own` is used instead when no context is bound (an operator driven by hand).
+void *context_scratch(size_t bytes, const MemoryDevice &device, Tensor &own);
 
 // Stream of the DeviceContext bound to the calling thread (nullptr = default stream when an
 // operator is driven without a Workbench).

@@ -42,6 +42,36 @@ inline bool format_is_nchw(const Operator &op) {
     return !op.has(name::format) || tensor::to_string(op.get(name::format)) == name::NCHW;
 }
 
+// Packed weights and staging workspace of one quantized-convolution operator instance.
+class PackedConv {
+public:
+    // The weights in MFMA operand order for geometry g: packed on first use, and again when another weight
+    // tensor, weight shape or device shows up.  The operator keeps a reference to the tensor the pack was made
+    // from: while it lives its address cannot be handed to a different tensor, so "same address and shape"
+    // does mean "same weights" (weights are constant graph data, src/runtime/instruction.cpp:143-150).
+    const void *packed(const tsx_conv2d_geom &g, const Tensor &w, const MemoryDevice &device, void *stream, const char *who) {
+        const size_t bytes = tsx_conv2d_i8_packed_weight_bytes(&g);
+        if (bytes == 0) TS_LOG_ERROR << "[hip] " << who << ": " << tsx_last_error() << eject;
+        const bool same = !m_packed.empty() && m_bytes == bytes && m_packed.device() == device && !m_source.empty() &&
+                          m_source.data() == w.data() && m_source.device() == w.device() && m_source.sizes() == w.sizes();
+        if (!same) {
+            m_packed = byte_tensor(device, bytes);
+            check(tsx_conv2d_i8_pack_weights(&g, w.data<int8_t>(), m_packed.data(), stream), "tsx_conv2d_i8_pack_weights");
+            m_source = w;
+            m_bytes = bytes;
+        }
+        return m_packed.data();
+    }
+
+    // staging scratch for the activations: the context's shared buffer (nothing allocated in the steady state,
+    // one buffer of the largest layer's size per context instead of one per operator)
+    void *workspace(size_t bytes, const MemoryDevice &device) { return context_scratch(bytes ? bytes : 16, device, m_workspace); }
+
+private:
+    Tensor m_packed, m_source, m_workspace;
+    size_t m_bytes = 0;
+};
+
 // Host vector -> device tensor, cached while the host values stay the same (parameters such as
 // quantize_scale / dequantize_scales are fixed at init(); the reference hands them to the core by
 // value on every run).

@@ -51,12 +51,12 @@ public:
         const int cout = kernel.size(0), cin = kernel.size(1);
         const bool f23 = mode == F2X2_3X3;
         const size_t bytes = f23 ? tsx_winograd_f23_kernel_bytes(cout, cin) : tsx_winograd_f63_kernel_bytes(cout, cin);
-        m_u = Tensor(kernel.device(), FLOAT32, Shape({int32_t(bytes / sizeof(float))}));
+        m_u = byte_tensor(kernel.device(), bytes);
         if (f23)
-            check(tsx_winograd_f23_transform_kernel(cout, cin, kernel.data<float>(), m_u.data<float>(), current_stream()),
+            check(tsx_winograd_f23_transform_kernel(cout, cin, kernel.data<float>(), static_cast<float *>(m_u.data()), current_stream()),
                   "tsx_winograd_f23_transform_kernel");
         else
-            check(tsx_winograd_f63_transform_kernel(cout, cin, kernel.data<float>(), m_u.data<float>(), current_stream()),
+            check(tsx_winograd_f63_transform_kernel(cout, cin, kernel.data<float>(), static_cast<float *>(m_u.data()), current_stream()),
                   "tsx_winograd_f63_transform_kernel");
         m_mode = mode;
         m_cout = cout;
@@ -85,13 +85,13 @@ public:
         const size_t ws_bytes = f23 ? tsx_winograd_f23_workspace_bytes(&g) : tsx_winograd_f63_workspace_bytes(&g);
         if (ws_bytes == 0) TS_LOG_ERROR << "[hip] conv2d_winograd: " << tsx_last_error() << eject;
         if (m_workspace.empty() || size_t(m_workspace.count()) < ws_bytes)
-            m_workspace = Tensor(out.device(), INT8, Shape({int32_t(ws_bytes)}));
+            m_workspace = byte_tensor(out.device(), ws_bytes);
         if (f23)
-            check(tsx_conv2d_winograd_f23_nchw(&g, x.data<float>(), m_u.data<float>(), padding_value, nullptr, TSX_ACT_NONE,
+            check(tsx_conv2d_winograd_f23_nchw(&g, x.data<float>(), static_cast<float *>(m_u.data()), padding_value, nullptr, TSX_ACT_NONE,
                                                0.f, out.data<float>(), m_workspace.data(), ws_bytes, current_stream()),
                   "tsx_conv2d_winograd_f23_nchw");
         else
-            check(tsx_conv2d_winograd_f63_nchw(&g, x.data<float>(), m_u.data<float>(), padding_value, nullptr, TSX_ACT_NONE,
+            check(tsx_conv2d_winograd_f63_nchw(&g, x.data<float>(), static_cast<float *>(m_u.data()), padding_value, nullptr, TSX_ACT_NONE,
                                                0.f, out.data<float>(), m_workspace.data(), ws_bytes, current_stream()),
                   "tsx_conv2d_winograd_f63_nchw");
     }

@@ -77,25 +77,16 @@ public:
         if (with_bias) bias = stack[2].view(device);
         Tensor out = *stack.push(proto, device);
         void *stream = current_stream();
-        const size_t packed_bytes = tsx_conv2d_i8_packed_weight_bytes(&g);
-        if (packed_bytes == 0) TS_LOG_ERROR << "[hip] conv2d_quantized_fused: " << tsx_last_error() << eject;
-        if (m_packed.empty() || m_packed_from != w.data() || size_t(m_packed.count()) != packed_bytes || m_packed_cin != g.c) {
-            m_packed = Tensor(device, INT8, Shape({int32_t(packed_bytes)}));
-            check(tsx_conv2d_i8_pack_weights(&g, w.data<int8_t>(), m_packed.data(), stream), "tsx_conv2d_i8_pack_weights");
-            m_packed_from = w.data();
-            m_packed_cin = g.c;
-        }
+        const void *packed = m_state.packed(g, w, device, stream, "conv2d_quantized_fused");
         const size_t ws_bytes = tsx_conv2d_i8_workspace_bytes(&g);
-        if (m_workspace.empty() || size_t(m_workspace.count()) < ws_bytes || m_workspace.device() != device)
-            m_workspace = Tensor(device, INT8, Shape({int32_t(ws_bytes ? ws_bytes : 16)}));
+        void *workspace = m_state.workspace(ws_bytes, device);
         tsx_epilogue ep{};
         ep.dq_dev = m_dq_dev.get(m_dq, device);
         ep.bias_dev = with_bias ? bias.data<float>() : nullptr;
         ep.act = m_act;
         ep.slope = m_slope;
-        check(tsx_quantize_conv2d_i8_nchw(&g, x.data<float>(), m_q_dev.get(m_q, device), int32_t(m_q.size()), m_packed.data(),
-                                          m_padding_value, &ep, out.data<float>(), nullptr, nullptr, m_workspace.data(), ws_bytes,
-                                          stream),
+        check(tsx_quantize_conv2d_i8_nchw(&g, x.data<float>(), m_q_dev.get(m_q, device), int32_t(m_q.size()), packed,
+                                          m_padding_value, &ep, out.data<float>(), nullptr, nullptr, workspace, ws_bytes, stream),
               "tsx_quantize_conv2d_i8_nchw");
         return 1;
     }
@@ -136,9 +127,7 @@ private:
     int m_act = TSX_ACT_NONE;
     std::vector<float> m_dq, m_q;
     DeviceFloats m_dq_dev, m_q_dev;
-    Tensor m_packed, m_workspace;
-    const void *m_packed_from = nullptr;
-    int m_packed_cin = 0;
+    PackedConv m_state;
 };
 
 }  // namespace hip

@@ -43,37 +43,22 @@ public:
         if (x.dtype() != INT8) TS_LOG_ERROR << "Conv2D_quantized not support this data type: " << type_str(x.dtype()) << eject;
         const tsx_conv2d_geom g = make_geom(x, w, padding, stride, dilation);
         void *stream = current_stream();
-        // Weights are constant graph data: pack them into MFMA operand tiles once per weight
-        // tensor and geometry, on first use (the pack translator leaves them unpacked for a
-        // device that registers its own operator).
-        const size_t packed_bytes = tsx_conv2d_i8_packed_weight_bytes(&g);
-        if (packed_bytes == 0) TS_LOG_ERROR << "[hip] conv2d_quantized: " << tsx_last_error() << eject;
-        if (m_packed.empty() || m_packed_from != w.data() || size_t(m_packed.count()) != packed_bytes || m_packed_cin != g.c) {
-            m_packed = Tensor(out.device(), INT8, Shape({int32_t(packed_bytes)}));
-            check(tsx_conv2d_i8_pack_weights(&g, w.data<int8_t>(), m_packed.data(), stream), "tsx_conv2d_i8_pack_weights");
-            m_packed_from = w.data();
-            m_packed_cin = g.c;
-        }
-        // staging scratch for the activations: kept across runs instead of taken from the stack's
-        // scratch frame, so the steady state allocates nothing
+        // Weights are constant graph data: packed into MFMA operand tiles once per weight tensor and geometry,
+        // on first use (the pack translator leaves them unpacked for a device that registers its own operator).
+        const void *packed = m_state.packed(g, w, out.device(), stream, "conv2d_quantized");
         const size_t ws_bytes = tsx_conv2d_i8_workspace_bytes(&g);
-        if (m_workspace.empty() || size_t(m_workspace.count()) < ws_bytes || m_workspace.device() != out.device())
-            m_workspace = Tensor(out.device(), INT8, Shape({int32_t(ws_bytes ? ws_bytes : 16)}));
-        Tensor &workspace = m_workspace;
+        void *workspace = m_state.workspace(ws_bytes, out.device());
         (void) stack;
         tsx_epilogue ep{};
         ep.dq_dev = m_dq.get(dequantize_scale, out.device());
         ep.act = TSX_ACT_NONE;
-        check(tsx_conv2d_i8_nchw(&g, x.data<int8_t>(), m_packed.data(), padding_value, &ep, out.data<float>(), nullptr,
-                                 nullptr, workspace.data(), ws_bytes, stream),
+        check(tsx_conv2d_i8_nchw(&g, x.data<int8_t>(), packed, padding_value, &ep, out.data<float>(), nullptr, nullptr,
+                                 workspace, ws_bytes, stream),
               "tsx_conv2d_i8_nchw");
     }
 
 private:
-    Tensor m_packed;
-    Tensor m_workspace;
-    const void *m_packed_from = nullptr;
-    int m_packed_cin = 0;
+    PackedConv m_state;
     DeviceFloats m_dq;
 };
 

@@ -47,10 +47,17 @@ public:
         std::vector<Node> bias;      // empty or the add_bias node's constant
         if (cur.bubble().op() == name::layer::add_bias()) {
             if (cur.inputs().size() != 2 || cur.input(1).bubble().op() != Bubble::Const) return false;
+            // the axis as AddBias::init resolves it (src/backend/base/base_add_bias.cpp:27-40): from the format's
+            // 'C', overridden by dim when that is set too; the fused epilogue adds along the channel axis 1 only
             const Bubble &b = cur.bubble();
-            const bool on_channels = (b.has(name::format) && tensor::to_string(b.get(name::format)) == name::NCHW) ||
-                                     (b.has(name::dim) && tensor::to_int(b.get(name::dim)) == 1);
-            if (!on_channels) return false;
+            int axis = -1;
+            if (b.has(name::format)) {
+                const std::string format = tensor::to_string(b.get(name::format));
+                if (format != name::NCHW && format != name::NHWC) return false;
+                axis = int(format.find('C'));
+            }
+            if (b.has(name::dim)) axis = tensor::to_int(b.get(name::dim));
+            if (axis != 1) return false;
             bias.push_back(cur.input(1));
             cur = cur.input(0);
             if (cur.outputs().size() != 1) return false;
@@ -60,6 +67,19 @@ public:
         if (q.bubble().op() != name::layer::quantize() || q.inputs().size() != 1 || w.bubble().op() != Bubble::Const) return false;
         const Bubble &conv = cur.bubble();
         if (!conv.has(name::format) || tensor::to_string(conv.get(name::format)) != name::NCHW) return false;
+        // what the fused operator checks at run time, checked here where the graph shows it, so that a chain which
+        // ran unfused is not turned into one that ejects: int8 OIHW weights, one float32 bias value per output
+        // channel, and -- where the graph carries the inferred type -- a float32 tensor in front of the quantize
+        if (!w.bubble().has(name::value)) return false;
+        const Tensor weights = w.bubble().get(name::value);
+        if (weights.dtype() != INT8 || weights.dims() != 4) return false;
+        if (!bias.empty()) {
+            if (!bias[0].bubble().has(name::value)) return false;
+            const Tensor b = bias[0].bubble().get(name::value);
+            if (b.dtype() != FLOAT32 || b.count() != weights.size(0)) return false;
+        }
+        const Bubble &source = q.input(0).bubble();
+        if (source.has("#dtype") && DTYPE(tensor::to_int(source.get("#dtype"))) != FLOAT32) return false;
 
         std::vector<Node> inputs = {q.input(0), w};
         inputs.insert(inputs.end(), bias.begin(), bias.end());

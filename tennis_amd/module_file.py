@@ -217,8 +217,22 @@ def fuse_quantized_chains(module):
         bi = only_user(last, "add_bias")
         if bi is not None:
             b = nodes[bi]
-            on_channels = b.params.get("format") == "NCHW" or int(np.asarray(b.params.get("dim", -99)).ravel()[0]) == 1
-            if len(b.inputs) == 2 and nodes[b.inputs[1]].op == CONST and on_channels:
+            # the axis as AddBias::init resolves it (src/backend/base/base_add_bias.cpp:27-40): from the format's 'C',
+            # overridden by dim when that is set too; the fused epilogue adds along the channel axis 1 only
+            axis = -1
+            fmt = b.params.get("format")
+            if isinstance(fmt, bytes):
+                fmt = fmt.decode()
+            if fmt in ("NCHW", "NHWC"):
+                axis = fmt.index("C")
+            if "dim" in b.params:
+                axis = int(np.asarray(b.params["dim"]).ravel()[0])
+            bias_ok = False
+            if len(b.inputs) == 2 and nodes[b.inputs[1]].op == CONST:
+                value = np.asarray(nodes[b.inputs[1]].params.get("value"))
+                wvalue = np.asarray(nodes[conv.inputs[1]].params.get("value"))
+                bias_ok = value.dtype == np.float32 and wvalue.ndim == 4 and value.size == wvalue.shape[0]
+            if bias_ok and axis == 1 and (fmt is None or fmt in ("NCHW", "NHWC")):
                 inputs.append(b.inputs[1])
                 last = bi
         ai = only_user(last, "relu")

@@ -301,3 +301,37 @@ def test_inputs_a_hip_class_does_not_cover_run_the_host_operator(ts):
             ts.run_op_intree(device, "pooling2d", p, [xn], xn.nbytes)
         errors.append(str(e.value).split("only support")[-1])
     assert errors[0] == errors[1] and "NCHW" in errors[0]
+
+
+def test_zipper_option_resolves_the_bias_axis_like_add_bias(ts, tmp_path):
+    """add_bias with format NCHW AND dim 3: AddBias::init lets dim override the format (base_add_bias.cpp:27-40), so
+    the bias runs along W.  The rewrite must not take it for a channel bias: it folds quantize + convolution only
+    and leaves the add_bias node in the graph; values as on TenniS's CPU device."""
+    import sys, os
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"))
+    from make_modules import conv_params
+    from tennis_amd import module_file as mf
+    rng = np.random.default_rng(78)
+    n, c, h, w, co = 2, 8, 6, 10, 10          # cout == w: a channel bias would have the same length
+    wq = rng.integers(-127, 128, (co, c, 3, 3)).astype(np.int8)
+    N = mf.Node
+    nodes = [N(mf.PARAMETER, "x"), N("quantize", "q", {"quantize_scale": np.array([9.0, 11.0], np.float32)}, [0]),
+             N(mf.CONST, "w", {"value": wq}),
+             N("conv2d_quantized", "conv", dict(conv_params((1, 1, 1, 1)),
+                                                dequantize_scales=rng.uniform(1e-4, 1e-3, co).astype(np.float32)), [1, 2]),
+             N(mf.CONST, "b", {"value": rng.standard_normal(w).astype(np.float32)}),
+             N("add_bias", "bias_w", {"format": "NCHW", "dim": np.array([3], np.int32)}, [3, 4]),
+             N("relu", "act", {}, [5])]
+    module = mf.Module(nodes, [0], [6])
+    path = str(tmp_path / "bias_axis.tsm")
+    mf.write_module(path, module)
+    x = (rng.standard_normal((n, c, h, w)) * 6).astype(np.float32)
+    cpu = ts.run_module_intree("cpu", path, [x])
+    fused0 = ts.fused_chain_count_intree()
+    hip = ts.run_module_intree("hip", path, [x])
+    assert ts.fused_chain_count_intree() == fused0 + 1
+    assert np.array_equal(bits(hip), bits(cpu))
+    fused = mf.fuse_quantized_chains(module)
+    assert [m.op for m in fused.nodes].count("add_bias") == 1
+    (own,) = mf.run_module(fused, [x])
+    assert np.array_equal(bits(own), bits(cpu))

@@ -131,6 +131,25 @@ def test_fusing_rewrite_structure():
     fg = mf.fuse_quantized_chains(g)
     assert [n.op for n in fg.nodes].count("add_bias") == 1 and [n.op for n in fg.nodes].count(mf.FUSED) == 1
 
+    # the bias axis as AddBias::init resolves it: dim overrides the format's 'C' (base_add_bias.cpp:27-40), and only
+    # axis 1 with one float32 value per output channel is a channel bias the fused epilogue can add
+    def chain(bias_params, bias_value):
+        return mf.Module([N("<param>", "x"), N("quantize", "q", {"quantize_scale": np.ones(1, np.float32)}, [0]),
+                          N("<const>", "w", {"value": w}), N("conv2d_quantized", "c", conv, [1, 2]),
+                          N("<const>", "b", {"value": bias_value}), N("add_bias", "ab", bias_params, [3, 4])], [0], [5])
+
+    def bias_fused(bias_params, bias_value=np.zeros(4, np.float32)):
+        ops = [n.op for n in mf.fuse_quantized_chains(chain(bias_params, bias_value)).nodes]
+        assert ops.count(mf.FUSED) == 1
+        return "add_bias" not in ops
+
+    one, three = np.array([1], np.int32), np.array([3], np.int32)
+    assert bias_fused({"format": "NCHW"}) and bias_fused({"dim": one}) and bias_fused({"format": "NHWC", "dim": one})
+    assert not bias_fused({"format": "NCHW", "dim": three})       # dim wins: the bias runs along W
+    assert not bias_fused({"format": "NHWC"}) and not bias_fused({"dim": three})
+    assert not bias_fused({"format": "NCHW"}, np.zeros(4, np.float64))
+    assert not bias_fused({"format": "NCHW"}, np.zeros(1, np.float32))
+
 
 @pytest.mark.gpu
 def test_fused_module_equals_the_unfused_one(hip_device):
