@@ -211,6 +211,21 @@ int tsx_add_bias_f32(const float *x_dev, int64_t pre, int32_t channels, int64_t 
 int tsx_relu_f32(const float *x_dev, int64_t count, float *out_dev, void *stream);
 int tsx_leaky_relu_f32(const float *x_dev, int64_t count, float scale, float *out_dev, void *stream);
 
+/* Batch normalisation nodes of graphs whose BN was not folded into the convolution, x = [pre][channels][inner]:
+ *   tsx_batch_norm_f32        cpu::BatchNorm      (src/kernels/cpu/batch_norm.cpp:61-105; interface
+ *                             include/backend/base/base_batch_norm.h): (x - mean[c]) * (1 / sqrt(variance[c] + epsilon))
+ *   tsx_batch_scale_f32       cpu::BatchScale     (src/kernels/cpu/batch_scale.cpp:57-97): x * scale[c] + bias[c]
+ *   tsx_fused_batch_norm_f32  cpu::FusedBatchNorm (src/kernels/cpu/fused_batch_norm.cpp:70-125): the two in one pass
+ * Same roundings as the reference's AVX2/FMA build (reciprocal root evaluated in double and rounded once, the
+ * scale-and-shift a single fused multiply-add): results match it bit for bit. */
+int tsx_batch_norm_f32(const float *x_dev, int64_t pre, int32_t channels, int64_t inner, const float *mean_dev,
+                       const float *variance_dev, float epsilon, float *out_dev, void *stream);
+int tsx_batch_scale_f32(const float *x_dev, int64_t pre, int32_t channels, int64_t inner, const float *scale_dev,
+                        const float *bias_dev, float *out_dev, void *stream);
+int tsx_fused_batch_norm_f32(const float *x_dev, int64_t pre, int32_t channels, int64_t inner, const float *mean_dev,
+                             const float *variance_dev, const float *scale_dev, const float *bias_dev, float epsilon,
+                             float *out_dev, void *stream);
+
 /* ---------------------------------------------------------------- glue between convolutions
  * The HBM-bound operators that sit between the convolutions of whole networks, so that a graph stays
  * on the device:

@@ -216,6 +216,50 @@ void orc_add_bias_f32(const float *x, int64_t pre, int channels, int64_t inner, 
     for (int64_t i = 0; i < total; ++i) out[i] = x[i] + bias[(i / inner) % channels];
 }
 
+// ---------------------------------------------------------------------------
+// batch_norm / batch_scale / fused_batch_norm on fp32, layout [pre][channels][inner]:
+// src/kernels/cpu/batch_norm.cpp:61-105, batch_scale.cpp:57-97, fused_batch_norm.cpp:70-125.
+// The reciprocal standard deviation is float(1) / sqrt(var + float(eps)) with the sum in float and the
+// unqualified sqrt taking it as a double: root and quotient are computed in double and rounded to float once.
+// x * scale + bias is one fused multiply-add in the reference's FMA build, in its 4-wide body and in its
+// scalar tail alike (gcc contracts both); (x - mean) * inv has nothing to contract.
+// ---------------------------------------------------------------------------
+static inline float inv_std(float variance, float epsilon) {
+    const float sum = variance + epsilon;
+    return float(1.0 / std::sqrt(double(sum)));
+}
+
+void orc_batch_norm_f32(const float *x, int64_t pre, int channels, int64_t inner, const float *mean,
+                        const float *variance, float epsilon, float *out) {
+    const int64_t total = pre * channels * inner;
+#pragma omp parallel for num_threads(g_threads)
+    for (int64_t i = 0; i < total; ++i) {
+        const int c = int((i / inner) % channels);
+        out[i] = (x[i] - mean[c]) * inv_std(variance[c], epsilon);
+    }
+}
+
+void orc_batch_scale_f32(const float *x, int64_t pre, int channels, int64_t inner, const float *scale,
+                         const float *bias, float *out) {
+    const int64_t total = pre * channels * inner;
+#pragma omp parallel for num_threads(g_threads)
+    for (int64_t i = 0; i < total; ++i) {
+        const int c = int((i / inner) % channels);
+        out[i] = std::fmaf(x[i], scale[c], bias[c]);
+    }
+}
+
+void orc_fused_batch_norm_f32(const float *x, int64_t pre, int channels, int64_t inner, const float *mean,
+                              const float *variance, const float *scale, const float *bias, float epsilon, float *out) {
+    const int64_t total = pre * channels * inner;
+#pragma omp parallel for num_threads(g_threads)
+    for (int64_t i = 0; i < total; ++i) {
+        const int c = int((i / inner) % channels);
+        const float t = (x[i] - mean[c]) * inv_std(variance[c], epsilon);
+        out[i] = std::fmaf(t, scale[c], bias[c]);
+    }
+}
+
 void orc_relu_f32(const float *x, int64_t count, float *out) {
     const int64_t body = count / 4 * 4;
 #pragma omp parallel for num_threads(g_threads)

@@ -35,6 +35,9 @@ def lib():
         L.orc_conv2d_quantized.argtypes = [_vp, _i, _i, _i, _i, _vp] + [_i] * 11 + [_f, _vp, _vp, _vp, _i]
         L.orc_add_bias_f32.argtypes = [_vp, _i64, _i, _i64, _vp, _vp]
         L.orc_relu_f32.argtypes = [_vp, _i64, _vp]
+        L.orc_batch_norm_f32.argtypes = [_vp, _i64, _i, _i64, _vp, _vp, _f, _vp]
+        L.orc_batch_scale_f32.argtypes = [_vp, _i64, _i, _i64, _vp, _vp, _vp]
+        L.orc_fused_batch_norm_f32.argtypes = [_vp, _i64, _i, _i64, _vp, _vp, _vp, _vp, _f, _vp]
         L.orc_leaky_relu_f32.argtypes = [_vp, _i64, _f, _vp]
         L.orc_epilogue.argtypes = [_vp, _i64, _i, _i64, _vp, _vp, _vp, _i, _f, _vp, _vp, _i, _vp]
         L.orc_conv2d_i8_fused.argtypes = ([_vp, _i, _i, _i, _i, _vp] + [_i] * 11 +
@@ -128,6 +131,41 @@ def add_bias(x, bias, dim=1):
     inner = int(np.prod(x.shape[dim + 1:], dtype=np.int64))
     out = np.empty_like(x)
     lib().orc_add_bias_f32(_p(x), pre, x.shape[dim], inner, _p(bias), _p(out))
+    return out
+
+
+def _channel_args(x, dim):
+    pre = int(np.prod(x.shape[:dim], dtype=np.int64))
+    inner = int(np.prod(x.shape[dim + 1:], dtype=np.int64))
+    return pre, x.shape[dim], inner
+
+
+def batch_norm(x, mean, variance, epsilon=1e-5, dim=1):
+    """cpu::BatchNorm (src/kernels/cpu/batch_norm.cpp:61-105): (x - mean[c]) / sqrt(variance[c] + epsilon)."""
+    x = _c(x, np.float32)
+    out = np.empty_like(x)
+    pre, ch, inner = _channel_args(x, dim)
+    lib().orc_batch_norm_f32(_p(x), pre, ch, inner, _p(_c(mean, np.float32)), _p(_c(variance, np.float32)),
+                             float(epsilon), _p(out))
+    return out
+
+
+def batch_scale(x, scale, bias, dim=1):
+    """cpu::BatchScale (src/kernels/cpu/batch_scale.cpp:57-97): x * scale[c] + bias[c]."""
+    x = _c(x, np.float32)
+    out = np.empty_like(x)
+    pre, ch, inner = _channel_args(x, dim)
+    lib().orc_batch_scale_f32(_p(x), pre, ch, inner, _p(_c(scale, np.float32)), _p(_c(bias, np.float32)), _p(out))
+    return out
+
+
+def fused_batch_norm(x, mean, variance, scale, bias, epsilon=1e-5, dim=1):
+    """cpu::FusedBatchNorm (src/kernels/cpu/fused_batch_norm.cpp:70-125): batch_norm followed by batch_scale."""
+    x = _c(x, np.float32)
+    out = np.empty_like(x)
+    pre, ch, inner = _channel_args(x, dim)
+    lib().orc_fused_batch_norm_f32(_p(x), pre, ch, inner, _p(_c(mean, np.float32)), _p(_c(variance, np.float32)),
+                                   _p(_c(scale, np.float32)), _p(_c(bias, np.float32)), float(epsilon), _p(out))
     return out
 
 

@@ -160,6 +160,63 @@ protected:
     bool covers(Stack &stack) override { return inputs_are(stack, 1, FLOAT32); }
 };
 
+// ---------------------------------------------------------------- batch_norm / batch_scale / fused_batch_norm
+// Graphs whose batch normalisation was not folded into the convolution carry these nodes behind it
+// (src/kernels/cpu/batch_norm.cpp, batch_scale.cpp, fused_batch_norm.cpp; device classes
+// src/kernels/gpu/batch_norm.cu, batch_scale.cu, fused_batch_norm.cu).  One HBM-bound pass each, the
+// reference's roundings; other element types than fp32 run the host operator.
+namespace {
+void channel_layout(const Tensor &x, int dim, int64_t &pre, int64_t &inner) {
+    pre = inner = 1;
+    for (int i = 0; i < dim; ++i) pre *= x.size(size_t(i));
+    for (size_t i = size_t(dim) + 1; i < x.dims(); ++i) inner *= x.size(i);
+}
+}  // namespace
+
+class BatchNorm : public OperatorOnHip<base::BatchNorm> {
+public:
+    void batch_norm(const Tensor &x, const Tensor &mean, const Tensor &variance, int dim, float epsilon, Tensor &out) override {
+        int64_t pre, inner;
+        channel_layout(x, dim, pre, inner);
+        check(tsx_batch_norm_f32(x.data<float>(), pre, x.size(size_t(dim)), inner, mean.data<float>(), variance.data<float>(),
+                                 epsilon, out.data<float>(), current_stream()),
+              "tsx_batch_norm_f32");
+    }
+
+protected:
+    bool covers(Stack &stack) override { return inputs_are(stack, 3, FLOAT32); }
+};
+
+class BatchScale : public OperatorOnHip<base::BatchScale> {
+public:
+    void batch_scale(const Tensor &x, const Tensor &scale, const Tensor &bias, int dim, Tensor &out) override {
+        int64_t pre, inner;
+        channel_layout(x, dim, pre, inner);
+        check(tsx_batch_scale_f32(x.data<float>(), pre, x.size(size_t(dim)), inner, scale.data<float>(), bias.data<float>(),
+                                  out.data<float>(), current_stream()),
+              "tsx_batch_scale_f32");
+    }
+
+protected:
+    bool covers(Stack &stack) override { return inputs_are(stack, 3, FLOAT32); }
+};
+
+class FusedBatchNorm : public OperatorOnHip<base::FusedBatchNorm> {
+public:
+    void batch_norm(const Tensor &x, const Tensor &mean, const Tensor &variance, const Tensor &scale, const Tensor &bias, int dim,
+                    float epsilon, Tensor &out) override {
+        int64_t pre, inner;
+        channel_layout(x, dim, pre, inner);
+        check(tsx_fused_batch_norm_f32(x.data<float>(), pre, x.size(size_t(dim)), inner, mean.data<float>(),
+                                       variance.data<float>(), scale.data<float>(), bias.data<float>(), epsilon,
+                                       out.data<float>(), current_stream()),
+              "tsx_fused_batch_norm_f32");
+    }
+
+protected:
+    bool covers(Stack &stack) override { return inputs_are(stack, 5, FLOAT32); }
+};
+
 }  // namespace hip
 }  // namespace ts
 
@@ -171,3 +228,6 @@ TS_REGISTER_OPERATOR(InnerProd, ts::hip::DEVICE, name::layer::inner_prod())
 TS_REGISTER_OPERATOR(AddBias, ts::hip::DEVICE, name::layer::add_bias())
 TS_REGISTER_OPERATOR(ReLU, ts::hip::DEVICE, name::layer::relu())
 TS_REGISTER_OPERATOR(LeakyReLU, ts::hip::DEVICE, "leaky_relu")
+TS_REGISTER_OPERATOR(BatchNorm, ts::hip::DEVICE, "batch_norm")
+TS_REGISTER_OPERATOR(BatchScale, ts::hip::DEVICE, "batch_scale")
+TS_REGISTER_OPERATOR(FusedBatchNorm, ts::hip::DEVICE, "fused_batch_norm")

@@ -10,6 +10,9 @@
 #include <backend/base/base_quantize.h>
 #endif
 #ifdef TSX_TS_FLOAT_OPS
+#include <backend/base/base_batch_norm.h>
+#include <backend/base/base_batch_scale.h>
+#include <backend/base/base_fused_batch_norm.h>
 #include <backend/base/base_add_bias.h>
 #include <backend/base/base_activation.h>
 #include <backend/base/base_conv2d.h>

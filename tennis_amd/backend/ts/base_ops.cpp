@@ -481,6 +481,110 @@ int AddBias::run(Stack &stack) {
     return 1;
 }
 
+// ---------------------------------------------------------------- batch_norm / batch_scale / fused_batch_norm
+namespace {
+// the checks of BatchNorm::check_inputs and its two siblings: `count` vectors of x.size(dim) values behind x
+void check_channel_vectors(Stack &stack, size_t count, int dim, const char *const *names) {
+    TS_AUTO_CHECK(stack.size() == count + 1);
+    auto &x = stack[0];
+    TS_AUTO_CHECK(dim < int(x.dims()));
+    for (size_t i = 1; i <= count; ++i) {
+        auto &v = stack[int(i)];
+        if (!v.has_shape(x.size(size_t(dim))))
+            TS_LOG_ERROR << "Miss matched: x:" << to_string(x.sizes()) << ", dim=" << dim << ", " << names[i - 1] << ":"
+                         << to_string(v.sizes()) << eject;
+    }
+    for (size_t i = 1; i <= count; ++i) TS_AUTO_CHECK(x.dtype() == stack[int(i)].dtype());
+}
+const char *const kNormNames[] = {"mean", "variance", "scale", "bias"};
+const char *const kScaleNames[] = {"scale", "bias"};
+}  // namespace
+
+BatchNorm::BatchNorm() {
+    field(name::epsilon, OPTIONAL);
+    field(name::dim, REQUIRED);
+}
+
+void BatchNorm::init() {
+    supper::init();
+    if (has(name::epsilon)) m_epsilon = tensor::to_float(get(name::epsilon));
+    m_dim = tensor::to_int(get(name::dim));
+    TS_AUTO_CHECK(m_dim >= 0);
+}
+
+int BatchNorm::infer(Stack &stack, std::vector<Tensor::Prototype> &output) {
+    check_channel_vectors(stack, 2, m_dim, kNormNames);
+    output.assign(1, stack[0].proto());
+    return 1;
+}
+
+int BatchNorm::run(Stack &stack) {
+    check_channel_vectors(stack, 2, m_dim, kNormNames);
+    auto memory_device = running_memory_device();
+    auto x = stack[0].view(memory_device);
+    auto mean = stack[1].view(memory_device);
+    auto variance = stack[2].view(memory_device);
+    auto out = *stack.push(x.proto(), memory_device);
+    batch_norm(x, mean, variance, m_dim, m_epsilon, out);
+    return 1;
+}
+
+BatchScale::BatchScale() { field(name::dim, REQUIRED); }
+
+void BatchScale::init() {
+    supper::init();
+    m_dim = tensor::to_int(get(name::dim));
+    TS_AUTO_CHECK(m_dim >= 0);
+}
+
+int BatchScale::infer(Stack &stack, std::vector<Tensor::Prototype> &output) {
+    check_channel_vectors(stack, 2, m_dim, kScaleNames);
+    output.assign(1, stack[0].proto());
+    return 1;
+}
+
+int BatchScale::run(Stack &stack) {
+    check_channel_vectors(stack, 2, m_dim, kScaleNames);
+    auto memory_device = running_memory_device();
+    auto x = stack[0].view(memory_device);
+    auto scale = stack[1].view(memory_device);
+    auto bias = stack[2].view(memory_device);
+    auto out = *stack.push(x.proto(), memory_device);
+    batch_scale(x, scale, bias, m_dim, out);
+    return 1;
+}
+
+FusedBatchNorm::FusedBatchNorm() {
+    field(name::epsilon, OPTIONAL);
+    field(name::dim, REQUIRED);
+}
+
+void FusedBatchNorm::init() {
+    supper::init();
+    if (has(name::epsilon)) m_epsilon = tensor::to_float(get(name::epsilon));
+    m_dim = tensor::to_int(get(name::dim));
+    TS_AUTO_CHECK(m_dim >= 0);
+}
+
+int FusedBatchNorm::infer(Stack &stack, std::vector<Tensor::Prototype> &output) {
+    check_channel_vectors(stack, 4, m_dim, kNormNames);
+    output.assign(1, stack[0].proto());
+    return 1;
+}
+
+int FusedBatchNorm::run(Stack &stack) {
+    check_channel_vectors(stack, 4, m_dim, kNormNames);
+    auto memory_device = running_memory_device();
+    auto x = stack[0].view(memory_device);
+    auto mean = stack[1].view(memory_device);
+    auto variance = stack[2].view(memory_device);
+    auto scale = stack[3].view(memory_device);
+    auto bias = stack[4].view(memory_device);
+    auto out = *stack.push(x.proto(), memory_device);
+    batch_norm(x, mean, variance, scale, bias, m_dim, m_epsilon, out);
+    return 1;
+}
+
 // ---------------------------------------------------------------- activations
 int Activation::infer(Stack &stack, std::vector<Tensor::Prototype> &output) {
     TS_AUTO_CHECK(stack.size() == 1);

@@ -172,6 +172,50 @@ private:
     std::string m_format;
 };
 
+// base::BatchNorm / BatchScale / FusedBatchNorm (src/backend/base/base_batch_norm.cpp, base_batch_scale.cpp,
+// base_fused_batch_norm.cpp): one parameter vector per extent of axis `dim`, same dtype as x.
+class BatchNorm : public OperatorOnDevice {
+public:
+    using supper = OperatorOnDevice;
+    BatchNorm();
+    void init() override;
+    int run(Stack &stack) override;
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override;
+    virtual void batch_norm(const Tensor &x, const Tensor &mean, const Tensor &variance, int dim, float epsilon, Tensor &out) = 0;
+
+private:
+    float m_epsilon = 1e-5f;
+    int m_dim = -1;
+};
+
+class BatchScale : public OperatorOnDevice {
+public:
+    using supper = OperatorOnDevice;
+    BatchScale();
+    void init() override;
+    int run(Stack &stack) override;
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override;
+    virtual void batch_scale(const Tensor &x, const Tensor &scale, const Tensor &bias, int dim, Tensor &out) = 0;
+
+private:
+    int m_dim = -1;
+};
+
+class FusedBatchNorm : public OperatorOnDevice {
+public:
+    using supper = OperatorOnDevice;
+    FusedBatchNorm();
+    void init() override;
+    int run(Stack &stack) override;
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override;
+    virtual void batch_norm(const Tensor &x, const Tensor &mean, const Tensor &variance, const Tensor &scale, const Tensor &bias,
+                            int dim, float epsilon, Tensor &out) = 0;
+
+private:
+    float m_epsilon = 1e-5f;
+    int m_dim = -1;
+};
+
 class Activation : public OperatorOnDevice {
 public:
     using supper = OperatorOnDevice;

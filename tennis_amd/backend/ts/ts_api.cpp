@@ -468,6 +468,7 @@ const char *const stride = "stride";
 const char *const dilation = "dilation";
 const char *const kernel_packed = "kernel_packed";
 const char *const dim = "dim";
+const char *const epsilon = "epsilon";
 const char *const scale = "scale";
 const char *const quantize_scale = "quantize_scale";
 const char *const dequantize_scales = "dequantize_scales";

@@ -484,6 +484,7 @@ extern const char *const stride;
 extern const char *const dilation;
 extern const char *const kernel_packed;
 extern const char *const dim;
+extern const char *const epsilon;
 extern const char *const scale;
 extern const char *const quantize_scale;
 extern const char *const dequantize_scales;

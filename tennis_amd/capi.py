@@ -77,6 +77,9 @@ SIGNATURES = {
     "tsx_inner_prod_f32": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp]),
     "tsx_add_bias_f32": (ctypes.c_int, [_vp, _i64, _i32, _i64, _vp, _vp, _vp]),
     "tsx_relu_f32": (ctypes.c_int, [_vp, _i64, _vp, _vp]),
+    "tsx_batch_norm_f32": (ctypes.c_int, [_vp, _i64, _i32, _i64, _vp, _vp, _f32, _vp, _vp]),
+    "tsx_batch_scale_f32": (ctypes.c_int, [_vp, _i64, _i32, _i64, _vp, _vp, _vp, _vp]),
+    "tsx_fused_batch_norm_f32": (ctypes.c_int, [_vp, _i64, _i32, _i64, _vp, _vp, _vp, _vp, _f32, _vp, _vp]),
     "tsx_leaky_relu_f32": (ctypes.c_int, [_vp, _i64, _f32, _vp, _vp]),
     "tsx_max_pooling2d_i8_staged": (ctypes.c_int, [_vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
     "tsx_add_f32": (ctypes.c_int, [_vp, _vp, _i64, _i32, _f32, _vp, _vp]),
@@ -428,6 +431,44 @@ def add_bias(x, bias, dim=1):
         inner *= d
     out = torch.empty_like(x)
     check(lib().tsx_add_bias_f32(_ptr(x), pre, x.shape[dim], inner, _ptr(bias), _ptr(out), _stream()))
+    return out
+
+
+def _channel_layout(x, dim):
+    pre = 1
+    for d in x.shape[:dim]:
+        pre *= d
+    inner = 1
+    for d in x.shape[dim + 1:]:
+        inner *= d
+    return pre, x.shape[dim], inner
+
+
+def batch_norm(x, mean, variance, epsilon=1e-5, dim=1):
+    x = _dev(x, torch.float32)
+    pre, ch, inner = _channel_layout(x, dim)
+    out = torch.empty_like(x)
+    check(lib().tsx_batch_norm_f32(_ptr(x), pre, ch, inner, _ptr(_dev(mean, torch.float32)), _ptr(_dev(variance, torch.float32)),
+                                   float(epsilon), _ptr(out), _stream()))
+    return out
+
+
+def batch_scale(x, scale, bias, dim=1):
+    x = _dev(x, torch.float32)
+    pre, ch, inner = _channel_layout(x, dim)
+    out = torch.empty_like(x)
+    check(lib().tsx_batch_scale_f32(_ptr(x), pre, ch, inner, _ptr(_dev(scale, torch.float32)), _ptr(_dev(bias, torch.float32)),
+                                    _ptr(out), _stream()))
+    return out
+
+
+def fused_batch_norm(x, mean, variance, scale, bias, epsilon=1e-5, dim=1):
+    x = _dev(x, torch.float32)
+    pre, ch, inner = _channel_layout(x, dim)
+    out = torch.empty_like(x)
+    check(lib().tsx_fused_batch_norm_f32(_ptr(x), pre, ch, inner, _ptr(_dev(mean, torch.float32)),
+                                         _ptr(_dev(variance, torch.float32)), _ptr(_dev(scale, torch.float32)),
+                                         _ptr(_dev(bias, torch.float32)), float(epsilon), _ptr(out), _stream()))
     return out
 
 

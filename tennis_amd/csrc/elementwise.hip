@@ -93,6 +93,79 @@ int launch(const float *x, int64_t count, const float *bias, int channels, int64
     return 0;
 }
 
+// batch_norm / batch_scale / fused_batch_norm on [pre][channels][inner] (src/kernels/cpu/batch_norm.cpp:61-105,
+// batch_scale.cpp:57-97, fused_batch_norm.cpp:70-125), 4 elements per lane.  The reference's arithmetic, rounding
+// for rounding: 1 / sqrt(var + eps) with the sum in float, root and quotient in double, rounded to float once;
+// (x - mean) * that; x * scale + bias as ONE fused multiply-add (its FMA build contracts the 4-wide body and the
+// scalar tail alike).  NORM: 0 = batch_scale, 1 = batch_norm, 2 = fused_batch_norm.
+template <int NORM>
+__global__ __launch_bounds__(256) void channel_affine_kernel(const float *__restrict__ x, int64_t count, int channels,
+                                                            int64_t inner, const float *__restrict__ mean,
+                                                            const float *__restrict__ variance,
+                                                            const float *__restrict__ scale, const float *__restrict__ bias,
+                                                            float epsilon, float *__restrict__ out, bool vec) {
+    auto apply = [&](float v, int c) -> float {
+        if (NORM != 0) {
+            const float sum = __fadd_rn(variance[c], epsilon);
+            const float inv = float(1.0 / sqrt(double(sum)));
+            v = __fmul_rn(__fsub_rn(v, mean[c]), inv);
+        }
+        if (NORM != 1) v = __builtin_fmaf(v, scale[c], bias[c]);
+        return v;
+    };
+    const int64_t stride = int64_t(gridDim.x) * blockDim.x * 4;
+    for (int64_t base = (int64_t(blockIdx.x) * blockDim.x + threadIdx.x) * 4; base < count; base += stride) {
+        if (vec && base + 4 <= count) {
+            const v4f in = *reinterpret_cast<const v4f *>(x + base);
+            v4f o;
+            if ((inner & 3) == 0) {   // the lane's four elements share their channel
+                const int c = count < (int64_t(1) << 32) ? int((unsigned(base) / unsigned(inner)) % unsigned(channels))
+                                                         : int((base / inner) % channels);
+                float m = 0.f, inv = 0.f, sc = 0.f, bi = 0.f;
+                if (NORM != 0) {
+                    m = mean[c];
+                    inv = float(1.0 / sqrt(double(__fadd_rn(variance[c], epsilon))));
+                }
+                if (NORM != 1) {
+                    sc = scale[c];
+                    bi = bias[c];
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float v = in[j];
+                    if (NORM != 0) v = __fmul_rn(__fsub_rn(v, m), inv);
+                    if (NORM != 1) v = __builtin_fmaf(v, sc, bi);
+                    o[j] = v;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) o[j] = apply(in[j], int(((base + j) / inner) % channels));
+            }
+            *reinterpret_cast<v4f *>(out + base) = o;
+        } else {
+            for (int j = 0; j < 4; ++j)
+                if (base + j < count) out[base + j] = apply(x[base + j], int(((base + j) / inner) % channels));
+        }
+    }
+}
+
+template <int NORM>
+int launch_affine(const char *who, const float *x, int64_t pre, int channels, int64_t inner, const float *mean,
+                  const float *variance, const float *scale, const float *bias, float epsilon, float *out, void *stream) {
+    TSX_REQUIRE(pre >= 0 && channels > 0 && inner > 0, "%s: bad extent", who);
+    TSX_REQUIRE((NORM == 0 || (mean && variance)) && (NORM == 1 || (scale && bias)), "%s: null parameter vector", who);
+    const int64_t count = pre * channels * inner;
+    if (count == 0) return 0;
+    TSX_REQUIRE(x && out, "%s: null pointer", who);
+    const bool vec = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    int64_t blocks = tsx::ceil_div(tsx::ceil_div(count, 4), 256);
+    if (blocks > 256 * 8) blocks = 256 * 8;
+    hipLaunchKernelGGL(channel_affine_kernel<NORM>, dim3(unsigned(blocks)), dim3(256), 0, tsx::as_stream(stream), x, count,
+                       channels, inner, mean, variance, scale, bias, epsilon, out, vec);
+    TSX_LAUNCH_CHECK("channel_affine_kernel");
+    return 0;
+}
+
 // out = lhs + rhs (MUL: lhs * rhs) with numpy-style broadcasting over up to 8 aligned axes (an extent of 1 repeats).
 // One lane per output element; an operand's stride is 0 on the axes it is broadcast along.
 struct BroadcastGeom {
@@ -153,6 +226,25 @@ int tsx_add_bias_f32(const float *x_dev, int64_t pre, int32_t channels, int64_t 
                      float *out_dev, void *stream) {
     TSX_REQUIRE(pre >= 0 && channels > 0 && inner > 0 && bias_dev, "add_bias: bad argument");
     return launch<0>(x_dev, pre * channels * inner, bias_dev, channels, inner, 0.f, out_dev, stream);
+}
+
+int tsx_batch_norm_f32(const float *x_dev, int64_t pre, int32_t channels, int64_t inner, const float *mean_dev,
+                       const float *variance_dev, float epsilon, float *out_dev, void *stream) {
+    return launch_affine<1>("batch_norm", x_dev, pre, channels, inner, mean_dev, variance_dev, nullptr, nullptr, epsilon,
+                            out_dev, stream);
+}
+
+int tsx_batch_scale_f32(const float *x_dev, int64_t pre, int32_t channels, int64_t inner, const float *scale_dev,
+                        const float *bias_dev, float *out_dev, void *stream) {
+    return launch_affine<0>("batch_scale", x_dev, pre, channels, inner, nullptr, nullptr, scale_dev, bias_dev, 0.f, out_dev,
+                            stream);
+}
+
+int tsx_fused_batch_norm_f32(const float *x_dev, int64_t pre, int32_t channels, int64_t inner, const float *mean_dev,
+                             const float *variance_dev, const float *scale_dev, const float *bias_dev, float epsilon,
+                             float *out_dev, void *stream) {
+    return launch_affine<2>("fused_batch_norm", x_dev, pre, channels, inner, mean_dev, variance_dev, scale_dev, bias_dev,
+                            epsilon, out_dev, stream);
 }
 
 int tsx_relu_f32(const float *x_dev, int64_t count, float *out_dev, void *stream) {

@@ -116,6 +116,17 @@ def main():
     for name, v in samples.items():
         ref.save_tensor(os.path.join(OUT, "sample.%s.t" % name), v)
 
+    # batch normalisation nodes (their own generator, so that the cases above keep their bytes)
+    rng = np.random.default_rng(20241)
+    xb = (rng.standard_normal((2, 6, 5, 7)) * 2).astype(np.float32)
+    mean, var = rng.standard_normal(6).astype(np.float32), rng.uniform(0.05, 3, 6).astype(np.float32)
+    scale, bias = rng.standard_normal(6).astype(np.float32), rng.standard_normal(6).astype(np.float32)
+    dim1 = {"dim": np.array([1], np.int32)}
+    eps = dict(dim1, epsilon=np.array([1e-3], np.float32))
+    save_case("batch_norm/nchw", "batch_norm", eps, [xb, mean, var])
+    save_case("batch_scale/nchw", "batch_scale", dim1, [xb, scale, bias])
+    save_case("fused_batch_norm/nchw", "fused_batch_norm", eps, [xb, mean, var, scale, bias])
+
 
 if __name__ == "__main__":
     main()

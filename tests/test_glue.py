@@ -122,3 +122,76 @@ def test_hip_pooling_rejects_bad_arguments(tsx):
     assert rc < 0 and b"outside" in tsx.lib().tsx_last_error()
     rc = tsx.lib().tsx_pooling2d_f32(x.data_ptr(), 1, 4, 4, 2, 0, 0, 3, 3, 2, 2, 0, out.data_ptr(), 2, 2, None)
     assert rc < 0
+
+
+# ---------------------------------------------------------------- batch_norm / batch_scale / fused_batch_norm
+
+@pytest.mark.parametrize("shape,dim", [((2, 5, 7, 9), 1), ((3, 6, 4, 4), 1), ((2, 3, 1, 1), 1), ((4, 10), 1), ((2, 3, 5, 6), 3),
+                                       ((1, 8, 13, 3), 2), ((6,), 0)])
+def test_batch_norm_family_against_the_compiled_reference(port, ref, shape, dim):
+    """Bitwise against cpu::BatchNorm / BatchScale / FusedBatchNorm, on inner extents that are and are not
+    multiples of their 4-wide body (body and tail contract x * scale + bias to one fma alike), with variances whose
+    reciprocal root differs between float and double evaluation (the reference's is the double one)."""
+    rng = np.random.default_rng(700 + len(shape) + dim)
+    c = shape[dim]
+    x = (rng.standard_normal(shape) * 3).astype(np.float32)
+    mean, var = rng.standard_normal(c).astype(np.float32), rng.uniform(1e-3, 4, c).astype(np.float32)
+    scale, bias = rng.standard_normal(c).astype(np.float32), rng.standard_normal(c).astype(np.float32)
+    d = {"dim": np.array([dim], np.int32)}
+    for eps in (1e-5, 1e-3):
+        e = dict(d, epsilon=np.array([eps], np.float32))
+        assert np.array_equal(bits(port.batch_norm(x, mean, var, eps, dim)), bits(ref.run_op("batch_norm", e, [x, mean, var], x.nbytes)))
+        assert np.array_equal(bits(port.fused_batch_norm(x, mean, var, scale, bias, eps, dim)),
+                              bits(ref.run_op("fused_batch_norm", e, [x, mean, var, scale, bias], x.nbytes)))
+    assert np.array_equal(bits(port.batch_scale(x, scale, bias, dim)), bits(ref.run_op("batch_scale", d, [x, scale, bias], x.nbytes)))
+    # the default epsilon (include/backend/base/base_batch_norm.h:33)
+    assert np.array_equal(bits(port.batch_norm(x, mean, var, 1e-5, dim)), bits(ref.run_op("batch_norm", d, [x, mean, var], x.nbytes)))
+
+
+def test_batch_norm_family_closed_forms(port):
+    """Without the reference: the definitions in float64 bound the fp32 results, batch_scale is exactly one fused
+    multiply-add per element, and fused_batch_norm is batch_scale applied to batch_norm."""
+    rng = np.random.default_rng(710)
+    x = (rng.standard_normal((3, 7, 5, 6)) * 2).astype(np.float32)
+    mean, var = rng.standard_normal(7).astype(np.float32), rng.uniform(0.05, 3, 7).astype(np.float32)
+    scale, bias = rng.standard_normal(7).astype(np.float32), rng.standard_normal(7).astype(np.float32)
+    sh = (1, 7, 1, 1)
+    bn = port.batch_norm(x, mean, var, 1e-3)
+    exact = (x.astype(np.float64) - mean.reshape(sh)) / np.sqrt(var.reshape(sh).astype(np.float64) + np.float32(1e-3))
+    assert np.abs(bn - exact).max() <= 4e-7 * np.abs(exact).max()
+    bs = port.batch_scale(x, scale, bias)
+    fma = (x.astype(np.float64) * scale.reshape(sh).astype(np.float64) + bias.reshape(sh).astype(np.float64)).astype(np.float32)
+    assert np.count_nonzero(bits(bs) != bits(fma)) <= 2      # float64 evaluation rounds twice in rare ties
+    assert np.array_equal(bits(port.fused_batch_norm(x, mean, var, scale, bias, 1e-3)), bits(port.batch_scale(bn, scale, bias)))
+    assert np.array_equal(bits(port.batch_norm(x, np.zeros(7, np.float32), np.ones(7, np.float32), 0.0)), bits(x))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape,dim", [((2, 5, 7, 9), 1), ((3, 6, 4, 4), 1), ((2, 3, 1, 1), 1), ((4, 10), 1), ((2, 3, 5, 6), 3),
+                                       ((32, 64, 56, 56), 1), ((3, 1000), 1)])
+def test_hip_batch_norm_family(tsx, port, shape, dim):
+    """tsx_batch_norm_f32 / tsx_batch_scale_f32 / tsx_fused_batch_norm_f32 through the C ABI: bit-exact against the
+    oracle (which is bit-exact against the compiled reference), inner extents with and without whole 4-element
+    groups, an unaligned view of the input."""
+    rng = np.random.default_rng(720 + len(shape) + dim)
+    c = shape[dim]
+    x = (rng.standard_normal(shape) * 3).astype(np.float32)
+    mean, var = rng.standard_normal(c).astype(np.float32), rng.uniform(1e-3, 4, c).astype(np.float32)
+    scale, bias = rng.standard_normal(c).astype(np.float32), rng.standard_normal(c).astype(np.float32)
+    xd, md, vd, sd, bd = (_dev(a) for a in (x, mean, var, scale, bias))
+    for eps in (1e-5, 1e-3):
+        assert np.array_equal(bits(tsx.batch_norm(xd, md, vd, eps, dim).cpu().numpy()), bits(port.batch_norm(x, mean, var, eps, dim)))
+        assert np.array_equal(bits(tsx.fused_batch_norm(xd, md, vd, sd, bd, eps, dim).cpu().numpy()),
+                              bits(port.fused_batch_norm(x, mean, var, scale, bias, eps, dim)))
+    assert np.array_equal(bits(tsx.batch_scale(xd, sd, bd, dim).cpu().numpy()), bits(port.batch_scale(x, scale, bias, dim)))
+
+
+@pytest.mark.gpu
+def test_hip_batch_norm_rejects_bad_arguments(tsx):
+    import torch
+    x = torch.zeros((2, 3, 4), device="cuda")
+    v = torch.ones(3, device="cuda")
+    L = tsx.lib()
+    assert L.tsx_batch_norm_f32(tsx._ptr(x), 2, 0, 4, tsx._ptr(v), tsx._ptr(v), 1e-5, tsx._ptr(x), None) == -1
+    assert L.tsx_batch_scale_f32(tsx._ptr(x), 2, 3, 4, None, tsx._ptr(v), tsx._ptr(x), None) == -1
+    assert b"batch_scale" in L.tsx_last_error()

@@ -335,3 +335,27 @@ def test_zipper_option_resolves_the_bias_axis_like_add_bias(ts, tmp_path):
     assert [m.op for m in fused.nodes].count("add_bias") == 1
     (own,) = mf.run_module(fused, [x])
     assert np.array_equal(bits(own), bits(cpu))
+
+
+def test_batch_norm_family_in_tennis_workbench(ts):
+    """batch_norm / batch_scale / fused_batch_norm created with strict device lookup, so the "hip" classes run:
+    bitwise against TenniS's CPU operators; fp64 inputs go through the host delegate."""
+    rng = np.random.default_rng(907)
+    for shape, dim in (((2, 6, 7, 9), 1), ((3, 5, 4, 4), 1), ((4, 10), 1), ((2, 3, 5, 6), 3)):
+        c = shape[dim]
+        x = (rng.standard_normal(shape) * 3).astype(np.float32)
+        mean, var = rng.standard_normal(c).astype(np.float32), rng.uniform(1e-3, 4, c).astype(np.float32)
+        scale, bias = rng.standard_normal(c).astype(np.float32), rng.standard_normal(c).astype(np.float32)
+        d = {"dim": np.array([dim], np.int32)}
+        e = dict(d, epsilon=np.array([1e-3], np.float32))
+        for op, params, inputs in (("batch_norm", e, [x, mean, var]), ("batch_norm", d, [x, mean, var]),
+                                   ("batch_scale", d, [x, scale, bias]), ("fused_batch_norm", e, [x, mean, var, scale, bias])):
+            cpu = ts.run_op_intree("cpu", op, params, inputs, x.nbytes)
+            hip = ts.run_op_intree("hip", op, params, inputs, x.nbytes, strict=True)
+            assert np.array_equal(bits(cpu), bits(hip)), (op, shape)
+    xd = rng.standard_normal((2, 4, 3, 3))
+    vd = rng.uniform(0.5, 2, 4)
+    d = {"dim": np.array([1], np.int32)}
+    cpu = ts.run_op_intree("cpu", "batch_scale", d, [xd, vd, vd], xd.nbytes)
+    hip = ts.run_op_intree("hip", "batch_scale", d, [xd, vd, vd], xd.nbytes, strict=True)
+    assert hip.dtype == np.float64 and np.array_equal(cpu.view(np.uint8), hip.view(np.uint8))

@@ -74,7 +74,7 @@ def test_case_loader():
     assert tc.output[0][0] == tensor_file.FLOAT32 and tc.output[0][1].shape == (2, 12, 7, 7)
     assert run_test.TestCase.load(CASES) is None            # sample files only: not a case
     found = [d for d in run_test.find_cases(CASES) if run_test.TestCase.load(os.path.join(CASES, d))]
-    assert len(found) == 31
+    assert len(found) == 34
 
 
 def test_broken_cases_are_reported(tmp_path):
@@ -110,8 +110,8 @@ def test_reference_cases_pass_on_hip(hip_device):
     text = out.getvalue()
     assert not results[run_test.FAILED] and not results[run_test.WARNING], text
     assert results[run_test.SKIP] == [os.path.join("softmax", "not_on_device")], text
-    assert len(results[run_test.OK]) == 30, text
-    assert "[OK]: 30, [SKIP]: 1, [WARNING]: 0, [FAILED]: 0" in text
+    assert len(results[run_test.OK]) == 33, text
+    assert "[OK]: 33, [SKIP]: 1, [WARNING]: 0, [FAILED]: 0" in text
 
 
 @pytest.mark.gpu
@@ -121,7 +121,8 @@ def test_integer_and_bit_exact_cases_match_exactly(hip_device):
     for sub in ("quantize/per_image", "quantize/single_scale", "conv2d_quantized/3x3_pad1", "conv2d_quantized/1x1_s2",
                 "relu/4d", "add_bias/nchw", "add/broadcast", "pooling2d/max_3x3_s2", "conv2d_winograd/auto_mode",
                 "conv2d_winograd_v2/auto_mode", "pooling2d_v2/avg_3x2", "concat/channels", "concat/last_axis",
-                "_resize2d/nearest_up", "_resize2d/nearest_odd", "mul/broadcast", "mul/same_shape"):
+                "_resize2d/nearest_up", "_resize2d/nearest_odd", "mul/broadcast", "mul/same_shape", "batch_norm/nchw",
+                "batch_scale/nchw", "fused_batch_norm/nchw"):
         tc = run_test.TestCase.load(os.path.join(CASES, *sub.split("/")))
         got = operators.run_op(tc.op, {k: v for k, (_, v) in tc.param.items()}, [tc.input[i][1] for i in range(tc.input_count)])
         want = tc.output[0][1]
