@@ -28,6 +28,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, 5.0 POP/s
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, 8 TB/s
+PEAK_FP32_TFLOPS = 157.3  # MI355X dense fp32 MFMA
 
 CFG = dict(n=32, c=256, h=28, w=28, cout=256, k=3, pad=1)
 
@@ -86,6 +87,83 @@ def cpu_baseline(x, x_scales, wq, dq, bias, pad, images):
     return {"value": 2.0 * macs / dt / 1e12, "unit": "TOPS", "cores": cores, "kind": kind,
             "sample": "%d of %d images of the same layer, %.2f s; %s" % (images, x.shape[0], dt, note),
             "host_cpus": os.cpu_count()}
+
+
+def cpu_baseline_all_cores(x, x_scales, wq, dq, bias, pad):
+    """The same operator chain with OpenMP on every loop, on all host cores: the CPU restatement (oracle/,
+    checked bit for bit against the compiled reference), whose int8 GEMM and dequantize loops are parallel --
+    the reference's own are single-threaded / racy above one thread.  A second baseline beside the faithful one."""
+    from oracle import port
+    threads = min(port.max_threads(), os.cpu_count() or 1, 16)
+    port.set_threads(threads)
+    pads = (pad, pad, pad, pad)
+    port.conv2d_i8_fused(port.quantize(x[:2], x_scales[:2]), wq, dq, bias, "relu", pads=pads)     # warm-up
+    t0 = time.perf_counter()
+    xq = port.quantize(x, x_scales)
+    port.conv2d_i8_fused(xq, wq, dq, bias, "relu", pads=pads)
+    dt = time.perf_counter() - t0
+    macs = x.shape[0] * wq.shape[0] * x.shape[2] * x.shape[3] * wq.shape[1] * wq.shape[2] * wq.shape[3]
+    return {"value": 2.0 * macs / dt / 1e12, "unit": "TOPS", "cores": threads, "kind": "port",
+            "sample": "all %d images of the layer, %.2f s; CPU restatement built -O3 -fopenmp -mavx2 -mfma, OpenMP on "
+                      "every loop" % (x.shape[0], dt), "host_cpus": os.cpu_count()}
+
+
+def config1_leg(reps=50):
+    """BASELINE config 1: fp32 conv2d 1x64x56x56 * 64x64x3x3, stride 1, pad 1, bias + ReLU -- the implicit im2col
+    GEMM on the fp32 MFMA and both Winograd modes (credited the direct convolution's flops), time per launch from
+    HIP events around back-to-back launches."""
+    import torch
+    from tennis_amd import capi
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.rand((1, 64, 56, 56), device=dev, generator=g) * 2 - 1
+    w = torch.randn((64, 64, 3, 3), device=dev, generator=g) * (2.0 / 576) ** 0.5
+    b = torch.randn(64, device=dev, generator=g) * 0.01
+    flops = 2.0 * 64 * 56 * 56 * 64 * 9
+    w63, w23 = capi.WinogradF63(w, (1, 1, 1, 1)), capi.WinogradF23(w, (1, 1, 1, 1))
+    rows = {}
+    for name, fn in (("im2col_gemm", lambda: capi.conv2d_f32(x, w, (1, 1, 1, 1), bias=b, act="relu")),
+                     ("winograd_f63", lambda: w63(x, bias=b, act="relu")), ("winograd_f23", lambda: w23(x, bias=b, act="relu"))):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        t = e0.elapsed_time(e1) * 1e-3 / reps
+        rows[name] = {"us": t * 1e6, "GFLOPS": flops / t / 1e9, "frac_of_fp32_mfma_peak": flops / t / 1e12 / PEAK_FP32_TFLOPS}
+    return {"workload": "BASELINE config 1: fp32 conv2d 1x64x56x56 * 64x64x3x3 s1 p1 + bias + ReLU; 231.2 MFLOP per launch "
+                        "(Winograd credited the same), 49 tiles of 64x64: a batch of one cannot fill 256 CUs", "reps": reps,
+            "peak_TFLOPS": PEAK_FP32_TFLOPS, **rows}
+
+
+def tennis_runtime_leg(reps=5):
+    """The ResNet-50-shaped network (BASELINE config 4) as a `.tsm` module through TenniS's own loader, graph compiler
+    and Workbench on ComputingDevice("hip") -- the operator boundary as a TenniS user meets it (in-tree build of the
+    backend, oracle/ref.mk `intree`; absent where that library was not built)."""
+    import tempfile
+    from oracle import ref
+    from tennis_amd import module_file as mf, resnet50
+    if not ref.intree_available():
+        return None
+    n = 32
+    desc, params = resnet50.make_parameters(seed=0)
+    module = resnet50.to_module(desc, params, batch=n)
+    x = np.random.default_rng(1).random((n, 3, 224, 224), dtype=np.float32)
+    with tempfile.TemporaryDirectory() as tmp:
+        path = os.path.join(tmp, "resnet50_int8_bs32.tsm")
+        mf.write_module(path, module)
+        fused0 = ref.fused_chain_count_intree()
+        ms, logits = ref.time_module_intree("hip", path, [x], warmup=2, reps=reps)
+        fused = ref.fused_chain_count_intree() - fused0
+    return {"workload": "BASELINE config 4 network as a .tsm module (every activation quantized with one fixed multiplier) "
+                        "in TenniS's Workbench on device hip: quantize+conv+bias+relu chains fused by the backend's zipper "
+                        "option, fp32 NCHW between nodes, fp32 inner_prod classifier; each run ends with the logits on the host",
+            "img_per_s": n / (ms * 1e-3), "ms_per_batch": ms, "reps": reps, "chains_fused_by_the_graph_compiler": fused,
+            "logits_finite": bool(np.isfinite(logits).all())}
 
 
 def resnet_leg(steps=20):
@@ -199,8 +277,6 @@ def gemm_leg(reps=20):
     return {"workload": "BASELINE config 3: int8 GEMM sweep, per-row x per-output-channel dequantize + bias, fp32 out",
             "launches_per_figure": 3 * reps, "shapes": rows}
 
-
-PEAK_FP32_TFLOPS = 157.3   # MI355X dense fp32 MFMA
 
 
 def kernels_leg(reps=20):
@@ -352,7 +428,7 @@ def main():
     launch_mode = "direct C-ABI calls on one stream"
 
     # The same step captured once in a HIP graph and replayed: what a serving loop that fixes its shapes does.
-    # The faster of the two launch modes is the step time reported (both are printed).
+    # Reported beside the direct-call time, which is the step time `value` is computed from.
     ms_direct, ms_graph = ms_per_step, None
     if not args.profile:
         side = torch.cuda.Stream()
@@ -374,9 +450,6 @@ def main():
             graph.replay()
         torch.cuda.synchronize()
         ms_graph = (time.perf_counter() - t0) / args.steps * 1e3
-        if ms_graph < ms_per_step:
-            ms_per_step = ms_graph
-            launch_mode = "HIP graph of the step (2 kernels), one replay per step"
 
     def event_time(fn, reps):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -447,9 +520,11 @@ def main():
                                "out; step = quantize+stage kernel + i8-MFMA implicit-GEMM kernel",
                    "algorithmic_ops_per_step": ops, "pct_of_int8_mfma_peak_whole_step": 100.0 * tops / PEAK_INT8_TOPS,
                    "launch": launch_mode, "ms_per_step_direct_calls": ms_direct, "ms_per_step_graph_replay": ms_graph},
-        "roofline": {"bound": "mfma", "kernel": "conv_i8_ws_kernel", "achieved": kernel_tops, "peak": PEAK_INT8_TOPS,
-                     "unit": "TFLOP/s", "frac": kernel_tops / PEAK_INT8_TOPS, "traffic": TRAFFIC_CONV_BYTES,
-                     "traffic_unit": "HBM bytes per launch (rocprofv3 counters; algorithmic 33.65e6)",
+        "roofline": {"bound": "mfma", "kernel": "conv_i8_fl_kernel", "achieved": kernel_tops, "peak": PEAK_INT8_TOPS,
+                     "unit": "TOP/s", "frac": kernel_tops / PEAK_INT8_TOPS, "traffic": TRAFFIC_CONV_BYTES,
+                     "traffic_unit": "HBM bytes per launch, a constant taken from rocprofv3 FETCH_SIZE / WRITE_SIZE of this "
+                                     "kernel on this workload (profiles/conv2d_i8_config2_hbm_traffic.txt), not measured "
+                                     "by this run; algorithmic 33.65e6",
                      "note": "int8 multiply-accumulate ops (TOP/s); 2*N*Cout*Ho*Wo*Cin*9 = %.4g ops per launch, "
                              "avg launch %.2f us over %d back-to-back launches" % (ops, t_mfma * 1e6, reps)},
         "sustained_mfma": None if args.profile else {
@@ -469,8 +544,13 @@ def main():
         result["yolov4_int8_bs8"] = yolo_leg()
     if not args.no_gemm and not args.profile:
         result["gemm_i8_sweep"] = gemm_leg()
+    if not args.profile:
+        result["conv2d_f32_config1"] = config1_leg()
+    if not args.no_resnet and not args.profile:
+        result["resnet50_int8_bs32_tennis_runtime"] = tennis_runtime_leg()
     if args.cpu_images > 0 and not args.profile:
         result["cpu_baseline"] = cpu_baseline(x, x_scales, wq, dq, bias, pad, min(args.cpu_images, cfg["n"]))
+        result["cpu_baseline_openmp_all"] = cpu_baseline_all_cores(x, x_scales, wq, dq, bias, pad)
     print(json.dumps(result))
 
 

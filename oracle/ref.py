@@ -115,6 +115,25 @@ def run_module_intree(device, path, inputs, out_bytes=1 << 24, threads=1):
     return buf[:out.bytes].view(_TS2NP[out.dtype]).reshape(shape).copy()
 
 
+def time_module_intree(device, path, inputs, warmup=2, reps=10, out_bytes=1 << 24, threads=1):
+    """ms per run of a `.tsm` module in a TenniS Workbench on ``device`` of the in-tree build (module loaded and
+    compiled once; each run ends with output 0 read back), and that output."""
+    L = intree_lib()
+    keep = []
+    i = (_Tensor * max(len(inputs), 1))(*[_pack("", v, keep) for v in inputs])
+    buf = np.empty(out_bytes, dtype=np.uint8)
+    out = _Output()
+    out.data = buf.ctypes.data
+    out.capacity = out_bytes
+    ms = ctypes.c_double(0.0)
+    rc = L.ref_time_module(str(path).encode(), device.encode(), len(inputs), i, int(threads), int(warmup), int(reps),
+                           ctypes.byref(ms), ctypes.byref(out))
+    if rc != 0:
+        raise RuntimeError("TenniS raised: " + L.ref_last_error().decode(errors="replace"))
+    shape = tuple(out.shape[k] for k in range(out.ndim))
+    return ms.value, buf[:out.bytes].view(_TS2NP[out.dtype]).reshape(shape).copy()
+
+
 def _pack(name, value, keep):
     """Turn a python value into a _Tensor; ``keep`` holds the buffers alive."""
     if isinstance(value, str):

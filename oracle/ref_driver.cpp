@@ -11,6 +11,7 @@
 // (src/kernels/cpu/winograd_algorithm.cpp:846-947) and the int8 GEMM primitive
 // (src/kernels/cpu/math_cpu.cpp:238-244).
 #include <cstdint>
+#include <chrono>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -193,6 +194,37 @@ int ref_run_module(const char *path, const char *device, int ninputs, const ref_
         for (int i = 0; i < ninputs; ++i) bench->input(i, make_tensor(inputs[i]));
         bench->run();
         ts::Tensor y = bench->output(0).view(ts::MemoryDevice(ts::CPU));
+        out->dtype = int32_t(y.dtype());
+        out->ndim = int32_t(y.dims());
+        for (int i = 0; i < out->ndim && i < 8; ++i) out->shape[i] = y.size(i);
+        out->bytes = int64_t(y.count()) * ts::type_bytes(y.dtype());
+        if (out->bytes > out->capacity) throw std::runtime_error("output buffer too small");
+        std::memcpy(out->data, y.data(), size_t(out->bytes));
+    });
+}
+
+// The same, timed: the module is loaded and compiled once, run `warmup` times, then `reps` times against the wall
+// clock; every run ends with output 0 read back to the host (the one synchronisation a caller of the runtime
+// sees).  Inputs are bound once: their device copies are cached by the runtime's SyncMemory after the first run.
+int ref_time_module(const char *path, const char *device, int ninputs, const ref_tensor *inputs, int threads, int warmup,
+                    int reps, double *ms_per_run, ref_output *out) {
+    return guarded([&] {
+        auto module = ts::Module::Load(path);
+        auto bench = ts::Workbench::Load(module, ts::ComputingDevice(device, 0));
+        bench->runtime().set_computing_thread_number(threads);
+        for (int i = 0; i < ninputs; ++i) bench->input(i, make_tensor(inputs[i]));
+        ts::Tensor y;
+        for (int r = 0; r < warmup; ++r) {
+            bench->run();
+            y = bench->output(0).view(ts::MemoryDevice(ts::CPU));
+        }
+        const auto t0 = std::chrono::steady_clock::now();
+        for (int r = 0; r < reps; ++r) {
+            bench->run();
+            y = bench->output(0).view(ts::MemoryDevice(ts::CPU));
+        }
+        const auto t1 = std::chrono::steady_clock::now();
+        *ms_per_run = std::chrono::duration<double, std::milli>(t1 - t0).count() / (reps > 0 ? reps : 1);
         out->dtype = int32_t(y.dtype());
         out->ndim = int32_t(y.dims());
         for (int i = 0; i < out->ndim && i < 8; ++i) out->shape[i] = y.size(i);
