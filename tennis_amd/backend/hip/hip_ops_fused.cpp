@@ -7,9 +7,13 @@
 // are its zipper options, src/compiler/option/winograd_zipper_option.cpp:16-96); tennis_amd/module_file.py holds
 // that rewrite for module graphs.  Values are those of the chain, bit for bit.
 //
-// Inputs: x fp32 NCHW, w int8 OIHW[, bias fp32 [cout]].  Parameters: those of conv2d_quantized (format, padding
-// [4,2], padding_value, stride [4], dilation [4], dequantize_scales [cout]) plus quantize_scale [n] (the
-// quantize node's) and, optionally, activation ("relu" or "leaky_relu") with scale (leaky_relu's slope).
+// Inputs: x fp32 NCHW, w int8 OIHW[, bias fp32 [cout]][, residual fp32].  Parameters: those of conv2d_quantized
+// (format, padding [4,2], padding_value, stride [4], dilation [4], dequantize_scales [cout]) plus quantize_scale
+// [n] (the quantize node's) and, optionally, activation ("relu" or "leaky_relu") with scale (leaky_relu's slope)
+// and residual: 1 = the last input is the other operand of an `add` node (src/kernels/cpu/add.cpp) that joined
+// the chain in front of the activation, act(y + residual) -- a ResNet block's join --, 2 = behind it,
+// act(y) + residual -- a darknet shortcut.  A residual of the output's shape is added in the MFMA kernel's
+// epilogue; one that broadcasts into it (the general `add`) takes a broadcast pass behind the convolution.
 #define TSX_TS_QUANTIZED_OPS   // Padding2D / Stride2D / Dilation2D come with the quantized skeleton
 #include "hip_ops_common.h"
 
@@ -35,6 +39,7 @@ public:
         field(name::quantize_scale, REQUIRED);
         field("activation", OPTIONAL, tensor::from("none"));
         field(name::scale, OPTIONAL, tensor::from(0.0f));
+        field("residual", OPTIONAL, tensor::from(int(0)));
     }
 
     void init() override {
@@ -58,6 +63,8 @@ public:
         else if (act == "leaky_relu") m_act = TSX_ACT_LEAKY_RELU;
         else TS_LOG_ERROR << "conv2d_quantized_fused: activation must be none, relu or leaky_relu, got " << act << eject;
         m_slope = tensor::to_float(get(name::scale));
+        m_residual = tensor::to_int(get("residual"));
+        if (m_residual < 0 || m_residual > 2) TS_LOG_ERROR << "conv2d_quantized_fused: residual must be 0, 1 or 2" << eject;
     }
 
     int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override {
@@ -72,9 +79,12 @@ public:
         auto &context = ctx::ref<DeviceContext>();
         const MemoryDevice device = context.memory_device;
         Tensor x = stack[0].view(device), w = stack[1].view(device);
-        Tensor bias;
-        const bool with_bias = stack.size() == 3;
+        Tensor bias, residual;
+        const int extra = int(stack.size()) - 2 - (m_residual ? 1 : 0);
+        const bool with_bias = extra == 1;
         if (with_bias) bias = stack[2].view(device);
+        if (m_residual) residual = stack[int(stack.size()) - 1].view(device);
+        const bool same_shape = m_residual && residual.sizes() == proto.sizes();
         Tensor out = *stack.push(proto, device);
         void *stream = current_stream();
         const void *packed = m_state.packed(g, w, device, stream, "conv2d_quantized_fused");
@@ -83,11 +93,30 @@ public:
         tsx_epilogue ep{};
         ep.dq_dev = m_dq_dev.get(m_dq, device);
         ep.bias_dev = with_bias ? bias.data<float>() : nullptr;
-        ep.act = m_act;
+        // a residual that needs broadcasting joins in a pass of its own: the activation in front of it (mode 2) stays
+        // in the epilogue, the one behind it (mode 1) follows that pass
+        const bool split = m_residual && !same_shape;
+        ep.act = (split && m_residual == 1) ? TSX_ACT_NONE : m_act;
         ep.slope = m_slope;
+        if (same_shape) {
+            ep.residual_dev = residual.data<float>();
+            ep.residual_after_act = m_residual == 2 ? 1 : 0;
+        }
         check(tsx_quantize_conv2d_i8_nchw(&g, x.data<float>(), m_q_dev.get(m_q, device), int32_t(m_q.size()), packed,
                                           m_padding_value, &ep, out.data<float>(), nullptr, nullptr, workspace, ws_bytes, stream),
               "tsx_quantize_conv2d_i8_nchw");
+        if (split) {
+            std::vector<int32_t> lhs(proto.sizes().begin(), proto.sizes().end()), rhs(lhs.size(), 1);
+            const Shape &rs = residual.sizes();
+            for (size_t i = 0; i < rs.size(); ++i) rhs[lhs.size() - rs.size() + i] = rs[i];
+            check(tsx_add_broadcast_f32(out.data<float>(), lhs.data(), residual.data<float>(), rhs.data(), int32_t(lhs.size()),
+                                        out.data<float>(), stream),
+                  "tsx_add_broadcast_f32");
+            if (m_residual == 1 && m_act == TSX_ACT_RELU)
+                check(tsx_relu_f32(out.data<float>(), out.count(), out.data<float>(), stream), "tsx_relu_f32");
+            else if (m_residual == 1 && m_act == TSX_ACT_LEAKY_RELU)
+                check(tsx_leaky_relu_f32(out.data<float>(), out.count(), m_slope, out.data<float>(), stream), "tsx_leaky_relu_f32");
+        }
         return 1;
     }
 
@@ -100,8 +129,10 @@ private:
 
     // checks the inputs against the parameters; fills the geometry; returns the output prototype
     Tensor::Prototype out_proto(Stack &stack, tsx_conv2d_geom &g) {
-        if (stack.size() != 2 && stack.size() != 3)
-            TS_LOG_ERROR << "conv2d_quantized_fused expects 2 or 3 inputs (x, w[, bias]), got " << stack.size() << eject;
+        const size_t fixed = m_residual ? 3 : 2;
+        if (stack.size() != fixed && stack.size() != fixed + 1)
+            TS_LOG_ERROR << "conv2d_quantized_fused expects " << fixed << " or " << fixed + 1 << " inputs (x, w[, bias]"
+                         << (m_residual ? ", residual" : "") << "), got " << stack.size() << eject;
         const Tensor &x = stack[0], &w = stack[1];
         if (x.dims() != 4 || w.dims() != 4 || x.dtype() != FLOAT32 || w.dtype() != INT8)
             TS_LOG_ERROR << "conv2d_quantized_fused: x must be float32 NCHW and w int8 OIHW" << eject;
@@ -111,7 +142,7 @@ private:
             TS_LOG_ERROR << "conv2d_quantized_fused: " << m_dq.size() << " dequantize scales for " << w.size(0) << " output channels" << eject;
         if (int32_t(m_q.size()) != x.size(0))      // base_quantize.cpp:26
             TS_LOG_ERROR << "conv2d_quantized_fused: " << m_q.size() << " quantize scales for a batch of " << x.size(0) << eject;
-        if (stack.size() == 3 && !(stack[2].dtype() == FLOAT32 && stack[2].count() == w.size(0)))
+        if (stack.size() == fixed + 1 && !(stack[2].dtype() == FLOAT32 && stack[2].count() == w.size(0)))
             TS_LOG_ERROR << "conv2d_quantized_fused: bias must hold one float32 per output channel" << eject;
         g = make_geom(x, w, Padding2D(m_pad[0], m_pad[1], m_pad[2], m_pad[3]), Stride2D(m_stride[0], m_stride[1]),
                       Dilation2D(m_dil[0], m_dil[1]));
@@ -119,12 +150,26 @@ private:
         const int ho = (g.h + g.pad_top + g.pad_bottom - (g.dilation_h * (g.kh - 1) + 1)) / g.stride_h + 1;
         const int wo = (g.w + g.pad_left + g.pad_right - (g.dilation_w * (g.kw - 1) + 1)) / g.stride_w + 1;
         if (ho <= 0 || wo <= 0) TS_LOG_ERROR << "conv2d_quantized_fused: empty output " << ho << "x" << wo << eject;
-        return Tensor::Prototype(FLOAT32, Shape({x.size(0), w.size(0), ho, wo}));
+        const Shape out({x.size(0), w.size(0), ho, wo});
+        if (m_residual) {
+            // the other operand of the `add` this node absorbed: the output's shape, or one that broadcasts into it
+            const Tensor &r = stack[int(stack.size()) - 1];
+            bool fits = r.dtype() == FLOAT32 && r.dims() <= out.size();
+            for (size_t i = 0; fits && i < r.dims(); ++i) {
+                const int32_t extent = r.size(i), target = out[out.size() - r.dims() + i];
+                fits = extent == target || extent == 1;
+            }
+            if (!fits)
+                TS_LOG_ERROR << "conv2d_quantized_fused: residual " << to_string(r.sizes()) << " does not broadcast into "
+                             << to_string(out) << eject;
+        }
+        return Tensor::Prototype(FLOAT32, out);
     }
 
     std::vector<int32_t> m_pad, m_stride, m_dil;
     float m_padding_value = 0.f, m_slope = 0.f;
     int m_act = TSX_ACT_NONE;
+    int m_residual = 0;   // 0: none; 1: act(y + residual); 2: act(y) + residual
     std::vector<float> m_dq, m_q;
     DeviceFloats m_dq_dev, m_q_dev;
     PackedConv m_state;

@@ -26,25 +26,35 @@ extern "C" __attribute__((visibility("default"))) long tsx_hip_fused_chain_count
 namespace ts {
 namespace hip {
 
-class FusedQuantizedConvOption : public ZipperOption {
-public:
-    bool zip(const ComputingDevice &device, Node node, Node &zipped_node) const final {
-        if (device.type() != DeviceType(DEVICE)) return false;
-        Node cur = node;
-        std::string activation = "none";
-        Tensor slope;
-        const std::string tail = cur.bubble().op();
-        if (tail == name::layer::relu() || tail == "leaky_relu") {
-            if (cur.inputs().size() != 1) return false;
-            if (tail == "leaky_relu") {
+namespace {
+
+bool is_activation(const std::string &op) { return op == name::layer::relu() || op == "leaky_relu"; }
+
+// A chain  quantize -> conv2d_quantized [-> add_bias (channel axis, constant bias)] [-> relu | leaky_relu]
+// matched backwards from its last node; the tensors inside it have no reader outside it.
+struct Chain {
+    std::vector<Node> nodes;         // quantize, conv2d_quantized, weights constant (Node has no empty state)
+    const Node &quantize() const { return nodes[0]; }
+    const Node &conv() const { return nodes[1]; }
+    const Node &weights() const { return nodes[2]; }
+    std::vector<Node> bias;          // empty or the add_bias node's constant
+    std::string activation = "none";
+    Tensor slope;
+
+    // `tail` is the chain's last node; with allow_activation = false a trailing activation does not match
+    bool match(Node tail, bool allow_activation) {
+        Node cur = tail;
+        const std::string op = cur.bubble().op();
+        if (is_activation(op)) {
+            if (!allow_activation || cur.inputs().size() != 1) return false;
+            if (op == "leaky_relu") {
                 if (!cur.bubble().has(name::scale)) return false;
                 slope = cur.bubble().get(name::scale);
             }
-            activation = tail;
+            activation = op;
             cur = cur.input(0);
             if (cur.outputs().size() != 1) return false;       // someone else reads the tensor in front of the activation
         }
-        std::vector<Node> bias;      // empty or the add_bias node's constant
         if (cur.bubble().op() == name::layer::add_bias()) {
             if (cur.inputs().size() != 2 || cur.input(1).bubble().op() != Bubble::Const) return false;
             // the axis as AddBias::init resolves it (src/backend/base/base_add_bias.cpp:27-40): from the format's
@@ -63,34 +73,92 @@ public:
             if (cur.outputs().size() != 1) return false;
         }
         if (cur.bubble().op() != name::layer::conv2d_quantized() || cur.inputs().size() != 2) return false;
-        Node q = cur.input(0), w = cur.input(1);
-        if (q.bubble().op() != name::layer::quantize() || q.inputs().size() != 1 || w.bubble().op() != Bubble::Const) return false;
-        const Bubble &conv = cur.bubble();
-        if (!conv.has(name::format) || tensor::to_string(conv.get(name::format)) != name::NCHW) return false;
+        nodes = {cur.input(0), cur, cur.input(1)};
+        if (quantize().bubble().op() != name::layer::quantize() || quantize().inputs().size() != 1 ||
+            weights().bubble().op() != Bubble::Const)
+            return false;
+        const Bubble &c = conv().bubble();
+        if (!c.has(name::format) || tensor::to_string(c.get(name::format)) != name::NCHW) return false;
         // what the fused operator checks at run time, checked here where the graph shows it, so that a chain which
         // ran unfused is not turned into one that ejects: int8 OIHW weights, one float32 bias value per output
         // channel, and -- where the graph carries the inferred type -- a float32 tensor in front of the quantize
-        if (!w.bubble().has(name::value)) return false;
-        const Tensor weights = w.bubble().get(name::value);
-        if (weights.dtype() != INT8 || weights.dims() != 4) return false;
+        if (!weights().bubble().has(name::value)) return false;
+        const Tensor w = weights().bubble().get(name::value);
+        if (w.dtype() != INT8 || w.dims() != 4) return false;
         if (!bias.empty()) {
             if (!bias[0].bubble().has(name::value)) return false;
             const Tensor b = bias[0].bubble().get(name::value);
-            if (b.dtype() != FLOAT32 || b.count() != weights.size(0)) return false;
+            if (b.dtype() != FLOAT32 || b.count() != w.size(0)) return false;
         }
-        const Bubble &source = q.input(0).bubble();
+        const Bubble &source = quantize().input(0).bubble();
         if (source.has("#dtype") && DTYPE(tensor::to_int(source.get("#dtype"))) != FLOAT32) return false;
+        return true;
+    }
+};
 
-        std::vector<Node> inputs = {q.input(0), w};
-        inputs.insert(inputs.end(), bias.begin(), bias.end());
+}  // namespace
+
+class FusedQuantizedConvOption : public ZipperOption {
+public:
+    bool zip(const ComputingDevice &device, Node node, Node &zipped_node) const final {
+        if (device.type() != DeviceType(DEVICE)) return false;
+        // Three shapes of the same rewrite, all ending in `node`:
+        //   chain                               -> fused(x, w[, bias])
+        //   [relu | leaky_relu <-] add(chain without activation, other)   -> fused(..., other), residual = 1:
+        //                                          the join of a residual block, act(y + other), in the epilogue
+        //   add(chain with activation, other)   -> fused(..., other), residual = 2: act(y) + other (darknet shortcut)
+        // `add` broadcasts; the fused operator adds an operand of the output's shape in the MFMA kernel's epilogue
+        // and any other in a broadcast pass of its own, so every add that ran still runs.
+        Chain chain;
+        std::vector<Node> residual;
+        int residual_mode = 0;
+        std::string activation = "none";
+        Tensor slope;
+        Node cur = node;
+        if (is_activation(cur.bubble().op()) && cur.inputs().size() == 1 && cur.input(0).bubble().op() == name::layer::add() &&
+            cur.input(0).outputs().size() == 1) {
+            activation = cur.bubble().op();
+            if (activation == "leaky_relu") {
+                if (!cur.bubble().has(name::scale)) return false;
+                slope = cur.bubble().get(name::scale);
+            }
+            cur = cur.input(0);
+        }
+        if (cur.bubble().op() == name::layer::add() && cur.inputs().size() == 2) {
+            for (int k = 0; k < 2 && !residual_mode; ++k) {
+                Node candidate = cur.input(k), other = cur.input(1 - k);
+                if (candidate.outputs().size() != 1 || candidate == other) continue;
+                Chain c;
+                if (!c.match(candidate, activation == "none")) continue;   // never two activations in one epilogue
+                chain = c;
+                residual.push_back(other);
+                residual_mode = c.activation != "none" ? 2 : 1;
+                if (residual_mode == 2) {
+                    activation = c.activation;
+                    slope = c.slope;
+                }
+            }
+            if (!residual_mode) return false;
+        } else {
+            if (cur != node) return false;          // an activation behind an add that did not fold: not a chain's end
+            if (!chain.match(node, true)) return false;
+            activation = chain.activation;
+            slope = chain.slope;
+        }
+
+        std::vector<Node> inputs = {chain.quantize().input(0), chain.weights()};
+        inputs.insert(inputs.end(), chain.bias.begin(), chain.bias.end());
+        inputs.insert(inputs.end(), residual.begin(), residual.end());
         zipped_node = bubble::op(node.bubble().name(), "conv2d_quantized_fused", inputs);
         Bubble &fused = zipped_node.bubble();
+        const Bubble &conv = chain.conv().bubble();
         for (const std::string &param : {name::format, name::padding, name::padding_value, name::stride, name::dilation,
                                          name::typo::dialations, name::dequantize_scales})
             if (conv.has(param)) fused.set(param, conv.get(param));
-        fused.set(name::quantize_scale, q.bubble().get(name::quantize_scale));
+        fused.set(name::quantize_scale, chain.quantize().bubble().get(name::quantize_scale));
         fused.set("activation", tensor::from(activation));
         if (activation == "leaky_relu") fused.set(name::scale, slope);
+        if (residual_mode) fused.set("residual", tensor::from(int(residual_mode)));
         ++g_fused_chains;
         return true;
     }

@@ -188,7 +188,8 @@ def fuse_quantized_chains(module):
         quantize -> conv2d_quantized [-> add_bias (channel axis, constant bias)] [-> relu | leaky_relu]
 
     whose intermediate tensors have no other consumer becomes one `conv2d_quantized_fused` node (two kernels
-    instead of up to four operators exchanging fp32 / int8 tensors; same values bit for bit).  A quantize node that
+    instead of up to four operators exchanging fp32 / int8 tensors; same values bit for bit), and an `add` that joins
+    such a chain to another tensor -- with the activation behind it -- moves into the node's epilogue as well.  A quantize node that
     feeds several convolutions is folded into each of them.  Returns a new Module without the dead nodes; TenniS's
     counterpart of such a pass is a zipper option of its graph compiler
     (src/compiler/option/winograd_zipper_option.cpp:16-96)."""
@@ -247,6 +248,42 @@ def fuse_quantized_chains(module):
                 last = ai
         # the fused node takes the place of the chain's last node, so its consumers keep their links
         nodes[last] = Node(FUSED, nodes[last].name, params, inputs)
+    # second pass: an `add` that joins a fused chain to another tensor (the residual join of a ResNet block, a darknet
+    # shortcut) moves into that chain's epilogue, with the activation behind it:
+    #   [relu | leaky_relu <-] add(chain without activation, other) -> residual = 1: act(y + other)
+    #   add(chain with activation, other)                          -> residual = 2: act(y) + other
+    users = {}
+    for i, n in enumerate(nodes):
+        for j in n.inputs:
+            users.setdefault(j, []).append(i)
+    for j in module.outputs:
+        users.setdefault(j, []).append(-1)
+    for ai, add in enumerate(list(nodes)):
+        if add.op != "add" or len(add.inputs) != 2:
+            continue
+        for k in (0, 1):
+            ci, other = add.inputs[k], add.inputs[1 - k]
+            cand = nodes[ci]
+            if cand.op != FUSED or users.get(ci) != [ai] or ci == other or "residual" in cand.params:
+                continue
+            params = dict(cand.params)
+            last = ai
+            if params.get("activation", "none") != "none":
+                params["residual"] = np.array([2], np.int32)
+            else:
+                params["residual"] = np.array([1], np.int32)
+                act = only_user(ai, "relu")
+                if act is not None:
+                    params["activation"] = "relu"
+                    last = act
+                else:
+                    act = only_user(ai, "leaky_relu")
+                    if act is not None and "scale" in nodes[act].params:
+                        params["activation"] = "leaky_relu"
+                        params["scale"] = nodes[act].params["scale"]
+                        last = act
+            nodes[last] = Node(FUSED, nodes[last].name, params, list(cand.inputs) + [other])
+            break
     # drop what no output reaches any more, renumber
     keep, stack = set(), list(module.outputs) + list(module.inputs)
     while stack:

@@ -359,3 +359,58 @@ def test_batch_norm_family_in_tennis_workbench(ts):
     cpu = ts.run_op_intree("cpu", "batch_scale", d, [xd, vd, vd], xd.nbytes)
     hip = ts.run_op_intree("hip", "batch_scale", d, [xd, vd, vd], xd.nbytes, strict=True)
     assert hip.dtype == np.float64 and np.array_equal(cpu.view(np.uint8), hip.view(np.uint8))
+
+
+def test_zipper_option_folds_residual_joins(ts, tmp_path):
+    """add + relu behind a chain (a residual block's join, the other operand another chain's output), a darknet-style
+    shortcut behind an activated chain, and an add whose other operand broadcasts: TenniS's compiler folds all three
+    into conv2d_quantized_fused nodes, values as on its CPU device bit for bit."""
+    import sys, os
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"))
+    from make_modules import conv_params
+    from tennis_amd import module_file as mf
+    rng = np.random.default_rng(79)
+    n, c, h, w, co = 2, 16, 9, 11, 12
+    N = mf.Node
+    nodes = [N(mf.PARAMETER, "x")]
+
+    def chain(name, src, k, pad, act=None):
+        wq = rng.integers(-127, 128, (co, c, k, k)).astype(np.int8)
+        nodes.append(N("quantize", name + ".q", {"quantize_scale": np.array([7.5, 12.0], np.float32)}, [src]))
+        nodes.append(N(mf.CONST, name + ".w", {"value": wq}))
+        nodes.append(N("conv2d_quantized", name, dict(conv_params((pad,) * 4),
+                                                      dequantize_scales=rng.uniform(1e-4, 1e-3, co).astype(np.float32)),
+                       [len(nodes) - 2, len(nodes) - 1]))
+        nodes.append(N(mf.CONST, name + ".b", {"value": rng.standard_normal(co).astype(np.float32)}))
+        nodes.append(N("add_bias", name + ".bias", {"format": "NCHW"}, [len(nodes) - 2, len(nodes) - 1]))
+        if act:
+            nodes.append(N(act, name + ".act", {"scale": np.array([0.1], np.float32)} if act == "leaky_relu" else {},
+                           [len(nodes) - 1]))
+        return len(nodes) - 1
+
+    a = chain("main", 0, 3, 1)
+    b = chain("proj", 0, 1, 0)
+    nodes.append(N("add", "join", {}, [a, b]))
+    nodes.append(N("relu", "join.relu", {}, [len(nodes) - 1]))
+    join = len(nodes) - 1
+    d = chain("dark", 0, 3, 1, "leaky_relu")
+    nodes.append(N("add", "shortcut", {}, [join, d]))
+    shortcut = len(nodes) - 1
+    e = chain("scaled", 0, 1, 0)
+    nodes.append(N(mf.CONST, "offsets", {"value": rng.standard_normal((1, co, 1, 1)).astype(np.float32)}))
+    nodes.append(N("add", "offset", {}, [e, len(nodes) - 1]))
+    nodes.append(N("concat", "out", {"dim": np.array([1], np.int32)}, [shortcut, len(nodes) - 1]))
+    module = mf.Module(nodes, [0], [len(nodes) - 1])
+    path = str(tmp_path / "residual_cases.tsm")
+    mf.write_module(path, module)
+    x = (rng.standard_normal((n, c, h, w)) * 6).astype(np.float32)
+    cpu = ts.run_module_intree("cpu", path, [x])
+    fused0 = ts.fused_chain_count_intree()
+    hip = ts.run_module_intree("hip", path, [x])
+    assert ts.fused_chain_count_intree() == fused0 + 4     # main (+ join), proj, dark (+ shortcut), scaled (+ offset)
+    assert cpu.shape == (n, 2 * co, h, w)
+    assert np.array_equal(bits(hip), bits(cpu))
+    fused = mf.fuse_quantized_chains(module)
+    assert "add" not in [m.op for m in fused.nodes]
+    (own,) = mf.run_module(fused, [x])
+    assert np.array_equal(bits(own), bits(cpu))

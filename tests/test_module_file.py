@@ -185,3 +185,64 @@ def test_fused_operator_against_the_operator_chain(hip_device):
         ops.run_op(mf.FUSED, dict(fused, quantize_scale=qs[:2]), [x, w, bias])
     with pytest.raises(ops.OperatorError, match="activation must be"):
         ops.run_op(mf.FUSED, dict(fused, activation="gelu"), [x, w, bias])
+
+
+def test_fusing_rewrite_folds_residual_joins():
+    """add (+ relu) behind a chain moves into the fused node: a ResNet-shaped module keeps no add and no relu node;
+    a darknet-style shortcut behind an activated chain becomes residual = 2; an add whose chain operand has a second
+    reader stays."""
+    from tennis_amd import resnet50
+    desc, params = resnet50.make_parameters(seed=3, width=0.25, blocks=(2, 1, 1, 1), classes=10)
+    f = mf.fuse_quantized_chains(resnet50.to_module(desc, params, batch=2))
+    ops = [n.op for n in f.nodes]
+    assert "add" not in ops and "relu" not in ops and "quantize" not in ops
+    joins = [n for n in f.nodes if n.op == mf.FUSED and "residual" in n.params]
+    assert len(joins) == 5 and all(int(n.params["residual"][0]) == 1 and n.params["activation"] == "relu" for n in joins)
+    assert all(len(n.inputs) == 4 for n in joins)             # x, w, bias, the other branch
+    mf.parse_module(mf.serialize_module(f))
+    N = mf.Node
+    w = np.zeros((4, 8, 1, 1), np.int8)
+    conv = {"format": "NCHW", "padding": np.zeros((4, 2), np.int32), "padding_value": np.zeros(1, np.float32),
+            "stride": np.ones(4, np.int32), "dilation": np.ones(4, np.int32), "dequantize_scales": np.ones(4, np.float32)}
+    g = mf.Module([N("<param>", "x"), N("<param>", "s"), N("quantize", "q", {"quantize_scale": np.ones(1, np.float32)}, [0]),
+                   N("<const>", "w", {"value": w}), N("conv2d_quantized", "c", conv, [2, 3]),
+                   N("leaky_relu", "act", {"scale": np.array([0.1], np.float32)}, [4]), N("add", "shortcut", {}, [1, 5])], [0, 1], [6])
+    fg = mf.fuse_quantized_chains(g)
+    fused = [n for n in fg.nodes if n.op == mf.FUSED]
+    assert len(fused) == 1 and int(fused[0].params["residual"][0]) == 2 and fused[0].params["activation"] == "leaky_relu"
+    assert [fg.nodes[i].name for i in fused[0].inputs] == ["x", "w", "s"] and "add" not in [n.op for n in fg.nodes]
+    g2 = mf.Module(g.nodes + [N("relu", "second_reader", {}, [5]), N("add", "sum", {}, [6, 7])], [0, 1], [8])
+    ops2 = [n.op for n in mf.fuse_quantized_chains(g2).nodes]
+    assert ops2.count("add") == 2 and ops2.count(mf.FUSED) == 1
+
+
+@pytest.mark.gpu
+def test_fused_operator_with_residual_against_the_operator_chain(hip_device):
+    """conv2d_quantized_fused with a residual input against quantize -> conv2d_quantized -> add_bias -> [act] -> add
+    [-> act] run operator by operator: residual of the output's shape (the MFMA kernel's epilogue) and residuals that
+    broadcast into it (the broadcast pass), both join orders."""
+    from tennis_amd import operators as ops
+    rng = np.random.default_rng(43)
+    x = (rng.standard_normal((2, 24, 9, 11)) * 6).astype(np.float32)
+    w = rng.integers(-127, 128, (130, 24, 3, 3)).astype(np.int8)
+    bias = rng.standard_normal(130).astype(np.float32)
+    qs = np.array([7.0, 9.5], np.float32)
+    conv = dict(ops.conv_params((1, 1, 1, 1)), dequantize_scales=rng.uniform(1e-4, 1e-3, 130).astype(np.float32))
+    y0 = ops.run_op("add_bias", {"format": "NCHW"},
+                    [ops.run_op("conv2d_quantized", conv, [ops.run_op("quantize", {"quantize_scale": qs}, [x]), w]), bias])
+    slope = {"scale": np.array([0.1], np.float32)}
+    for shape in ((2, 130, 9, 11), (1, 130, 1, 1), (9, 11), (1,)):
+        r = rng.standard_normal(shape).astype(np.float32)
+        for act in ("none", "relu", "leaky_relu"):
+            apply = lambda t: t if act == "none" else ops.run_op(act, slope if act == "leaky_relu" else {}, [t])
+            want1 = apply(ops.run_op("add", {}, [y0, r]))                    # act(y + r)
+            want2 = ops.run_op("add", {}, [apply(y0), r])                    # act(y) + r
+            base = dict(conv, quantize_scale=qs, activation=act, scale=slope["scale"])
+            got1 = ops.run_op(mf.FUSED, dict(base, residual=np.array([1], np.int32)), [x, w, bias, r])
+            assert np.array_equal(bits(got1), bits(want1)), (shape, act, 1)
+            got2 = ops.run_op(mf.FUSED, dict(base, residual=np.array([2], np.int32)), [x, w, bias, r])
+            assert np.array_equal(bits(got2), bits(want2)), (shape, act, 2)
+    with pytest.raises(ops.OperatorError, match="does not broadcast into"):
+        ops.run_op(mf.FUSED, dict(base, residual=np.array([1], np.int32)), [x, w, bias, np.zeros((3, 130, 9, 11), np.float32)])
+    with pytest.raises(ops.OperatorError, match="inputs"):
+        ops.run_op(mf.FUSED, dict(base, residual=np.array([1], np.int32)), [x, w])
