@@ -167,6 +167,12 @@ int tsx_conv2d_i8_staged(const tsx_conv2d_geom *g, const void *staged_dev, const
 int tsx_conv2d_i8_staged_dims(const tsx_conv2d_geom *g, int32_t *hs, int32_t *ws, int32_t *cp);
 int tsx_conv2d_i8_stage_fill(const tsx_conv2d_geom *g, float padding_value, void *staged_dev, size_t staged_bytes,
                              void *stream);
+/*   stage_fill_halo : the same for a buffer of exactly tsx_conv2d_i8_workspace_bytes(g) bytes whose interior a
+ *                 producer's epilogue is about to write: only the halo pixels and the channel padding are
+ *                 written (nothing at all for a layer without either) -- for callers whose staged buffer is fresh
+ *                 memory on every run, such as an operator output. */
+int tsx_conv2d_i8_stage_fill_halo(const tsx_conv2d_geom *g, float padding_value, void *staged_dev, size_t staged_bytes,
+                                  void *stream);
 int tsx_conv2d_i8_staged_at(const tsx_conv2d_geom *g, const void *staged_dev, int32_t staged_hs, int32_t staged_ws,
                             const void *packed_w_dev, const tsx_epilogue *ep, float *out_f32_dev, int8_t *out_i8_dev,
                             int32_t *out_acc_dev, void *stream);

@@ -14,6 +14,16 @@
 // the chain in front of the activation, act(y + residual) -- a ResNet block's join --, 2 = behind it,
 // act(y) + residual -- a darknet shortcut.  A residual of the output's shape is added in the MFMA kernel's
 // epilogue; one that broadcasts into it (the general `add`) takes a broadcast pass behind the convolution.
+//
+// Two such nodes in a row -- the first's output read by the second's quantize and by nothing else -- exchange the
+// activation as int8 in the second's staged layout (pixel-major, channel-blocked, halo included;
+// tsx_conv2d_i8_staged_dims) instead of fp32 NCHW: the producer carries the consumer's quantize_scale and
+// convolution geometry as next_quantize_scale, next_ksize [2], next_padding [top, bottom, left, right],
+// next_stride [2], next_dilation [2], next_padding_value, requantizes in its epilogue
+// (quantize(act(...)) of the consumer's quantize node, value for value) and returns an INT8 tensor
+// [n, hs, ws, cp]; the consumer is marked staged_input = 1 and runs the MFMA kernel on that tensor directly.
+// No staging pass, a quarter of the bytes.  The reference leaves this to a TODO
+// (src/backend/base/base_conv2d_quantized.cpp:163).
 #define TSX_TS_QUANTIZED_OPS   // Padding2D / Stride2D / Dilation2D come with the quantized skeleton
 #include "hip_ops_common.h"
 
@@ -40,6 +50,13 @@ public:
         field("activation", OPTIONAL, tensor::from("none"));
         field(name::scale, OPTIONAL, tensor::from(0.0f));
         field("residual", OPTIONAL, tensor::from(int(0)));
+        field("staged_input", OPTIONAL, tensor::from(int(0)));
+        field("next_quantize_scale", OPTIONAL);
+        field("next_ksize", OPTIONAL);
+        field("next_padding", OPTIONAL);
+        field("next_stride", OPTIONAL);
+        field("next_dilation", OPTIONAL);
+        field("next_padding_value", OPTIONAL, tensor::from(0.0f));
     }
 
     void init() override {
@@ -65,17 +82,27 @@ public:
         m_slope = tensor::to_float(get(name::scale));
         m_residual = tensor::to_int(get("residual"));
         if (m_residual < 0 || m_residual > 2) TS_LOG_ERROR << "conv2d_quantized_fused: residual must be 0, 1 or 2" << eject;
+        m_staged_input = tensor::to_int(get("staged_input")) != 0;
+        m_next = has("next_quantize_scale");
+        if (m_next) {
+            m_next_q = tensor::array::to_float(get("next_quantize_scale"));
+            m_next_ksize = ints("next_ksize", 2);
+            m_next_pad = ints("next_padding", 4);
+            m_next_stride = ints("next_stride", 2);
+            m_next_dil = ints("next_dilation", 2);
+            m_next_padding_value = tensor::to_float(get("next_padding_value"));
+        }
     }
 
     int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override {
-        tsx_conv2d_geom g;
-        output.assign(1, out_proto(stack, g));
+        tsx_conv2d_geom g, gn;
+        output.assign(1, out_proto(stack, g, gn));
         return 1;
     }
 
     int run(Stack &stack) override {
-        tsx_conv2d_geom g;
-        const Tensor::Prototype proto = out_proto(stack, g);
+        tsx_conv2d_geom g, gn;
+        const Tensor::Prototype proto = out_proto(stack, g, gn);
         auto &context = ctx::ref<DeviceContext>();
         const MemoryDevice device = context.memory_device;
         Tensor x = stack[0].view(device), w = stack[1].view(device);
@@ -84,12 +111,11 @@ public:
         const bool with_bias = extra == 1;
         if (with_bias) bias = stack[2].view(device);
         if (m_residual) residual = stack[int(stack.size()) - 1].view(device);
-        const bool same_shape = m_residual && residual.sizes() == proto.sizes();
+        const Shape conv_shape({g.n, g.cout, m_ho, m_wo});
+        const bool same_shape = m_residual && residual.sizes() == conv_shape;
         Tensor out = *stack.push(proto, device);
         void *stream = current_stream();
         const void *packed = m_state.packed(g, w, device, stream, "conv2d_quantized_fused");
-        const size_t ws_bytes = tsx_conv2d_i8_workspace_bytes(&g);
-        void *workspace = m_state.workspace(ws_bytes, device);
         tsx_epilogue ep{};
         ep.dq_dev = m_dq_dev.get(m_dq, device);
         ep.bias_dev = with_bias ? bias.data<float>() : nullptr;
@@ -102,9 +128,33 @@ public:
             ep.residual_dev = residual.data<float>();
             ep.residual_after_act = m_residual == 2 ? 1 : 0;
         }
-        check(tsx_quantize_conv2d_i8_nchw(&g, x.data<float>(), m_q_dev.get(m_q, device), int32_t(m_q.size()), packed,
-                                          m_padding_value, &ep, out.data<float>(), nullptr, nullptr, workspace, ws_bytes, stream),
-              "tsx_quantize_conv2d_i8_nchw");
+        float *out_f32 = out.data<float>();
+        if (m_next) {
+            if (split) TS_LOG_ERROR << "conv2d_quantized_fused: a residual that broadcasts cannot be combined with next_*" << eject;
+            // the consumer's staged input: halo and channel padding first (the tensor is fresh memory every run),
+            // then the interior from the epilogue
+            const size_t bytes = size_t(out.count());
+            check(tsx_conv2d_i8_stage_fill_halo(&gn, m_next_padding_value, out.data(), bytes, stream), "tsx_conv2d_i8_stage_fill_halo");
+            ep.q_scales_dev = m_next_q_dev.get(m_next_q, device);
+            ep.n_qscales = int32_t(m_next_q.size());
+            ep.staged_out_dev = static_cast<int8_t *>(out.data());
+            ep.staged_hs = out.size(1);
+            ep.staged_ws = out.size(2);
+            ep.staged_cp = out.size(3);
+            ep.staged_pad_top = gn.pad_top;
+            ep.staged_pad_left = gn.pad_left;
+            out_f32 = nullptr;
+        }
+        if (m_staged_input) {
+            check(tsx_conv2d_i8_staged_at(&g, x.data(), x.size(1), x.size(2), packed, &ep, out_f32, nullptr, nullptr, stream),
+                  "tsx_conv2d_i8_staged_at");
+        } else {
+            const size_t ws_bytes = tsx_conv2d_i8_workspace_bytes(&g);
+            void *workspace = m_state.workspace(ws_bytes, device);
+            check(tsx_quantize_conv2d_i8_nchw(&g, x.data<float>(), m_q_dev.get(m_q, device), int32_t(m_q.size()), packed,
+                                              m_padding_value, &ep, out_f32, nullptr, nullptr, workspace, ws_bytes, stream),
+                  "tsx_quantize_conv2d_i8_nchw");
+        }
         if (split) {
             std::vector<int32_t> lhs(proto.sizes().begin(), proto.sizes().end()), rhs(lhs.size(), 1);
             const Shape &rs = residual.sizes();
@@ -127,30 +177,52 @@ private:
         return v;
     }
 
-    // checks the inputs against the parameters; fills the geometry; returns the output prototype
-    Tensor::Prototype out_proto(Stack &stack, tsx_conv2d_geom &g) {
+    // checks the inputs against the parameters; fills the geometry (and, with next_*, the consumer's); returns the
+    // output prototype
+    Tensor::Prototype out_proto(Stack &stack, tsx_conv2d_geom &g, tsx_conv2d_geom &gn) {
         const size_t fixed = m_residual ? 3 : 2;
         if (stack.size() != fixed && stack.size() != fixed + 1)
             TS_LOG_ERROR << "conv2d_quantized_fused expects " << fixed << " or " << fixed + 1 << " inputs (x, w[, bias]"
                          << (m_residual ? ", residual" : "") << "), got " << stack.size() << eject;
         const Tensor &x = stack[0], &w = stack[1];
-        if (x.dims() != 4 || w.dims() != 4 || x.dtype() != FLOAT32 || w.dtype() != INT8)
-            TS_LOG_ERROR << "conv2d_quantized_fused: x must be float32 NCHW and w int8 OIHW" << eject;
-        if (x.size(1) != w.size(1))
-            TS_LOG_ERROR << "conv2d_quantized_fused: x has " << x.size(1) << " channels, w " << w.size(1) << eject;
+        if (w.dims() != 4 || w.dtype() != INT8) TS_LOG_ERROR << "conv2d_quantized_fused: w must be int8 OIHW" << eject;
+        const Padding2D padding(m_pad[0], m_pad[1], m_pad[2], m_pad[3]);
+        if (m_staged_input) {
+            // x is this convolution's staged input [n, hs, ws, cp], written by the producing node
+            if (x.dims() != 4 || x.dtype() != INT8)
+                TS_LOG_ERROR << "conv2d_quantized_fused: staged_input expects an int8 tensor [n, hs, ws, cp]" << eject;
+            // a map of hs - pads by ws - pads reads exactly the staged rows and columns (the producer's true extent may
+            // be up to stride - 1 larger: those rows and columns lie behind the last window)
+            g = tsx_conv2d_geom{x.size(0), w.size(1), x.size(1) - m_pad[0] - m_pad[1], x.size(2) - m_pad[2] - m_pad[3],
+                                w.size(0), w.size(2), w.size(3), m_pad[0], m_pad[1], m_pad[2], m_pad[3],
+                                m_stride[0], m_stride[1], m_dil[0], m_dil[1]};
+            if (g.h < 1 || g.w < 1) TS_LOG_ERROR << "conv2d_quantized_fused: staged input smaller than the padding" << eject;
+            int32_t hs = 0, ws = 0, cp = 0;
+            if (tsx_conv2d_i8_staged_dims(&g, &hs, &ws, &cp) != 0)
+                TS_LOG_ERROR << "[hip] conv2d_quantized_fused: " << tsx_last_error() << eject;
+            if (hs > x.size(1) || ws > x.size(2) || cp != x.size(3))
+                TS_LOG_ERROR << "conv2d_quantized_fused: staged input " << to_string(x.sizes()) << " does not hold the [" << hs << ", "
+                             << ws << ", " << cp << "] this convolution reads" << eject;
+        } else {
+            if (x.dims() != 4 || x.dtype() != FLOAT32)
+                TS_LOG_ERROR << "conv2d_quantized_fused: x must be float32 NCHW and w int8 OIHW" << eject;
+            if (x.size(1) != w.size(1))
+                TS_LOG_ERROR << "conv2d_quantized_fused: x has " << x.size(1) << " channels, w " << w.size(1) << eject;
+            g = make_geom(x, w, padding, Stride2D(m_stride[0], m_stride[1]), Dilation2D(m_dil[0], m_dil[1]));
+        }
         if (int32_t(m_dq.size()) != w.size(0))
             TS_LOG_ERROR << "conv2d_quantized_fused: " << m_dq.size() << " dequantize scales for " << w.size(0) << " output channels" << eject;
         if (int32_t(m_q.size()) != x.size(0))      // base_quantize.cpp:26
             TS_LOG_ERROR << "conv2d_quantized_fused: " << m_q.size() << " quantize scales for a batch of " << x.size(0) << eject;
         if (stack.size() == fixed + 1 && !(stack[2].dtype() == FLOAT32 && stack[2].count() == w.size(0)))
             TS_LOG_ERROR << "conv2d_quantized_fused: bias must hold one float32 per output channel" << eject;
-        g = make_geom(x, w, Padding2D(m_pad[0], m_pad[1], m_pad[2], m_pad[3]), Stride2D(m_stride[0], m_stride[1]),
-                      Dilation2D(m_dil[0], m_dil[1]));
         // include/backend/common_function.h:30-40
         const int ho = (g.h + g.pad_top + g.pad_bottom - (g.dilation_h * (g.kh - 1) + 1)) / g.stride_h + 1;
         const int wo = (g.w + g.pad_left + g.pad_right - (g.dilation_w * (g.kw - 1) + 1)) / g.stride_w + 1;
         if (ho <= 0 || wo <= 0) TS_LOG_ERROR << "conv2d_quantized_fused: empty output " << ho << "x" << wo << eject;
-        const Shape out({x.size(0), w.size(0), ho, wo});
+        m_ho = ho;
+        m_wo = wo;
+        const Shape out({g.n, w.size(0), ho, wo});
         if (m_residual) {
             // the other operand of the `add` this node absorbed: the output's shape, or one that broadcasts into it
             const Tensor &r = stack[int(stack.size()) - 1];
@@ -163,13 +235,27 @@ private:
                 TS_LOG_ERROR << "conv2d_quantized_fused: residual " << to_string(r.sizes()) << " does not broadcast into "
                              << to_string(out) << eject;
         }
-        return Tensor::Prototype(FLOAT32, out);
+        if (!m_next) return Tensor::Prototype(FLOAT32, out);
+        // the consumer's staged input
+        if (int32_t(m_next_q.size()) != g.n)
+            TS_LOG_ERROR << "conv2d_quantized_fused: " << m_next_q.size() << " next_quantize_scale values for a batch of " << g.n << eject;
+        gn = tsx_conv2d_geom{g.n, w.size(0), ho, wo, 1, m_next_ksize[0], m_next_ksize[1], m_next_pad[0], m_next_pad[1],
+                             m_next_pad[2], m_next_pad[3], m_next_stride[0], m_next_stride[1], m_next_dil[0], m_next_dil[1]};
+        int32_t hs = 0, ws = 0, cp = 0;
+        if (tsx_conv2d_i8_staged_dims(&gn, &hs, &ws, &cp) != 0) TS_LOG_ERROR << "[hip] conv2d_quantized_fused: " << tsx_last_error() << eject;
+        return Tensor::Prototype(INT8, Shape({g.n, hs, ws, cp}));
     }
 
     std::vector<int32_t> m_pad, m_stride, m_dil;
     float m_padding_value = 0.f, m_slope = 0.f;
     int m_act = TSX_ACT_NONE;
     int m_residual = 0;   // 0: none; 1: act(y + residual); 2: act(y) + residual
+    bool m_staged_input = false, m_next = false;
+    std::vector<float> m_next_q;
+    std::vector<int32_t> m_next_ksize, m_next_pad, m_next_stride, m_next_dil;
+    float m_next_padding_value = 0.f;
+    int m_ho = 0, m_wo = 0;
+    DeviceFloats m_next_q_dev;
     std::vector<float> m_dq, m_q;
     DeviceFloats m_dq_dev, m_q_dev;
     PackedConv m_state;

@@ -146,11 +146,64 @@ public:
             slope = chain.slope;
         }
 
-        std::vector<Node> inputs = {chain.quantize().input(0), chain.weights()};
+        zipped_node = build(chain, activation, slope, residual, residual_mode, nullptr, node.bubble().name());
+        return true;
+    }
+
+private:
+    // What a producer has to know about the chain that reads its output to write that chain's staged int8 input.
+    struct Next {
+        Tensor quantize_scale, ksize, padding, stride, dilation, padding_value;
+    };
+
+    static Tensor int_vector(std::initializer_list<int32_t> values) {
+        const std::vector<int32_t> v(values);
+        return tensor::build(INT32, Shape({int32_t(v.size())}), v.data());
+    }
+
+    // The consumer side of an int8 hand-over, from the chain's conv2d_quantized node; false when the layer cannot
+    // read a staged buffer a producer wrote (few input channels under a large kernel are staged by im2col).
+    static bool describe(const Chain &chain, Next &next) {
+        const Bubble &conv = chain.conv().bubble();
+        const Tensor w = chain.weights().bubble().get(name::value);
+        const int c = w.size(1), kh = w.size(2), kw = w.size(3);
+        if (kh * kw > 1 && c <= 8 && c * kh * kw <= 512) return false;
+        if (!conv.has(name::padding) || !conv.has(name::stride)) return false;
+        const std::vector<int32_t> pad = tensor::array::to_int(conv.get(name::padding));
+        const std::vector<int32_t> stride = tensor::array::to_int(conv.get(name::stride));
+        const std::string dil_name = conv.has(name::dilation) ? name::dilation : name::typo::dialations;
+        if (!conv.has(dil_name)) return false;
+        const std::vector<int32_t> dil = tensor::array::to_int(conv.get(dil_name));
+        if (pad.size() != 8 || stride.size() != 4 || dil.size() != 4) return false;
+        next.quantize_scale = chain.quantize().bubble().get(name::quantize_scale);
+        next.ksize = int_vector({kh, kw});
+        next.padding = int_vector({pad[4], pad[5], pad[6], pad[7]});
+        next.stride = int_vector({stride[2], stride[3]});
+        next.dilation = int_vector({dil[2], dil[3]});
+        next.padding_value = conv.has(name::padding_value) ? conv.get(name::padding_value) : tensor::from(0.0f);
+        return true;
+    }
+
+    // The conv2d_quantized_fused node for `chain`.  When the tensor in front of the chain's quantize is itself the
+    // end of a chain and nothing else reads it, that chain is built here too, as a producer that writes this one's
+    // staged int8 input (and so on up the line): consecutive quantized convolutions exchange int8 in the consumer's
+    // layout, with no staging pass and no fp32 tensor in between.
+    static Node build(const Chain &chain, const std::string &activation, const Tensor &slope, const std::vector<Node> &residual,
+                      int residual_mode, const Next *next, const std::string &node_name) {
+        Node source = chain.quantize().input(0);
+        bool staged_input = false;
+        Next mine;
+        Chain producer;
+        if (chain.quantize().outputs().size() == 1 && source.outputs().size() == 1 && describe(chain, mine) &&
+            producer.match(source, true)) {
+            source = build(producer, producer.activation, producer.slope, {}, 0, &mine, source.bubble().name());
+            staged_input = true;
+        }
+        std::vector<Node> inputs = {source, chain.weights()};
         inputs.insert(inputs.end(), chain.bias.begin(), chain.bias.end());
         inputs.insert(inputs.end(), residual.begin(), residual.end());
-        zipped_node = bubble::op(node.bubble().name(), "conv2d_quantized_fused", inputs);
-        Bubble &fused = zipped_node.bubble();
+        Node made = bubble::op(node_name, "conv2d_quantized_fused", inputs);
+        Bubble &fused = made.bubble();
         const Bubble &conv = chain.conv().bubble();
         for (const std::string &param : {name::format, name::padding, name::padding_value, name::stride, name::dilation,
                                          name::typo::dialations, name::dequantize_scales})
@@ -159,8 +212,17 @@ public:
         fused.set("activation", tensor::from(activation));
         if (activation == "leaky_relu") fused.set(name::scale, slope);
         if (residual_mode) fused.set("residual", tensor::from(int(residual_mode)));
+        if (staged_input) fused.set("staged_input", tensor::from(int(1)));
+        if (next) {
+            fused.set("next_quantize_scale", next->quantize_scale);
+            fused.set("next_ksize", next->ksize);
+            fused.set("next_padding", next->padding);
+            fused.set("next_stride", next->stride);
+            fused.set("next_dilation", next->dilation);
+            fused.set("next_padding_value", next->padding_value);
+        }
         ++g_fused_chains;
-        return true;
+        return made;
     }
 };
 

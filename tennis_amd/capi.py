@@ -67,6 +67,7 @@ SIGNATURES = {
     "tsx_conv2d_i8_staged_dims": (ctypes.c_int, [ctypes.POINTER(ConvGeom), ctypes.POINTER(_i32), ctypes.POINTER(_i32),
                                                  ctypes.POINTER(_i32)]),
     "tsx_conv2d_i8_stage_fill": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _f32, _vp, _sz, _vp]),
+    "tsx_conv2d_i8_stage_fill_halo": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _f32, _vp, _sz, _vp]),
     "tsx_conv2d_i8_staged_at": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _i32, _i32, _vp, ctypes.POINTER(Epilogue), _vp,
                                                _vp, _vp, _vp]),
     "tsx_gemm_i8_packed_weight_bytes": (_sz, [_i32, _i32]),
@@ -192,15 +193,18 @@ class StagedInput:
     """The staged (channel-blocked, padded) int8 input of one convolution for one input shape: producers write
     their requantized output straight into it, the convolution (and other consumers of the same tensor) read it."""
 
-    def __init__(self, conv, x_shape):
+    def __init__(self, conv, x_shape, halo_only=False):
+        """halo_only: the buffer starts as garbage and only what a producer does not write is set (what an
+        operator whose output tensor is fresh memory on every run does)."""
         geom, _, ws_bytes = conv._plan(tuple(x_shape))
         hs, ws, cp = _i32(), _i32(), _i32()
         check(lib().tsx_conv2d_i8_staged_dims(ctypes.byref(geom), ctypes.byref(hs), ctypes.byref(ws), ctypes.byref(cp)))
         self.x_shape = tuple(x_shape)
         self.hs, self.ws, self.cp = hs.value, ws.value, cp.value
         self.pad_top, self.pad_left = conv.pads[0], conv.pads[2]
-        self.buf = torch.empty(max(ws_bytes, 16), dtype=torch.int8, device=conv.w.device)
-        check(lib().tsx_conv2d_i8_stage_fill(ctypes.byref(geom), conv.padding_value, _ptr(self.buf), ws_bytes, _stream()))
+        self.buf = torch.full((max(ws_bytes, 16),), 0x55, dtype=torch.int8, device=conv.w.device)
+        fill = lib().tsx_conv2d_i8_stage_fill_halo if halo_only else lib().tsx_conv2d_i8_stage_fill
+        check(fill(ctypes.byref(geom), conv.padding_value, _ptr(self.buf), ws_bytes, _stream()))
 
 
 class StagedPlain:

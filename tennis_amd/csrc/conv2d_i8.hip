@@ -22,6 +22,7 @@
 // r of lane l holds row 8*(r/4) + 4*(l/32) + (r%4), column l % 32.
 #include "igemm_i8.hpp"
 
+#include <algorithm>
 #include <cmath>
 #include <mutex>
 
@@ -519,6 +520,31 @@ __global__ __launch_bounds__(256) void stage_fill_kernel(int8_t *__restrict__ xs
     const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
     if (id >= chunks) return;
     const int c0 = int((id * 16) % cp);
+    uint32_t words[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        uint32_t word = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (c0 + v * 4 + j < c) word |= uint32_t(pad_value & 0xff) << (8 * j);
+        words[v] = word;
+    }
+    *reinterpret_cast<uint4 *>(xs + id * 16) = make_uint4(words[0], words[1], words[2], words[3]);
+}
+
+// The same for a buffer whose interior a producer is about to write: only the halo pixels and the channel padding
+// (every 16-byte chunk that is not wholly real channels of an interior pixel; the producer's epilogue writes
+// those, 16 channels at a time).
+__global__ __launch_bounds__(256) void stage_fill_halo_kernel(int8_t *__restrict__ xs, int64_t chunks, int hs, int ws, int cp, int c,
+                                                             int pad_top, int pad_left, int h, int w, int pad_value) {
+    const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id >= chunks) return;
+    const int cpc = cp / 16;
+    const int64_t pixel = id / cpc;
+    const int c0 = int(id - pixel * cpc) * 16;
+    const int col = int(pixel % ws), row = int((pixel / ws) % hs);
+    const bool inside = row >= pad_top && row < pad_top + h && col >= pad_left && col < pad_left + w;
+    if (inside && c0 + 16 <= c) return;
     uint32_t words[4];
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
@@ -1247,6 +1273,27 @@ int tsx_conv2d_i8_stage_fill(const tsx_conv2d_geom *g, float padding_value, void
     hipLaunchKernelGGL(stage_fill_kernel, dim3(unsigned(tsx::ceil_div(chunks, 256))), dim3(256), 0, tsx::as_stream(stream),
                        static_cast<int8_t *>(staged_dev), chunks, pl.cp, g->c, int(int8_t(padding_value)));
     TSX_LAUNCH_CHECK("stage_fill_kernel");
+    return 0;
+}
+
+int tsx_conv2d_i8_stage_fill_halo(const tsx_conv2d_geom *g, float padding_value, void *staged_dev, size_t staged_bytes,
+                                  void *stream) {
+    Plan pl;
+    int rc = make_plan(g, &pl);
+    if (rc) return rc;
+    TSX_REQUIRE(!pl.im2col, "stage_fill_halo: this layer stages by im2col; a producer cannot write its input");
+    TSX_REQUIRE(staged_dev && reinterpret_cast<uintptr_t>(staged_dev) % 16 == 0, "stage_fill_halo: buffer must be 16-byte aligned");
+    TSX_REQUIRE(staged_bytes == pl.staged_bytes, "stage_fill_halo: the buffer must be this layer's own staged input (%zu bytes, got %zu)",
+                pl.staged_bytes, staged_bytes);
+    // rows and columns of the map the convolution reads (its last rows / columns may lie behind the last window)
+    const int h = std::min(g->h, pl.hs - g->pad_top), w = std::min(g->w, pl.ws - g->pad_left);
+    if (pl.hs == h && pl.ws == w && g->c % 16 == 0 && pl.cp == g->c) return 0;   // no halo, no channel padding: nothing to write
+    // channels [c rounded down to 16, cp) of interior pixels are written here; the producer's 16-channel stores cover the rest
+    const int64_t chunks = int64_t(staged_bytes / 16);
+    hipLaunchKernelGGL(stage_fill_halo_kernel, dim3(unsigned(tsx::ceil_div(chunks, 256))), dim3(256), 0, tsx::as_stream(stream),
+                       static_cast<int8_t *>(staged_dev), chunks, pl.hs, pl.ws, pl.cp, g->c, g->pad_top, g->pad_left, h, w,
+                       int(int8_t(padding_value)));
+    TSX_LAUNCH_CHECK("stage_fill_halo_kernel");
     return 0;
 }
 

@@ -284,6 +284,50 @@ def fuse_quantized_chains(module):
                         last = act
             nodes[last] = Node(FUSED, nodes[last].name, params, list(cand.inputs) + [other])
             break
+    # third pass: a fused node whose output only another fused node reads hands it over as int8 in that node's
+    # staged layout (next_* parameters on the producer, staged_input on the consumer): no staging pass, no fp32
+    # tensor in between
+    live, todo = set(), list(module.outputs)
+    while todo:                        # the chains' inner nodes are dead by now and must not count as readers
+        i = todo.pop()
+        if i not in live:
+            live.add(i)
+            todo.extend(nodes[i].inputs)
+    users = {}
+    for i in sorted(live):
+        for j in nodes[i].inputs:
+            users.setdefault(j, []).append(i)
+    for j in module.outputs:
+        users.setdefault(j, []).append(-1)
+    for ci, cons in enumerate(nodes):
+        if ci not in live:
+            continue
+        if cons.op != FUSED or "staged_input" in cons.params:
+            continue
+        pi = cons.inputs[0]
+        prod = nodes[pi]
+        if prod.op != FUSED or users.get(pi) != [ci] or "residual" in prod.params or "next_quantize_scale" in prod.params:
+            continue
+        wv = np.asarray(nodes[cons.inputs[1]].params.get("value"))
+        if wv.ndim != 4:
+            continue
+        c, kh, kw = wv.shape[1], wv.shape[2], wv.shape[3]
+        if kh * kw > 1 and c <= 8 and c * kh * kw <= 512:      # staged by im2col: cannot read a producer's buffer
+            continue
+        dil = cons.params.get("dilation", cons.params.get("dialations"))
+        if dil is None or "padding" not in cons.params or "stride" not in cons.params:
+            continue
+        pad = np.asarray(cons.params["padding"]).reshape(4, 2)
+        stride, dil = np.asarray(cons.params["stride"]).ravel(), np.asarray(dil).ravel()
+        pp = dict(prod.params)
+        pp["next_quantize_scale"] = cons.params["quantize_scale"]
+        pp["next_ksize"] = np.array([kh, kw], np.int32)
+        pp["next_padding"] = np.array([pad[2, 0], pad[2, 1], pad[3, 0], pad[3, 1]], np.int32)
+        pp["next_stride"] = np.array([stride[2], stride[3]], np.int32)
+        pp["next_dilation"] = np.array([dil[2], dil[3]], np.int32)
+        pp["next_padding_value"] = np.asarray(cons.params.get("padding_value", np.zeros(1, np.float32)), np.float32).reshape(-1)[:1]
+        nodes[pi] = Node(FUSED, prod.name, pp, prod.inputs)
+        nodes[ci] = Node(FUSED, cons.name, dict(cons.params, staged_input=np.array([1], np.int32)), cons.inputs)
     # drop what no output reaches any more, renumber
     keep, stack = set(), list(module.outputs) + list(module.inputs)
     while stack:

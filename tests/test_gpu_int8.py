@@ -291,6 +291,12 @@ def test_conv2d_i8_staged_hand_over(tsx, port, cmid, a_strides):
     exp_q2 = port.conv2d_i8_fused((xq // 2).astype(np.int8), wa, dqa, ba, "relu", 0.0, qs, (1, 1, 1, 1), a_strides)[1]
     got_b2 = B.run_staged(sb, _dev(dqb))[0].cpu().numpy()
     assert np.array_equal(bits(got_b2), bits(port.conv2d_quantized(exp_q2, wb, dqb, (1, 1, 1, 1))))
+    # fresh memory with only halo and channel padding set, then the producer: the same bytes as the full fill
+    for consumer, full in ((B, sb), (C1, sc)):
+        part = tsx.StagedInput(consumer, tuple(ya_q.shape), halo_only=True)
+        A(_dev((xq // 2).astype(np.int8)), dq=_dev(dqa), bias=_dev(ba), act="relu", q_scales=_dev(qs), staged_out=part)
+        A(_dev((xq // 2).astype(np.int8)), dq=_dev(dqa), bias=_dev(ba), act="relu", q_scales=_dev(qs), staged_out=full)
+        assert torch.equal(part.buf, full.buf)
     with pytest.raises(tsx.TsxError):                # a buffer too small for the producer's output
         small = tsx.StagedInput(tsx.Conv2dI8(_dev(wb)), (n, cmid, 4, 4))
         A(_dev(xq), dq=_dev(dqa), q_scales=_dev(qs), staged_out=small)

@@ -246,3 +246,24 @@ def test_fused_operator_with_residual_against_the_operator_chain(hip_device):
         ops.run_op(mf.FUSED, dict(base, residual=np.array([1], np.int32)), [x, w, bias, np.zeros((3, 130, 9, 11), np.float32)])
     with pytest.raises(ops.OperatorError, match="inputs"):
         ops.run_op(mf.FUSED, dict(base, residual=np.array([1], np.int32)), [x, w])
+
+
+def test_fusing_rewrite_hands_int8_over_between_chains():
+    """c1 -> c2 -> c3 of a bottleneck: c1 and c2 become producers (next_* of their consumer), c2 and c3 consumers
+    (staged_input); the block's first convolution and its projection read the fp32 block input as before."""
+    from tennis_amd import resnet50
+    desc, params = resnet50.make_parameters(seed=3, width=0.25, blocks=(1, 1, 1, 1), classes=10)
+    f = mf.fuse_quantized_chains(resnet50.to_module(desc, params, batch=2))
+    fused = [n for n in f.nodes if n.op == mf.FUSED]
+    assert len(fused) == 17
+    producers = [n for n in fused if "next_quantize_scale" in n.params]
+    consumers = [n for n in fused if "staged_input" in n.params]
+    assert len(producers) == 8 and len(consumers) == 8          # two hand-overs per block
+    c2 = next(n for n in fused if n.name == "s1b0.c2.relu")
+    assert "staged_input" in c2.params and list(c2.params["next_ksize"]) == [1, 1] and list(c2.params["next_padding"]) == [0, 0, 0, 0]
+    c1 = f.nodes[c2.inputs[0]]
+    assert c1.op == mf.FUSED and list(c1.params["next_ksize"]) == [3, 3] and list(c1.params["next_padding"]) == [1, 1, 1, 1]
+    assert np.array_equal(c1.params["next_quantize_scale"], c2.params["quantize_scale"]) and "staged_input" not in c1.params
+    stem = next(n for n in fused if n.name.startswith("stem"))
+    assert "next_quantize_scale" not in stem.params             # a pooling node reads the stem
+    mf.parse_module(mf.serialize_module(f))
