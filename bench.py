@@ -34,8 +34,8 @@ CFG = dict(n=32, c=256, h=28, w=28, cout=256, k=3, pad=1)
 
 # HBM bytes per launch of the two kernels on this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a
 # known-size copy (profiles/conv2d_i8_config2_hbm_traffic.txt); a profiler figure, not measured by this script.
-TRAFFIC_CONV_BYTES = 45.19e6
-TRAFFIC_STAGE_BYTES = 33.62e6
+TRAFFIC_CONV_BYTES = 43.99e6
+TRAFFIC_STAGE_BYTES = 33.44e6
 
 
 def make_inputs(cfg, seed=1234):
