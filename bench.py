@@ -157,12 +157,18 @@ def tennis_runtime_leg(reps=5):
         path = os.path.join(tmp, "resnet50_int8_bs32.tsm")
         mf.write_module(path, module)
         fused0 = ref.fused_chain_count_intree()
-        ms, logits = ref.time_module_intree("hip", path, [x], warmup=2, reps=reps)
+        hand0 = ref.handover_counts_intree()
+        ms, logits = ref.time_module_intree("hip", path, [x], warmup=2, reps=reps, resident=True)
         fused = ref.fused_chain_count_intree() - fused0
+        hand = tuple(a - b for a, b in zip(ref.handover_counts_intree(), hand0))
+        ms_upload, _ = ref.time_module_intree("hip", path, [x], warmup=2, reps=reps, resident=False)
     return {"workload": "BASELINE config 4 network as a .tsm module (every activation quantized with one fixed multiplier) "
-                        "in TenniS's Workbench on device hip: quantize+conv+bias+relu chains fused by the backend's zipper "
-                        "option, fp32 NCHW between nodes, fp32 inner_prod classifier; each run ends with the logits on the host",
+                        "in TenniS's Workbench on device hip: quantize+conv+bias+relu chains (and residual joins) fused by "
+                        "the backend's zipper option, int8 hand-over between fused nodes, fp32 inner_prod classifier; input "
+                        "bound from device memory, each run ends with the logits on the host",
             "img_per_s": n / (ms * 1e-3), "ms_per_batch": ms, "reps": reps, "chains_fused_by_the_graph_compiler": fused,
+            "int8_hand_overs": hand[0], "dual_output_nodes": hand[1],
+            "ms_per_batch_input_uploaded_every_run": ms_upload,
             "logits_finite": bool(np.isfinite(logits).all())}
 
 

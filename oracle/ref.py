@@ -98,6 +98,15 @@ def fused_chain_count_intree():
     return int(L.ref_hip_fused_chain_count())
 
 
+def handover_counts_intree():
+    """(fused nodes that write a staged int8 output for the convolutions behind them, those of them that return
+    the fp32 form as well) so far in the in-tree library."""
+    L = intree_lib()
+    L.ref_hip_handover_count.restype = ctypes.c_long
+    L.ref_hip_dual_output_count.restype = ctypes.c_long
+    return int(L.ref_hip_handover_count()), int(L.ref_hip_dual_output_count())
+
+
 def run_module_intree(device, path, inputs, out_bytes=1 << 24, threads=1):
     """Load a `.tsm` file into a TenniS Workbench on ``device`` ("cpu" or "hip") of the in-tree build: TenniS's own
     module loader, graph compiler and runtime, with this repository's backend serving device "hip"."""
@@ -115,9 +124,10 @@ def run_module_intree(device, path, inputs, out_bytes=1 << 24, threads=1):
     return buf[:out.bytes].view(_TS2NP[out.dtype]).reshape(shape).copy()
 
 
-def time_module_intree(device, path, inputs, warmup=2, reps=10, out_bytes=1 << 24, threads=1):
+def time_module_intree(device, path, inputs, warmup=2, reps=10, out_bytes=1 << 24, threads=1, resident=False):
     """ms per run of a `.tsm` module in a TenniS Workbench on ``device`` of the in-tree build (module loaded and
-    compiled once; each run ends with output 0 read back), and that output."""
+    compiled once; each run ends with output 0 read back), and that output.  ``resident``: the inputs are moved to
+    the device before the timed loop instead of being uploaded by every run."""
     L = intree_lib()
     keep = []
     i = (_Tensor * max(len(inputs), 1))(*[_pack("", v, keep) for v in inputs])
@@ -127,7 +137,7 @@ def time_module_intree(device, path, inputs, warmup=2, reps=10, out_bytes=1 << 2
     out.capacity = out_bytes
     ms = ctypes.c_double(0.0)
     rc = L.ref_time_module(str(path).encode(), device.encode(), len(inputs), i, int(threads), int(warmup), int(reps),
-                           ctypes.byref(ms), ctypes.byref(out))
+                           int(bool(resident)), ctypes.byref(ms), ctypes.byref(out))
     if rc != 0:
         raise RuntimeError("TenniS raised: " + L.ref_last_error().decode(errors="replace"))
     shape = tuple(out.shape[k] for k in range(out.ndim))

@@ -30,6 +30,7 @@
 #include "kernels/cpu/winograd_algorithm.h"
 #include "kernels/cpu/math_cpu.h"
 #include "global/setup.h"
+#include "global/memory_device.h"
 #include "utils/ctxmgr_lite.h"
 
 extern "C" {
@@ -205,14 +206,25 @@ int ref_run_module(const char *path, const char *device, int ninputs, const ref_
 
 // The same, timed: the module is loaded and compiled once, run `warmup` times, then `reps` times against the wall
 // clock; every run ends with output 0 read back to the host (the one synchronisation a caller of the runtime
-// sees).  Inputs are bound once: their device copies are cached by the runtime's SyncMemory after the first run.
+// sees).  Inputs are bound once.  A host tensor bound to a Workbench is copied to the device by the first operator
+// that reads it, on EVERY run (new data each run is the normal case); with resident != 0 the inputs are moved to
+// the device's memory before the loop and bound from there, the case of a caller whose data is already on the
+// device.
 int ref_time_module(const char *path, const char *device, int ninputs, const ref_tensor *inputs, int threads, int warmup,
-                    int reps, double *ms_per_run, ref_output *out) {
+                    int reps, int resident, double *ms_per_run, ref_output *out) {
     return guarded([&] {
         auto module = ts::Module::Load(path);
-        auto bench = ts::Workbench::Load(module, ts::ComputingDevice(device, 0));
+        const ts::ComputingDevice computing(device, 0);
+        auto bench = ts::Workbench::Load(module, computing);
         bench->runtime().set_computing_thread_number(threads);
-        for (int i = 0; i < ninputs; ++i) bench->input(i, make_tensor(inputs[i]));
+        for (int i = 0; i < ninputs; ++i) {
+            ts::Tensor t = make_tensor(inputs[i]);
+            if (resident) {
+                BindAll bind(*bench);   // the converters need the device context
+                t = t.view(ts::ComputingMemory::Query(computing));
+            }
+            bench->input(i, t);
+        }
         ts::Tensor y;
         for (int r = 0; r < warmup; ++r) {
             bench->run();
@@ -274,5 +286,10 @@ int ref_gemm_f32(int m, int n, int k, const float *a, const float *bm, float *c,
 // Chains replaced by the "hip" device's zipper option so far (in-tree build); -1 where the library holds no such option.
 long tsx_hip_fused_chain_count() __attribute__((weak));
 long ref_hip_fused_chain_count() { return tsx_hip_fused_chain_count ? tsx_hip_fused_chain_count() : -1; }
+// ... of which write a staged int8 output for the convolutions behind them / return the fp32 form as well
+long tsx_hip_handover_count() __attribute__((weak));
+long tsx_hip_dual_output_count() __attribute__((weak));
+long ref_hip_handover_count() { return tsx_hip_handover_count ? tsx_hip_handover_count() : -1; }
+long ref_hip_dual_output_count() { return tsx_hip_dual_output_count ? tsx_hip_dual_output_count() : -1; }
 
 }  // extern "C"

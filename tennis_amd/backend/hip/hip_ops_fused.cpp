@@ -23,7 +23,10 @@
 // (quantize(act(...)) of the consumer's quantize node, value for value) and returns an INT8 tensor
 // [n, hs, ws, cp]; the consumer is marked staged_input = 1 and runs the MFMA kernel on that tensor directly.
 // No staging pass, a quarter of the bytes.  The reference leaves this to a TODO
-// (src/backend/base/base_conv2d_quantized.cpp:163).
+// (src/backend/base/base_conv2d_quantized.cpp:163).  With dual_output = 1 as well the node returns BOTH forms as
+// one packed tensor -- field 0 the fp32 NCHW result, field 1 the staged int8 one -- for a tensor that quantized
+// convolutions and other nodes (a later residual join) both read; `_field` nodes pick the form
+// (src/runtime/instruction/tensor_instruction.cpp:38-61).
 #define TSX_TS_QUANTIZED_OPS   // Padding2D / Stride2D / Dilation2D come with the quantized skeleton
 #include "hip_ops_common.h"
 
@@ -57,6 +60,7 @@ public:
         field("next_stride", OPTIONAL);
         field("next_dilation", OPTIONAL);
         field("next_padding_value", OPTIONAL, tensor::from(0.0f));
+        field("dual_output", OPTIONAL, tensor::from(int(0)));
     }
 
     void init() override {
@@ -92,12 +96,17 @@ public:
             m_next_dil = ints("next_dilation", 2);
             m_next_padding_value = tensor::to_float(get("next_padding_value"));
         }
+        m_dual = tensor::to_int(get("dual_output")) != 0;
+        if (m_dual && !m_next) TS_LOG_ERROR << "conv2d_quantized_fused: dual_output needs the next_* parameters" << eject;
     }
 
     int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override {
         tsx_conv2d_geom g, gn;
-        output.assign(1, out_proto(stack, g, gn));
-        return 1;
+        const Tensor::Prototype proto = out_proto(stack, g, gn);
+        output.clear();
+        if (m_dual) output.push_back(Tensor::Prototype(FLOAT32, Shape({g.n, g.cout, m_ho, m_wo})));
+        output.push_back(proto);
+        return int(output.size());
     }
 
     int run(Stack &stack) override {
@@ -113,7 +122,10 @@ public:
         if (m_residual) residual = stack[int(stack.size()) - 1].view(device);
         const Shape conv_shape({g.n, g.cout, m_ho, m_wo});
         const bool same_shape = m_residual && residual.sizes() == conv_shape;
-        Tensor out = *stack.push(proto, device);
+        // dual output: the staged int8 tensor as usual plus the fp32 one, pushed as one packed tensor at the end
+        Tensor out = m_dual ? stack.make(proto, device) : *stack.push(proto, device);
+        Tensor out_plain;
+        if (m_dual) out_plain = stack.make(Tensor::Prototype(FLOAT32, conv_shape), device);
         void *stream = current_stream();
         const void *packed = m_state.packed(g, w, device, stream, "conv2d_quantized_fused");
         tsx_epilogue ep{};
@@ -143,7 +155,7 @@ public:
             ep.staged_cp = out.size(3);
             ep.staged_pad_top = gn.pad_top;
             ep.staged_pad_left = gn.pad_left;
-            out_f32 = nullptr;
+            out_f32 = m_dual ? out_plain.data<float>() : nullptr;
         }
         if (m_staged_input) {
             check(tsx_conv2d_i8_staged_at(&g, x.data(), x.size(1), x.size(2), packed, &ep, out_f32, nullptr, nullptr, stream),
@@ -167,6 +179,7 @@ public:
             else if (m_residual == 1 && m_act == TSX_ACT_LEAKY_RELU)
                 check(tsx_leaky_relu_f32(out.data<float>(), out.count(), m_slope, out.data<float>(), stream), "tsx_leaky_relu_f32");
         }
+        if (m_dual) stack.push(Tensor::Pack({out_plain, out}));
         return 1;
     }
 
@@ -250,7 +263,7 @@ private:
     float m_padding_value = 0.f, m_slope = 0.f;
     int m_act = TSX_ACT_NONE;
     int m_residual = 0;   // 0: none; 1: act(y + residual); 2: act(y) + residual
-    bool m_staged_input = false, m_next = false;
+    bool m_staged_input = false, m_next = false, m_dual = false;
     std::vector<float> m_next_q;
     std::vector<int32_t> m_next_ksize, m_next_pad, m_next_stride, m_next_dil;
     float m_next_padding_value = 0.f;

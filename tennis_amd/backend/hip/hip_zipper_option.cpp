@@ -13,15 +13,23 @@
 #include <module/menu.h>
 
 #include <atomic>
+#include <cstring>
+#include <iterator>
+#include <mutex>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "hip_device.h"
 
-static std::atomic<long> g_fused_chains{0};
+static std::atomic<long> g_fused_chains{0}, g_handovers{0}, g_dual_outputs{0};
 
 // how many chains the option has replaced in this process (tests read it to see that the option fired)
 extern "C" __attribute__((visibility("default"))) long tsx_hip_fused_chain_count() { return g_fused_chains.load(); }
+// ... how many of them write a staged int8 output for the quantized convolutions behind them, and how many of
+// those return the fp32 form as well (dual output)
+extern "C" __attribute__((visibility("default"))) long tsx_hip_handover_count() { return g_handovers.load(); }
+extern "C" __attribute__((visibility("default"))) long tsx_hip_dual_output_count() { return g_dual_outputs.load(); }
 
 namespace ts {
 namespace hip {
@@ -72,6 +80,12 @@ struct Chain {
             cur = cur.input(0);
             if (cur.outputs().size() != 1) return false;
         }
+        return core(cur);
+    }
+
+    // the part of the match that does not depend on what follows the convolution: every conv2d_quantized node
+    // that passes it ends up inside a fused node, whichever way the walker reaches it
+    bool core(Node cur) {
         if (cur.bubble().op() != name::layer::conv2d_quantized() || cur.inputs().size() != 2) return false;
         nodes = {cur.input(0), cur, cur.input(1)};
         if (quantize().bubble().op() != name::layer::quantize() || quantize().inputs().size() != 1 ||
@@ -96,24 +110,22 @@ struct Chain {
     }
 };
 
-}  // namespace
+// What ends at a node: a chain, or a chain joined with another tensor by an `add` (activation in front of or
+// behind the add).  Three shapes of the same rewrite:
+//   chain                               -> fused(x, w[, bias])
+//   [relu | leaky_relu <-] add(chain without activation, other)   -> fused(..., other), residual = 1:
+//                                          the join of a residual block, act(y + other), in the epilogue
+//   add(chain with activation, other)   -> fused(..., other), residual = 2: act(y) + other (darknet shortcut)
+// `add` broadcasts; the fused operator adds an operand of the output's shape in the MFMA kernel's epilogue
+// and any other in a broadcast pass of its own, so every add that ran still runs.
+struct Pattern {
+    Chain chain;
+    std::vector<Node> residual;
+    int residual_mode = 0;
+    std::string activation = "none";
+    Tensor slope;
 
-class FusedQuantizedConvOption : public ZipperOption {
-public:
-    bool zip(const ComputingDevice &device, Node node, Node &zipped_node) const final {
-        if (device.type() != DeviceType(DEVICE)) return false;
-        // Three shapes of the same rewrite, all ending in `node`:
-        //   chain                               -> fused(x, w[, bias])
-        //   [relu | leaky_relu <-] add(chain without activation, other)   -> fused(..., other), residual = 1:
-        //                                          the join of a residual block, act(y + other), in the epilogue
-        //   add(chain with activation, other)   -> fused(..., other), residual = 2: act(y) + other (darknet shortcut)
-        // `add` broadcasts; the fused operator adds an operand of the output's shape in the MFMA kernel's epilogue
-        // and any other in a broadcast pass of its own, so every add that ran still runs.
-        Chain chain;
-        std::vector<Node> residual;
-        int residual_mode = 0;
-        std::string activation = "none";
-        Tensor slope;
+    bool match(Node node) {
         Node cur = node;
         if (is_activation(cur.bubble().op()) && cur.inputs().size() == 1 && cur.input(0).bubble().op() == name::layer::add() &&
             cur.input(0).outputs().size() == 1) {
@@ -138,70 +150,201 @@ public:
                     slope = c.slope;
                 }
             }
-            if (!residual_mode) return false;
-        } else {
-            if (cur != node) return false;          // an activation behind an add that did not fold: not a chain's end
-            if (!chain.match(node, true)) return false;
-            activation = chain.activation;
-            slope = chain.slope;
+            return residual_mode != 0;
         }
+        if (cur != node) return false;          // an activation behind an add that did not fold: not a chain's end
+        if (!chain.match(node, true)) return false;
+        activation = chain.activation;
+        slope = chain.slope;
+        return true;
+    }
+};
 
-        zipped_node = build(chain, activation, slope, residual, residual_mode, nullptr, node.bubble().name());
+// What a producer has to know about the chains that read its output to write their staged int8 input.
+struct Next {
+    Tensor quantize_scale, ksize, padding, stride, dilation, padding_value;
+};
+
+Tensor int_vector(std::initializer_list<int32_t> values) {
+    const std::vector<int32_t> v(values);
+    return tensor::build(INT32, Shape({int32_t(v.size())}), v.data());
+}
+
+bool same_values(const Tensor &a, const Tensor &b) {
+    if (a.dtype() != b.dtype() || a.count() != b.count()) return false;
+    const Tensor ha = a.view(MemoryDevice(CPU)), hb = b.view(MemoryDevice(CPU));
+    return std::memcmp(ha.data(), hb.data(), size_t(a.count()) * type_bytes(a.dtype())) == 0;
+}
+
+// The consumer side of an int8 hand-over, from the chain's conv2d_quantized node; false when the layer cannot
+// read a staged buffer a producer wrote (few input channels under a large kernel are staged by im2col).
+bool describe(const Chain &chain, Next &next) {
+    const Bubble &conv = chain.conv().bubble();
+    const Tensor w = chain.weights().bubble().get(name::value);
+    const int c = w.size(1), kh = w.size(2), kw = w.size(3);
+    if (kh * kw > 1 && c <= 8 && c * kh * kw <= 512) return false;
+    if (!conv.has(name::padding) || !conv.has(name::stride)) return false;
+    if (!chain.quantize().bubble().has(name::quantize_scale)) return false;
+    const std::vector<int32_t> pad = tensor::array::to_int(conv.get(name::padding));
+    const std::vector<int32_t> stride = tensor::array::to_int(conv.get(name::stride));
+    const std::string dil_name = conv.has(name::dilation) ? name::dilation : name::typo::dialations;
+    if (!conv.has(dil_name)) return false;
+    const std::vector<int32_t> dil = tensor::array::to_int(conv.get(dil_name));
+    if (pad.size() != 8 || stride.size() != 4 || dil.size() != 4) return false;
+    next.quantize_scale = chain.quantize().bubble().get(name::quantize_scale);
+    next.ksize = int_vector({kh, kw});
+    next.padding = int_vector({pad[4], pad[5], pad[6], pad[7]});
+    next.stride = int_vector({stride[2], stride[3]});
+    next.dilation = int_vector({dil[2], dil[3]});
+    next.padding_value = conv.has(name::padding_value) ? conv.get(name::padding_value) : tensor::from(0.0f);
+    return true;
+}
+
+// How the value of one original node is computed in the rewritten graph: by a conv2d_quantized_fused node
+// whose output is the fp32 tensor (`plain`), the staged int8 input of the quantized convolutions that read it
+// (`staged`), or both (a dual-output node behind two `_field` nodes).
+struct Product {
+    std::vector<Node> plain, staged;    // empty or one node
+    std::vector<Node> staged_readers;   // the conv2d_quantized nodes that take the staged form
+    bool alive() const {
+        for (const Node &n : plain) if (n.ptr() == nullptr) return false;
+        for (const Node &n : staged) if (n.ptr() == nullptr) return false;
+        return !(plain.empty() && staged.empty());
+    }
+};
+
+std::mutex g_memo_mutex;
+// per graph under compilation (ctx Graph) and original node; entries of finished compilations hold expired nodes
+std::unordered_map<const void *, std::unordered_map<Node, Product>> g_memo;
+
+}  // namespace
+
+class FusedQuantizedConvOption : public ZipperOption {
+public:
+    bool zip(const ComputingDevice &device, Node node, Node &zipped_node) const final {
+        if (device.type() != DeviceType(DEVICE)) return false;
+        std::lock_guard<std::mutex> lock(g_memo_mutex);
+        Product product;
+        if (!produce(node, product)) return false;
+        if (!product.plain.empty()) {
+            zipped_node = product.plain[0];
+            return true;
+        }
+        // every reader seen in the graph takes the staged form, yet the walker asks for the tensor itself (a graph
+        // output): a node of its own for the fp32 form
+        Pattern p;
+        if (!p.match(node)) return false;
+        zipped_node = build(p, nullptr, false, node.bubble().name());
         return true;
     }
 
 private:
-    // What a producer has to know about the chain that reads its output to write that chain's staged int8 input.
-    struct Next {
-        Tensor quantize_scale, ksize, padding, stride, dilation, padding_value;
-    };
-
-    static Tensor int_vector(std::initializer_list<int32_t> values) {
-        const std::vector<int32_t> v(values);
-        return tensor::build(INT32, Shape({int32_t(v.size())}), v.data());
-    }
-
-    // The consumer side of an int8 hand-over, from the chain's conv2d_quantized node; false when the layer cannot
-    // read a staged buffer a producer wrote (few input channels under a large kernel are staged by im2col).
-    static bool describe(const Chain &chain, Next &next) {
-        const Bubble &conv = chain.conv().bubble();
-        const Tensor w = chain.weights().bubble().get(name::value);
-        const int c = w.size(1), kh = w.size(2), kw = w.size(3);
-        if (kh * kw > 1 && c <= 8 && c * kh * kw <= 512) return false;
-        if (!conv.has(name::padding) || !conv.has(name::stride)) return false;
-        const std::vector<int32_t> pad = tensor::array::to_int(conv.get(name::padding));
-        const std::vector<int32_t> stride = tensor::array::to_int(conv.get(name::stride));
-        const std::string dil_name = conv.has(name::dilation) ? name::dilation : name::typo::dialations;
-        if (!conv.has(dil_name)) return false;
-        const std::vector<int32_t> dil = tensor::array::to_int(conv.get(dil_name));
-        if (pad.size() != 8 || stride.size() != 4 || dil.size() != 4) return false;
-        next.quantize_scale = chain.quantize().bubble().get(name::quantize_scale);
-        next.ksize = int_vector({kh, kw});
-        next.padding = int_vector({pad[4], pad[5], pad[6], pad[7]});
-        next.stride = int_vector({stride[2], stride[3]});
-        next.dilation = int_vector({dil[2], dil[3]});
-        next.padding_value = conv.has(name::padding_value) ? conv.get(name::padding_value) : tensor::from(0.0f);
+    // The quantized convolutions that read `node` through a quantize node of their own (or a shared one), when
+    // they can all read ONE staged buffer: the same quantize scale, kernel extent, padding, dilation and padding
+    // value (strides may differ: a strided reader skips pixels of the same buffer), `next` from the reader with
+    // the smallest stride, which must be 1 when strides differ.  `others` = whether anything else reads the node.
+    static bool staged_readers(const Node &node, std::vector<Node> &convs, Next &next, bool &others) {
+        convs.clear();
+        others = false;
+        std::vector<Next> all;
+        for (const Node &reader : node.outputs()) {
+            bool chains = reader.bubble().op() == name::layer::quantize() && reader.inputs().size() == 1 &&
+                          !reader.outputs().empty();
+            std::vector<Node> mine;
+            std::vector<Next> mine_next;
+            if (chains)
+                for (const Node &conv : reader.outputs()) {
+                    Chain c;
+                    Next n;
+                    if (!c.core(conv) || !describe(c, n)) {
+                        chains = false;
+                        break;
+                    }
+                    mine.push_back(conv);
+                    mine_next.push_back(n);
+                }
+            if (!chains) {
+                others = true;
+                continue;
+            }
+            convs.insert(convs.end(), mine.begin(), mine.end());
+            all.insert(all.end(), mine_next.begin(), mine_next.end());
+        }
+        if (convs.empty()) return false;
+        size_t primary = 0;
+        auto area = [](const Next &n) {
+            const std::vector<int32_t> s = tensor::array::to_int(n.stride);
+            return s[0] * s[1];
+        };
+        bool strides_differ = false;
+        for (size_t i = 1; i < all.size(); ++i) {
+            if (!same_values(all[i].quantize_scale, all[0].quantize_scale) || !same_values(all[i].ksize, all[0].ksize) ||
+                !same_values(all[i].padding, all[0].padding) || !same_values(all[i].dilation, all[0].dilation) ||
+                !same_values(all[i].padding_value, all[0].padding_value))
+                return false;
+            if (!same_values(all[i].stride, all[0].stride)) strides_differ = true;
+            if (area(all[i]) < area(all[primary])) primary = i;
+        }
+        if (strides_differ && area(all[primary]) != 1) return false;
+        next = all[primary];
         return true;
     }
 
-    // The conv2d_quantized_fused node for `chain`.  When the tensor in front of the chain's quantize is itself the
-    // end of a chain and nothing else reads it, that chain is built here too, as a producer that writes this one's
-    // staged int8 input (and so on up the line): consecutive quantized convolutions exchange int8 in the consumer's
-    // layout, with no staging pass and no fp32 tensor in between.
-    static Node build(const Chain &chain, const std::string &activation, const Tensor &slope, const std::vector<Node> &residual,
-                      int residual_mode, const Next *next, const std::string &node_name) {
+    // Fills `product` for original node `node`; false when no fused node computes it.
+    static bool produce(const Node &node, Product &product) {
+        auto &memo = g_memo[ctx::get<Graph>()];
+        for (auto it = memo.begin(); it != memo.end();)     // entries of an earlier compilation at this address
+            it = (it->first.ptr() == nullptr || !it->second.alive()) ? memo.erase(it) : std::next(it);
+        auto hit = memo.find(node);
+        if (hit != memo.end()) {
+            product = hit->second;
+            return true;
+        }
+        Pattern p;
+        if (!p.match(node)) return false;
+        Next next;
+        bool others = false;
+        Product made;
+        const std::string name = node.bubble().name();
+        if (!staged_readers(node, made.staged_readers, next, others)) {
+            made.plain.push_back(build(p, nullptr, false, name));
+        } else if (!others) {
+            made.staged.push_back(build(p, &next, false, name));
+            ++g_handovers;
+        } else {
+            Node dual = build(p, &next, true, name);
+            Node f32 = bubble::op(name, name::layer::field(), {dual});
+            f32.bubble().set(name::offset, tensor::from(int(0)));
+            Node i8 = bubble::op(name + "#staged", name::layer::field(), {dual});
+            i8.bubble().set(name::offset, tensor::from(int(1)));
+            made.plain.push_back(f32);
+            made.staged.push_back(i8);
+            ++g_handovers;
+            ++g_dual_outputs;
+        }
+        memo.insert(std::make_pair(node, made));
+        product = made;
+        return true;
+    }
+
+    // The conv2d_quantized_fused node for pattern `p`.  When the tensor in front of the chain's quantize is itself
+    // computed by a fused node that hands this convolution its staged int8 input, that node is built here too (and
+    // so on up the line): consecutive quantized convolutions exchange int8 in the consumer's layout, with no staging
+    // pass and no fp32 tensor in between.
+    static Node build(const Pattern &p, const Next *next, bool dual, const std::string &node_name) {
+        const Chain &chain = p.chain;
         Node source = chain.quantize().input(0);
         bool staged_input = false;
-        Next mine;
-        Chain producer;
-        if (chain.quantize().outputs().size() == 1 && source.outputs().size() == 1 && describe(chain, mine) &&
-            producer.match(source, true)) {
-            source = build(producer, producer.activation, producer.slope, {}, 0, &mine, source.bubble().name());
-            staged_input = true;
-        }
+        Product from;
+        if (produce(source, from) && !from.staged.empty())
+            for (const Node &reader : from.staged_readers)
+                if (reader == chain.conv()) {
+                    source = from.staged[0];
+                    staged_input = true;
+                }
         std::vector<Node> inputs = {source, chain.weights()};
         inputs.insert(inputs.end(), chain.bias.begin(), chain.bias.end());
-        inputs.insert(inputs.end(), residual.begin(), residual.end());
+        inputs.insert(inputs.end(), p.residual.begin(), p.residual.end());
         Node made = bubble::op(node_name, "conv2d_quantized_fused", inputs);
         Bubble &fused = made.bubble();
         const Bubble &conv = chain.conv().bubble();
@@ -209,9 +352,9 @@ private:
                                          name::typo::dialations, name::dequantize_scales})
             if (conv.has(param)) fused.set(param, conv.get(param));
         fused.set(name::quantize_scale, chain.quantize().bubble().get(name::quantize_scale));
-        fused.set("activation", tensor::from(activation));
-        if (activation == "leaky_relu") fused.set(name::scale, slope);
-        if (residual_mode) fused.set("residual", tensor::from(int(residual_mode)));
+        fused.set("activation", tensor::from(p.activation));
+        if (p.activation == "leaky_relu") fused.set(name::scale, p.slope);
+        if (p.residual_mode) fused.set("residual", tensor::from(int(p.residual_mode)));
         if (staged_input) fused.set("staged_input", tensor::from(int(1)));
         if (next) {
             fused.set("next_quantize_scale", next->quantize_scale);
@@ -221,6 +364,7 @@ private:
             fused.set("next_dilation", next->dilation);
             fused.set("next_padding_value", next->padding_value);
         }
+        if (dual) fused.set("dual_output", tensor::from(int(1)));
         ++g_fused_chains;
         return made;
     }

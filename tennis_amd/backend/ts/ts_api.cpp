@@ -213,6 +213,23 @@ Tensor Tensor::view(const MemoryDevice &device) const {
     m_sync->copies[device] = dst;
     return out;
 }
+Tensor Tensor::Pack(const std::vector<Tensor> &fields) {
+    if (fields.empty()) return Tensor();
+    Tensor packed = fields[0];
+    packed.m_fields.assign(fields.begin() + 1, fields.end());
+    return packed;
+}
+
+Tensor Tensor::field(size_t offset) const {
+    if (offset >= fields_count()) TS_LOG_ERROR << "Tensor offset output range error. Access index " << offset << " in range(" << fields_count() << ")" << eject;
+    if (offset == 0) {
+        Tensor first = *this;
+        first.m_fields.clear();
+        return first;
+    }
+    return m_fields[offset - 1];
+}
+
 Tensor Tensor::clone() const {
     if (!m_sync) return Tensor();
     Tensor out(m_device, m_proto);

@@ -317,6 +317,12 @@ public:
     // marks this device's copy as the current one: cached copies on other devices are dropped
     void broadcast() const;
 
+    // Packed tensors (include/core/tensor.h:230-242): an operator with several results pushes ONE tensor whose
+    // fields are the results; field 0 is the tensor itself, `_field` nodes pick the others.
+    static Tensor Pack(const std::vector<Tensor> &fields);
+    Tensor field(size_t offset) const;
+    size_t fields_count() const { return empty() ? 0 : 1 + m_fields.size(); }
+
 private:
     struct Sync {
         MemoryDevice home;
@@ -325,6 +331,7 @@ private:
     std::shared_ptr<Sync> m_sync;
     MemoryDevice m_device;   // the copy this handle reads
     Prototype m_proto;
+    std::vector<Tensor> m_fields;   // fields 1.. of a packed tensor
 };
 
 // ---------------------------------------------------------------- small parameter helpers

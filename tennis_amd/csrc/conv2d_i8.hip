@@ -557,6 +557,40 @@ __global__ __launch_bounds__(256) void stage_fill_halo_kernel(int8_t *__restrict
     *reinterpret_cast<uint4 *>(xs + id * 16) = make_uint4(words[0], words[1], words[2], words[3]);
 }
 
+// ... and when the layer has no channel padding at all, one lane per 16-byte chunk of a HALO pixel only: the lanes
+// of the scan above that land on interior pixels are most of a large map.
+__global__ __launch_bounds__(256) void stage_fill_halo_only_kernel(int8_t *__restrict__ xs, int64_t chunks, int hs, int ws, int cp,
+                                                                  int pad_top, int pad_left, int h, int w, int pad_value) {
+    const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (id >= chunks) return;
+    const int cpc = cp / 16;
+    const int halo_px = hs * ws - h * w;                  // per image
+    const int64_t hp_all = id / cpc;
+    const int chunk = int(id - hp_all * cpc);
+    const int img = int(hp_all / halo_px);
+    int hp = int(hp_all - int64_t(img) * halo_px);
+    int row, col;
+    const int above = pad_top * ws, below = (hs - pad_top - h) * ws;
+    if (hp < above) {
+        row = hp / ws;
+        col = hp - row * ws;
+    } else if (hp < above + below) {
+        hp -= above;
+        row = hp / ws;
+        col = hp - row * ws;
+        row += pad_top + h;
+    } else {
+        hp -= above + below;
+        const int side = ws - w;                          // halo pixels beside one interior row
+        row = hp / side;
+        const int k = hp - row * side;
+        row += pad_top;
+        col = k < pad_left ? k : w + k;
+    }
+    const uint32_t word = uint32_t(pad_value & 0xff) * 0x01010101u;
+    *reinterpret_cast<uint4 *>(xs + ((int64_t(img) * hs + row) * ws + col) * cp + chunk * 16) = make_uint4(word, word, word, word);
+}
+
 // ------------------------------------------------------------------ weight packing
 
 // packed[ks][frag][half][lane][16]: ks = tap * cblocks + cb (tap = kh*KW + kw),
@@ -1288,6 +1322,14 @@ int tsx_conv2d_i8_stage_fill_halo(const tsx_conv2d_geom *g, float padding_value,
     // rows and columns of the map the convolution reads (its last rows / columns may lie behind the last window)
     const int h = std::min(g->h, pl.hs - g->pad_top), w = std::min(g->w, pl.ws - g->pad_left);
     if (pl.hs == h && pl.ws == w && g->c % 16 == 0 && pl.cp == g->c) return 0;   // no halo, no channel padding: nothing to write
+    if (pl.cp == g->c) {
+        const int64_t halo_chunks = int64_t(g->n) * (pl.hs * pl.ws - h * w) * (pl.cp / 16);
+        hipLaunchKernelGGL(stage_fill_halo_only_kernel, dim3(unsigned(tsx::ceil_div(halo_chunks, 256))), dim3(256), 0,
+                           tsx::as_stream(stream), static_cast<int8_t *>(staged_dev), halo_chunks, pl.hs, pl.ws, pl.cp, g->pad_top,
+                           g->pad_left, h, w, int(int8_t(padding_value)));
+        TSX_LAUNCH_CHECK("stage_fill_halo_only_kernel");
+        return 0;
+    }
     // channels [c rounded down to 16, cp) of interior pixels are written here; the producer's 16-channel stores cover the rest
     const int64_t chunks = int64_t(staged_bytes / 16);
     hipLaunchKernelGGL(stage_fill_halo_kernel, dim3(unsigned(tsx::ceil_div(chunks, 256))), dim3(256), 0, tsx::as_stream(stream),

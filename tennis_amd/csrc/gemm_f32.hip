@@ -226,6 +226,95 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmArgs g, Loader ld
     });
 }
 
+// inner_prod with few rows (a classifier behind a batch of 32: M = 32, K = 2048, N = 1000).  The tiled kernel
+// above gives such a problem 32 workgroups that each walk all of K chunk by chunk, one global round trip per
+// chunk.  Here a workgroup owns a 16 x 16 output tile on v_mfma_f32_16x16x4_f32, its four wavefronts take a
+// quarter of K each, operands go from global memory straight into the MFMA operand registers (no LDS staging)
+// with four 16-deep K blocks in flight per wavefront, and the quarters are summed through LDS in a fixed order
+// (results do not depend on timing).  Lane l holds A[row l%16][4 consecutive k of group l/16] as one 16-byte
+// load, and B[those k][col l%16]; the four MFMAs of a block take k group by group -- the sum over k does not
+// care which k an MFMA step carries.  Accumulator register r of lane l is row 4*(l/16) + r, column l%16.
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+struct SkinnyArgs {
+    const float *a, *b;
+    float *c;
+    int m, n, k;
+    int64_t ld_k, ld_n;   // element (k, n) of the right operand at b[k*ld_k + n*ld_n]
+};
+
+constexpr int SK_DEPTH = 4;   // K blocks (16 k each) in flight per wavefront
+
+__global__ __launch_bounds__(256) void inner_prod_skinny_kernel(SkinnyArgs g) {
+    __shared__ float part[3][256];
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int row = min(int(blockIdx.y) * 16 + lane % 16, g.m - 1);      // rows / columns beyond the edge repeat the
+    const int col = min(int(blockIdx.x) * 16 + lane % 16, g.n - 1);      // last one: computed, never stored
+    const int kgrp = (lane / 16) * 4;
+    const int blocks = (g.k + 15) / 16;
+    const int per_wave = (blocks + 3) / 4;
+    const int b0 = wave * per_wave, b1 = min(blocks, b0 + per_wave);
+    const float *ap = g.a + int64_t(row) * g.k;
+    const float *bp = g.b + int64_t(col) * g.ld_n;
+    const bool a_vec = g.k % 4 == 0 && reinterpret_cast<uintptr_t>(g.a) % 16 == 0;
+
+    float av[SK_DEPTH][4], bv[SK_DEPTH][4];
+    auto load = [&](auto slot, int blk) __attribute__((always_inline)) {
+        constexpr int s = decltype(slot)::value;
+        const int k0 = blk * 16 + kgrp;
+        // unconditional loads from clamped addresses, zeroed afterwards where k lies beyond K or the block beyond
+        // this wavefront's range: a load behind a branch is waited for before the next one is issued
+        const bool live = blk < b1;
+        if (a_vec) {
+            const int kc = min(k0, g.k - 4);
+            const v4f t = *reinterpret_cast<const v4f *>(ap + kc);
+            static_for<0, 4>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                av[s][i] = (live && k0 + i < g.k) ? t[i] : 0.f;   // kc == k0 whenever k0 + 3 < K, and K % 4 == 0
+            });
+        } else {
+            static_for<0, 4>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                const float t = ap[min(k0 + i, g.k - 1)];
+                av[s][i] = (live && k0 + i < g.k) ? t : 0.f;
+            });
+        }
+        static_for<0, 4>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            const float t = bp[int64_t(min(k0 + i, g.k - 1)) * g.ld_k];
+            bv[s][i] = (live && k0 + i < g.k) ? t : 0.f;
+        });
+    };
+
+    v4f acc = {0.f, 0.f, 0.f, 0.f};
+    static_for<0, SK_DEPTH - 1>([&](auto sc) { load(sc, b0 + decltype(sc)::value); });
+    for (int blk = b0; blk < b1; blk += SK_DEPTH) {
+        static_for<0, SK_DEPTH>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            load(std::integral_constant<int, (u + SK_DEPTH - 1) % SK_DEPTH>{}, blk + u + SK_DEPTH - 1);
+            static_for<0, 4>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u][i], bv[u][i], acc, 0, 0, 0);
+            });
+        });
+    }
+
+    if (wave > 0) {
+        static_for<0, 4>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            part[wave - 1][r * 64 + lane] = acc[r];
+        });
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    const int orow = int(blockIdx.y) * 16 + 4 * (lane / 16), ocol = int(blockIdx.x) * 16 + lane % 16;
+    static_for<0, 4>([&](auto rc) {
+        constexpr int r = decltype(rc)::value;
+        const float v = ((acc[r] + part[0][r * 64 + lane]) + part[1][r * 64 + lane]) + part[2][r * 64 + lane];
+        if (orow + r < g.m && ocol < g.n) g.c[int64_t(orow + r) * g.n + ocol] = v;
+    });
+}
+
 template <class Loader>
 int launch(const GemmArgs &g, const Loader &ld, int batches, hipStream_t stream) {
     // Big problems: 64x64 tiles, no K split.  Small ones (fewer tiles than SIMDs): 32x32 tiles
@@ -315,6 +404,14 @@ int tsx_inner_prod_f32(int32_t m, int32_t n, int32_t k, const float *lhs_dev, co
                        float *out_dev, void *stream) {
     TSX_REQUIRE(m > 0 && n > 0 && k > 0, "inner_prod_f32: non-positive extent");
     TSX_REQUIRE(lhs_dev && rhs_dev && out_dev, "inner_prod_f32: null argument");
+    if (m <= 64 && k >= 256) {
+        // few rows: the tiled kernel would run on m/32 * n/32 workgroups, each walking all of K
+        tsx::SkinnyArgs s{lhs_dev, rhs_dev, out_dev, m, n, k, transpose ? 1 : int64_t(n), transpose ? int64_t(k) : 1};
+        hipLaunchKernelGGL(tsx::inner_prod_skinny_kernel, dim3(unsigned(tsx::ceil_div(n, 16)), unsigned(tsx::ceil_div(m, 16))),
+                           dim3(256), 0, tsx::as_stream(stream), s);
+        TSX_LAUNCH_CHECK("inner_prod_skinny_kernel");
+        return 0;
+    }
     tsx::GemmArgs g{};
     g.a = lhs_dev;
     g.c = out_dev;

@@ -78,7 +78,8 @@ def test_conv2d_f32_padding_value_and_exact_integers(tsx, port):
     assert np.array_equal(bits(got), bits(exp))
 
 
-@pytest.mark.parametrize("m,k,n", [(1, 64, 32), (3, 70, 33), (32, 1024, 1000), (130, 200, 260), (12, 2048, 1000)])
+@pytest.mark.parametrize("m,k,n", [(1, 64, 32), (3, 70, 33), (32, 1024, 1000), (130, 200, 260), (12, 2048, 1000),
+                                   (17, 301, 45), (64, 259, 16), (5, 1000, 7), (33, 4096, 130)])   # the few-rows kernel's edges
 @pytest.mark.parametrize("transpose", [False, True])
 def test_inner_prod_f32(tsx, port, m, k, n, transpose):
     rng = np.random.default_rng(402)

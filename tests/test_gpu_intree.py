@@ -182,22 +182,29 @@ def test_module_file_in_tennis_workbench_on_hip(ts):
 
 
 def test_resnet_shaped_module_in_tennis_workbench_on_hip(ts, tmp_path):
-    """A ResNet-50-shaped int8 network (quarter width, one bottleneck per stage: 17 quantized convolutions, 4
+    """A ResNet-50-shaped int8 network (quarter width, 2 + 1 + 2 + 1 bottlenecks: 23 quantized convolutions, 6
     residual joins, pooling, global pooling, classifier) written as a `.tsm` module and run (a) by TenniS's own
     runtime on its CPU device, (b) by TenniS's own runtime on ComputingDevice("hip"), (c) by this repository's
     operator-by-operator module runner, plain and with the chain-fusing rewrite.  Everything up to the fp32
     classifier is exact arithmetic shared by all four; the classifier's MFMA summation order differs from the
     host's, hence the fp32 tolerance of 1e-4 relative + 1e-5 absolute on the logits."""
     from tennis_amd import module_file as mf, resnet50
-    desc, params = resnet50.make_parameters(seed=3, width=0.25, blocks=(1, 1, 1, 1), classes=10)
+    desc, params = resnet50.make_parameters(seed=3, width=0.25, blocks=(2, 1, 2, 1), classes=10)
     module = resnet50.to_module(desc, params, batch=2)
     path = str(tmp_path / "resnet_shaped.tsm")
     mf.write_module(path, module)
     x = np.random.default_rng(1).random((2, 3, 64, 64), dtype=np.float32)
     cpu = ts.run_module_intree("cpu", path, [x])
     fused0 = ts.fused_chain_count_intree()
+    hand0, dual0 = ts.handover_counts_intree()
     hip = ts.run_module_intree("hip", path, [x])
-    assert ts.fused_chain_count_intree() == fused0 + 17   # every quantized convolution of the network, fused by TenniS's compiler
+    assert ts.fused_chain_count_intree() == fused0 + 23   # every quantized convolution of the network, fused by TenniS's compiler
+    # int8 hand-overs: c1 -> c2 -> c3 inside each of the 6 blocks (12), and each join that another block reads
+    # (5: the last one feeds the pooling).  The joins in front of the two identity blocks are read by the next
+    # block's first convolution AND its residual add, so they return both forms (dual output); the ones in front
+    # of a projection block are read by two convolutions of different stride sharing one staged tensor.
+    hand, dual = ts.handover_counts_intree()
+    assert (hand - hand0, dual - dual0) == (17, 2)
     assert cpu.shape == (2, 10) and hip.shape == (2, 10) and np.abs(cpu).max() > 0.1
     assert close(hip, cpu)
     (own,) = mf.run_module(module, [x])
