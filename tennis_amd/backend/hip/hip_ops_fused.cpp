@@ -122,8 +122,24 @@ public:
         if (m_residual) residual = stack[int(stack.size()) - 1].view(device);
         const Shape conv_shape({g.n, g.cout, m_ho, m_wo});
         const bool same_shape = m_residual && residual.sizes() == conv_shape;
-        // dual output: the staged int8 tensor as usual plus the fp32 one, pushed as one packed tensor at the end
-        Tensor out = m_dual ? stack.make(proto, device) : *stack.push(proto, device);
+        // The staged int8 output lives in a tensor this operator keeps from run to run: its halo and channel padding
+        // are written once, when it is allocated, and every run's epilogue overwrites exactly the interior -- a
+        // tensor from the stack is fresh memory each time and would need the halo filled again (one more launch per
+        // node and run).  Readers run behind this node on the same stream and the next run's epilogue behind them.
+        // Dual output: that tensor plus the fp32 one, pushed as one packed tensor at the end.
+        Tensor out;
+        bool fill_halo = false;
+        if (m_next) {
+            if (m_staged_out.empty() || m_staged_out.device() != device || m_staged_out.dtype() != proto.dtype() ||
+                !(m_staged_out.sizes() == proto.sizes())) {
+                m_staged_out = Tensor(device, proto.dtype(), proto.sizes());
+                fill_halo = true;
+            }
+            out = m_staged_out;
+            if (!m_dual) stack.push(out);
+        } else {
+            out = *stack.push(proto, device);
+        }
         Tensor out_plain;
         if (m_dual) out_plain = stack.make(Tensor::Prototype(FLOAT32, conv_shape), device);
         void *stream = current_stream();
@@ -143,10 +159,10 @@ public:
         float *out_f32 = out.data<float>();
         if (m_next) {
             if (split) TS_LOG_ERROR << "conv2d_quantized_fused: a residual that broadcasts cannot be combined with next_*" << eject;
-            // the consumer's staged input: halo and channel padding first (the tensor is fresh memory every run),
-            // then the interior from the epilogue
-            const size_t bytes = size_t(out.count());
-            check(tsx_conv2d_i8_stage_fill_halo(&gn, m_next_padding_value, out.data(), bytes, stream), "tsx_conv2d_i8_stage_fill_halo");
+            // the consumer's staged input: halo and channel padding (once), then the interior from the epilogue
+            if (fill_halo)
+                check(tsx_conv2d_i8_stage_fill_halo(&gn, m_next_padding_value, out.data(), size_t(out.count()), stream),
+                      "tsx_conv2d_i8_stage_fill_halo");
             ep.q_scales_dev = m_next_q_dev.get(m_next_q, device);
             ep.n_qscales = int32_t(m_next_q.size());
             ep.staged_out_dev = static_cast<int8_t *>(out.data());
@@ -269,9 +285,100 @@ private:
     float m_next_padding_value = 0.f;
     int m_ho = 0, m_wo = 0;
     DeviceFloats m_next_q_dev;
+    Tensor m_staged_out;
     std::vector<float> m_dq, m_q;
     DeviceFloats m_dq_dev, m_q_dev;
     PackedConv m_state;
+};
+
+// max_pooling2d_staged: a MAX pooling2d node (src/kernels/cpu/pooling2d_core.cpp:48-93) between a fused producer and
+// quantized convolutions, on the producer's requantized int8 output instead of its fp32 one: quantize is monotone,
+// so pooling the int8 values gives what pooling2d -> quantize gives, byte for byte (tsx_max_pooling2d_i8_staged).
+// Input: INT8 [n, h, w, cp], the producer's staged output without halo (next_ksize 1x1, no padding).  Parameters:
+// ksize [2], stride [2], padding [top, bottom, left, right] of the pooling, and the reading convolutions' geometry
+// as next_ksize / next_padding / next_stride / next_dilation / next_padding_value.  Output: their staged input,
+// INT8 [n, hs, ws, cp], in a tensor the operator keeps (halo written once, see conv2d_quantized_fused).
+class MaxPooling2DStaged : public Operator {
+public:
+    using self = MaxPooling2DStaged;
+    using supper = Operator;
+
+    MaxPooling2DStaged() {
+        field(name::ksize, REQUIRED);
+        field(name::stride, REQUIRED);
+        field(name::padding, REQUIRED);
+        field("next_ksize", REQUIRED);
+        field("next_padding", REQUIRED);
+        field("next_stride", REQUIRED);
+        field("next_dilation", REQUIRED);
+        field("next_padding_value", OPTIONAL, tensor::from(0.0f));
+    }
+
+    void init() override {
+        supper::init();
+        m_ksize = ints(name::ksize, 2);
+        m_stride = ints(name::stride, 2);
+        m_pad = ints(name::padding, 4);
+        m_next_ksize = ints("next_ksize", 2);
+        m_next_pad = ints("next_padding", 4);
+        m_next_stride = ints("next_stride", 2);
+        m_next_dil = ints("next_dilation", 2);
+        m_next_padding_value = tensor::to_float(get("next_padding_value"));
+    }
+
+    int infer(Stack &stack, std::vector<Tensor::Prototype> &output) override {
+        tsx_conv2d_geom gn;
+        int32_t oh, ow;
+        output.assign(1, out_proto(stack, gn, oh, ow));
+        return 1;
+    }
+
+    int run(Stack &stack) override {
+        tsx_conv2d_geom gn;
+        int32_t oh = 0, ow = 0;
+        const Tensor::Prototype proto = out_proto(stack, gn, oh, ow);
+        const MemoryDevice device = ctx::ref<DeviceContext>().memory_device;
+        Tensor x = stack[0].view(device);
+        void *stream = current_stream();
+        if (m_out.empty() || m_out.device() != device || !(m_out.sizes() == proto.sizes())) {
+            m_out = Tensor(device, proto.dtype(), proto.sizes());
+            check(tsx_conv2d_i8_stage_fill(&gn, m_next_padding_value, m_out.data(), size_t(m_out.count()), stream),
+                  "tsx_conv2d_i8_stage_fill");
+        }
+        const tsx_staged_map src{x.data(), x.size(0), x.size(1), x.size(2), x.size(3), 0, 0, x.size(1), x.size(2), x.size(3)};
+        const tsx_staged_map dst{m_out.data(), m_out.size(0), m_out.size(1), m_out.size(2), m_out.size(3),
+                                 gn.pad_top, gn.pad_left, oh, ow, x.size(3)};
+        check(tsx_max_pooling2d_i8_staged(&src, &dst, m_ksize[0], m_ksize[1], m_pad[0], m_pad[2], m_stride[0], m_stride[1], stream),
+              "tsx_max_pooling2d_i8_staged");
+        stack.push(m_out);
+        return 1;
+    }
+
+private:
+    std::vector<int32_t> ints(const std::string &param, size_t count) {
+        const std::vector<int32_t> v = tensor::array::to_int(get(param));
+        if (v.size() != count) TS_LOG_ERROR << "max_pooling2d_staged: " << param << " must hold " << count << " integers" << eject;
+        return v;
+    }
+
+    Tensor::Prototype out_proto(Stack &stack, tsx_conv2d_geom &gn, int32_t &oh, int32_t &ow) {
+        if (stack.size() != 1) TS_LOG_ERROR << "max_pooling2d_staged expects 1 input, got " << stack.size() << eject;
+        const Tensor &x = stack[0];
+        if (x.dims() != 4 || x.dtype() != INT8 || x.size(3) % 64 != 0)
+            TS_LOG_ERROR << "max_pooling2d_staged expects an int8 tensor [n, h, w, cp]" << eject;
+        if (tsx_pooling2d_out_size(x.size(1), x.size(2), m_ksize[0], m_ksize[1], m_pad[0], m_pad[1], m_pad[2], m_pad[3], m_stride[0],
+                                   m_stride[1], &oh, &ow) != 0)
+            TS_LOG_ERROR << "[hip] max_pooling2d_staged: " << tsx_last_error() << eject;
+        gn = tsx_conv2d_geom{x.size(0), x.size(3), oh, ow, 1, m_next_ksize[0], m_next_ksize[1], m_next_pad[0], m_next_pad[1],
+                             m_next_pad[2], m_next_pad[3], m_next_stride[0], m_next_stride[1], m_next_dil[0], m_next_dil[1]};
+        int32_t hs = 0, ws = 0, cp = 0;
+        if (tsx_conv2d_i8_staged_dims(&gn, &hs, &ws, &cp) != 0) TS_LOG_ERROR << "[hip] max_pooling2d_staged: " << tsx_last_error() << eject;
+        return Tensor::Prototype(INT8, Shape({x.size(0), hs, ws, cp}));
+    }
+
+    std::vector<int32_t> m_ksize, m_stride, m_pad, m_next_ksize, m_next_pad, m_next_stride, m_next_dil;
+    float m_next_padding_value = 0.f;
+    Tensor m_out;
 };
 
 }  // namespace hip
@@ -280,3 +387,4 @@ private:
 using namespace ts;
 using namespace ts::hip;
 TS_REGISTER_OPERATOR(Conv2DQuantizedFused, ts::hip::DEVICE, "conv2d_quantized_fused")
+TS_REGISTER_OPERATOR(MaxPooling2DStaged, ts::hip::DEVICE, "max_pooling2d_staged")

@@ -300,6 +300,13 @@ private:
             product = hit->second;
             return true;
         }
+        if (node.bubble().op() == name::layer::pooling2d()) {
+            Product pooled;
+            if (!through_max_pooling(node, pooled)) return false;
+            memo.insert(std::make_pair(node, pooled));
+            product = pooled;
+            return true;
+        }
         Pattern p;
         if (!p.match(node)) return false;
         Next next;
@@ -324,6 +331,50 @@ private:
         }
         memo.insert(std::make_pair(node, made));
         product = made;
+        return true;
+    }
+
+    // pattern -> MAX pooling2d -> quantized convolutions only (a ResNet stem): quantize is monotone, so it commutes
+    // with max -- the producer requantizes in its epilogue into a staged tensor without halo, max_pooling2d_staged
+    // pools the int8 values straight into the convolutions' staged input.  Nothing else may read either tensor.
+    static bool through_max_pooling(const Node &node, Product &made) {
+        const Bubble &b = node.bubble();
+        if (node.inputs().size() != 1) return false;
+        for (const std::string &param : {name::format, name::type, name::padding, name::ksize, name::stride})
+            if (!b.has(param)) return false;
+        if (tensor::to_string(b.get(name::format)) != name::NCHW || tensor::to_int(b.get(name::type)) != 0) return false;
+        const std::vector<int32_t> pad = tensor::array::to_int(b.get(name::padding));
+        const std::vector<int32_t> ksize = tensor::array::to_int(b.get(name::ksize));
+        const std::vector<int32_t> stride = tensor::array::to_int(b.get(name::stride));
+        if (pad.size() != 8 || ksize.size() != 4 || stride.size() != 4) return false;
+        if (pad[0] || pad[1] || pad[2] || pad[3] || ksize[0] != 1 || ksize[1] != 1 || stride[0] != 1 || stride[1] != 1) return false;
+        if (pad[4] < 0 || pad[6] < 0 || pad[4] >= ksize[2] || pad[6] >= ksize[3] || stride[2] < 1 || stride[3] < 1) return false;
+        Node source = node.input(0);
+        if (source.outputs().size() != 1) return false;
+        Pattern p;
+        if (!p.match(source)) return false;
+        Next next;
+        bool others = false;
+        if (!staged_readers(node, made.staged_readers, next, others) || others) return false;
+        Next flat = next;                       // the producer's side: the same scale into [n][h][w][cp], no halo
+        flat.ksize = int_vector({1, 1});
+        flat.padding = int_vector({0, 0, 0, 0});
+        flat.stride = int_vector({1, 1});
+        flat.dilation = int_vector({1, 1});
+        flat.padding_value = tensor::from(0.0f);
+        Node producer = build(p, &flat, false, source.bubble().name());
+        Node pool = bubble::op(node.bubble().name(), "max_pooling2d_staged", {producer});
+        Bubble &staged = pool.bubble();
+        staged.set(name::ksize, int_vector({ksize[2], ksize[3]}));
+        staged.set(name::stride, int_vector({stride[2], stride[3]}));
+        staged.set(name::padding, int_vector({pad[4], pad[5], pad[6], pad[7]}));
+        staged.set("next_ksize", next.ksize);
+        staged.set("next_padding", next.padding);
+        staged.set("next_stride", next.stride);
+        staged.set("next_dilation", next.dilation);
+        staged.set("next_padding_value", next.padding_value);
+        made.staged.push_back(pool);
+        g_handovers += 2;
         return true;
     }
 

@@ -228,9 +228,10 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmArgs g, Loader ld
 
 // inner_prod with few rows (a classifier behind a batch of 32: M = 32, K = 2048, N = 1000).  The tiled kernel
 // above gives such a problem 32 workgroups that each walk all of K chunk by chunk, one global round trip per
-// chunk.  Here a workgroup owns a 16 x 16 output tile on v_mfma_f32_16x16x4_f32, its four wavefronts take a
-// quarter of K each, operands go from global memory straight into the MFMA operand registers (no LDS staging)
-// with four 16-deep K blocks in flight per wavefront, and the quarters are summed through LDS in a fixed order
+// chunk.  Here a workgroup owns a 16 x 16 output tile on v_mfma_f32_16x16x4_f32, its eight wavefronts take an
+// eighth of K each, operands go from global memory straight into the MFMA operand registers (no LDS staging)
+// with seven 16-deep K blocks in flight per wavefront (the right operand streams from HBM once: what bounds the
+// kernel is how many bytes are in flight), and the eighths are summed through LDS in a fixed order
 // (results do not depend on timing).  Lane l holds A[row l%16][4 consecutive k of group l/16] as one 16-byte
 // load, and B[those k][col l%16]; the four MFMAs of a block take k group by group -- the sum over k does not
 // care which k an MFMA step carries.  Accumulator register r of lane l is row 4*(l/16) + r, column l%16.
@@ -243,58 +244,59 @@ struct SkinnyArgs {
     int64_t ld_k, ld_n;   // element (k, n) of the right operand at b[k*ld_k + n*ld_n]
 };
 
-constexpr int SK_DEPTH = 4;   // K blocks (16 k each) in flight per wavefront
+constexpr int SK_DEPTH = 8;   // ring of K blocks (16 k each) per wavefront: SK_DEPTH - 1 in flight
+constexpr int SK_WAVES = 8;
 
-__global__ __launch_bounds__(256) void inner_prod_skinny_kernel(SkinnyArgs g) {
-    __shared__ float part[3][256];
+__global__ __launch_bounds__(64 * SK_WAVES) void inner_prod_skinny_kernel(SkinnyArgs g) {
+    __shared__ float part[SK_WAVES - 1][256];
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const int row = min(int(blockIdx.y) * 16 + lane % 16, g.m - 1);      // rows / columns beyond the edge repeat the
     const int col = min(int(blockIdx.x) * 16 + lane % 16, g.n - 1);      // last one: computed, never stored
     const int kgrp = (lane / 16) * 4;
     const int blocks = (g.k + 15) / 16;
-    const int per_wave = (blocks + 3) / 4;
+    const int per_wave = (blocks + SK_WAVES - 1) / SK_WAVES;
     const int b0 = wave * per_wave, b1 = min(blocks, b0 + per_wave);
     const float *ap = g.a + int64_t(row) * g.k;
     const float *bp = g.b + int64_t(col) * g.ld_n;
     const bool a_vec = g.k % 4 == 0 && reinterpret_cast<uintptr_t>(g.a) % 16 == 0;
 
     float av[SK_DEPTH][4], bv[SK_DEPTH][4];
+    // Unconditional loads from clamped addresses (a load behind a branch is waited for before the next one is
+    // issued); what lies beyond K or beyond this wavefront's range is zeroed where the block is USED, so that
+    // nothing between a load and its use seven blocks later needs the loaded value.
     auto load = [&](auto slot, int blk) __attribute__((always_inline)) {
         constexpr int s = decltype(slot)::value;
         const int k0 = blk * 16 + kgrp;
-        // unconditional loads from clamped addresses, zeroed afterwards where k lies beyond K or the block beyond
-        // this wavefront's range: a load behind a branch is waited for before the next one is issued
-        const bool live = blk < b1;
         if (a_vec) {
-            const int kc = min(k0, g.k - 4);
-            const v4f t = *reinterpret_cast<const v4f *>(ap + kc);
-            static_for<0, 4>([&](auto ic) {
-                constexpr int i = decltype(ic)::value;
-                av[s][i] = (live && k0 + i < g.k) ? t[i] : 0.f;   // kc == k0 whenever k0 + 3 < K, and K % 4 == 0
-            });
+            const v4f t = *reinterpret_cast<const v4f *>(ap + max(0, min(k0, g.k - 4)));
+            static_for<0, 4>([&](auto ic) { av[s][decltype(ic)::value] = t[decltype(ic)::value]; });
         } else {
             static_for<0, 4>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
-                const float t = ap[min(k0 + i, g.k - 1)];
-                av[s][i] = (live && k0 + i < g.k) ? t : 0.f;
+                av[s][i] = ap[min(k0 + i, g.k - 1)];
             });
         }
         static_for<0, 4>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
-            const float t = bp[int64_t(min(k0 + i, g.k - 1)) * g.ld_k];
-            bv[s][i] = (live && k0 + i < g.k) ? t : 0.f;
+            bv[s][i] = bp[int64_t(min(k0 + i, g.k - 1)) * g.ld_k];
         });
     };
 
     v4f acc = {0.f, 0.f, 0.f, 0.f};
     static_for<0, SK_DEPTH - 1>([&](auto sc) { load(sc, b0 + decltype(sc)::value); });
     for (int blk = b0; blk < b1; blk += SK_DEPTH) {
+        // all SK_DEPTH blocks of this round inside the wavefront's range and inside K: no masking
+        const bool whole = blk + SK_DEPTH <= b1 && (blk + SK_DEPTH) * 16 <= g.k;
         static_for<0, SK_DEPTH>([&](auto uc) {
             constexpr int u = decltype(uc)::value;
             load(std::integral_constant<int, (u + SK_DEPTH - 1) % SK_DEPTH>{}, blk + u + SK_DEPTH - 1);
+            const int k0 = (blk + u) * 16 + kgrp;
+            const bool live = blk + u < b1;
             static_for<0, 4>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
-                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u][i], bv[u][i], acc, 0, 0, 0);
+                // with K % 4 == 0 the clamped 16-byte load is the lane's own four values whenever any of them is inside K
+                const bool ok = whole || (live && k0 + i < g.k);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ok ? av[u][i] : 0.f, ok ? bv[u][i] : 0.f, acc, 0, 0, 0);
             });
         });
     }
@@ -310,7 +312,8 @@ __global__ __launch_bounds__(256) void inner_prod_skinny_kernel(SkinnyArgs g) {
     const int orow = int(blockIdx.y) * 16 + 4 * (lane / 16), ocol = int(blockIdx.x) * 16 + lane % 16;
     static_for<0, 4>([&](auto rc) {
         constexpr int r = decltype(rc)::value;
-        const float v = ((acc[r] + part[0][r * 64 + lane]) + part[1][r * 64 + lane]) + part[2][r * 64 + lane];
+        float v = acc[r];
+        static_for<0, SK_WAVES - 1>([&](auto wc) { v += part[decltype(wc)::value][r * 64 + lane]; });
         if (orow + r < g.m && ocol < g.n) g.c[int64_t(orow + r) * g.n + ocol] = v;
     });
 }
@@ -408,7 +411,7 @@ int tsx_inner_prod_f32(int32_t m, int32_t n, int32_t k, const float *lhs_dev, co
         // few rows: the tiled kernel would run on m/32 * n/32 workgroups, each walking all of K
         tsx::SkinnyArgs s{lhs_dev, rhs_dev, out_dev, m, n, k, transpose ? 1 : int64_t(n), transpose ? int64_t(k) : 1};
         hipLaunchKernelGGL(tsx::inner_prod_skinny_kernel, dim3(unsigned(tsx::ceil_div(n, 16)), unsigned(tsx::ceil_div(m, 16))),
-                           dim3(256), 0, tsx::as_stream(stream), s);
+                           dim3(64 * tsx::SK_WAVES), 0, tsx::as_stream(stream), s);
         TSX_LAUNCH_CHECK("inner_prod_skinny_kernel");
         return 0;
     }
