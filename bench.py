@@ -140,6 +140,71 @@ def config1_leg(reps=50):
             "peak_TFLOPS": PEAK_FP32_TFLOPS, **rows}
 
 
+def ceiling_evidence(L, conv_launch, event_time, conv_ops, dev, stream):
+    """What bounds the config-2 MFMA kernel, measured: (1) the rate of a register-only MFMA loop against the number of
+    busy CUs and the operand data (the clock the part grants falls with both), (2) where one launch of the kernel
+    spends its time, per wavefront, from wall-clock and shader-clock stamps the kernel writes when asked
+    (tsx_debug_phase_stamps).  `python bench.py --ceiling`; under rocprofv3 --pmc GRBM_GUI_ACTIVE the same run gives
+    cycles / duration for the probe and the kernel from the counters' side."""
+    import torch
+    from tennis_amd import capi
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    iters = 20000
+    probe = []
+    for data in ("random int8", "zeros"):
+        if data == "zeros":
+            operands = torch.zeros(32768, dtype=torch.int8, device=dev)
+        else:
+            operands = torch.randint(-128, 128, (32768,), dtype=torch.int8, device=dev)
+        for blocks in (64, 128, 224, 256, 512, 1024):
+            t = event_time(lambda: capi.check(L.tsx_probe_mfma_i8(capi._ptr(operands), iters, blocks, capi._ptr(sink), stream)), 3)
+            rate = blocks * 4 * iters * 8 * 65536.0 / t
+            simds = min(blocks * 4, 1024)      # a workgroup of 4 wavefronts fills one CU's SIMDs; beyond 256 they queue up
+            probe.append({"operands": data, "workgroups": blocks, "POP_per_s": rate / 1e15,
+                          "GHz_equivalent_per_busy_simd": rate / simds / 2048 / 1e9})
+    t_conv = event_time(conv_launch, 50)
+    slots = 8192 * 8
+    stamps = torch.zeros(slots, dtype=torch.int64, device=dev)
+    capi.check(L.tsx_debug_phase_stamps(capi._ptr(stamps), slots * 8))
+    try:
+        t_stamped = event_time(conv_launch, 20)      # the stamps of the last of 21 back-to-back launches remain
+    finally:
+        capi.check(L.tsx_debug_phase_stamps(None, 0))
+    st = stamps.cpu().numpy().reshape(-1, 8, 8)      # [workgroup][wavefront][4 x (wall, clock)]
+    st = st[st[:, 0, 0] != 0]                        # workgroups beyond the last tile leave at once
+    wall, clk = st[:, :, 0::2].astype(np.float64) * 10.0, st[:, :, 1::2].astype(np.float64)   # ns (100 MHz), cycles
+    t_first = wall[:, :, 0].min()
+
+    def stats(v):
+        return {"mean": float(v.mean()), "min": float(v.min()), "max": float(v.max())}
+
+    phases = {}
+    for name, waves in (("wavefronts 0-3 (4 fragments)", slice(0, 4)), ("wavefronts 4-7 (3 fragments)", slice(4, 8))):
+        w, c = wall[:, waves], clk[:, waves]
+        loop_ns = w[:, :, 2] - w[:, :, 1]
+        phases[name] = {
+            "entry_after_first_wavefront_ns": stats(w[:, :, 0] - t_first),
+            "prologue_ns": stats(w[:, :, 1] - w[:, :, 0]),
+            "k_loop_ns": stats(loop_ns),
+            "epilogue_until_stores_left_ns": stats(w[:, :, 3] - w[:, :, 2]),
+            "end_after_first_wavefront_ns": stats(w[:, :, 3] - t_first),
+            "k_loop_shader_cycles": stats(c[:, :, 2] - c[:, :, 1]),
+            "k_loop_clock_GHz": float(((c[:, :, 2] - c[:, :, 1]) / loop_ns).mean()),
+            "prologue_clock_GHz": float(((c[:, :, 1] - c[:, :, 0]) / (w[:, :, 1] - w[:, :, 0])).mean()),
+            "epilogue_clock_GHz": float(((c[:, :, 3] - c[:, :, 2]) / (w[:, :, 3] - w[:, :, 2])).mean()),
+        }
+    steps_per_simd = 36 * 2 * 7      # K-steps x halves x fragments of the two wavefronts of a SIMD
+    return {"workload": "BASELINE config 2 MFMA kernel (conv_i8_fl_kernel<4,3>): ceiling evidence",
+            "mfma_probe": probe,
+            "kernel_us": t_conv * 1e6, "kernel_us_with_stamps": t_stamped * 1e6,
+            "kernel_TOP_per_s": conv_ops / t_conv / 1e12,
+            "workgroups_with_stamps": int(st.shape[0]),
+            "phases": phases,
+            "k_loop_mfma_cycles_per_simd": steps_per_simd * 32,
+            "note": "wall clock = s_memrealtime (10 ns ticks), shader clock = s_memtime; k_loop_mfma_cycles_per_simd is "
+                    "what the loop's MFMAs alone occupy a SIMD's pipe for (504 v_mfma_i32_32x32x32_i8 x 32 cycles)"}
+
+
 def tennis_runtime_leg(reps=5):
     """The ResNet-50-shaped network (BASELINE config 4) as a `.tsm` module through TenniS's own loader, graph compiler
     and Workbench on ComputingDevice("hip") -- the operator boundary as a TenniS user meets it (in-tree build of the
@@ -366,6 +431,8 @@ def main():
     ap.add_argument("--no-resnet", action="store_true", help="skip the ResNet-50-shaped network leg")
     ap.add_argument("--no-yolo", action="store_true", help="skip the YOLOv4-shaped network leg")
     ap.add_argument("--no-gemm", action="store_true", help="skip the int8 GEMM sweep leg")
+    ap.add_argument("--ceiling", action="store_true",
+                    help="only the ceiling evidence of the config-2 MFMA kernel: MFMA probe rates and per-phase stamps")
     ap.add_argument("--profile", action="store_true",
                     help="for runs under a profiler: skip the int8-output variant (same kernel name as the roofline "
                          "kernel), the MFMA-rate probe and the CPU baseline, so per-kernel statistics cover the timed "
@@ -468,6 +535,11 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / reps * 1e-3   # seconds per launch
 
+    if args.ceiling:
+        conv_ops = 2.0 * cfg["n"] * cfg["cout"] * ho * wo * cfg["c"] * cfg["k"] * cfg["k"]
+        print(json.dumps(ceiling_evidence(L, mfma_only, event_time, conv_ops, dev, stream)))
+        return
+
     reps = max(args.steps, 50)
     t_mfma = event_time(mfma_only, reps)
     t_stage = event_time(stage_only, reps)
@@ -503,11 +575,19 @@ def main():
         calib_dst.copy_(calib_src)
     torch.cuda.synchronize()
 
+    stage_bytes = 4.0 * x.size + float(ws_bytes)
+    # What the device's own copy reaches on a transfer of the staging kernel's size (half read, half written): the
+    # practical HBM rate for a single launch this small, launch and ramp included -- the figure to hold the staging
+    # kernel's rate against, next to the 8 TB/s peak.
+    half = int(stage_bytes) // 2
+    copy_src = torch.empty(half, dtype=torch.uint8, device=dev).fill_(3)
+    copy_dst = torch.empty_like(copy_src)
+    t_copy = event_time(lambda: copy_dst.copy_(copy_src), reps)
+
     macs = cfg["n"] * cfg["cout"] * ho * wo * cfg["c"] * cfg["k"] * cfg["k"]
     ops = 2.0 * macs
     tops = ops / (ms_per_step * 1e-3) / 1e12
     kernel_tops = ops / t_mfma / 1e12
-    stage_bytes = 4.0 * x.size + float(ws_bytes)
 
     result = {
         "metric": "int8 conv2d TOPS & % MFMA peak; ResNet-50-shape img/s at bs=32, 1 MI355X",
@@ -542,7 +622,11 @@ def main():
             "note": "same kernel, epilogue requantizes to int8 for a following quantized layer"},
         "stage_kernel": {"bound": "hbm", "kernel": "stage_rows_kernel<quantize>", "achieved": stage_bytes / t_stage / 1e9,
                          "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": stage_bytes / t_stage / 1e9 / PEAK_HBM_GBS,
-                         "us": t_stage * 1e6, "bytes": stage_bytes, "traffic": TRAFFIC_STAGE_BYTES},
+                         "us": t_stage * 1e6, "bytes": stage_bytes, "traffic": TRAFFIC_STAGE_BYTES,
+                         "device_copy_of_the_same_bytes": {"us": t_copy * 1e6, "GB_per_s": 2.0 * half / t_copy / 1e9,
+                                                           "note": "torch copy_ of %d bytes device to device (read + "
+                                                                   "written = the staging kernel's bytes), timed the "
+                                                                   "same way" % half}},
     }
     if not args.no_resnet and not args.profile:
         result["resnet50_int8_bs32"] = resnet_leg()

@@ -42,6 +42,15 @@ int tsx_device_cu_count(void);
  * of random operands, so it is well below the nominal peak).  ops = blocks * 4 * iters * 8 * 65536. */
 int tsx_probe_mfma_i8(const void *operands_dev, int32_t iters, int32_t blocks, int32_t *sink_dev, void *stream);
 
+/* Measurement aid with no counterpart in the reference.  While a buffer is set (NULL switches it off; process-wide),
+ * every wavefront of the flat-tile int8 convolution kernel (the kernel of large multi-tap layers such as BASELINE
+ * config 2) writes four (wall clock at 100 MHz, shader clock) pairs to
+ * buffer[(workgroup * 8 + wavefront) * 8 ...]: at kernel entry, at K-loop entry, at K-loop exit and after its last
+ * store has left the wavefront -- where a launch's time goes, and the shader clock of each phase (shader cycles /
+ * wall time).  Workgroup = blockIdx.y * gridDim.x + blockIdx.x; wavefronts whose slot lies beyond `bytes` write
+ * nothing.  Costs a few scalar instructions per wavefront when set, one predictable branch when not. */
+int tsx_debug_phase_stamps(void *buffer_dev, size_t bytes);
+
 /* Geometry of one 2-D convolution, as base::Conv2D / base::Conv2DQuantized hand it to
  * their core: x [n,c,h,w], w [cout,c,kh,kw], Padding2D{top,bottom,left,right},
  * Stride2D, Dilation2D (include/backend/common_structure.h:10-62).  Output size follows

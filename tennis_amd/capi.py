@@ -67,6 +67,7 @@ SIGNATURES = {
     "tsx_conv2d_i8_staged_dims": (ctypes.c_int, [ctypes.POINTER(ConvGeom), ctypes.POINTER(_i32), ctypes.POINTER(_i32),
                                                  ctypes.POINTER(_i32)]),
     "tsx_conv2d_i8_stage_fill": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _f32, _vp, _sz, _vp]),
+    "tsx_debug_phase_stamps": (ctypes.c_int, [_vp, _sz]),
     "tsx_conv2d_i8_stage_fill_halo": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _f32, _vp, _sz, _vp]),
     "tsx_conv2d_i8_staged_at": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _i32, _i32, _vp, ctypes.POINTER(Epilogue), _vp,
                                                _vp, _vp, _vp]),

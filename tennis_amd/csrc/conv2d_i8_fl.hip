@@ -18,6 +18,20 @@
 
 #include <cstdlib>
 
+#include <atomic>
+
+// phase-stamp buffer of tsx_debug_phase_stamps (null = off)
+static std::atomic<unsigned long long *> g_stamps{nullptr};
+static std::atomic<size_t> g_stamp_slots{0};
+
+extern "C" int tsx_debug_phase_stamps(void *buffer_dev, size_t bytes) {
+    if (buffer_dev && (bytes < 64 || reinterpret_cast<uintptr_t>(buffer_dev) % 8 != 0))
+        return tsx::fail(TSX_E_INVALID, "debug_phase_stamps: buffer must be 8-byte aligned and hold at least one wavefront's 64 bytes");
+    g_stamp_slots.store(buffer_dev ? bytes / 8 : 0);
+    g_stamps.store(static_cast<unsigned long long *>(buffer_dev));
+    return 0;
+}
+
 namespace tsx {
 
 void fl_plan(const WsGeom &g, WsPlan *pl) {
@@ -114,6 +128,8 @@ int fl_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t 
     p.tiles_per_xcd = int((pl.fl_tiles + 7) / 8);
     p.positions = int(int64_t(g.n) * g.ho * g.wo);
     p.resident = pl.fl_resident ? 1 : 0;
+    p.stamps = g_stamps.load();
+    p.stamp_slots = int(g_stamp_slots.load());
     // an output of L2 size or more that no fused consumer reads: stream it
     p.stream_out = (!ep.residual && !ep.st_out && ep.out_f32 && int64_t(g.n) * g.cout * g.ho * g.wo * 4 >= (int64_t(16) << 20)) ? 1 : 0;
     const dim3 grid(unsigned(p.tiles_per_xcd * 8), unsigned((g.cout + 127) / 128));

@@ -29,6 +29,11 @@ struct FlParams : EpiParams {
     int positions;          // n * ho * wo
     int stream_out;         // fp32 output written with streaming stores
     int resident;           // every channel block's window in LDS at once (cblocks buffers instead of 2)
+    // measurement aid (tsx_debug_phase_stamps): when set, every wavefront writes 8 values at
+    // stamps[(workgroup * 8 + wave) * 8]: wall clock (100 MHz) and shader clock at kernel entry, K-loop entry,
+    // K-loop exit and after its last store has left
+    unsigned long long *stamps;
+    int stamp_slots;
 };
 
 template <int NTA, int NTB>
@@ -64,6 +69,14 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
     const int m0 = (blockIdx.y * 4 + wave_m) * 32;   // first cout of this wavefront
     const int taps = p.kh * p.kw;
     const int win_bytes = p.wr * p.rowp;
+    const int stamp_slot = ((blockIdx.y * gridDim.x + blockIdx.x) * 8 + threadIdx.x / 64) * 8;
+    auto stamp = [&](int phase) __attribute__((always_inline)) {
+        if (p.stamps && lane == 0 && stamp_slot + 8 <= p.stamp_slots) {
+            p.stamps[stamp_slot + 2 * phase] = wall_clock64();
+            p.stamps[stamp_slot + 2 * phase + 1] = clock64();
+        }
+    };
+    stamp(0);
 
     // ---- window fill bookkeeping: chunk q = tid + i*512 -> pixel q / 4, 16-byte chunk q % 4
     const int8_t *fill_src[FL_MAX_FILL];
@@ -163,6 +176,7 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
     };
     int toff = 0;   // buf * win_bytes + tap shift
     b_read(b0, toff);
+    stamp(1);
 
     for (int ks0 = 0; ks0 < p.ksteps_p; ks0 += FL_RING) {
         static_for<0, FL_RING>([&](auto uc) {
@@ -215,6 +229,13 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
                 acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[u][1], b1[j], acc[j], 0, 0, 0);
             });
         });
+    }
+
+    if (p.stamps) {
+        // the accumulators are written by the MFMAs still in flight: wait for them, so that the stamp marks the end
+        // of the multiplication rather than the issue of its last instruction
+        asm volatile("; accumulators complete" ::"v"(acc[0][15]), "v"(acc[NT - 1][15]) : "memory");
+        stamp(2);
     }
 
     // ---- epilogue: accumulator register r of lane l = cout 8*(r/4) + 4*(l/32) + r%4, position l%32
@@ -357,6 +378,10 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
                 if (pok[j] && co0 + dco < p.cout) emit(p, acc[j][r], base + int64_t(dco) * howo, dq[r], bias[r], 0.f);
             });
         });
+    }
+    if (p.stamps) {
+        __builtin_amdgcn_s_waitcnt(0);   // every store of this wavefront has left
+        stamp(3);
     }
 }
 
