@@ -132,7 +132,7 @@ struct StageRow {
 // keeps the mapping division-free; loads are issued in batches of NB quads before any is consumed.
 // RMODE says how the row's elements round: 0 = all half away from zero (the reference's scalar loop),
 // 1 = all half to even (its AVX body), 2 = per element (the one row that holds the body/tail border).
-template <bool QUANT, int VW, int RMODE>
+template <bool QUANT, int VW, int RMODE, bool UNIFORM = false>
 __device__ __forceinline__ void stage_quads(const StageGeom &g, const StageRow &r, int8_t *tile, int tid) {
     typedef float vf __attribute__((ext_vector_type(VW == 1 ? 2 : VW)));   // VW == 1 uses scalars
     constexpr int NB = VW == 4 ? 2 : 4;
@@ -201,9 +201,9 @@ __device__ __forceinline__ void stage_quads(const StageGeom &g, const StageRow &
                     if (QUANT) {
                         float sc = r.row_scale;
                         bool half_even = RMODE == 1;
-                        if (RMODE == 2 || !r.uniform_scale) {   // the element's linear index is only needed here
+                        if (RMODE == 2 || (!UNIFORM && !r.uniform_scale)) {   // the element's linear index is only needed here
                             const int64_t e = row_base + int64_t(c + j) * plane + v;
-                            if (!r.uniform_scale) sc = c + j < r.creal ? r.scales[e / r.group_len] : 0.f;
+                            if (!UNIFORM && !r.uniform_scale) sc = c + j < r.creal ? r.scales[e / r.group_len] : 0.f;
                             if (RMODE == 2) half_even = e < r.bulk8;
                         }
                         q[j] = tsx::quantize_value(__fmul_rn(fv[u][j][v], sc), half_even);
@@ -222,7 +222,12 @@ __device__ __forceinline__ void stage_quads(const StageGeom &g, const StageRow &
     }
 }
 
-template <bool QUANT>
+// FAST: what the launcher has checked for the whole launch -- rows of a multiple of 4 elements from a 16-byte
+// aligned tensor (4-byte aligned for int8), at most 256 of them, one scale per image and more than one image (so
+// every element rounds half away from zero, base_quantize / quantize.cpp's scalar path).  The general kernel
+// carries the per-element 64-bit divisions and the three rounding variants of every load width inline, ~47 000
+// instructions of which a row executes a few hundred scattered over 40 KiB of code; this one is the row's own code.
+template <bool QUANT, bool FAST = false>
 __global__ __launch_bounds__(256) void stage_rows_kernel(const void *__restrict__ src, StageGeom g,
                                                         const float *__restrict__ scales, int n_scales,
                                                         int64_t group_len, int64_t bulk8,
@@ -251,14 +256,14 @@ __global__ __launch_bounds__(256) void stage_rows_kernel(const void *__restrict_
         const uintptr_t addr = reinterpret_cast<uintptr_t>(src);
         const int esz = QUANT ? 4 : 1;
         int vw = 1;
-        if (g.w % 4 == 0 && addr % (4 * esz) == 0) vw = 4;
+        if (FAST || (g.w % 4 == 0 && addr % (4 * esz) == 0)) vw = 4;
         else if (g.w % 2 == 0 && addr % (2 * esz) == 0) vw = 2;
         int wl = 1;
         while (wl * vw < g.w) wl <<= 1;
         // stage_quads writes every dword of the interior pixels up to the last real channel quad, so
         // on that path the pre-fill only has to cover the halo pixels and the channel padding: the
         // two write disjoint dwords and need no barrier between them.
-        const bool quad_path = row_inside && wl <= 64;
+        const bool quad_path = row_inside && (FAST || wl <= 64);
         const int real_words = (creal + 3) / 4;
         // pre-fill: halo value for real channels, zero for channel padding
         const int wpr = cg / 4;   // dwords per pixel
@@ -293,7 +298,10 @@ __global__ __launch_bounds__(256) void stage_rows_kernel(const void *__restrict_
             __syncthreads();
         }
         if (row_inside) {
-            if (quad_path) {
+            if constexpr (FAST) {
+                const StageRow r{src, scales, n_scales, group_len, bulk8, true, row_scale, ni, hi, c0, creal};
+                stage_quads<QUANT, 4, 0, true>(g, r, tile, tid);
+            } else if (quad_path) {
                 const StageRow r{src, scales, n_scales, group_len, bulk8, uniform_scale, row_scale, ni, hi, c0, creal};
                 // how this row's elements round: linear indices run from lo to hi_e, the AVX body ends at bulk8
                 int rmode = 0;
@@ -1094,15 +1102,24 @@ int run_stage(const tsx_conv2d_geom *g, const Plan &pl, const void *x, bool x_is
         TSX_REQUIRE(n_x_scales == g->n, "quantize_conv2d_i8: n_x_scales (%d) must equal the batch (%d)", n_x_scales, g->n);
         const int64_t count = int64_t(g->n) * g->c * g->h * g->w;
         const int64_t group_len = int64_t(std::ceil(static_cast<float>(count) / static_cast<float>(n_x_scales)));
-        if (by_rows)
-            hipLaunchKernelGGL(stage_rows_kernel<true>, dim3(row_blocks), dim3(256), row_lds, stream, x, sg, x_scales,
+        const bool fast = by_rows && n_x_scales > 1 && g->w % 4 == 0 && g->w <= 256 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
+        if (fast)
+            hipLaunchKernelGGL((stage_rows_kernel<true, true>), dim3(row_blocks), dim3(256), row_lds, stream, x, sg, x_scales,
+                               n_x_scales, group_len, (count >> 3) << 3, static_cast<int8_t *>(staged));
+        else if (by_rows)
+            hipLaunchKernelGGL((stage_rows_kernel<true, false>), dim3(row_blocks), dim3(256), row_lds, stream, x, sg, x_scales,
                                n_x_scales, group_len, (count >> 3) << 3, static_cast<int8_t *>(staged));
         else
             hipLaunchKernelGGL(stage_nchw_kernel<true>, dim3(stage_blocks), dim3(256), 0, stream, x, sg, x_scales,
                                n_x_scales, group_len, (count >> 3) << 3, static_cast<int8_t *>(staged));
     } else {
-        if (by_rows)
-            hipLaunchKernelGGL(stage_rows_kernel<false>, dim3(row_blocks), dim3(256), row_lds, stream, x, sg,
+        const bool fast = by_rows && g->w % 4 == 0 && g->w <= 256 && reinterpret_cast<uintptr_t>(x) % 4 == 0;
+        if (fast)
+            hipLaunchKernelGGL((stage_rows_kernel<false, true>), dim3(row_blocks), dim3(256), row_lds, stream, x, sg,
+                               static_cast<const float *>(nullptr), 1, int64_t(1), int64_t(0),
+                               static_cast<int8_t *>(staged));
+        else if (by_rows)
+            hipLaunchKernelGGL((stage_rows_kernel<false, false>), dim3(row_blocks), dim3(256), row_lds, stream, x, sg,
                                static_cast<const float *>(nullptr), 1, int64_t(1), int64_t(0),
                                static_cast<int8_t *>(staged));
         else
