@@ -110,8 +110,8 @@ def cpu_baseline_all_cores(x, x_scales, wq, dq, bias, pad):
 
 def config1_leg(reps=50):
     """BASELINE config 1: fp32 conv2d 1x64x56x56 * 64x64x3x3, stride 1, pad 1, bias + ReLU -- the implicit im2col
-    GEMM on the fp32 MFMA and both Winograd modes (credited the direct convolution's flops), time per launch from
-    HIP events around back-to-back launches."""
+    GEMM on the fp32 MFMA, both Winograd modes in their bit-exact form and F(6,3) as one MFMA launch (all credited the
+    direct convolution's flops), time per launch from HIP events around back-to-back launches."""
     import torch
     from tennis_amd import capi
     dev = torch.device("cuda:0")
@@ -123,7 +123,8 @@ def config1_leg(reps=50):
     w63, w23 = capi.WinogradF63(w, (1, 1, 1, 1)), capi.WinogradF23(w, (1, 1, 1, 1))
     rows = {}
     for name, fn in (("im2col_gemm", lambda: capi.conv2d_f32(x, w, (1, 1, 1, 1), bias=b, act="relu")),
-                     ("winograd_f63", lambda: w63(x, bias=b, act="relu")), ("winograd_f23", lambda: w23(x, bias=b, act="relu"))):
+                     ("winograd_f63", lambda: w63(x, bias=b, act="relu")), ("winograd_f23", lambda: w23(x, bias=b, act="relu")),
+                     ("winograd_f63_fast", lambda: w63(x, bias=b, act="relu", fast=True))):
         for _ in range(3):
             fn()
         torch.cuda.synchronize()

@@ -329,6 +329,17 @@ size_t tsx_winograd_f63_workspace_bytes(const tsx_conv2d_geom *g);
 int tsx_conv2d_winograd_f63_nchw(const tsx_conv2d_geom *g, const float *x_dev, const float *u_dev, float padding_value,
                                  const float *bias_dev, int32_t act, float slope, float *out_dev, void *workspace_dev,
                                  size_t workspace_bytes, void *stream);
+/* The same operator (same u_dev, same arguments) with the 64 frequency GEMMs on the fp32 MFMA and the output
+ * transform fused behind them: two launches instead of three, the products M never reach memory, workspace = the
+ * transformed input only (tsx_winograd_f63_fast_workspace_bytes).  The MFMA sums the channel products in another
+ * order than the reference's FMA chains, so this entry is held to a floating-point bar -- the one TenniS's own
+ * backend test applies between devices, max 1e-4 / mean 1e-5 (tools/run_test/test_case.hpp:491-503) -- against
+ * winograd_f63 (src/kernels/cpu/winograd_algorithm.cpp:846-947), not to its bits; tsx_conv2d_winograd_f63_nchw is
+ * the bit-exact one. */
+size_t tsx_winograd_f63_fast_workspace_bytes(const tsx_conv2d_geom *g);
+int tsx_conv2d_winograd_f63_fast_nchw(const tsx_conv2d_geom *g, const float *x_dev, const float *u_dev, float padding_value,
+                                      const float *bias_dev, int32_t act, float slope, float *out_dev, void *workspace_dev,
+                                      size_t workspace_bytes, void *stream);
 
 /* ---------------------------------------------------------------- Winograd F(2x2, 3x3) fp32 conv2d
  * Conv2dWinogradAlgorithm<float>::winograd_f23 (src/kernels/cpu/winograd_algorithm.cpp:347-459), the

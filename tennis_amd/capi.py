@@ -104,6 +104,9 @@ SIGNATURES = {
     "tsx_winograd_f23_workspace_bytes": (_sz, [ctypes.POINTER(ConvGeom)]),
     "tsx_conv2d_winograd_f23_nchw": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, _f32, _vp, _i32, _f32, _vp, _vp,
                                                     _sz, _vp]),
+    "tsx_winograd_f63_fast_workspace_bytes": (_sz, [ctypes.POINTER(ConvGeom)]),
+    "tsx_conv2d_winograd_f63_fast_nchw": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, _f32, _vp, _i32, _f32, _vp, _vp,
+                                                         _sz, _vp]),
     "tsx_conv2d_winograd_f63_nchw": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, _f32, _vp, _i32, _f32, _vp, _vp,
                                                     _sz, _vp]),
 }
@@ -399,19 +402,23 @@ class Winograd:
         check(self._transform(cout, cin, _ptr(self.w), _ptr(self.u), _stream()))
         self._workspace = None
 
-    def __call__(self, x, bias=None, act=None, slope=0.0):
+    def __call__(self, x, bias=None, act=None, slope=0.0, fast=False):
+        """fast (f63 only): the MFMA form, held to the fp32 tolerance instead of the reference's bits."""
         x = _dev(x, torch.float32)
         bias = _dev(bias, torch.float32)
         geom = make_geom(tuple(x.shape), tuple(self.w.shape), self.pads)
         ho, wo = conv_out_size(geom)
-        nbytes = self._workspace_bytes(ctypes.byref(geom))
+        if fast:
+            assert self.mode == "f63"
+        nbytes = (lib().tsx_winograd_f63_fast_workspace_bytes if fast else self._workspace_bytes)(ctypes.byref(geom))
         if nbytes == 0:
             raise TsxError("winograd: " + lib().tsx_last_error().decode())
         if self._workspace is None or self._workspace.numel() < nbytes:
             self._workspace = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
         out = torch.empty((x.shape[0], self.w.shape[0], ho, wo), dtype=torch.float32, device=x.device)
-        check(self._conv(ctypes.byref(geom), _ptr(x), _ptr(self.u), self.padding_value, _ptr(bias), _ACT[act],
-                         float(slope), _ptr(out), _ptr(self._workspace), nbytes, _stream()))
+        conv = lib().tsx_conv2d_winograd_f63_fast_nchw if fast else self._conv
+        check(conv(ctypes.byref(geom), _ptr(x), _ptr(self.u), self.padding_value, _ptr(bias), _ACT[act],
+                   float(slope), _ptr(out), _ptr(self._workspace), nbytes, _stream()))
         return out
 
 

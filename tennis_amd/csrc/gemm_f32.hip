@@ -221,7 +221,7 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmArgs g, Loader ld
             const int64_t idx = col_base + int64_t(row) * row_stride;
             float v = acc[r];
             if (g.bias) v = __fadd_rn(v, g.bias[row]);
-            c[idx] = apply_act(v, g.act, g.slope, idx < g.act_body);
+            c[idx] = apply_act_basic(v, g.act, g.slope, idx < g.act_body);   // the entry points take none / relu / leaky_relu
         }
     });
 }

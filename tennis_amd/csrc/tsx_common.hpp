@@ -81,7 +81,10 @@ __device__ __forceinline__ int quantize_value(float v, bool half_even) {
 // tensor): SIMD body vs scalar tail of src/kernels/cpu/relu.cpp:30-52 and
 // leaky_relu.cpp:41-66.  Body: max(x,0) returns +0 for -0 and NaN; the leaky form is one
 // fused multiply-add in the reference's FMA build.  Tail: std::max / ternary.
-__device__ __forceinline__ float apply_act(float v, int act, float slope, bool in_body) {
+// none / relu / leaky_relu only: for kernels that unroll the call many times -- the Mish branch below is a few hundred
+// instructions (double-precision log), and dozens of inlined copies of it put the taken branches of the cheap
+// activations an instruction-cache miss apart.
+__device__ __forceinline__ float apply_act_basic(float v, int act, float slope, bool in_body) {
     if (act == TSX_ACT_RELU) {
         return in_body ? (v > 0.f ? v : 0.f) : (v < 0.f ? 0.f : v);
     }
@@ -93,7 +96,12 @@ __device__ __forceinline__ float apply_act(float v, int act, float slope, bool i
         }
         return v > 0.f ? v : __fmul_rn(v, slope);
     }
-    if (act == TSX_ACT_MISH) {
+    return v;
+}
+
+__device__ __forceinline__ float apply_act(float v, int act, float slope, bool in_body) {
+    if (act != TSX_ACT_MISH) return apply_act_basic(v, act, slope, in_body);
+    {
         // x * tanh(softplus(x)) as TenniS graphs compose it: softplus = float(log(double(expf(x)) + 1.0))
         // (src/kernels/cpu/softplus.cpp:30-39), tanh = 2 * (1 / (1 + expf(-2y))) - 1 in float
         // (src/kernels/cpu/tanh.cpp:14-23), then mul.  Same formulas; expf/log are this device's
@@ -102,7 +110,6 @@ __device__ __forceinline__ float apply_act(float v, int act, float slope, bool i
         const float t = __fsub_rn(__fmul_rn(2.f, __fdiv_rn(1.f, __fadd_rn(1.f, expf(-__fmul_rn(2.f, sp))))), 1.f);
         return __fmul_rn(v, t);
     }
-    return v;
 }
 
 #endif  // __HIPCC__

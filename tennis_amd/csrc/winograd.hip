@@ -25,6 +25,8 @@
 // All kernels here are memory/latency-bound elementwise or small-GEMM kernels.
 #include "tsx_common.hpp"
 
+#include <atomic>
+
 namespace tsx {
 namespace {
 
@@ -294,6 +296,8 @@ int launch_gemm_f32_seq(const float *a, const float *b, float *c, int m, int n, 
 
 // One thread per (image, cout, tile): Y = A^T M A, cut to the true output, then the optional
 // add_bias / activation that follow the convolution in the graph.
+// MISH: whether the activation may be Mish (see apply_act_basic for why that is a compile-time matter here)
+template <bool MISH>
 __global__ __launch_bounds__(256) void wino_output_transform_kernel(const float *__restrict__ mm, WinoGeom g,
                                                                    const float *__restrict__ bias, int act,
                                                                    float slope, int64_t act_body,
@@ -331,7 +335,159 @@ __global__ __launch_bounds__(256) void wino_output_transform_kernel(const float 
                 float val = o[r];
                 if (bias) val = __fadd_rn(val, bv);
                 const int64_t idx = (int64_t(img) * g.cout + co) * g.ho * g.wo + hh * g.wo + ww;
-                dst[hh * g.wo + ww] = apply_act(val, act, slope, idx < act_body);
+                dst[hh * g.wo + ww] = MISH ? apply_act(val, act, slope, idx < act_body) : apply_act_basic(val, act, slope, idx < act_body);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------- F(6,3), fast path
+// The same algorithm on the fp32 MFMA, for callers that hold the path to its floating-point tolerance rather than
+// to its bits (the MFMA sums the channel products in another order than the reference's FMA chains): the input
+// transform kernel above, then ONE kernel for the 64 frequency GEMMs and the output transform -- M never exists in
+// memory.  A workgroup owns 16 tiles x 16 output channels and all 64 frequencies; wavefront w multiplies
+// frequencies 16w .. 16w+15 on v_mfma_f32_16x16x4_f32 with both operands loaded from global memory (L2: U and V
+// are a few MB) straight into the MFMA operand registers, four 16-channel blocks in flight: lane l holds
+// U_f[cout l%16][4 consecutive channels of group l/16] as one 16-byte load and V_f[those channels][tile l%16]; the
+// four MFMAs of a block take the channels group by group (a sum does not care which k a step carries).
+// Accumulator register r of lane l is output channel 4*(l/16) + r, tile l%16.  The 64 products of every (output
+// channel, tile) then go through LDS to one thread, which applies A^T M A, bias and activation and stores the 6x6
+// outputs.
+constexpr int WF_TILES = 16, WF_COUT = 16;
+constexpr int WF_DEPTH = 4;   // ring of 16-channel blocks per wavefront: WF_DEPTH - 1 in flight
+
+typedef float wf_v4f __attribute__((ext_vector_type(4)));
+
+// BLOCKS = C / 16 when C is 64, 128 or 256 (then the whole walk over frequencies and channel blocks is unrolled
+// around a 16-slot ring, 15 blocks in flight: with one wavefront per SIMD nothing else hides an L2 round trip),
+// 0 for any other channel count (rounds of WF_DEPTH blocks per frequency).
+template <int BLOCKS, bool MISH>
+__global__ __launch_bounds__(256) void wino_f63_gemm_output_kernel(const float *__restrict__ v, const float *__restrict__ u,
+                                                                  WinoGeom g, const float *__restrict__ bias, int act, float slope,
+                                                                  int64_t act_body, float *__restrict__ out) {
+    __shared__ float ms[64 * WF_COUT * WF_TILES];           // M[f][cout][tile]
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const int total_tiles = g.n * g.tiles;
+    const int t0 = blockIdx.x * WF_TILES, co0 = blockIdx.y * WF_COUT;
+    // operand rows / columns of this lane (beyond the edge: the last one again; computed, never stored)
+    const int a_co = min(co0 + lane % 16, g.cout - 1);
+    const int b_t = min(t0 + lane % 16, total_tiles - 1);
+    const int b_img = b_t / g.tiles, b_tile = b_t - b_img * g.tiles;
+    const int kgrp = (lane / 16) * 4;
+    const bool a_vec = g.c % 4 == 0 && reinterpret_cast<uintptr_t>(u) % 16 == 0;
+    wf_v4f acc[16];
+#pragma unroll
+    for (int f = 0; f < 16; ++f) acc[f] = wf_v4f{0.f, 0.f, 0.f, 0.f};
+    if constexpr (BLOCKS > 0) {
+        constexpr int RING = 16, STEPS = 16 * BLOCKS;
+        float av[RING][4], bv[RING][4];
+        auto load = [&](auto stepc) __attribute__((always_inline)) {
+            constexpr int step = decltype(stepc)::value;
+            constexpr int s = step % RING;
+            const int f = wave * 16 + step / BLOCKS, k0 = (step % BLOCKS) * 16 + kgrp;
+            const wf_v4f t = *reinterpret_cast<const wf_v4f *>(u + (int64_t(f) * g.cout + a_co) * g.c + k0);
+            static_for<0, 4>([&](auto ic) { av[s][decltype(ic)::value] = t[decltype(ic)::value]; });
+            const float *bp = v + ((int64_t(b_img) * 64 + f) * g.c + k0) * g.tiles + b_tile;
+            static_for<0, 4>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                bv[s][i] = bp[int64_t(i) * g.tiles];
+            });
+        };
+        static_for<0, RING - 1>([&](auto sc) { load(sc); });
+        static_for<0, STEPS>([&](auto stepc) {
+            constexpr int step = decltype(stepc)::value;
+            if constexpr (step + RING - 1 < STEPS) load(std::integral_constant<int, step + RING - 1>{});
+            static_for<0, 4>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                acc[step / BLOCKS] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[step % RING][i], bv[step % RING][i], acc[step / BLOCKS], 0, 0, 0);
+            });
+        });
+    } else {
+    // 16-channel blocks per frequency, rounded up to whole rounds of the ring (blocks beyond C multiply zeros)
+    const int blocks = (g.c + 16 * WF_DEPTH - 1) / (16 * WF_DEPTH) * WF_DEPTH;
+    const int steps = 16 * blocks;            // (frequency, block) pairs of this wavefront, frequency-major
+
+    float av[WF_DEPTH][4], bv[WF_DEPTH][4];
+    // unconditional loads from clamped addresses; what lies beyond C is zeroed where the block is used
+    auto load = [&](auto slot, int step) __attribute__((always_inline)) {
+        constexpr int s = decltype(slot)::value;
+        if (step >= steps) step = steps - 1;
+        const int f = wave * 16 + step / blocks, k0 = (step % blocks) * 16 + kgrp;
+        const float *ap = u + (int64_t(f) * g.cout + a_co) * g.c;
+        const float *bp = v + ((int64_t(b_img) * 64 + f) * g.c) * g.tiles + b_tile;
+        if (a_vec) {
+            const wf_v4f t = *reinterpret_cast<const wf_v4f *>(ap + max(0, min(k0, g.c - 4)));
+            static_for<0, 4>([&](auto ic) { av[s][decltype(ic)::value] = t[decltype(ic)::value]; });
+        } else {
+            static_for<0, 4>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                av[s][i] = ap[min(k0 + i, g.c - 1)];
+            });
+        }
+        static_for<0, 4>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            bv[s][i] = bp[int64_t(min(k0 + i, g.c - 1)) * g.tiles];
+        });
+    };
+
+    static_for<0, WF_DEPTH - 1>([&](auto sc) { load(sc, decltype(sc)::value); });
+    int step = 0;
+    static_for<0, 16>([&](auto fc) {
+        constexpr int fl = decltype(fc)::value;
+        for (int blk = 0; blk < blocks; blk += WF_DEPTH) {
+            static_for<0, WF_DEPTH>([&](auto uc) {
+                constexpr int uu = decltype(uc)::value;       // = step % WF_DEPTH: every frequency starts a round
+                load(std::integral_constant<int, (uu + WF_DEPTH - 1) % WF_DEPTH>{}, step + WF_DEPTH - 1);
+                const int k0 = (blk + uu) * 16 + kgrp;
+                static_for<0, 4>([&](auto ic) {
+                    constexpr int i = decltype(ic)::value;
+                    const bool ok = k0 + i < g.c;
+                    acc[fl] = __builtin_amdgcn_mfma_f32_16x16x4f32(ok ? av[uu][i] : 0.f, ok ? bv[uu][i] : 0.f, acc[fl], 0, 0, 0);
+                });
+                ++step;
+            });
+        }
+    });
+    }
+
+    // ---- M[f][cout][tile] into LDS, then one thread per (cout, tile)
+#pragma unroll
+    for (int fl = 0; fl < 16; ++fl) {
+        const int f = wave * 16 + fl;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) ms[(f * WF_COUT + 4 * (lane / 16) + r) * WF_TILES + lane % 16] = acc[fl][r];
+    }
+    __syncthreads();
+    const int co = co0 + tid / WF_TILES;
+    const int my_t = t0 + tid % WF_TILES;
+    if (my_t >= total_tiles || co >= g.cout) return;
+    const int my_img = my_t / g.tiles, my_tile = my_t - my_img * g.tiles;
+    const int my_ty = my_tile / g.tw, my_tx = my_tile - my_ty * g.tw;
+    float tmpa[8][6];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        float t8[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) t8[j] = ms[((i * 8 + j) * WF_COUT + tid / WF_TILES) * WF_TILES + tid % WF_TILES];
+        at_pass(t8, tmpa[i]);
+    }
+    const float bvv = bias ? bias[co] : 0.f;
+    const int64_t plane = (int64_t(my_img) * g.cout + co) * g.ho * g.wo;
+#pragma unroll
+    for (int i = 0; i < 6; ++i) {
+        float t8[8], o[6];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) t8[r] = tmpa[r][i];
+        at_pass(t8, o);
+        const int ww = my_tx * 6 + i;
+#pragma unroll
+        for (int r = 0; r < 6; ++r) {
+            const int hh = my_ty * 6 + r;
+            if (hh < g.ho && ww < g.wo) {
+                float val = o[r];
+                if (bias) val = __fadd_rn(val, bvv);
+                const int64_t idx = plane + hh * g.wo + ww;
+                out[idx] = MISH ? apply_act(val, act, slope, idx < act_body) : apply_act_basic(val, act, slope, idx < act_body);
             }
         }
     }
@@ -405,6 +561,7 @@ __global__ __launch_bounds__(256) void wino23_input_transform_kernel(const float
 }
 
 // Y = A^T M A (winograd_algorithm.cpp:262-330), cut to the true output, + optional bias / activation.
+template <bool MISH>
 __global__ __launch_bounds__(256) void wino23_output_transform_kernel(const float *__restrict__ mm, WinoGeom g,
                                                                      const float *__restrict__ bias, int act,
                                                                      float slope, int64_t act_body,
@@ -441,7 +598,7 @@ __global__ __launch_bounds__(256) void wino23_output_transform_kernel(const floa
                 float val = o[r * 2 + i];
                 if (bias) val = __fadd_rn(val, bv);
                 const int64_t idx = plane + hh * g.wo + ww;
-                out[idx] = apply_act(val, act, slope, idx < act_body);
+                out[idx] = MISH ? apply_act(val, act, slope, idx < act_body) : apply_act_basic(val, act, slope, idx < act_body);
             }
         }
 }
@@ -521,9 +678,55 @@ int tsx_conv2d_winograd_f63_nchw(const tsx_conv2d_geom *q, const float *x_dev, c
 
     const int64_t out_threads = int64_t(g.n) * g.cout * g.tiles;
     const int64_t count = int64_t(g.n) * g.cout * g.ho * g.wo;
-    hipLaunchKernelGGL(tsx::wino_output_transform_kernel, dim3(unsigned(tsx::ceil_div(out_threads, 256))), dim3(256), 0,
-                       stream, mm, g, bias_dev, act, slope, count / 4 * 4, out_dev);
+    if (act == TSX_ACT_MISH)
+        hipLaunchKernelGGL(tsx::wino_output_transform_kernel<true>, dim3(unsigned(tsx::ceil_div(out_threads, 256))), dim3(256), 0,
+                           stream, mm, g, bias_dev, act, slope, count / 4 * 4, out_dev);
+    else
+        hipLaunchKernelGGL(tsx::wino_output_transform_kernel<false>, dim3(unsigned(tsx::ceil_div(out_threads, 256))), dim3(256), 0,
+                           stream, mm, g, bias_dev, act, slope, count / 4 * 4, out_dev);
     TSX_LAUNCH_CHECK("wino_output_transform_kernel");
+    return 0;
+}
+
+size_t tsx_winograd_f63_fast_workspace_bytes(const tsx_conv2d_geom *q) {
+    tsx::WinoGeom g;
+    if (tsx::make_geom(q, 0.f, &g)) return 0;
+    return size_t(g.n) * 64 * g.tiles * size_t(g.c) * sizeof(float);
+}
+
+int tsx_conv2d_winograd_f63_fast_nchw(const tsx_conv2d_geom *q, const float *x_dev, const float *u_dev, float padding_value,
+                                      const float *bias_dev, int32_t act, float slope, float *out_dev, void *workspace_dev,
+                                      size_t workspace_bytes, void *stream_) {
+    tsx::WinoGeom g;
+    int rc = tsx::make_geom(q, padding_value, &g);
+    if (rc) return rc;
+    TSX_REQUIRE(x_dev && u_dev && out_dev, "winograd: null argument");
+    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_MISH, "winograd: unknown activation %d", act);
+    const size_t need = tsx_winograd_f63_fast_workspace_bytes(q);
+    if (!workspace_dev || workspace_bytes < need)
+        return tsx::fail(TSX_E_WORKSPACE, "winograd: workspace %zu < %zu bytes", workspace_bytes, need);
+    const int64_t total_tiles = int64_t(g.n) * g.tiles;
+    TSX_REQUIRE(total_tiles < (int64_t(1) << 31) - tsx::WF_TILES, "winograd: too many tiles");
+    hipStream_t stream = tsx::as_stream(stream_);
+    float *v = static_cast<float *>(workspace_dev);
+    const int64_t in_threads = int64_t(g.n) * g.c * g.tiles;
+    hipLaunchKernelGGL(tsx::wino_input_transform_kernel, dim3(unsigned(tsx::ceil_div(in_threads, 256))), dim3(256), 0,
+                       stream, x_dev, g, v);
+    TSX_LAUNCH_CHECK("wino_input_transform_kernel");
+    const int64_t count = int64_t(g.n) * g.cout * g.ho * g.wo;
+    const dim3 grid(unsigned(tsx::ceil_div(total_tiles, int64_t(tsx::WF_TILES))), unsigned(tsx::ceil_div(g.cout, tsx::WF_COUT)));
+    const bool aligned = reinterpret_cast<uintptr_t>(u_dev) % 16 == 0;
+    const int blocks = aligned && (g.c == 64 || g.c == 128 || g.c == 256) ? g.c / 16 : 0;
+    const bool mish = act == TSX_ACT_MISH;
+#define TSX_WF_LAUNCH(B, M)                                                                                         \
+    hipLaunchKernelGGL((tsx::wino_f63_gemm_output_kernel<B, M>), grid, dim3(256), 0, stream, v, u_dev, g, bias_dev, act, \
+                       slope, count / 4 * 4, out_dev)
+    if (blocks == 4) { if (mish) TSX_WF_LAUNCH(4, true); else TSX_WF_LAUNCH(4, false); }
+    else if (blocks == 8) { if (mish) TSX_WF_LAUNCH(8, true); else TSX_WF_LAUNCH(8, false); }
+    else if (blocks == 16) { if (mish) TSX_WF_LAUNCH(16, true); else TSX_WF_LAUNCH(16, false); }
+    else { if (mish) TSX_WF_LAUNCH(0, true); else TSX_WF_LAUNCH(0, false); }
+#undef TSX_WF_LAUNCH
+    TSX_LAUNCH_CHECK("wino_f63_gemm_output_kernel");
     return 0;
 }
 
@@ -572,8 +775,12 @@ int tsx_conv2d_winograd_f23_nchw(const tsx_conv2d_geom *q, const float *x_dev, c
 
     const int64_t out_threads = int64_t(g.n) * g.cout * g.tiles;
     const int64_t count = int64_t(g.n) * g.cout * g.ho * g.wo;
-    hipLaunchKernelGGL(tsx::wino23_output_transform_kernel, dim3(unsigned(tsx::ceil_div(out_threads, 256))), dim3(256), 0,
-                       stream, mm, g, bias_dev, act, slope, count / 4 * 4, out_dev);
+    if (act == TSX_ACT_MISH)
+        hipLaunchKernelGGL(tsx::wino23_output_transform_kernel<true>, dim3(unsigned(tsx::ceil_div(out_threads, 256))), dim3(256), 0,
+                           stream, mm, g, bias_dev, act, slope, count / 4 * 4, out_dev);
+    else
+        hipLaunchKernelGGL(tsx::wino23_output_transform_kernel<false>, dim3(unsigned(tsx::ceil_div(out_threads, 256))), dim3(256), 0,
+                           stream, mm, g, bias_dev, act, slope, count / 4 * 4, out_dev);
     TSX_LAUNCH_CHECK("wino23_output_transform_kernel");
     return 0;
 }

@@ -116,6 +116,33 @@ def test_winograd(tsx, port, case, mode):
     assert np.array_equal(bits(got), bits(exp)), (bits(got) != bits(exp)).mean()
 
 
+@pytest.mark.parametrize("case", WINO_CASES + [(3, 20, 31, 13, 50, (1, 0, 2, 1)), (2, 64, 28, 28, 96, (1, 1, 1, 1))])
+def test_winograd_f63_fast_path(tsx, port, case):
+    """The MFMA form of F(6,3) against the reference's F(6,3) values (the oracle is bit-exact to them),
+    with bias, activation and a non-zero padding value; channel counts and tile counts that are not multiples of the
+    kernel's 16-wide blocks included.  Two F(6,3) evaluations that sum the channel products in different orders
+    differ by the method's own fp32 noise (its transforms multiply by up to 32 and cancel again), ~1e-5 absolute on
+    O(1) outputs, so the bar is the one TenniS's own backend test applies between devices (tools/run_test/
+    test_case.hpp:491-503): max |diff| <= 1e-4 and mean |diff| <= 1e-5; on top of it, all but a small share of the
+    elements must meet the strict per-element bar 1e-4 |exp| + 1e-5."""
+    n, c, h, w, cout, pads = case
+    rng = np.random.default_rng(405)
+    x = rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)
+    wt = (rng.standard_normal((cout, c, 3, 3)) * np.sqrt(2.0 / (c * 9))).astype(np.float32)
+    bias = (rng.standard_normal(cout) * 0.1).astype(np.float32)
+    op = tsx.Winograd(_dev(wt), pads, padding_value=0.25, mode="f63")
+    got = op(_dev(x), bias=_dev(bias), act="relu", fast=True).cpu().numpy()
+    exp = port.relu(port.add_bias(port.winograd_f63(x, wt, pads, padding_value=0.25), bias))
+    assert got.shape == exp.shape
+    diff = np.abs(got.astype(np.float64) - exp)
+    assert diff.max() <= 1e-4 and diff.mean() <= 1e-5, (diff.max(), diff.mean())
+    strict = diff <= ABS + REL * np.abs(exp)
+    assert strict.mean() >= 0.999, (1.0 - strict.mean(), diff.max())
+    # and against the direct convolution in fp64, to see that the tolerance is not hiding a wrong transform
+    exact = port.relu(port.add_bias(port.conv2d_f32(x, wt, pads, padding_value=0.25), bias))
+    assert np.abs(got - exact).max() < 2e-4
+
+
 @pytest.mark.parametrize("mode", ["f63", "f23"])
 def test_winograd_padding_value_bias_relu(tsx, port, mode):
     rng = np.random.default_rng(404)
