@@ -223,12 +223,31 @@ class StagedPlain:
         self.buf = torch.zeros(n * h * w * self.cp, dtype=torch.int8, device=device)
 
 
+class StagedSlice:
+    """Channels [c0, c0 + channels) of a StagedInput, as the staged output of ONE producer of a channel concatenation:
+    every producer's epilogue writes its requantized output into its own run of channels of the consumer's staged
+    input (quantized with the consumer's scale, which was calibrated on the concatenated tensor), so the concatenated
+    tensor never exists in fp32 and is never staged.  c0 must be a multiple of 16 (the epilogue stores 16 bytes)."""
+
+    def __init__(self, staged, c0, channels):
+        n, c, h, w = staged.x_shape
+        if c0 % 16 != 0 or c0 < 0 or c0 + channels > c:
+            raise TsxError("channels [%d, %d) are not a 16-aligned run inside the %d of the staged tensor" % (c0, c0 + channels, c))
+        self.x_shape = (n, channels, h, w)
+        self.hs, self.ws, self.cp = staged.hs, staged.ws, staged.cp
+        self.pad_top, self.pad_left = staged.pad_top, staged.pad_left
+        self.full_buf, self.c0 = staged.buf, c0
+        self.buf = staged.buf[c0:]          # the epilogue takes the address of channel c0 of the first pixel
+
+
 def staged_interior(staged, images):
     """The map inside a staged buffer (StagedInput / StagedPlain) as an int8 NCHW tensor of the given images:
     a copy, for checkers that compare a producer's requantized hand-over with the operator chain's values."""
     n, c, h, w = staged.x_shape
-    t = staged.buf[: n * staged.hs * staged.ws * staged.cp].view(n, staged.hs, staged.ws, staged.cp)
-    t = t[list(images), staged.pad_top:staged.pad_top + h, staged.pad_left:staged.pad_left + w, :c]
+    c0 = getattr(staged, "c0", 0)
+    buf = getattr(staged, "full_buf", staged.buf)
+    t = buf[: n * staged.hs * staged.ws * staged.cp].view(n, staged.hs, staged.ws, staged.cp)
+    t = t[list(images), staged.pad_top:staged.pad_top + h, staged.pad_left:staged.pad_left + w, c0:c0 + c]
     return t.permute(0, 3, 1, 2).contiguous()
 
 

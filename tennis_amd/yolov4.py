@@ -213,6 +213,29 @@ class YoloV4Int8:
                 a, b = rsrcs[i]
                 if L[a]["type"] == "conv" and consumers[a] == [i] and a not in heads and a != b:
                     folded[i] = a
+        # Channel concatenations (routes with several sources) whose sources are all convolution outputs that nothing
+        # else reads and whose one consumer is a convolution that can read a staged buffer: every source convolution
+        # writes its requantized output into its run of channels of that consumer's staged input (the CSP stages'
+        # two-branch joins).  concat_of: source convolution -> (route, consumer, first channel, total channels).
+        self._concat_of, self._concat_routes = {}, {}
+        for i, l in enumerate(L):
+            if l["type"] != "route" or len(self.srcs[i]) < 2 or i in heads:
+                continue
+            cons = consumers[i]
+            if len(cons) != 1 or L[cons[0]]["type"] != "conv" or not self._stageable(cons[0]):
+                continue
+            s = rsrcs[i]
+            ok = all(j >= 0 and L[j]["type"] == "conv" and consumers[j] == [i] and j not in heads and j not in folded.values()
+                     for j in s) and len(set(s)) == len(s)
+            if not ok:
+                continue
+            offsets = [sum(L[j]["filters"] for j in s[:m]) for m in range(len(s))]
+            if any(o % 16 for o in offsets):
+                continue
+            total = sum(L[j]["filters"] for j in s)
+            for j, o in zip(s, offsets):
+                self._concat_of[j] = (i, cons[0], o, total)
+            self._concat_routes[i] = cons[0]
         return rsrcs, consumers, heads, folded
 
     def _run_chained(self, x):
@@ -269,9 +292,17 @@ class YoloV4Int8:
                     assert self.scales[k] == self.scales[served[0]]   # calibrated on the same tensor
                     staged_for[k] = target
                 want_f32 = bool(others) or out_id in heads or any(k not in served for k in conv_cons)
+                q_layer = served[0] if served else None
+                if i in self._concat_of and out_id == i:
+                    # one branch of a channel concatenation: straight into its channels of the consumer's staged input
+                    route, k, c0, total = self._concat_of[i]
+                    whole = staged_input(k, (n, total, ho, wo))
+                    target = capi.StagedSlice(whole, c0, l["filters"])
+                    staged_for[k] = whole
+                    want_f32, q_layer = False, k
                 kw = dict(dq=self.dq[i], bias=self.bias[i], act=l["act"], slope=0.1, want_f32=want_f32)
                 if target is not None:
-                    kw.update(q_scales=self.sx[served[0]], staged_out=target)
+                    kw.update(q_scales=self.sx[q_layer], staged_out=target)
                 if i in absorbed:
                     kw.update(residual=outs[rsrcs[absorbed[i]][1]], residual_after_act=True)
                 if i in staged_for:
@@ -287,7 +318,7 @@ class YoloV4Int8:
                         "residual": None if res is None else res[idx].cpu().numpy(),
                         "out_f32": None if y is None else y[idx].cpu().numpy(),
                         "out_q": None if target is None else capi.staged_interior(target, idx).cpu().numpy(),
-                        "q_layer": served[0] if served else None})
+                        "q_layer": q_layer})
                 outs[out_id] = y
                 if out_id != i:
                     outs[i] = None
@@ -301,6 +332,10 @@ class YoloV4Int8:
                 if len(self.srcs[i]) == 1:
                     outs[i] = None                                 # looked through
                     self._shapes[i] = self._shapes[s[0]]
+                elif i in self._concat_routes:
+                    outs[i] = None                                 # its sources wrote the consumer's staged input
+                    first = self._shapes[s[0]]
+                    self._shapes[i] = (first[0], sum(L[j]["filters"] for j in s), first[2], first[3])
                 else:
                     outs[i] = capi.concat_channels([outs[j] for j in s])
                     self._shapes[i] = tuple(outs[i].shape)
