@@ -59,7 +59,7 @@ __global__ __launch_bounds__(256) void elementwise_kernel(const float *__restric
             } else if (MODE == 4) {
                 v[j] = tsx::apply_act(v[j], TSX_ACT_MISH, 0.f, true);
             } else if (MODE == 5) {
-                v[j] = float(log(double(expf(v[j])) + 1.0));
+                v[j] = tsx::softplus_value(v[j]);
             } else if (MODE == 6) {
                 v[j] = __fsub_rn(__fmul_rn(2.f, __fdiv_rn(1.f, __fadd_rn(1.f, expf(-__fmul_rn(2.f, v[j]))))), 1.f);
             } else if (MODE == 7) {

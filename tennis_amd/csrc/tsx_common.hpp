@@ -99,17 +99,52 @@ __device__ __forceinline__ float apply_act_basic(float v, int act, float slope, 
     return v;
 }
 
+// cpu::Softplus (src/kernels/cpu/softplus.cpp:30-39): float(log(double(expf(x)) + 1.0)).  The host goes through double
+// only to round log(1 + e) to float well; here log1pf does that in single precision (within an ulp or two of the
+// correctly rounded value) at a fraction of the cost -- a double-precision logarithm per element made the Mish
+// epilogue, not memory or the MFMAs, the bound of every Mish layer.  expf / log1pf are this device's library
+// routines in either form, so Mish values agree with the host's to a few ulp, not bit for bit.
+__device__ __forceinline__ float softplus_value(float x) { return log1pf(expf(x)); }
+
+// e^x for the Mish epilogue: the hardware's 2^a (v_exp_f32, 1 ulp) on a = x * log2(e) carried in two floats, so that
+// the product's rounding does not reach the result: 2^(ah + al) = 2^ah * (1 + al ln2 + ...).  About 1.5 ulp, no range
+// handling: arguments are below 89 in magnitude where the result matters (see mish_value).
+__device__ __forceinline__ float mish_exp(float x) {
+    const float ah = __fmul_rn(x, 1.4426950216293335f);
+    const float al = __builtin_fmaf(x, 1.925963033500011e-08f, __builtin_fmaf(x, 1.4426950216293335f, -ah));
+    const float e = __builtin_amdgcn_exp2f(ah);
+    return __builtin_fmaf(e, __fmul_rn(al, 0.6931471824645996f), e);
+}
+
+// Mish as TenniS graphs compose it, x * tanh(softplus(x)) with softplus = float(log(double(expf(x)) + 1.0))
+// (src/kernels/cpu/softplus.cpp:30-39) and tanh(y) = 2 * (1 / (1 + expf(-2y))) - 1 in float
+// (src/kernels/cpu/tanh.cpp:14-23): the same chain of rounded intermediates -- e, softplus, expf(-2 softplus), the
+// quotient, 2q - 1, the product -- each within an ulp or two of the host's, evaluated on the hardware's exp2 / log2 /
+// reciprocal instead of the library routines: ~45 issue slots against ~160 (two expf, a log1pf and an IEEE division
+// with all their range handling), which was what bounded every Mish layer.
+//   softplus: s = 1 + e with its rounding error c kept (two-sum), log(s) = log2(s) ln2 (constant in two floats) + c / s;
+//             for e below 2^-24 this is e itself, as log1p gives.
+//   quotient: reciprocal with one Newton step (correctly rounded but for rare ties).
+// Limits as the host's: x large -> x, x very negative -> -0 or 0, NaN -> NaN.
+__device__ __forceinline__ float mish_value(float x) {
+    const float e = mish_exp(fminf(x, 88.f));              // beyond 88 the host's expf overflows to inf and tanh gives 1: so does this
+    const float hi = fmaxf(e, 1.f), lo = fminf(e, 1.f);
+    const float s = __fadd_rn(hi, lo);
+    const float c = __fsub_rn(lo, __fsub_rn(s, hi));       // s + c = 1 + e exactly
+    const float l2 = __builtin_amdgcn_logf(s);             // log2(s), 1 ulp
+    const float rs = __builtin_amdgcn_rcpf(s);
+    const float sp = __builtin_fmaf(l2, 0.6931471824645996f, __builtin_fmaf(l2, -1.9046542121259336e-09f, __fmul_rn(c, rs)));
+    const float u = mish_exp(__fmul_rn(-2.f, sp));
+    const float d = __fadd_rn(1.f, u);
+    const float r0 = __builtin_amdgcn_rcpf(d);
+    const float q = __builtin_fmaf(r0, __builtin_fmaf(-d, r0, 1.f), r0);
+    const float t = __builtin_fmaf(2.f, q, -1.f);          // 2q is exact: one rounding, as fl(fl(2q) - 1)
+    return __fmul_rn(x, t);
+}
+
 __device__ __forceinline__ float apply_act(float v, int act, float slope, bool in_body) {
     if (act != TSX_ACT_MISH) return apply_act_basic(v, act, slope, in_body);
-    {
-        // x * tanh(softplus(x)) as TenniS graphs compose it: softplus = float(log(double(expf(x)) + 1.0))
-        // (src/kernels/cpu/softplus.cpp:30-39), tanh = 2 * (1 / (1 + expf(-2y))) - 1 in float
-        // (src/kernels/cpu/tanh.cpp:14-23), then mul.  Same formulas; expf/log are this device's
-        // library routines, so results agree with the host's to a few ulp, not bit for bit.
-        const float sp = float(log(double(expf(v)) + 1.0));
-        const float t = __fsub_rn(__fmul_rn(2.f, __fdiv_rn(1.f, __fadd_rn(1.f, expf(-__fmul_rn(2.f, sp))))), 1.f);
-        return __fmul_rn(v, t);
-    }
+    return mish_value(v);
 }
 
 #endif  // __HIPCC__

@@ -253,7 +253,8 @@ def test_concat_and_resize2d_operators(ops, port):
 def test_mish_composition_operators(ops, port):
     """softplus, tanh and mul -- the nodes TenniS graphs compose Mish from.  mul is one IEEE multiplication per
     element (bitwise); softplus and tanh use the device's expf / log: a few ulp from the host's, checked to
-    1e-6 relative + 1e-6 absolute against the oracle, and the composition equals the fused Mish kernel bit for bit."""
+    1e-6 relative + 1e-6 absolute against the oracle; the fused Mish kernel (the same chain of rounded intermediates
+    on the hardware's exp2 / log2 / reciprocal) stays within 1e-6 relative + 1e-6 absolute of their composition."""
     from tennis_amd import capi
     rng = np.random.default_rng(509)
     x = (rng.standard_normal((2, 5, 13, 11)) * 4).astype(np.float32)
@@ -269,6 +270,7 @@ def test_mish_composition_operators(ops, port):
     mish = ops.run_op("mul", {}, [x, ops.run_op("tanh", {}, [sp])])
     import torch
     fused = capi.mish(torch.from_numpy(x).cuda()).cpu().numpy()
-    assert np.array_equal(bits(mish), bits(fused))
+    assert np.allclose(fused, mish, rtol=1e-6, atol=1e-6), np.abs(fused - mish).max()
+    assert np.array_equal(bits(fused.flat[:6]), bits(mish.flat[:6]))      # the limits: 0, -0, large, very negative
     with pytest.raises(ops.OperatorError):
         ops.run_op("softplus", {}, [x.astype(np.float64)])
