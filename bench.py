@@ -34,8 +34,8 @@ CFG = dict(n=32, c=256, h=28, w=28, cout=256, k=3, pad=1)
 
 # HBM bytes per launch of the two kernels on this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a
 # known-size copy (profiles/conv2d_i8_config2_hbm_traffic.txt); a profiler figure, not measured by this script.
-TRAFFIC_CONV_BYTES = 43.99e6
-TRAFFIC_STAGE_BYTES = 33.44e6
+TRAFFIC_CONV_BYTES = 43.93e6
+TRAFFIC_STAGE_BYTES = 33.15e6
 
 
 def make_inputs(cfg, seed=1234):
@@ -438,8 +438,9 @@ def main():
                     help="for runs under a profiler: skip the int8-output variant (same kernel name as the roofline "
                          "kernel), the MFMA-rate probe and the CPU baseline, so per-kernel statistics cover the timed "
                          "kernels only")
-    ap.add_argument("--network", choices=("resnet", "yolo"),
-                    help="run only that network leg and print its figures (for per-kernel profiles of a network)")
+    ap.add_argument("--network", choices=("resnet", "yolo", "tennis"),
+                    help="run only that network leg and print its figures (for per-kernel profiles of a network); "
+                         "tennis = the ResNet-50-shaped module through TenniS's own runtime on device hip")
     ap.add_argument("--kernels", action="store_true",
                     help="run only the one-by-one kernel leg (GEMM, fp32, Winograd, 1x1, depthwise, elementwise, pooling) "
                          "and print its figures (for per-kernel counters)")
@@ -458,7 +459,8 @@ def main():
     L = capi.lib()
     dev = torch.device("cuda:0")
     if args.network:
-        print(json.dumps(resnet_leg() if args.network == "resnet" else yolo_leg()))
+        leg = {"resnet": resnet_leg, "yolo": yolo_leg, "tennis": tennis_runtime_leg}[args.network]
+        print(json.dumps(leg()))
         return
     if args.kernels:
         print(json.dumps(kernels_leg()))
