@@ -34,6 +34,11 @@ extern "C" int tsx_debug_phase_stamps(void *buffer_dev, size_t bytes) {
 
 namespace tsx {
 
+void debug_phase_stamps(unsigned long long **buffer, int *slots) {
+    *buffer = g_stamps.load();
+    *slots = int(g_stamp_slots.load());
+}
+
 void fl_plan(const WsGeom &g, WsPlan *pl) {
     pl->flat = false;
     if (!pl->ok || g.gemm || g.kh * g.kw <= 1 || pl->wm != 4) return;

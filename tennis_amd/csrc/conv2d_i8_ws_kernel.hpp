@@ -28,7 +28,20 @@ struct WsParams : EpiParams {
     int pix, chunk_shift, stage_bytes, tap_row, tap_col;
     int stream_out;   // fp32 output written with streaming stores
     int rowmajor;     // GEMM: output index position * cout + channel, row_scale[position] applied behind dq
+    // measurement aid (tsx_debug_phase_stamps): when set, every wavefront writes 8 values at
+    // stamps[(workgroup * 8 + wave) * 8]: wall clock (100 MHz) and shader clock at kernel entry, K-loop entry,
+    // K-loop exit and after its last store
+    unsigned long long *stamps;
+    int stamp_slots;
+    // per-lane divisions by uniform divisors as one multiply-high: ceil(2^32 / d), 0 for d = 1 (see udiv)
+    unsigned wc_magic, tw_magic, ow_magic;
 };
+
+// ceil(2^32 / d) for d >= 2, 0 for d = 1: floor(n / d) = mulhi(n, magic) whenever n * d <= 2^32
+inline unsigned div_magic(int d) { return d <= 1 ? 0u : unsigned(((uint64_t(1) << 32) + unsigned(d) - 1) / unsigned(d)); }
+
+// buffer of tsx_debug_phase_stamps (null = off)
+void debug_phase_stamps(unsigned long long **buffer, int *slots);
 
 // One specialisation per fragment count, each defined by its own translation unit.
 template <int NT>
@@ -56,6 +69,10 @@ namespace {
 // [position][cout] row-major, and row_scale[position] multiplies behind dq (the per-row activation scale of a
 // quantized inner product).  A lane's accumulators 4g..4g+3 are 4 consecutive channels of its position, so
 // the fp32 output goes out as 16-byte stores; lanes l and l+32 and the four g complete a 128-byte line.
+// floor(n / d) through d's magic number (div_magic): window pixels, tile positions and map pixels times their
+// divisors stay far below 2^32
+__device__ __forceinline__ int udiv(int n, unsigned magic) { return magic ? int(__umulhi(unsigned(n), magic)) : n; }
+
 template <int NT, int FM, bool EXTRA, bool STREAM, bool ROWM>
 __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <= 4 ? 2 : 1))) void conv_i8_ws_kernel(WsParams p_in) {
     WsParams p = p_in;
@@ -65,7 +82,9 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
     }
     if (!ROWM) p.row_scale = nullptr;
     extern __shared__ __attribute__((aligned(16))) int8_t lds[];   // 2 x wpix x PIX
-    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    // the wavefront's index as a scalar: what derives from it (first cout, tile bases, the choice of epilogue path)
+    // then stays in scalar registers and branches uniformly
+    const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const int rtile = blockIdx.x / p.ctiles;
     const int col0 = (blockIdx.x - rtile * p.ctiles) * p.tw;   // first output column of the tile
     const int row0 = rtile * p.th;           // first output row of the tile, counted over the whole batch
@@ -79,33 +98,56 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
     const int m0 = (blockIdx.y * p.wm + wave_m) * (32 * FM);         // first cout of this wavefront
     const int taps = p.kh * p.kw;
     const int win_bytes = p.wpix * p.pix;
+    const int stamp_slot = ((blockIdx.y * gridDim.x + blockIdx.x) * 8 + wave) * 8;
+    auto stamp = [&](int phase) __attribute__((always_inline)) {
+        if (p.stamps && lane == 0 && stamp_slot + 8 <= p.stamp_slots) {
+            p.stamps[stamp_slot + 2 * phase] = wall_clock64();
+            p.stamps[stamp_slot + 2 * phase + 1] = clock64();
+        }
+    };
+    stamp(0);
 
     // ---- window fill bookkeeping: chunk q = tid + i*256 -> pixel q / chunks-per-pixel, 16-byte chunk q % ...
-    const int8_t *fill_src[MAX_FILL];
+    // A uniform 64-bit base (the window's first staged row and column) plus one 32-bit byte offset per chunk: the
+    // loads then take the base from scalar registers and need no address arithmetic of their own.
+    const int n_fill = ((p.wpix << p.chunk_shift) + WS_THREADS - 1) / WS_THREADS;   // <= MAX_FILL, uniform
+    // window row r is staged row (img * hs + th0 * stride) + r of the batch-wide staged row sequence
+    const int64_t row_base = int64_t(img) * p.hs + th0 * p.sh;
+    const int col_base = col0 * p.sw;
+    const int row_last = int(min(int64_t(p.n) * p.hs - 1 - row_base, int64_t(1) << 20));   // last tile: rows no stored output uses
+    const int col_last = p.ws - 1 - col_base;                                               // last column tile: likewise
+    const int8_t *xs_base = p.xs + (row_base * p.ws + col_base) * p.cp;
+    unsigned fill_off[MAX_FILL];
     int fill_dst[MAX_FILL];
     static_for<0, MAX_FILL>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        const int q = tid + i * WS_THREADS;
-        int pix = q >> p.chunk_shift;
-        const int chunk = q & ((1 << p.chunk_shift) - 1);
-        if (pix >= p.wpix) pix = p.wpix - 1;   // duplicates rewrite the same bytes
-        int wrow = pix / p.wc;
-        const int wcol = pix - wrow * p.wc;
-        // window row r is staged row (img * hs + th0 * stride) + r of the batch-wide staged row sequence
-        int64_t row = int64_t(img) * p.hs + th0 * p.sh + wrow;
-        if (row >= int64_t(p.n) * p.hs) row = int64_t(p.n) * p.hs - 1;   // last tile: rows no stored output uses
-        int col = col0 * p.sw + wcol;
-        if (col >= p.ws) col = p.ws - 1;                                 // last column tile: columns no stored output uses
-        fill_src[i] = p.xs + (row * p.ws + col) * p.cp + chunk * 16;
-        fill_dst[i] = pix * p.pix + chunk * 16;
+        fill_off[i] = 0;
+        fill_dst[i] = 0;
+        if (i < n_fill) {
+            const int q = tid + i * WS_THREADS;
+            int pix = q >> p.chunk_shift;
+            const int chunk = q & ((1 << p.chunk_shift) - 1);
+            if (pix >= p.wpix) pix = p.wpix - 1;   // duplicates rewrite the same bytes
+            const int wrow = udiv(pix, p.wc_magic);
+            const int wcol = pix - __mul24(wrow, p.wc);
+            // 24-bit multiplies (full rate): window rows, staged widths and pixel sizes are far below 2^24
+            fill_off[i] = unsigned(__mul24(__mul24(min(wrow, row_last), p.ws) + min(wcol, col_last), p.cp) + chunk * 16);
+            fill_dst[i] = __mul24(pix, p.pix) + chunk * 16;
+        }
     });
-    const int n_fill = ((p.wpix << p.chunk_shift) + WS_THREADS - 1) / WS_THREADS;   // <= MAX_FILL, uniform
     v4i wreg[MAX_FILL];   // native vectors: arrays of HIP's uint4 struct do not stay in registers
 
     auto window_load = [&](int cb) __attribute__((always_inline)) {
+        const int8_t *base = xs_base + cb * p.stage_bytes;
         static_for<0, MAX_FILL>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
-            if (i < n_fill) wreg[i] = *reinterpret_cast<const v4i *>(fill_src[i] + cb * p.stage_bytes);
+            if (i < n_fill) {
+                // the empty statement keeps the offset's widening next to the load, where instruction selection
+                // folds it into the scalar-base addressing mode
+                unsigned off = fill_off[i];
+                asm volatile("" : "+v"(off));
+                wreg[i] = *reinterpret_cast<const v4i *>(base + off);
+            }
         });
     };
     auto window_store = [&](int buf) __attribute__((always_inline)) {
@@ -121,9 +163,9 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
         constexpr int j = decltype(jc)::value;
         int pos = pos0 + j * 32 + lane % 32;
         if (pos >= p.th * p.tw) pos = 0;       // padding positions: computed, never stored
-        const int r = pos / p.tw, tc = pos - r * p.tw;
+        const int r = udiv(pos, p.tw_magic), tc = pos - __mul24(r, p.tw);
         const int wrow = r * p.sh + (th0 + r >= p.ho ? wrap : 0);   // positions of the next image sit below its halo rows
-        b_base[j] = (wrow * p.wc + tc * p.sw) * p.pix + (lane / 32) * 16;
+        b_base[j] = __mul24(__mul24(wrow, p.wc) + __mul24(tc, p.sw), p.pix) + (lane / 32) * 16;
     });
 
     // ---- A ring: the wavefront's FM fragments (32 cout each) x 2 halves of K-step ks, 1 KiB each
@@ -150,6 +192,35 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
     // ---- prologue
     window_load(0);
     static_for<0, RING - 1>([&](auto sc) { a_load(sc, decltype(sc)::value); });
+
+    // ---- epilogue operands, fetched while the first window is in flight: a wavefront that meets them only behind
+    // its K-loop waits a full memory latency there, with nothing else on its SIMD to hide it
+    const int tile_pos = p.th * p.tw;
+    const int howo = p.ho * p.wo;
+    const int64_t count = int64_t(p.n) * p.cout * howo;
+    // hot case: no raw accumulators wanted, every element inside the activation's SIMD-body range,
+    // a tensor small enough for 32-bit lane offsets, and -- for the requantized output -- one
+    // quantize group per image (or a single scale whose round-half-even bulk covers everything),
+    // so the consumer's scale is uniform for this tile and needs no per-element division
+    const bool want_q = p.out_i8 || p.st_out;
+    const bool q_uniform = !want_q || (p.n_qscales == 1 ? p.q_bulk8 == count : p.q_group_len == int64_t(p.cout) * howo);
+    // the GEMM form stores 4 consecutive channels at once, and its quantize groups are rows, not images
+    const bool rowm_ok = !ROWM || (!want_q && p.cout % 4 == 0 && reinterpret_cast<uintptr_t>(p.out_f32) % 16 == 0);
+    const bool fast = (p.out_f32 || want_q) && !p.out_acc && p.act_body == count && count < (int64_t(1) << 30) && q_uniform && rowm_ok;
+    // a tile may end in the next image: one consumer scale per image, selected per lane
+    const float q_scale_a = (fast && want_q) ? p.q_scales[p.n_qscales == 1 ? 0 : img] : 0.f;
+    const float q_scale_b = (fast && want_q) ? p.q_scales[p.n_qscales == 1 ? 0 : min(img + 1, p.n - 1)] : 0.f;
+    const bool q_even = p.n_qscales == 1;   // single-scale quantize rounds half to even in its bulk
+    // the wavefront's dequantize scales and biases are read behind the K-loop; touching their lines now leaves them
+    // in the caches by then (one load per array: 32 channels per fragment)
+    float touch = 0.f;
+    static_for<0, FM>([&](auto fc) {
+        const int co = min(m0 + decltype(fc)::value * 32 + lane % 32, p.cout - 1);
+        if (p.dq) touch += p.dq[co];
+        if (p.bias) touch += p.bias[co];
+    });
+    asm volatile("; epilogue operands touched" ::"v"(touch));
+
     window_store(0);
     __syncthreads();
     int cb = 0, tap = 0, kr = 0, kc = 0, buf = 0;
@@ -166,6 +237,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
     };
     int toff = 0;   // buf * win_bytes + tap shift
     b_read(b0, toff);
+    stamp(1);
 
     for (int ks0 = 0; ks0 < p.ksteps_p; ks0 += RING) {
         static_for<0, RING>([&](auto uc) {
@@ -209,62 +281,75 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
         });
     }
 
+    if (p.stamps) {
+        // wait for the MFMAs still in flight: the stamp marks the end of the multiplication, not its last issue
+        asm volatile("; accumulators complete" ::"v"(acc[0][0][15]), "v"(acc[FM - 1][NT - 1][15]) : "memory");
+        stamp(2);
+    }
+
     // ---- epilogue: accumulator register r of lane l = cout 8*(r/4) + 4*(l/32) + r%4, position l%32
-    const int tile_pos = p.th * p.tw;
-    const int howo = p.ho * p.wo;
-    const int64_t count = int64_t(p.n) * p.cout * howo;
-    // hot case: no raw accumulators wanted, every element inside the activation's SIMD-body range,
-    // a tensor small enough for 32-bit lane offsets, and -- for the requantized output -- one
-    // quantize group per image (or a single scale whose round-half-even bulk covers everything),
-    // so the consumer's scale is uniform for this tile and needs no per-element division
-    const bool want_q = p.out_i8 || p.st_out;
-    const bool q_uniform = !want_q || (p.n_qscales == 1 ? p.q_bulk8 == count : p.q_group_len == int64_t(p.cout) * howo);
-    // the GEMM form stores 4 consecutive channels at once, and its quantize groups are rows, not images
-    const bool rowm_ok = !ROWM || (!want_q && p.cout % 4 == 0 && reinterpret_cast<uintptr_t>(p.out_f32) % 16 == 0);
-    const bool fast = (p.out_f32 || want_q) && !p.out_acc && p.act_body == count && count < (int64_t(1) << 30) && q_uniform && rowm_ok;
-    // a tile may end in the next image: one consumer scale per image, selected per lane
-    const float q_scale_a = (fast && want_q) ? p.q_scales[p.n_qscales == 1 ? 0 : img] : 0.f;
-    const float q_scale_b = (fast && want_q) ? p.q_scales[p.n_qscales == 1 ? 0 : min(img + 1, p.n - 1)] : 0.f;
-    const bool q_even = p.n_qscales == 1;   // single-scale quantize rounds half to even in its bulk
     static_for<0, FM>([&](auto fc) {
         constexpr int f = decltype(fc)::value;
         const int cf = m0 + f * 32;   // first cout of this fragment (uniform)
+        // fast: all 32 channels exist, the loads need no bounds and combine into 16-byte ones
+        const bool fast_f = fast && cf + 32 <= p.cout;
+        // Loads without per-element branches: the fast case needs no bounds (consecutive channels combine into
+        // 16-byte loads); otherwise the index is clamped, and what a channel beyond cout loads is never stored.
         float dq[16], bias[16];
         static_for<0, 16>([&](auto rc) {
-            constexpr int r = decltype(rc)::value;
-            const int co = cf + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
-            const bool in = co < p.cout;
-            dq[r] = (in && p.dq) ? p.dq[co] : 0.f;
-            bias[r] = (in && p.bias) ? p.bias[co] : 0.f;
+            dq[decltype(rc)::value] = 0.f;
+            bias[decltype(rc)::value] = 0.f;
         });
-        // the other branch of a residual join: the loads of every fragment are in flight before the first use
-        float res[NT][16];
-        if (fast && cf + 32 <= p.cout && p.residual) {
-            const int64_t tile_base = (int64_t(img) * p.cout + cf) * howo;
+        const int co_lane = cf + 4 * (lane / 32);
+        if (fast_f) {
+            if (p.dq) static_for<0, 16>([&](auto rc) {
+                constexpr int r = decltype(rc)::value;
+                dq[r] = (p.dq + cf)[4 * (lane / 32) + 8 * (r / 4) + (r % 4)];
+            });
+            if (p.bias) static_for<0, 16>([&](auto rc) {
+                constexpr int r = decltype(rc)::value;
+                bias[r] = (p.bias + cf)[4 * (lane / 32) + 8 * (r / 4) + (r % 4)];
+            });
+        } else {
+            if (p.dq) static_for<0, 16>([&](auto rc) {
+                constexpr int r = decltype(rc)::value;
+                dq[r] = p.dq[min(co_lane + 8 * (r / 4) + (r % 4), p.cout - 1)];
+            });
+            if (p.bias) static_for<0, 16>([&](auto rc) {
+                constexpr int r = decltype(rc)::value;
+                bias[r] = p.bias[min(co_lane + 8 * (r / 4) + (r % 4), p.cout - 1)];
+            });
+        }
+        // One branch around the fragments, not one per fragment: inside it the compiler knows what is still in
+        // flight, and a fragment does not wait for the stores of the one before it.
+        if (fast_f) {
+            // the other branch of a residual join: the loads of every fragment are in flight before the first use
+            float res[NT][16];
+            if (EXTRA && p.residual) {
+                const int64_t tile_base = (int64_t(img) * p.cout + cf) * howo;
+                static_for<0, NT>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value;
+                    const int pos = pos0 + j * 32 + lane % 32;
+                    const int tr = udiv(pos, p.tw_magic), ow = col0 + pos - tr * p.tw;
+                    const bool wrapped = th0 + tr >= p.ho;                 // this position belongs to the next image
+                    const int oh = th0 + tr - (wrapped ? p.ho : 0);
+                    const bool pos_ok = pos < tile_pos && row0 + tr < rows_total && ow < p.wo;
+                    const unsigned lane_off = unsigned((wrapped ? p.cout * howo : 0) + (4 * (lane / 32)) * howo + oh * p.wo + ow);
+                    static_for<0, 16>([&](auto rc) {
+                        constexpr int r = decltype(rc)::value;
+                        constexpr int dco = 8 * (r / 4) + (r % 4);
+                        res[j][r] = pos_ok ? (p.residual + tile_base + int64_t(dco) * howo)[lane_off] : 0.f;
+                    });
+                });
+            }
             static_for<0, NT>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
                 const int pos = pos0 + j * 32 + lane % 32;
-                const int tr = pos / p.tw, ow = col0 + pos - tr * p.tw;
-                const bool wrapped = th0 + tr >= p.ho;
+                const int tr = udiv(pos, p.tw_magic), ow = col0 + pos - tr * p.tw;
+                const bool wrapped = th0 + tr >= p.ho;                 // this position belongs to the next image
                 const int oh = th0 + tr - (wrapped ? p.ho : 0);
                 const bool pos_ok = pos < tile_pos && row0 + tr < rows_total && ow < p.wo;
-                const unsigned lane_off = unsigned((wrapped ? p.cout * howo : 0) + (4 * (lane / 32)) * howo + oh * p.wo + ow);
-                static_for<0, 16>([&](auto rc) {
-                    constexpr int r = decltype(rc)::value;
-                    constexpr int dco = 8 * (r / 4) + (r % 4);
-                    res[j][r] = pos_ok ? (p.residual + tile_base + int64_t(dco) * howo)[lane_off] : 0.f;
-                });
-            });
-        }
-        static_for<0, NT>([&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-            const int pos = pos0 + j * 32 + lane % 32;
-            const int tr = pos / p.tw, ow = col0 + pos - tr * p.tw;
-            const bool wrapped = th0 + tr >= p.ho;                 // this position belongs to the next image
-            const int oh = th0 + tr - (wrapped ? p.ho : 0);
-            const bool pos_ok = pos < tile_pos && row0 + tr < rows_total && ow < p.wo;
-            const float q_scale = wrapped ? q_scale_b : q_scale_a;
-            if (fast && cf + 32 <= p.cout) {
+                const float q_scale = wrapped ? q_scale_b : q_scale_a;
                 // uniform base in scalar registers + one 32-bit lane offset: no per-store address math
                 const int64_t tile_base = (int64_t(img) * p.cout + cf) * howo;
                 const unsigned lane_off = unsigned((wrapped ? p.cout * howo : 0) + (4 * (lane / 32)) * howo + oh * p.wo + ow);
@@ -362,7 +447,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
                             const auto s13 = __builtin_amdgcn_permlane32_swap(word[1], word[3], false, false);
                             // the consumer's buffer is addressed by the real row/column (this kernel's rows may be virtual)
                             const int pix = oh * p.wo + ow;
-                            const int roh = p.wo == p.o_w ? oh : pix / p.o_w;
+                            const int roh = p.wo == p.o_w ? oh : udiv(pix, p.ow_magic);
                             const int row_ = p.wo == p.o_w ? ow : pix - roh * p.o_w;
                             int8_t *dst = p.st_out + ((int64_t(img + (wrapped ? 1 : 0)) * p.st_hs + roh + p.st_pt) * p.st_ws + row_ + p.st_pl) * p.st_cp +
                                           cf + 16 * (lane / 32);
@@ -371,7 +456,15 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
                         }
                     }
                 }
-            } else {
+            });
+        } else {
+            static_for<0, NT>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                const int pos = pos0 + j * 32 + lane % 32;
+                const int tr = udiv(pos, p.tw_magic), ow = col0 + pos - tr * p.tw;
+                const bool wrapped = th0 + tr >= p.ho;                 // this position belongs to the next image
+                const int oh = th0 + tr - (wrapped ? p.ho : 0);
+                const bool pos_ok = pos < tile_pos && row0 + tr < rows_total && ow < p.wo;
                 const int co0 = cf + 4 * (lane / 32);
                 const int64_t base = ROWM ? int64_t(row0 + tr) * p.cout + co0
                                           : (int64_t(img + (wrapped ? 1 : 0)) * p.cout + co0) * howo + oh * p.wo + ow;
@@ -383,9 +476,13 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
                     if (pos_ok && co0 + dco < p.cout)
                         emit(p, acc[f][j][r], base + int64_t(dco) * co_stride, dq[r], bias[r], rs);
                 });
-            }
-        });
+            });
+        }
     });
+    if (p.stamps) {
+        __builtin_amdgcn_s_waitcnt(0);   // every store of this wavefront has left
+        stamp(3);
+    }
 }
 
 }  // namespace
