@@ -133,6 +133,10 @@ int fl_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t 
     p.tiles_per_xcd = int((pl.fl_tiles + 7) / 8);
     p.positions = int(int64_t(g.n) * g.ho * g.wo);
     p.resident = pl.fl_resident ? 1 : 0;
+    p.wc_magic = div_magic(p.wc, FL_MAX_WP);
+    p.wo_magic = div_magic(p.wo, p.positions);
+    p.ho_magic = div_magic(p.ho, int64_t(g.n) * g.ho);
+    p.howo_magic = div_magic(p.ho * p.wo, p.positions);
     p.stamps = g_stamps.load();
     p.stamp_slots = int(g_stamp_slots.load());
     // an output of L2 size or more that no fused consumer reads: stream it

@@ -34,6 +34,8 @@ struct FlParams : EpiParams {
     // K-loop exit and after its last store has left
     unsigned long long *stamps;
     int stamp_slots;
+    // per-lane divisions by uniform divisors as one multiply-high (div_magic / udiv)
+    unsigned wc_magic, wo_magic, ho_magic, howo_magic;
 };
 
 template <int NTA, int NTB>
@@ -61,8 +63,8 @@ template <int NT, bool EXTRA, bool STREAM, bool RESIDENT>
 __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile, int wave_m, int frag0) {
     const int tid = threadIdx.x, lane = tid % 64;
     const int P0 = tile * p.frags * 32;   // first flat position (n, oh, ow) of the tile
-    const int R0 = P0 / p.wo;             // its row in the batch-wide row sequence
-    const int img0 = R0 / p.ho;
+    const int R0 = udiv(P0, p.wo, p.wo_magic);   // its row in the batch-wide row sequence
+    const int img0 = udiv(R0, p.ho, p.ho_magic);
     const int srow0 = img0 * p.hs + (R0 - img0 * p.ho) * p.sh;   // staged row of window row 0
     // staged rows from where output row `ho` of an image would start to the next image's first row
     const int wrap = p.hs - p.ho * p.sh;
@@ -79,28 +81,42 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
     stamp(0);
 
     // ---- window fill bookkeeping: chunk q = tid + i*512 -> pixel q / 4, 16-byte chunk q % 4
-    const int8_t *fill_src[FL_MAX_FILL];
+    // A uniform 64-bit base (the window's first staged row) plus one 32-bit byte offset per chunk: the loads take
+    // the base from scalar registers and need no address arithmetic of their own.
+    const int n_fill = (p.wpix * 4 + FL_THREADS - 1) / FL_THREADS;   // <= FL_MAX_FILL, uniform
+    const int row_last = int(min(int64_t(p.n) * p.hs - 1 - srow0, int64_t(1) << 20));   // last tile: rows no stored output uses
+    const int8_t *xs_base = p.xs + int64_t(srow0) * p.ws * p.cp;
+    unsigned fill_off[FL_MAX_FILL];
     int fill_dst[FL_MAX_FILL];
     static_for<0, FL_MAX_FILL>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        const int q = tid + i * FL_THREADS;
-        int pix = q >> 2;
-        const int chunk = q & 3;
-        if (pix >= p.wpix) pix = p.wpix - 1;   // duplicates rewrite the same bytes
-        const int wrow = pix / p.wc;
-        const int wcol = pix - wrow * p.wc;
-        int64_t row = int64_t(srow0) + wrow;
-        if (row >= int64_t(p.n) * p.hs) row = int64_t(p.n) * p.hs - 1;   // last tile: rows no stored output uses
-        fill_src[i] = p.xs + (row * p.ws + wcol) * p.cp + chunk * 16;
-        fill_dst[i] = wrow * p.rowp + wcol * FL_PIX + chunk * 16;
+        fill_off[i] = 0;
+        fill_dst[i] = 0;
+        if (i < n_fill) {
+            const int q = tid + i * FL_THREADS;
+            int pix = q >> 2;
+            const int chunk = q & 3;
+            if (pix >= p.wpix) pix = p.wpix - 1;   // duplicates rewrite the same bytes
+            const int wrow = udiv(pix, p.wc, p.wc_magic);
+            const int wcol = pix - __mul24(wrow, p.wc);
+            // 24-bit multiplies (full rate): window rows, staged widths and pixel sizes are far below 2^24
+            fill_off[i] = unsigned(__mul24(__mul24(min(wrow, row_last), p.ws) + wcol, p.cp) + chunk * 16);
+            fill_dst[i] = __mul24(wrow, p.rowp) + wcol * FL_PIX + chunk * 16;
+        }
     });
-    const int n_fill = (p.wpix * 4 + FL_THREADS - 1) / FL_THREADS;   // <= FL_MAX_FILL, uniform
     v4i wreg[FL_MAX_FILL];
 
+    // the empty statement keeps the offset's widening next to the load, where instruction selection folds it
+    // into the scalar-base addressing mode
+    auto fill_load = [&](int i, int cb) __attribute__((always_inline)) {
+        unsigned off = fill_off[i];
+        asm volatile("" : "+v"(off));
+        return *reinterpret_cast<const v4i *>(xs_base + cb * 64 + off);
+    };
     auto window_load = [&](int cb) __attribute__((always_inline)) {
         static_for<0, FL_MAX_FILL>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
-            if (i < n_fill) wreg[i] = *reinterpret_cast<const v4i *>(fill_src[i] + cb * 64);
+            if (i < n_fill) wreg[i] = fill_load(i, cb);
         });
     };
     auto window_store = [&](int buf) __attribute__((always_inline)) {
@@ -116,10 +132,10 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
         constexpr int j = decltype(jc)::value;
         int pp = P0 + (frag0 + j) * 32 + lane % 32;
         if (pp >= p.positions) pp = P0;       // beyond the last position: computed, never stored
-        const int R = pp / p.wo, ow = pp - R * p.wo;
-        const int img = R / p.ho;
+        const int R = udiv(pp, p.wo, p.wo_magic), ow = pp - R * p.wo;
+        const int img = udiv(R, p.ho, p.ho_magic);
         const int wrow = (R - R0) * p.sh + wrap * (img - img0);   // later images sit below their halo rows
-        b_base[j] = wrow * p.rowp + ow * p.sw * FL_PIX + (lane / 32) * 16;
+        b_base[j] = __mul24(wrow, p.rowp) + __mul24(ow, p.sw * FL_PIX) + (lane / 32) * 16;
     });
 
     // ---- A ring: 2 halves of K-step ks for the wavefront's 32 output channels, 1 KiB each.  Buffer loads:
@@ -159,7 +175,7 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
             const int c = 1 + b < p.cblocks ? 1 + b : p.cblocks - 1;
             static_for<0, FL_MAX_FILL>([&](auto ic) {
                 constexpr int i = decltype(ic)::value;
-                if (i < n_fill) wbat[b][i] = *reinterpret_cast<const v4i *>(fill_src[i] + c * 64);
+                if (i < n_fill) wbat[b][i] = fill_load(i, c);
             });
         });
     }
@@ -249,14 +265,34 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
     const bool fast = (p.out_f32 || want_q) && !p.out_acc && p.act_body == count && count < (int64_t(1) << 30) && q_uniform;
     const bool q_even = p.n_qscales == 1;   // single-scale quantize rounds half to even in its bulk
     const int cf = m0;                      // first cout of this wavefront's fragment (uniform)
+    // Loads without per-element branches: the fast case needs no bounds (consecutive channels combine into
+    // 16-byte loads); otherwise the index is clamped, and what a channel beyond cout loads is never stored.
+    const bool fast_f = fast && cf + 32 <= p.cout;
     float dq[16], bias[16];
     static_for<0, 16>([&](auto rc) {
-        constexpr int r = decltype(rc)::value;
-        const int co = cf + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
-        const bool in = co < p.cout;
-        dq[r] = (in && p.dq) ? p.dq[co] : 0.f;
-        bias[r] = (in && p.bias) ? p.bias[co] : 0.f;
+        dq[decltype(rc)::value] = 0.f;
+        bias[decltype(rc)::value] = 0.f;
     });
+    if (fast_f) {
+        if (p.dq) static_for<0, 16>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            dq[r] = (p.dq + cf)[4 * (lane / 32) + 8 * (r / 4) + (r % 4)];
+        });
+        if (p.bias) static_for<0, 16>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            bias[r] = (p.bias + cf)[4 * (lane / 32) + 8 * (r / 4) + (r % 4)];
+        });
+    } else {
+        const int co_lane = cf + 4 * (lane / 32);
+        if (p.dq) static_for<0, 16>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            dq[r] = p.dq[min(co_lane + 8 * (r / 4) + (r % 4), p.cout - 1)];
+        });
+        if (p.bias) static_for<0, 16>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            bias[r] = p.bias[min(co_lane + 8 * (r / 4) + (r % 4), p.cout - 1)];
+        });
+    }
     // per fragment: the lane's position as image and pixel
     int pimg[NT], prem[NT];
     bool pok[NT];
@@ -265,10 +301,10 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
         const int pp = P0 + (frag0 + j) * 32 + lane % 32;
         pok[j] = pp < p.positions;
         const int ps = pok[j] ? pp : P0;
-        pimg[j] = ps / howo;
+        pimg[j] = udiv(ps, howo, p.howo_magic);
         prem[j] = ps - pimg[j] * howo;
     });
-    if (fast && cf + 32 <= p.cout) {
+    if (fast_f) {
         // uniform base in scalar registers + one 32-bit lane offset: no per-store address math
         const int64_t base = int64_t(cf) * howo;
         // the other branch of a residual join: the loads of every fragment are in flight before the first use
@@ -359,7 +395,7 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
                     });
                     const auto s02 = __builtin_amdgcn_permlane32_swap(word[0], word[2], false, false);
                     const auto s13 = __builtin_amdgcn_permlane32_swap(word[1], word[3], false, false);
-                    const int oh = prem[j] / p.wo, ow = prem[j] - oh * p.wo;
+                    const int oh = udiv(prem[j], p.wo, p.wo_magic), ow = prem[j] - oh * p.wo;
                     int8_t *dst = p.st_out + ((int64_t(pimg[j]) * p.st_hs + oh + p.st_pt) * p.st_ws + ow + p.st_pl) * p.st_cp +
                                   cf + 16 * (lane / 32);
                     const v4i packed = {int(s02[0]), int(s02[1]), int(s13[0]), int(s13[1])};
@@ -405,7 +441,8 @@ __global__ __launch_bounds__(FL_THREADS) void conv_i8_fl_kernel(FlParams p_in) {
     // of 8, so the workgroups of one tile (blockIdx.y) land on the same XCD too.
     const int tile = (blockIdx.x & 7) * p.tiles_per_xcd + (blockIdx.x >> 3);
     if (tile >= p.tiles) return;   // the whole workgroup leaves
-    const int wave = threadIdx.x / 64;
+    // the wavefront's index as a scalar: what derives from it stays in scalar registers and branches uniformly
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     // The long wavefronts get the SIMD's issue priority: they run through K at the MFMA pipe's pace while the
     // short ones fill the gaps, finish first although they hold more fragments, and store the larger part of
     // the tile's output under the other group's K loop.

@@ -214,9 +214,9 @@ int ws_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t 
     p.rowmajor = g.gemm ? 1 : 0;
     if (g.gemm) p.stream_out = 0;
     debug_phase_stamps(&p.stamps, &p.stamp_slots);
-    p.wc_magic = div_magic(p.wc);
-    p.tw_magic = div_magic(p.tw);
-    p.ow_magic = div_magic(ep.o_w);
+    p.wc_magic = div_magic(p.wc, MAX_WP);
+    p.tw_magic = div_magic(p.tw, 4 * 7 * 32);
+    p.ow_magic = div_magic(ep.o_w, int64_t(p.ho) * p.wo);
     const int bm = 32 * WS_FM * pl.wm;
     const dim3 grid(unsigned(pl.tiles), unsigned((g.cout + bm - 1) / bm));
     const size_t lds_bytes = size_t(2) * pl.wp * (64 * pl.cbs + 16);

@@ -33,12 +33,9 @@ struct WsParams : EpiParams {
     // K-loop exit and after its last store
     unsigned long long *stamps;
     int stamp_slots;
-    // per-lane divisions by uniform divisors as one multiply-high: ceil(2^32 / d), 0 for d = 1 (see udiv)
+    // per-lane divisions by uniform divisors as one multiply-high (div_magic / udiv)
     unsigned wc_magic, tw_magic, ow_magic;
 };
-
-// ceil(2^32 / d) for d >= 2, 0 for d = 1: floor(n / d) = mulhi(n, magic) whenever n * d <= 2^32
-inline unsigned div_magic(int d) { return d <= 1 ? 0u : unsigned(((uint64_t(1) << 32) + unsigned(d) - 1) / unsigned(d)); }
 
 // buffer of tsx_debug_phase_stamps (null = off)
 void debug_phase_stamps(unsigned long long **buffer, int *slots);
@@ -69,10 +66,6 @@ namespace {
 // [position][cout] row-major, and row_scale[position] multiplies behind dq (the per-row activation scale of a
 // quantized inner product).  A lane's accumulators 4g..4g+3 are 4 consecutive channels of its position, so
 // the fp32 output goes out as 16-byte stores; lanes l and l+32 and the four g complete a 128-byte line.
-// floor(n / d) through d's magic number (div_magic): window pixels, tile positions and map pixels times their
-// divisors stay far below 2^32
-__device__ __forceinline__ int udiv(int n, unsigned magic) { return magic ? int(__umulhi(unsigned(n), magic)) : n; }
-
 template <int NT, int FM, bool EXTRA, bool STREAM, bool ROWM>
 __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <= 4 ? 2 : 1))) void conv_i8_ws_kernel(WsParams p_in) {
     WsParams p = p_in;
@@ -128,7 +121,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
             int pix = q >> p.chunk_shift;
             const int chunk = q & ((1 << p.chunk_shift) - 1);
             if (pix >= p.wpix) pix = p.wpix - 1;   // duplicates rewrite the same bytes
-            const int wrow = udiv(pix, p.wc_magic);
+            const int wrow = udiv(pix, p.wc, p.wc_magic);
             const int wcol = pix - __mul24(wrow, p.wc);
             // 24-bit multiplies (full rate): window rows, staged widths and pixel sizes are far below 2^24
             fill_off[i] = unsigned(__mul24(__mul24(min(wrow, row_last), p.ws) + min(wcol, col_last), p.cp) + chunk * 16);
@@ -163,7 +156,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
         constexpr int j = decltype(jc)::value;
         int pos = pos0 + j * 32 + lane % 32;
         if (pos >= p.th * p.tw) pos = 0;       // padding positions: computed, never stored
-        const int r = udiv(pos, p.tw_magic), tc = pos - __mul24(r, p.tw);
+        const int r = udiv(pos, p.tw, p.tw_magic), tc = pos - __mul24(r, p.tw);
         const int wrow = r * p.sh + (th0 + r >= p.ho ? wrap : 0);   // positions of the next image sit below its halo rows
         b_base[j] = __mul24(__mul24(wrow, p.wc) + __mul24(tc, p.sw), p.pix) + (lane / 32) * 16;
     });
@@ -330,7 +323,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
                 static_for<0, NT>([&](auto jc) {
                     constexpr int j = decltype(jc)::value;
                     const int pos = pos0 + j * 32 + lane % 32;
-                    const int tr = udiv(pos, p.tw_magic), ow = col0 + pos - tr * p.tw;
+                    const int tr = udiv(pos, p.tw, p.tw_magic), ow = col0 + pos - tr * p.tw;
                     const bool wrapped = th0 + tr >= p.ho;                 // this position belongs to the next image
                     const int oh = th0 + tr - (wrapped ? p.ho : 0);
                     const bool pos_ok = pos < tile_pos && row0 + tr < rows_total && ow < p.wo;
@@ -345,7 +338,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
             static_for<0, NT>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
                 const int pos = pos0 + j * 32 + lane % 32;
-                const int tr = udiv(pos, p.tw_magic), ow = col0 + pos - tr * p.tw;
+                const int tr = udiv(pos, p.tw, p.tw_magic), ow = col0 + pos - tr * p.tw;
                 const bool wrapped = th0 + tr >= p.ho;                 // this position belongs to the next image
                 const int oh = th0 + tr - (wrapped ? p.ho : 0);
                 const bool pos_ok = pos < tile_pos && row0 + tr < rows_total && ow < p.wo;
@@ -447,7 +440,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
                             const auto s13 = __builtin_amdgcn_permlane32_swap(word[1], word[3], false, false);
                             // the consumer's buffer is addressed by the real row/column (this kernel's rows may be virtual)
                             const int pix = oh * p.wo + ow;
-                            const int roh = p.wo == p.o_w ? oh : udiv(pix, p.ow_magic);
+                            const int roh = p.wo == p.o_w ? oh : udiv(pix, p.o_w, p.ow_magic);
                             const int row_ = p.wo == p.o_w ? ow : pix - roh * p.o_w;
                             int8_t *dst = p.st_out + ((int64_t(img + (wrapped ? 1 : 0)) * p.st_hs + roh + p.st_pt) * p.st_ws + row_ + p.st_pl) * p.st_cp +
                                           cf + 16 * (lane / 32);
@@ -461,7 +454,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
             static_for<0, NT>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
                 const int pos = pos0 + j * 32 + lane % 32;
-                const int tr = udiv(pos, p.tw_magic), ow = col0 + pos - tr * p.tw;
+                const int tr = udiv(pos, p.tw, p.tw_magic), ow = col0 + pos - tr * p.tw;
                 const bool wrapped = th0 + tr >= p.ho;                 // this position belongs to the next image
                 const int oh = th0 + tr - (wrapped ? p.ho : 0);
                 const bool pos_ok = pos < tile_pos && row0 + tr < rows_total && ow < p.wo;

@@ -25,6 +25,17 @@ struct EpiParams {
     int res_after;       // residual joins behind the activation instead of in front of it
 };
 
+// Division of a non-negative n by a uniform divisor d as one multiply-high: magic = ceil(2^32 / d) gives
+// floor(n / d) = mulhi(n, magic) whenever n * d <= 2^32.  0 = no magic number (d = 1, or n_max too large): the
+// kernel then divides.
+inline unsigned div_magic(int d, int64_t n_max) {
+    if (d <= 1 || n_max * d > (int64_t(1) << 32)) return 0u;
+    return unsigned(((uint64_t(1) << 32) + unsigned(d) - 1) / unsigned(d));
+}
+#ifdef __HIPCC__
+__device__ __forceinline__ int udiv(int n, int d, unsigned magic) { return magic ? int(__umulhi(unsigned(n), magic)) : n / d; }
+#endif
+
 // fp32 value of one accumulator after dequant -> row scale -> bias -> residual -> activation;
 // idx is the linear index in the output tensor.
 __device__ __forceinline__ float epi_value(const EpiParams &p, int acc, int64_t idx, float dq, float bias, float row_scale) {
