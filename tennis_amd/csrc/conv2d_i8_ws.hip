@@ -33,6 +33,8 @@
 // of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32.  Rows = cout, columns = positions.
 #include "conv2d_i8_ws_kernel.hpp"
 
+#include <algorithm>
+
 namespace tsx {
 namespace {
 
@@ -86,12 +88,13 @@ WsPlan ws_plan(const WsGeom &g_in) {
     // A tile is TH output rows of the batch-wide row sequence x TW output columns (whole rows when they fit),
     // at most MAX_NT fragments of 32 positions per wavefront.  Candidates are ranked by a model of the busiest
     // CU's time in units of one fragment's work,
-    //     (workgroups per CU) x (0.5 + fragments x slow),
+    //     (rounds of resident workgroups) x (overlap factor) x (0.5 + fragments x slow),
     // where 0.5 is the per-workgroup fixed cost and slow = 1.45 for tiles of more than 4 fragments
-    // (one workgroup per CU, so one wavefront per SIMD with nothing to hide its LDS/L2 waits).  The two
+    // (one workgroup per CU, so one wavefront per SIMD with nothing to hide its LDS/L2 waits).  The
     // constants come from a sweep over 32x256x28x28 (1/2/4/8-row tiles: 35 / 30.5 / 23.0 / 23.4 us) and the
-    // layers of a ResNet-50-shaped network, whose small maps want many small workgroups.  Ties go to the
-    // fewest total fragments (least padding).
+    // layers of a ResNet-50-shaped network, whose small maps want many small workgroups: 196 workgroups of 4
+    // fragments per wavefront (60 CUs idle) take 11.7 us on 32x512x28x28 -> 128 channels, 392 of 2 take 9.4.
+    // Ties go to the fewest total fragments (least padding).
     constexpr int MAX_NT = 7;
     // few output channels: fewer wavefronts along cout, the others take more positions of a larger tile
     const int wm = g.cout <= 32 ? 1 : g.cout <= 64 ? 2 : 4, wn = 4 / wm;
@@ -119,7 +122,14 @@ WsPlan ws_plan(const WsGeom &g_in) {
             if (wp > MAX_WP || size_t(2) * wp * PIX > 65536) continue;   // two windows must fit 64 KiB of LDS
             const int64_t wgs = tiles * (coutp / bm);
             const int64_t frags = tiles * nt * wn;
-            const double cost = double((wgs + 255) / 256) * (0.5 + nt * (nt > 4 ? 1.45 : 1.0));
+            // workgroups of up to 2 fragments per wavefront fit three to a CU, up to 4 two, larger ones one; those
+            // resident together overlap (each further one adds about half of a lone workgroup's time), the rest
+            // run in rounds -- so a layer that leaves CUs idle with large tiles takes tiles of half the size
+            const int64_t per_cu = (wgs + 255) / 256;
+            const int resident = nt <= 2 ? 3 : nt <= 4 ? 2 : 1;
+            const int64_t rounds = (per_cu + resident - 1) / resident;
+            const double together = 1.0 + 0.5 * double(std::min<int64_t>(per_cu, resident) - 1);
+            const double cost = double(rounds) * together * (0.5 + nt * (nt > 4 ? 1.45 : 1.0));
             // One or two K-steps (a 1x1 layer on 64 or 128 channels): the workgroup is all epilogue, its time is the
             // store traffic of its tile, and what pays is many small workgroups in flight per CU -- measured on
             // 32x64x56x56 -> 256 channels: 63 us with 4 fragments per wavefront and a residual join, 55 us with 2.
