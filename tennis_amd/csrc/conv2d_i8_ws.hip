@@ -202,6 +202,7 @@ int ws_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t 
     p.wc = pl.wc;
     p.wpix = pl.wp;
     p.ksteps_p = pl.ksteps_p;
+    p.ksteps = g.cblocks * g.kh * g.kw;
     p.wm = pl.wm;
     p.tw = pl.tw;
     p.ctiles = pl.ctiles;

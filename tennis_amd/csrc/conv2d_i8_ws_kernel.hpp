@@ -19,6 +19,7 @@ struct WsParams : EpiParams {
     const int8_t *wp;   // packed weights [ks_p][coutp/32][2 halves][64 lanes][16]
     int n, cout, coutp, ho, wo, hs, ws, cp, cblocks, kh, kw, dil_h, dil_w;
     int th, wr, wc, wpix, ksteps_p;
+    int ksteps;       // K-steps that hold weights (ksteps_p: padded to the A-ring size with zero steps)
     int wm;           // wavefronts along cout (4, 2 or 1: the other factor of 4 splits the tile's positions)
     int tw, ctiles;   // tile width in output columns, column tiles per row (1: whole rows)
     int sh, sw;       // strides
@@ -167,7 +168,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
     v4i areg[RING][2 * FM];
     auto a_load = [&](auto slot, int ks) __attribute__((always_inline)) {
         constexpr int s = decltype(slot)::value;
-        if (ks >= p.ksteps_p) ks = p.ksteps_p - 1;
+        if (ks >= p.ksteps) ks = p.ksteps - 1;   // beyond the last K-step: its lines again, never used
         const int8_t *src = a_ptr + ks * a_kstride;
         static_for<0, 2 * FM>([&](auto fc) {
             constexpr int f = decltype(fc)::value;
@@ -217,7 +218,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
     window_store(0);
     __syncthreads();
     int cb = 0, tap = 0, kr = 0, kc = 0, buf = 0;
-    window_load(p.cblocks > 1 ? 1 : 0);   // block cb+1, in flight during block cb's taps
+    if (p.cblocks > 1) window_load(1);   // block cb+1, in flight during block cb's taps
 
     // B fragments are read one half-step ahead of the MFMAs that use them (one wavefront per
     // SIMD: nothing else hides the LDS latency).
@@ -232,47 +233,57 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
     b_read(b0, toff);
     stamp(1);
 
-    for (int ks0 = 0; ks0 < p.ksteps_p; ks0 += RING) {
-        static_for<0, RING>([&](auto uc) {
-            constexpr int u = decltype(uc)::value;
-            // prefetch weights of K-step ks0+u+RING-1 into the slot freed by the previous step
-            a_load(std::integral_constant<int, (u + RING - 1) % RING>{}, ks0 + u + RING - 1);
-            b_read(b1, toff + 32);                       // second half of this K-step
-            static_for<0, FM>([&](auto ic) {
-                constexpr int i = decltype(ic)::value;
-                static_for<0, NT>([&](auto jc) {
-                    constexpr int j = decltype(jc)::value;
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[u][i * 2], b0[j], acc[i][j], 0, 0, 0);
-                });
+    // One K-step: both halves' MFMAs, the B reads one half-step ahead, the window swap on a channel-block boundary.
+    // PREFETCH: also load the weights of the K-step RING-1 ahead into the ring slot the previous step freed.
+    int ks = 0;
+    auto k_step = [&](auto uc, auto prefetch) __attribute__((always_inline)) {
+        constexpr int u = decltype(uc)::value;
+        if (decltype(prefetch)::value) a_load(std::integral_constant<int, (u + RING - 1) % RING>{}, ks + RING - 1);
+        b_read(b1, toff + 32);                       // second half of this K-step
+        static_for<0, FM>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            static_for<0, NT>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[u][i * 2], b0[j], acc[i][j], 0, 0, 0);
             });
-            // advance (cb, tap); on a channel-block boundary swap in the next window
-            ++tap;
-            if (++kc == p.kw) {
-                kc = 0;
-                ++kr;
-            }
-            if (tap == taps) {
-                tap = 0;
-                kr = 0;
-                kc = 0;
-                ++cb;
+        });
+        // advance (cb, tap); on a channel-block boundary swap in the next window (none behind the last K-step)
+        ++ks;
+        ++tap;
+        if (++kc == p.kw) {
+            kc = 0;
+            ++kr;
+        }
+        if (tap == taps) {
+            tap = 0;
+            kr = 0;
+            kc = 0;
+            ++cb;
+            if (ks < p.ksteps) {
                 window_store(buf ^ 1);
                 __syncthreads();
                 buf ^= 1;
                 const int next = cb + 1 < p.cblocks ? cb + 1 : p.cblocks - 1;
                 window_load(next);
             }
-            toff = buf * win_bytes + kr * p.tap_row + kc * p.tap_col;
-            b_read(b0, toff);                            // first half of the next K-step
-            static_for<0, FM>([&](auto ic) {
-                constexpr int i = decltype(ic)::value;
-                static_for<0, NT>([&](auto jc) {
-                    constexpr int j = decltype(jc)::value;
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[u][i * 2 + 1], b1[j], acc[i][j], 0, 0, 0);
-                });
+        }
+        toff = buf * win_bytes + kr * p.tap_row + kc * p.tap_col;
+        b_read(b0, toff);                            // first half of the next K-step
+        static_for<0, FM>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            static_for<0, NT>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[u][i * 2 + 1], b1[j], acc[i][j], 0, 0, 0);
             });
         });
-    }
+    };
+    // whole rounds of the ring, then the K-steps left over: their weights are in the ring already (the steps
+    // ahead of the last round), and the zero steps that pad the packed weights to a whole round are not multiplied
+    while (ks + RING <= p.ksteps) static_for<0, RING>([&](auto uc) { k_step(uc, std::true_type{}); });
+    const int left = p.ksteps - ks;
+    static_for<0, RING - 1>([&](auto uc) {
+        if (decltype(uc)::value < left) k_step(uc, std::false_type{});
+    });
 
     if (p.stamps) {
         // wait for the MFMAs still in flight: the stamp marks the end of the multiplication, not its last issue
