@@ -127,6 +127,7 @@ int fl_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t 
     p.wr = pl.fl_wr;
     p.rowp = pl.fl_rowp;
     p.ksteps_p = pl.ksteps_p;
+    p.ksteps = g.cblocks * g.kh * g.kw;
     p.tap_row = g.dil_h * pl.fl_rowp;
     p.tap_col = g.dil_w * FL_PIX;
     p.tiles = int(pl.fl_tiles);

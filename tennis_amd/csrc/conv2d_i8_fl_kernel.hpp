@@ -24,6 +24,7 @@ struct FlParams : EpiParams {
     int wc, wpix;           // window columns, window pixels
     int wr, rowp;           // window rows; LDS bytes per window row (>= wc * FL_PIX, see fl_plan)
     int ksteps_p;
+    int ksteps;             // K-steps that hold weights (ksteps_p: padded to the A-ring size with zero steps)
     int tap_row, tap_col;   // bytes into the window per kernel row / column
     int tiles, tiles_per_xcd;
     int positions;          // n * ho * wo
@@ -150,7 +151,7 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
     v4i areg[FL_RING][2];
     auto a_load = [&](auto slot, int ks) __attribute__((always_inline)) {
         constexpr int s = decltype(slot)::value;
-        if (ks >= p.ksteps_p) ks = p.ksteps_p - 1;
+        if (ks >= p.ksteps) ks = p.ksteps - 1;   // beyond the last K-step: its lines again, never used
         const int so = a_frag + ks * a_kstride;
         areg[s][0] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_lane, so, 0));
         areg[s][1] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_lane, so + 1024, 0));
@@ -181,7 +182,7 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
     }
     window_store(0);
     __syncthreads();
-    if (!RESIDENT) window_load(p.cblocks > 1 ? 1 : 0);   // block cb+1, in flight during block cb's taps
+    if (!RESIDENT && p.cblocks > 1) window_load(1);   // block cb+1, in flight during block cb's taps
 
     v4i b0[NT], b1[NT];
     auto b_read = [&](v4i(&dst)[NT], int off) __attribute__((always_inline)) {
@@ -194,58 +195,67 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
     b_read(b0, toff);
     stamp(1);
 
-    for (int ks0 = 0; ks0 < p.ksteps_p; ks0 += FL_RING) {
-        static_for<0, FL_RING>([&](auto uc) {
-            constexpr int u = decltype(uc)::value;
-            a_load(std::integral_constant<int, (u + FL_RING - 1) % FL_RING>{}, ks0 + u + FL_RING - 1);
-            b_read(b1, toff + 32);                       // second half of this K-step
-            static_for<0, NT>([&](auto jc) {
-                constexpr int j = decltype(jc)::value;
-                acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[u][0], b0[j], acc[j], 0, 0, 0);
-            });
-            ++tap;
-            if (++kc == p.kw) {
-                kc = 0;
-                ++kr;
-            }
-            if (tap == taps) {
-                tap = 0;
-                kr = 0;
-                kc = 0;
-                ++cb;
-                if (RESIDENT) {
-                    if (cb == 1 && p.cblocks > 1) {
-                        static_for<0, 3>([&](auto bc) {
-                            constexpr int b = decltype(bc)::value;
-                            const int c = 1 + b < p.cblocks ? 1 + b : p.cblocks - 1;
-                            static_for<0, FL_MAX_FILL>([&](auto ic) {
-                                constexpr int i = decltype(ic)::value;
-                                if (i < n_fill) *reinterpret_cast<v4i *>(&lds[c * win_bytes + fill_dst[i]]) = wbat[b][i];
-                            });
-                        });
-                        for (int c = 4; c < p.cblocks; ++c) {   // more than four blocks: the rest, one round trip each
-                            window_load(c);
-                            window_store(c);
-                        }
-                        __syncthreads();
-                    }
-                    buf = cb < p.cblocks ? cb : p.cblocks - 1;   // K-steps of the ring padding re-read the last block
-                } else {
-                    window_store(buf ^ 1);
-                    __syncthreads();
-                    buf ^= 1;
-                    const int next = cb + 1 < p.cblocks ? cb + 1 : p.cblocks - 1;
-                    window_load(next);
-                }
-            }
-            toff = buf * win_bytes + kr * p.tap_row + kc * p.tap_col;
-            b_read(b0, toff);                            // first half of the next K-step
-            static_for<0, NT>([&](auto jc) {
-                constexpr int j = decltype(jc)::value;
-                acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[u][1], b1[j], acc[j], 0, 0, 0);
-            });
+    // One K-step: both halves' MFMAs, the B reads one half-step ahead, the window change on a channel-block
+    // boundary.  PREFETCH: also load the weights of the K-step FL_RING-1 ahead into the slot the previous step freed.
+    int ks = 0;
+    auto k_step = [&](auto uc, auto prefetch) __attribute__((always_inline)) {
+        constexpr int u = decltype(uc)::value;
+        if (decltype(prefetch)::value) a_load(std::integral_constant<int, (u + FL_RING - 1) % FL_RING>{}, ks + FL_RING - 1);
+        b_read(b1, toff + 32);                       // second half of this K-step
+        static_for<0, NT>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[u][0], b0[j], acc[j], 0, 0, 0);
         });
-    }
+        ++ks;
+        ++tap;
+        if (++kc == p.kw) {
+            kc = 0;
+            ++kr;
+        }
+        if (tap == taps) {
+            tap = 0;
+            kr = 0;
+            kc = 0;
+            ++cb;
+            if (RESIDENT) {
+                if (cb == 1 && p.cblocks > 1) {
+                    static_for<0, 3>([&](auto bc) {
+                        constexpr int b = decltype(bc)::value;
+                        const int c = 1 + b < p.cblocks ? 1 + b : p.cblocks - 1;
+                        static_for<0, FL_MAX_FILL>([&](auto ic) {
+                            constexpr int i = decltype(ic)::value;
+                            if (i < n_fill) *reinterpret_cast<v4i *>(&lds[c * win_bytes + fill_dst[i]]) = wbat[b][i];
+                        });
+                    });
+                    for (int c = 4; c < p.cblocks; ++c) {   // more than four blocks: the rest, one round trip each
+                        window_load(c);
+                        window_store(c);
+                    }
+                    __syncthreads();
+                }
+                buf = cb < p.cblocks ? cb : p.cblocks - 1;   // the read ahead behind the last K-step stays in the last block
+            } else if (ks < p.ksteps) {                      // no window change behind the last K-step
+                window_store(buf ^ 1);
+                __syncthreads();
+                buf ^= 1;
+                const int next = cb + 1 < p.cblocks ? cb + 1 : p.cblocks - 1;
+                window_load(next);
+            }
+        }
+        toff = buf * win_bytes + kr * p.tap_row + kc * p.tap_col;
+        b_read(b0, toff);                            // first half of the next K-step
+        static_for<0, NT>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[u][1], b1[j], acc[j], 0, 0, 0);
+        });
+    };
+    // whole rounds of the ring, then the K-steps left over: their weights are in the ring already (the steps
+    // ahead of the last round), and the zero steps that pad the packed weights to a whole round are not multiplied
+    while (ks + FL_RING <= p.ksteps) static_for<0, FL_RING>([&](auto uc) { k_step(uc, std::true_type{}); });
+    const int left = p.ksteps - ks;
+    static_for<0, FL_RING - 1>([&](auto uc) {
+        if (decltype(uc)::value < left) k_step(uc, std::false_type{});
+    });
 
     if (p.stamps) {
         // the accumulators are written by the MFMAs still in flight: wait for them, so that the stamp marks the end
