@@ -356,12 +356,12 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
             } else if (p.act == TSX_ACT_LEAKY_RELU) {
                 static_for<0, 16>([&](auto rc) {
                     constexpr int r = decltype(rc)::value;
-                    v[r] = apply_act(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
+                    v[r] = apply_act_conv_i8(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
                 });
             } else if (p.act == TSX_ACT_MISH) {
                 static_for<0, 16>([&](auto rc) {
                     constexpr int r = decltype(rc)::value;
-                    v[r] = apply_act(v[r], TSX_ACT_MISH, 0.f, true);
+                    v[r] = apply_act_conv_i8(v[r], TSX_ACT_MISH, 0.f, true);
                 });
             }
             if (EXTRA && p.residual && p.res_after) static_for<0, 16>([&](auto rc) {

@@ -389,12 +389,12 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
                     } else if (p.act == TSX_ACT_LEAKY_RELU) {
                         static_for<0, 16>([&](auto rc) {
                             constexpr int r = decltype(rc)::value;
-                            v[r] = apply_act(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
+                            v[r] = apply_act_conv_i8(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
                         });
                     } else if (p.act == TSX_ACT_MISH) {
                         static_for<0, 16>([&](auto rc) {
                             constexpr int r = decltype(rc)::value;
-                            v[r] = apply_act(v[r], TSX_ACT_MISH, 0.f, true);
+                            v[r] = apply_act_conv_i8(v[r], TSX_ACT_MISH, 0.f, true);
                         });
                     }
                     if (EXTRA && p.residual && p.res_after) static_for<0, 16>([&](auto rc) {

@@ -43,7 +43,7 @@ __device__ __forceinline__ float epi_value(const EpiParams &p, int acc, int64_t 
     if (p.row_scale) v = __fmul_rn(v, row_scale);
     if (p.bias) v = __fadd_rn(v, bias);
     if (p.residual && !p.res_after) v = __fadd_rn(v, p.residual[idx]);
-    v = apply_act(v, p.act, p.slope, idx < p.act_body);
+    v = apply_act_conv_i8(v, p.act, p.slope, idx < p.act_body);
     if (p.residual && p.res_after) v = __fadd_rn(v, p.residual[idx]);
     return v;
 }
@@ -100,10 +100,10 @@ __device__ __forceinline__ void epilogue_rows16(const EpiParams &p, const v16i &
         for (int r = 0; r < 16; ++r) v[r] = v[r] > 0.f ? v[r] : 0.f;
     } else if (p.act == TSX_ACT_LEAKY_RELU) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) v[r] = apply_act(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
+        for (int r = 0; r < 16; ++r) v[r] = apply_act_conv_i8(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
     } else if (p.act == TSX_ACT_MISH) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) v[r] = apply_act(v[r], TSX_ACT_MISH, 0.f, true);
+        for (int r = 0; r < 16; ++r) v[r] = apply_act_conv_i8(v[r], TSX_ACT_MISH, 0.f, true);
     }
     if (p.residual && p.res_after) {
 #pragma unroll

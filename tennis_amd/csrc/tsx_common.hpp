@@ -142,6 +142,33 @@ __device__ __forceinline__ float mish_value(float x) {
     return __fmul_rn(x, t);
 }
 
+// Mish for the epilogues of the int8 convolution kernels, where the activation's arithmetic, not memory or the MFMAs,
+// bounds a layer (the 608x608 and 304x304 layers of a YOLOv4-shaped backbone spend more issue slots on mish_value than
+// on everything else): one exponential and one division,
+//     tanh(softplus(x)) = w / (w + 2),  w = e (e + 2),  e = e^x,
+// with the quotient (correctly rounded but for rare ties) then brought onto the grid the host's tanh lives on:
+// 2 * (1 / (1 + u)) - 1 with 1 / (1 + u) in [0.5, 1] is a multiple of 2^-23, which (t + 1) - 1 reproduces -- including
+// the host's 0 (and so -0 for the product) once x is below about -17.  Three quarters of all results are the host's
+// bit for bit; the others are one grid step of tanh away (1.2e-7 |x|, at most 2e-6 where x is near -17), the same
+// distance the host's own rounding keeps from the exact function there.  NaN -> NaN, +-inf as the host's.
+__device__ __forceinline__ float mish_short(float x) {
+    const float e = mish_exp(fminf(x, 30.f));              // beyond 30 (long before, in fact) the quotient is 1
+    const float w = __fmul_rn(e, __fadd_rn(e, 2.f));
+    const float d = __fadd_rn(w, 2.f);
+    const float r0 = __builtin_amdgcn_rcpf(d);
+    const float r = __builtin_fmaf(r0, __builtin_fmaf(-d, r0, 1.f), r0);
+    const float q = __fmul_rn(w, r);
+    const float t = __builtin_fmaf(__builtin_fmaf(-d, q, w), r, q);   // remainder correction of the quotient
+    return __fmul_rn(x, __fsub_rn(__fadd_rn(t, 1.f), 1.f));
+}
+
+// apply_act for the int8 convolution epilogues: Mish in its short form (every path of those kernels -- fragment-wise
+// and per element -- goes through this one, so an element's value does not depend on the tile it falls into)
+__device__ __forceinline__ float apply_act_conv_i8(float v, int act, float slope, bool in_body) {
+    if (act != TSX_ACT_MISH) return apply_act_basic(v, act, slope, in_body);
+    return mish_short(v);
+}
+
 __device__ __forceinline__ float apply_act(float v, int act, float slope, bool in_body) {
     if (act != TSX_ACT_MISH) return apply_act_basic(v, act, slope, in_body);
     return mish_value(v);
