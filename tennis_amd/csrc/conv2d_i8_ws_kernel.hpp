@@ -12,6 +12,7 @@ constexpr int PIX = 80;         // LDS bytes per window pixel (64 + 16 pad) when
 constexpr int WS_THREADS = 256;
 constexpr int WS_FM = 1;        // 32-cout fragments per wavefront
 constexpr int MAX_FILL = 7;     // window chunks per thread per channel block
+constexpr int SMALL_FILL = 4;   // ... of the kernels compiled for small windows (fewer registers: one more workgroup per CU)
 constexpr int MAX_WP = MAX_FILL * WS_THREADS / 4;   // 448 window pixels
 
 struct WsParams : EpiParams {
@@ -67,7 +68,11 @@ namespace {
 // [position][cout] row-major, and row_scale[position] multiplies behind dq (the per-row activation scale of a
 // quantized inner product).  A lane's accumulators 4g..4g+3 are 4 consecutive channels of its position, so
 // the fp32 output goes out as 16-byte stores; lanes l and l+32 and the four g complete a 128-byte line.
-template <int NT, int FM, bool EXTRA, bool STREAM, bool ROWM>
+//
+// FILL = chunks of 16 window bytes a thread copies per channel block (MAX_FILL, or SMALL_FILL for windows that need
+// no more: with up to 2 fragments the kernel then fits four wavefronts per SIMD, and the layers bound by their
+// epilogue's memory latency -- the residual joins on large maps -- keep a fourth workgroup in flight per CU).
+template <int NT, int FM, bool EXTRA, bool STREAM, bool ROWM, int FILL>
 __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <= 4 ? 2 : 1))) void conv_i8_ws_kernel(WsParams p_in) {
     WsParams p = p_in;
     if (!EXTRA) {
@@ -104,16 +109,16 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
     // ---- window fill bookkeeping: chunk q = tid + i*256 -> pixel q / chunks-per-pixel, 16-byte chunk q % ...
     // A uniform 64-bit base (the window's first staged row and column) plus one 32-bit byte offset per chunk: the
     // loads then take the base from scalar registers and need no address arithmetic of their own.
-    const int n_fill = ((p.wpix << p.chunk_shift) + WS_THREADS - 1) / WS_THREADS;   // <= MAX_FILL, uniform
+    const int n_fill = ((p.wpix << p.chunk_shift) + WS_THREADS - 1) / WS_THREADS;   // <= FILL, uniform
     // window row r is staged row (img * hs + th0 * stride) + r of the batch-wide staged row sequence
     const int64_t row_base = int64_t(img) * p.hs + th0 * p.sh;
     const int col_base = col0 * p.sw;
     const int row_last = int(min(int64_t(p.n) * p.hs - 1 - row_base, int64_t(1) << 20));   // last tile: rows no stored output uses
     const int col_last = p.ws - 1 - col_base;                                               // last column tile: likewise
     const int8_t *xs_base = p.xs + (row_base * p.ws + col_base) * p.cp;
-    unsigned fill_off[MAX_FILL];
-    int fill_dst[MAX_FILL];
-    static_for<0, MAX_FILL>([&](auto ic) {
+    unsigned fill_off[FILL];
+    int fill_dst[FILL];
+    static_for<0, FILL>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
         fill_off[i] = 0;
         fill_dst[i] = 0;
@@ -129,11 +134,11 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
             fill_dst[i] = __mul24(pix, p.pix) + chunk * 16;
         }
     });
-    v4i wreg[MAX_FILL];   // native vectors: arrays of HIP's uint4 struct do not stay in registers
+    v4i wreg[FILL];   // native vectors: arrays of HIP's uint4 struct do not stay in registers
 
     auto window_load = [&](int cb) __attribute__((always_inline)) {
         const int8_t *base = xs_base + cb * p.stage_bytes;
-        static_for<0, MAX_FILL>([&](auto ic) {
+        static_for<0, FILL>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
             if (i < n_fill) {
                 // the empty statement keeps the offset's widening next to the load, where instruction selection
@@ -145,7 +150,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
         });
     };
     auto window_store = [&](int buf) __attribute__((always_inline)) {
-        static_for<0, MAX_FILL>([&](auto ic) {
+        static_for<0, FILL>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
             if (i < n_fill) *reinterpret_cast<v4i *>(&lds[buf * win_bytes + fill_dst[i]]) = wreg[i];
         });
@@ -496,14 +501,22 @@ int ws_launch_nt<TSX_WS_NT>(const WsParams &p, dim3 grid, size_t lds_bytes, hipS
     constexpr int NT = TSX_WS_NT;
     // ROWM: the GEMM form of the epilogue; EXTRA: residual input and/or staged int8 output; STREAM: a large
     // fp32 output nothing reads back soon
-    if (p.rowmajor)
-        hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, false, false, true>), grid, dim3(WS_THREADS), lds_bytes, stream, p);
-    else if (p.residual || p.st_out)
-        hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, true, false, false>), grid, dim3(WS_THREADS), lds_bytes, stream, p);
-    else if (p.stream_out)
-        hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, false, true, false>), grid, dim3(WS_THREADS), lds_bytes, stream, p);
-    else
-        hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, false, false, false>), grid, dim3(WS_THREADS), lds_bytes, stream, p);
+    // small windows of small tiles: the variant with fewer fill registers
+    const bool small_fill = NT <= 2 && ((p.wpix << p.chunk_shift) + WS_THREADS - 1) / WS_THREADS <= SMALL_FILL;
+#define TSX_WS_LAUNCH(EXTRA, STREAM, ROWM)                                                                             \
+    do {                                                                                                               \
+        if (NT <= 2 && small_fill)                                                                                     \
+            hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, EXTRA, STREAM, ROWM, (NT <= 2 ? SMALL_FILL : MAX_FILL)>), grid, \
+                               dim3(WS_THREADS), lds_bytes, stream, p);                                               \
+        else                                                                                                           \
+            hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, EXTRA, STREAM, ROWM, MAX_FILL>), grid, dim3(WS_THREADS),  \
+                               lds_bytes, stream, p);                                                                  \
+    } while (0)
+    if (p.rowmajor) TSX_WS_LAUNCH(false, false, true);
+    else if (p.residual || p.st_out) TSX_WS_LAUNCH(true, false, false);
+    else if (p.stream_out) TSX_WS_LAUNCH(false, true, false);
+    else TSX_WS_LAUNCH(false, false, false);
+#undef TSX_WS_LAUNCH
     TSX_LAUNCH_CHECK("conv_i8_ws_kernel");
     return 0;
 }
