@@ -341,7 +341,16 @@ class YoloV4Int8:
                     self._shapes[i] = tuple(outs[i].shape)
             elif t == "maxpool":
                 k = l["size"]
-                outs[i] = capi.pooling2d(outs[rsrcs[i][0]], "max", (k, k), (1, 1), (k // 2,) * 4)
+                # An SPP block pools one map with growing odd windows at stride 1: the k x k maximum is the
+                # (k - k' + 1)-maximum of the k' x k' maxima already computed (windows clipped to the map on both
+                # levels; equal for finite values -- a tie between +0 and -0 may keep the other sign), so 9 and 13
+                # cost a 5 x 5 pass each instead of 81 and 169 elements per output.
+                src, kk = outs[rsrcs[i][0]], k
+                for m in range(i):
+                    if (L[m]["type"] == "maxpool" and rsrcs[m][0] == rsrcs[i][0] and outs[m] is not None
+                            and L[m]["size"] % 2 == 1 and k % 2 == 1 and L[m]["size"] < k and k - L[m]["size"] + 1 <= kk):
+                        src, kk = outs[m], k - L[m]["size"] + 1
+                outs[i] = capi.pooling2d(src, "max", (kk, kk), (1, 1), (kk // 2,) * 4)
                 self._shapes[i] = tuple(outs[i].shape)
             elif t == "upsample":
                 src = outs[rsrcs[i][0]]
