@@ -72,7 +72,12 @@ namespace {
 // FILL = chunks of 16 window bytes a thread copies per channel block (MAX_FILL, or SMALL_FILL for windows that need
 // no more: with up to 2 fragments the kernel then fits four wavefronts per SIMD, and the layers bound by their
 // epilogue's memory latency -- the residual joins on large maps -- keep a fourth workgroup in flight per CU).
-template <int NT, int FM, bool EXTRA, bool STREAM, bool ROWM, int FILL>
+//
+// LOOK: the B operands go through a register ring as deep as the weights', read RING - 1 K-steps ahead of their
+// MFMAs.  A wavefront with one fragment spends 2 MFMAs (64 cycles) on a K-step, half of an LDS read's latency: read
+// one half-step ahead (the other form), the small maps at the end of a network -- under one wavefront per SIMD,
+// nothing else to issue -- ran at one K-step per two LDS latencies.
+template <int NT, int FM, bool EXTRA, bool STREAM, bool ROWM, int FILL, bool LOOK>
 __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <= 4 ? 2 : 1))) void conv_i8_ws_kernel(WsParams p_in) {
     WsParams p = p_in;
     if (!EXTRA) {
@@ -222,73 +227,133 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
 
     window_store(0);
     __syncthreads();
-    int cb = 0, tap = 0, kr = 0, kc = 0, buf = 0;
+    int cb = 0, tap = 0, kc = 0, buf = 0;
+    int cb_ks = 0;   // K-steps the B read pointer has passed (LOOK)
+    // byte offset of the current tap in the LDS windows (buffer + kernel row and column), stepped with the taps: a
+    // column on, or to the first column of the next kernel row
+    int toff = 0;
+    const int row_step = p.tap_row - (p.kw - 1) * p.tap_col;
     if (p.cblocks > 1) window_load(1);   // block cb+1, in flight during block cb's taps
 
-    // B fragments are read one half-step ahead of the MFMAs that use them (one wavefront per
-    // SIMD: nothing else hides the LDS latency).
-    v4i b0[NT], b1[NT];
     auto b_read = [&](v4i(&dst)[NT], int off) __attribute__((always_inline)) {
         static_for<0, NT>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
             dst[j] = *reinterpret_cast<const v4i *>(&lds[b_base[j] + off]);
         });
     };
-    int toff = 0;   // buf * win_bytes + tap shift
-    b_read(b0, toff);
-    stamp(1);
-
-    // One K-step: both halves' MFMAs, the B reads one half-step ahead, the window swap on a channel-block boundary.
-    // PREFETCH: also load the weights of the K-step RING-1 ahead into the ring slot the previous step freed.
     int ks = 0;
-    auto k_step = [&](auto uc, auto prefetch) __attribute__((always_inline)) {
-        constexpr int u = decltype(uc)::value;
-        if (decltype(prefetch)::value) a_load(std::integral_constant<int, (u + RING - 1) % RING>{}, ks + RING - 1);
-        b_read(b1, toff + 32);                       // second half of this K-step
-        static_for<0, FM>([&](auto ic) {
-            constexpr int i = decltype(ic)::value;
-            static_for<0, NT>([&](auto jc) {
-                constexpr int j = decltype(jc)::value;
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[u][i * 2], b0[j], acc[i][j], 0, 0, 0);
-            });
-        });
-        // advance (cb, tap); on a channel-block boundary swap in the next window (none behind the last K-step)
-        ++ks;
-        ++tap;
-        if (++kc == p.kw) {
-            kc = 0;
-            ++kr;
-        }
-        if (tap == taps) {
-            tap = 0;
-            kr = 0;
-            kc = 0;
-            ++cb;
-            if (ks < p.ksteps) {
-                window_store(buf ^ 1);
-                __syncthreads();
-                buf ^= 1;
-                const int next = cb + 1 < p.cblocks ? cb + 1 : p.cblocks - 1;
-                window_load(next);
+    if constexpr (LOOK) {
+        // ---- K-loop with the B ring: slot u holds both halves of K-step (round start + u).  The read pointer runs
+        // RING - 1 K-steps ahead of the MFMAs and is the one that swaps the windows when it enters a channel block.
+        v4i bq[RING][2][NT];
+        auto b_ahead = [&](auto slot) __attribute__((always_inline)) {
+            constexpr int sl = decltype(slot)::value;
+            b_read(bq[sl][0], toff);
+            b_read(bq[sl][1], toff + 32);
+            ++cb_ks;
+            ++tap;
+            if (++kc == p.kw) {
+                kc = 0;
+                toff += row_step;
+            } else {
+                toff += p.tap_col;
             }
-        }
-        toff = buf * win_bytes + kr * p.tap_row + kc * p.tap_col;
-        b_read(b0, toff);                            // first half of the next K-step
-        static_for<0, FM>([&](auto ic) {
-            constexpr int i = decltype(ic)::value;
-            static_for<0, NT>([&](auto jc) {
-                constexpr int j = decltype(jc)::value;
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[u][i * 2 + 1], b1[j], acc[i][j], 0, 0, 0);
+            if (tap == taps) {
+                tap = 0;
+                kc = 0;
+                ++cb;
+                if (cb_ks < p.ksteps) {      // no window swap behind the last K-step (reads beyond it stay where they are)
+                    window_store(buf ^ 1);
+                    __syncthreads();
+                    buf ^= 1;
+                    const int next = cb + 1 < p.cblocks ? cb + 1 : p.cblocks - 1;
+                    window_load(next);
+                }
+                toff = buf * win_bytes;
+            }
+        };
+        static_for<0, RING - 1>([&](auto sc) { b_ahead(sc); });
+        stamp(1);
+        auto k_step = [&](auto uc, auto prefetch) __attribute__((always_inline)) {
+            constexpr int u = decltype(uc)::value;
+            if (decltype(prefetch)::value) a_load(std::integral_constant<int, (u + RING - 1) % RING>{}, ks + RING - 1);
+            b_ahead(std::integral_constant<int, (u + RING - 1) % RING>{});
+            static_for<0, 2>([&](auto hc) {
+                constexpr int h = decltype(hc)::value;
+                static_for<0, FM>([&](auto ic) {
+                    constexpr int i = decltype(ic)::value;
+                    static_for<0, NT>([&](auto jc) {
+                        constexpr int j = decltype(jc)::value;
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[u][i * 2 + h], bq[u][h][j], acc[i][j], 0, 0, 0);
+                    });
+                });
             });
+            ++ks;
+        };
+        while (ks + RING <= p.ksteps) static_for<0, RING>([&](auto uc) { k_step(uc, std::true_type{}); });
+        const int left = p.ksteps - ks;
+        static_for<0, RING - 1>([&](auto uc) {
+            if (decltype(uc)::value < left) k_step(uc, std::false_type{});
         });
-    };
-    // whole rounds of the ring, then the K-steps left over: their weights are in the ring already (the steps
-    // ahead of the last round), and the zero steps that pad the packed weights to a whole round are not multiplied
-    while (ks + RING <= p.ksteps) static_for<0, RING>([&](auto uc) { k_step(uc, std::true_type{}); });
-    const int left = p.ksteps - ks;
-    static_for<0, RING - 1>([&](auto uc) {
-        if (decltype(uc)::value < left) k_step(uc, std::false_type{});
-    });
+    } else {
+        // B fragments are read one half-step ahead of the MFMAs that use them (one wavefront per
+        // SIMD: nothing else hides the LDS latency).
+        v4i b0[NT], b1[NT];
+        b_read(b0, toff);
+        stamp(1);
+
+        // One K-step: both halves' MFMAs, the B reads one half-step ahead, the window swap on a channel-block boundary.
+        // PREFETCH: also load the weights of the K-step RING-1 ahead into the ring slot the previous step freed.
+        auto k_step = [&](auto uc, auto prefetch) __attribute__((always_inline)) {
+            constexpr int u = decltype(uc)::value;
+            if (decltype(prefetch)::value) a_load(std::integral_constant<int, (u + RING - 1) % RING>{}, ks + RING - 1);
+            b_read(b1, toff + 32);                       // second half of this K-step
+            static_for<0, FM>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                static_for<0, NT>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value;
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[u][i * 2], b0[j], acc[i][j], 0, 0, 0);
+                });
+            });
+            // advance (cb, tap); on a channel-block boundary swap in the next window (none behind the last K-step)
+            ++ks;
+            ++tap;
+            if (++kc == p.kw) {
+                kc = 0;
+                toff += row_step;
+            } else {
+                toff += p.tap_col;
+            }
+            if (tap == taps) {
+                tap = 0;
+                kc = 0;
+                ++cb;
+                if (ks < p.ksteps) {
+                    window_store(buf ^ 1);
+                    __syncthreads();
+                    buf ^= 1;
+                    const int next = cb + 1 < p.cblocks ? cb + 1 : p.cblocks - 1;
+                    window_load(next);
+                }
+                toff = buf * win_bytes;
+            }
+            b_read(b0, toff);                            // first half of the next K-step
+            static_for<0, FM>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                static_for<0, NT>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value;
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[u][i * 2 + 1], b1[j], acc[i][j], 0, 0, 0);
+                });
+            });
+        };
+        // whole rounds of the ring, then the K-steps left over: their weights are in the ring already (the steps
+        // ahead of the last round), and the zero steps that pad the packed weights to a whole round are not multiplied
+        while (ks + RING <= p.ksteps) static_for<0, RING>([&](auto uc) { k_step(uc, std::true_type{}); });
+        const int left = p.ksteps - ks;
+        static_for<0, RING - 1>([&](auto uc) {
+            if (decltype(uc)::value < left) k_step(uc, std::false_type{});
+        });
+    }
 
     if (p.stamps) {
         // wait for the MFMAs still in flight: the stamp marks the end of the multiplication, not its last issue
@@ -503,14 +568,21 @@ int ws_launch_nt<TSX_WS_NT>(const WsParams &p, dim3 grid, size_t lds_bytes, hipS
     // fp32 output nothing reads back soon
     // small windows of small tiles: the variant with fewer fill registers
     const bool small_fill = NT <= 2 && ((p.wpix << p.chunk_shift) + WS_THREADS - 1) / WS_THREADS <= SMALL_FILL;
+    // one fragment per wavefront, a K of two rounds or more, and few enough workgroups that a SIMD holds one or
+    // two wavefronts: the B ring (more registers: three workgroups per CU)
+    const bool look = NT == 1 && small_fill && p.ksteps >= 2 * RING && int64_t(grid.x) * grid.y <= 1024;
 #define TSX_WS_LAUNCH(EXTRA, STREAM, ROWM)                                                                             \
     do {                                                                                                               \
-        if (NT <= 2 && small_fill)                                                                                     \
-            hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, EXTRA, STREAM, ROWM, (NT <= 2 ? SMALL_FILL : MAX_FILL)>), grid, \
-                               dim3(WS_THREADS), lds_bytes, stream, p);                                               \
-        else                                                                                                           \
-            hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, EXTRA, STREAM, ROWM, MAX_FILL>), grid, dim3(WS_THREADS),  \
+        constexpr int F = NT <= 2 ? SMALL_FILL : MAX_FILL;                                                             \
+        if (NT == 1 && look)                                                                                           \
+            hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, EXTRA, STREAM, ROWM, F, NT == 1>), grid, dim3(WS_THREADS), \
                                lds_bytes, stream, p);                                                                  \
+        else if (NT <= 2 && small_fill)                                                                                \
+            hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, EXTRA, STREAM, ROWM, F, false>), grid, dim3(WS_THREADS),  \
+                               lds_bytes, stream, p);                                                                  \
+        else                                                                                                           \
+            hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, EXTRA, STREAM, ROWM, MAX_FILL, false>), grid,             \
+                               dim3(WS_THREADS), lds_bytes, stream, p);                                                \
     } while (0)
     if (p.rowmajor) TSX_WS_LAUNCH(false, false, true);
     else if (p.residual || p.st_out) TSX_WS_LAUNCH(true, false, false);
