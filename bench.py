@@ -34,7 +34,7 @@ CFG = dict(n=32, c=256, h=28, w=28, cout=256, k=3, pad=1)
 
 # HBM bytes per launch of the two kernels on this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a
 # known-size copy (profiles/conv2d_i8_config2_hbm_traffic.txt); a profiler figure, not measured by this script.
-TRAFFIC_CONV_BYTES = 43.93e6
+TRAFFIC_CONV_BYTES = 43.97e6
 TRAFFIC_STAGE_BYTES = 33.15e6
 
 
