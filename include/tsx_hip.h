@@ -105,6 +105,11 @@ typedef struct tsx_epilogue {
     int8_t *staged_out_dev;
     int32_t staged_hs, staged_ws, staged_cp, staged_pad_top, staged_pad_left;
     int32_t residual_after_act; /* 0: act(y + residual); 1: act(y) + residual */
+    /* 0 or 1: output pixel (oh, ow) goes to staged pixel (oh, ow) as described above.  2: a nearest-neighbour
+     * resize by 2 (cpu::Resize2D NEAREST at an integer factor, src/kernels/cpu/resize2d.cpp:186-215) is folded in:
+     * the pixel is written to the four staged pixels (2 oh + dy, 2 ow + dx), so that a convolution -> upsample ->
+     * (concatenation ->) convolution chain needs no fp32 tensor in between. */
+    int32_t staged_upsample;
 } tsx_epilogue;
 
 /* ---------------------------------------------------------------- quantize

@@ -34,7 +34,7 @@ class Epilogue(ctypes.Structure):
     _fields_ = [("dq_dev", _vp), ("row_scale_dev", _vp), ("bias_dev", _vp), ("act", _i32), ("slope", _f32),
                 ("q_scales_dev", _vp), ("n_qscales", _i32), ("residual_dev", _vp), ("staged_out_dev", _vp),
                 ("staged_hs", _i32), ("staged_ws", _i32), ("staged_cp", _i32), ("staged_pad_top", _i32),
-                ("staged_pad_left", _i32), ("residual_after_act", _i32)]
+                ("staged_pad_left", _i32), ("residual_after_act", _i32), ("staged_upsample", _i32)]
 
 
 class TsxError(RuntimeError):
@@ -191,6 +191,7 @@ class _EpilogueArgs:
             self.c.staged_out_dev = staged_out.buf.data_ptr()
             self.c.staged_hs, self.c.staged_ws, self.c.staged_cp = staged_out.hs, staged_out.ws, staged_out.cp
             self.c.staged_pad_top, self.c.staged_pad_left = staged_out.pad_top, staged_out.pad_left
+            self.c.staged_upsample = int(getattr(staged_out, "upsample", 1))
 
 
 class StagedInput:
@@ -229,10 +230,15 @@ class StagedSlice:
     input (quantized with the consumer's scale, which was calibrated on the concatenated tensor), so the concatenated
     tensor never exists in fp32 and is never staged.  c0 must be a multiple of 16 (the epilogue stores 16 bytes)."""
 
-    def __init__(self, staged, c0, channels):
+    def __init__(self, staged, c0, channels, upsample=1):
+        """upsample = 2: the producer's map is half the staged one's size and every pixel is written to the 2 x 2
+        staged pixels it becomes under a nearest-neighbour resize (the epilogue's staged_upsample)."""
         n, c, h, w = staged.x_shape
         if c0 % 16 != 0 or c0 < 0 or c0 + channels > c:
             raise TsxError("channels [%d, %d) are not a 16-aligned run inside the %d of the staged tensor" % (c0, c0 + channels, c))
+        if upsample not in (1, 2) or h % upsample or w % upsample:
+            raise TsxError("staged slice: upsample %r does not fit a %dx%d map" % (upsample, h, w))
+        self.upsample = upsample
         self.x_shape = (n, channels, h, w)
         self.hs, self.ws, self.cp = staged.hs, staged.ws, staged.cp
         self.pad_top, self.pad_left = staged.pad_top, staged.pad_left
@@ -248,6 +254,12 @@ def staged_interior(staged, images):
     buf = getattr(staged, "full_buf", staged.buf)
     t = buf[: n * staged.hs * staged.ws * staged.cp].view(n, staged.hs, staged.ws, staged.cp)
     t = t[list(images), staged.pad_top:staged.pad_top + h, staged.pad_left:staged.pad_left + w, c0:c0 + c]
+    if getattr(staged, "upsample", 1) == 2:
+        # the producer wrote every pixel four times: its own map is any of the four phases, and they must agree
+        phases = [t[:, dy::2, dx::2] for dy in (0, 1) for dx in (0, 1)]
+        if not all(torch.equal(phases[0], ph) for ph in phases[1:]):
+            raise TsxError("staged slice: the 2 x 2 pixels of an upsampled hand-over differ")
+        t = phases[0]
     return t.permute(0, 3, 1, 2).contiguous()
 
 

@@ -811,7 +811,8 @@ __global__ __launch_bounds__(WGM *WGN * 64) void igemm_i8_kernel(GemmParams p) {
                         if (p.st_out) {
                             const int rem = pos - n * p.howo;
                             const int oh = rem / p.wo, ow = rem - oh * p.wo;
-                            st_dst = p.st_out + ((int64_t(n) * p.st_hs + oh + p.st_pt) * p.st_ws + ow + p.st_pl) * p.st_cp + co0;
+                            const int up = p.st_up == 2 ? 2 : 1;
+                            st_dst = p.st_out + ((int64_t(n) * p.st_hs + up * oh + p.st_pt) * p.st_ws + up * ow + p.st_pl) * p.st_cp + co0;
                         }
                         const float qs = want_q ? p.q_scales[p.n_qscales == 1 ? 0 : n] : 0.f;
                         tsx::epilogue_rows16(p, acc[i][j], dq, bias, base[j] + int64_t(co0) * p.howo, p.howo, qs,
@@ -998,8 +999,10 @@ int check_epilogue(const tsx_epilogue *ep, const float *out_f32, const int8_t *o
         TSX_REQUIRE(cout > 0, "staged output is a convolution-only epilogue term");
         TSX_REQUIRE(ep->dq_dev && ep->q_scales_dev && ep->n_qscales == groups,
                     "staged output needs dequantize scales and one consumer quantize scale per image");
+        TSX_REQUIRE(ep->staged_upsample >= 0 && ep->staged_upsample <= 2, "staged output: upsample factor %d (1 or 2)", ep->staged_upsample);
+        const int up = ep->staged_upsample == 2 ? 2 : 1;
         TSX_REQUIRE(ep->staged_pad_top >= 0 && ep->staged_pad_left >= 0 && ep->staged_cp >= cout && ep->staged_cp % 64 == 0 &&
-                        ho + ep->staged_pad_top <= ep->staged_hs && wo + ep->staged_pad_left <= ep->staged_ws,
+                        up * ho + ep->staged_pad_top <= ep->staged_hs && up * wo + ep->staged_pad_left <= ep->staged_ws,
                     "staged output: %dx%dx%d does not fit [%d][%d][%d] at (%d,%d)", ho, wo, cout, ep->staged_hs,
                     ep->staged_ws, ep->staged_cp, ep->staged_pad_top, ep->staged_pad_left);
         TSX_REQUIRE(reinterpret_cast<uintptr_t>(ep->staged_out_dev) % 16 == 0, "staged output must be 16-byte aligned");
@@ -1041,6 +1044,7 @@ void fill_epilogue(tsx::EpiParams &p, const tsx_epilogue *ep, int64_t count, flo
         p.st_cp = ep->staged_cp;
         p.st_pt = ep->staged_pad_top;
         p.st_pl = ep->staged_pad_left;
+        p.st_up = ep->staged_upsample == 2 ? 2 : 1;
     }
 }
 

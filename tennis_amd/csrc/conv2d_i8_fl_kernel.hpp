@@ -406,10 +406,16 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
                     const auto s02 = __builtin_amdgcn_permlane32_swap(word[0], word[2], false, false);
                     const auto s13 = __builtin_amdgcn_permlane32_swap(word[1], word[3], false, false);
                     const int oh = udiv(prem[j], p.wo, p.wo_magic), ow = prem[j] - oh * p.wo;
-                    int8_t *dst = p.st_out + ((int64_t(pimg[j]) * p.st_hs + oh + p.st_pt) * p.st_ws + ow + p.st_pl) * p.st_cp +
+                    const int up = p.st_up == 2 ? 2 : 1;   // 2: a nearest-neighbour resize by 2 folded into the store
+                    int8_t *dst = p.st_out + ((int64_t(pimg[j]) * p.st_hs + up * oh + p.st_pt) * p.st_ws + up * ow + p.st_pl) * p.st_cp +
                                   cf + 16 * (lane / 32);
                     const v4i packed = {int(s02[0]), int(s02[1]), int(s13[0]), int(s13[1])};
                     *reinterpret_cast<v4i *>(dst) = packed;
+                    if (up == 2) {
+                        *reinterpret_cast<v4i *>(dst + p.st_cp) = packed;
+                        *reinterpret_cast<v4i *>(dst + int64_t(p.st_ws) * p.st_cp) = packed;
+                        *reinterpret_cast<v4i *>(dst + int64_t(p.st_ws + 1) * p.st_cp) = packed;
+                    }
                 }
             }
         });

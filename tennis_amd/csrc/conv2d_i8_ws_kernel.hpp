@@ -523,10 +523,16 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
                             const int pix = oh * p.wo + ow;
                             const int roh = p.wo == p.o_w ? oh : udiv(pix, p.o_w, p.ow_magic);
                             const int row_ = p.wo == p.o_w ? ow : pix - roh * p.o_w;
-                            int8_t *dst = p.st_out + ((int64_t(img + (wrapped ? 1 : 0)) * p.st_hs + roh + p.st_pt) * p.st_ws + row_ + p.st_pl) * p.st_cp +
+                            const int up = p.st_up == 2 ? 2 : 1;   // 2: a nearest-neighbour resize by 2 folded into the store
+                            int8_t *dst = p.st_out + ((int64_t(img + (wrapped ? 1 : 0)) * p.st_hs + up * roh + p.st_pt) * p.st_ws + up * row_ + p.st_pl) * p.st_cp +
                                           cf + 16 * (lane / 32);
                             const v4i packed = {int(s02[0]), int(s02[1]), int(s13[0]), int(s13[1])};
                             *reinterpret_cast<v4i *>(dst) = packed;
+                            if (up == 2) {
+                                *reinterpret_cast<v4i *>(dst + p.st_cp) = packed;
+                                *reinterpret_cast<v4i *>(dst + int64_t(p.st_ws) * p.st_cp) = packed;
+                                *reinterpret_cast<v4i *>(dst + int64_t(p.st_ws + 1) * p.st_cp) = packed;
+                            }
                         }
                     }
                 }

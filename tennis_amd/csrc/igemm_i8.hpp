@@ -21,6 +21,7 @@ struct EpiParams {
     // int8 output in the consumer's staged layout [n][st_hs][st_ws][st_cp] (convolutions only)
     int8_t *st_out;
     int st_hs, st_ws, st_cp, st_pt, st_pl;
+    int st_up;           // 2: every output pixel is written to the 2 x 2 staged pixels of a nearest-neighbour resize by 2
     int o_c, o_h, o_w;   // NCHW extents of the output, to decode a linear index
     int res_after;       // residual joins behind the activation instead of in front of it
 };
@@ -65,7 +66,15 @@ __device__ __forceinline__ void emit(const EpiParams &p, int acc, int64_t idx, f
             const int64_t t2 = t1 / p.o_h;
             const int co = int(t2 % p.o_c);
             const int64_t n = t2 / p.o_c;
-            p.st_out[((n * p.st_hs + oh + p.st_pt) * p.st_ws + ow + p.st_pl) * p.st_cp + co] = q;
+            if (p.st_up == 2) {
+                int8_t *d = p.st_out + ((n * p.st_hs + 2 * oh + p.st_pt) * p.st_ws + 2 * ow + p.st_pl) * p.st_cp + co;
+                d[0] = q;
+                d[p.st_cp] = q;
+                d[int64_t(p.st_ws) * p.st_cp] = q;
+                d[int64_t(p.st_ws + 1) * p.st_cp] = q;
+            } else {
+                p.st_out[((n * p.st_hs + oh + p.st_pt) * p.st_ws + ow + p.st_pl) * p.st_cp + co] = q;
+            }
         }
     }
 }
@@ -128,10 +137,16 @@ __device__ __forceinline__ void epilogue_rows16(const EpiParams &p, const v16i &
         }
         if (st_dst) {
 #pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4)
-                *reinterpret_cast<uint32_t *>(st_dst + 8 * g4) =
-                    uint32_t(qv[4 * g4] & 0xff) | (uint32_t(qv[4 * g4 + 1] & 0xff) << 8) |
-                    (uint32_t(qv[4 * g4 + 2] & 0xff) << 16) | (uint32_t(qv[4 * g4 + 3] & 0xff) << 24);
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const uint32_t w = uint32_t(qv[4 * g4] & 0xff) | (uint32_t(qv[4 * g4 + 1] & 0xff) << 8) |
+                                   (uint32_t(qv[4 * g4 + 2] & 0xff) << 16) | (uint32_t(qv[4 * g4 + 3] & 0xff) << 24);
+                *reinterpret_cast<uint32_t *>(st_dst + 8 * g4) = w;
+                if (p.st_up == 2) {   // st_dst is staged pixel (2 oh, 2 ow): the other three of the 2 x 2 block
+                    *reinterpret_cast<uint32_t *>(st_dst + p.st_cp + 8 * g4) = w;
+                    *reinterpret_cast<uint32_t *>(st_dst + int64_t(p.st_ws) * p.st_cp + 8 * g4) = w;
+                    *reinterpret_cast<uint32_t *>(st_dst + int64_t(p.st_ws + 1) * p.st_cp + 8 * g4) = w;
+                }
+            }
         }
     }
 }

@@ -217,25 +217,38 @@ class YoloV4Int8:
         # else reads and whose one consumer is a convolution that can read a staged buffer: every source convolution
         # writes its requantized output into its run of channels of that consumer's staged input (the CSP stages'
         # two-branch joins).  concat_of: source convolution -> (route, consumer, first channel, total channels).
-        self._concat_of, self._concat_routes = {}, {}
+        self._concat_of, self._concat_routes, self._concat_channels, self._folded_upsamples = {}, {}, {}, set()
         for i, l in enumerate(L):
             if l["type"] != "route" or len(self.srcs[i]) < 2 or i in heads:
                 continue
             cons = consumers[i]
             if len(cons) != 1 or L[cons[0]]["type"] != "conv" or not self._stageable(cons[0]):
                 continue
-            s = rsrcs[i]
-            ok = all(j >= 0 and L[j]["type"] == "conv" and consumers[j] == [i] and j not in heads and j not in folded.values()
-                     for j in s) and len(set(s)) == len(s)
+            # a source is a convolution nothing else reads, or the 2x upsampling of one (the convolution then writes
+            # every pixel to the 2 x 2 pixels it becomes: capi.StagedSlice(upsample=2))
+            s, prod = rsrcs[i], []
+            for j in s:
+                if j >= 0 and L[j]["type"] == "upsample" and consumers[j] == [i] and j not in heads:
+                    c = rsrcs[j][0]
+                    prod.append((c, 2) if c >= 0 and L[c]["type"] == "conv" and consumers[c] == [j] else None)
+                else:
+                    prod.append((j, 1) if j >= 0 and L[j]["type"] == "conv" and consumers[j] == [i] else None)
+            ok = all(pr is not None and pr[0] not in heads and pr[0] not in folded.values() for pr in prod) and \
+                len({pr[0] for pr in prod if pr}) == len(prod)
             if not ok:
                 continue
-            offsets = [sum(L[j]["filters"] for j in s[:m]) for m in range(len(s))]
+            filters = [L[pr[0]]["filters"] for pr in prod]
+            offsets = [sum(filters[:m]) for m in range(len(prod))]
             if any(o % 16 for o in offsets):
                 continue
-            total = sum(L[j]["filters"] for j in s)
-            for j, o in zip(s, offsets):
-                self._concat_of[j] = (i, cons[0], o, total)
+            total = sum(filters)
+            for (c, up), o in zip(prod, offsets):
+                self._concat_of[c] = (i, cons[0], o, total, up)
             self._concat_routes[i] = cons[0]
+            self._concat_channels[i] = total
+            for j in s:
+                if L[j]["type"] == "upsample":
+                    self._folded_upsamples.add(j)
         return rsrcs, consumers, heads, folded
 
     def _run_chained(self, x):
@@ -295,9 +308,9 @@ class YoloV4Int8:
                 q_layer = served[0] if served else None
                 if i in self._concat_of and out_id == i:
                     # one branch of a channel concatenation: straight into its channels of the consumer's staged input
-                    route, k, c0, total = self._concat_of[i]
-                    whole = staged_input(k, (n, total, ho, wo))
-                    target = capi.StagedSlice(whole, c0, l["filters"])
+                    route, k, c0, total, up = self._concat_of[i]
+                    whole = staged_input(k, (n, total, ho * up, wo * up))
+                    target = capi.StagedSlice(whole, c0, l["filters"], upsample=up)
                     staged_for[k] = whole
                     want_f32, q_layer = False, k
                 kw = dict(dq=self.dq[i], bias=self.bias[i], act=l["act"], slope=0.1, want_f32=want_f32)
@@ -335,7 +348,7 @@ class YoloV4Int8:
                 elif i in self._concat_routes:
                     outs[i] = None                                 # its sources wrote the consumer's staged input
                     first = self._shapes[s[0]]
-                    self._shapes[i] = (first[0], sum(L[j]["filters"] for j in s), first[2], first[3])
+                    self._shapes[i] = (first[0], self._concat_channels[i], first[2], first[3])
                 else:
                     outs[i] = capi.concat_channels([outs[j] for j in s])
                     self._shapes[i] = tuple(outs[i].shape)
@@ -353,9 +366,14 @@ class YoloV4Int8:
                 outs[i] = capi.pooling2d(src, "max", (kk, kk), (1, 1), (kk // 2,) * 4)
                 self._shapes[i] = tuple(outs[i].shape)
             elif t == "upsample":
-                src = outs[rsrcs[i][0]]
-                outs[i] = capi.resize_nearest(src, src.shape[2] * 2, src.shape[3] * 2)
-                self._shapes[i] = tuple(outs[i].shape)
+                if i in self._folded_upsamples:
+                    outs[i] = None                                 # the producing convolution wrote the upsampled pixels
+                    sh = self._shapes[rsrcs[i][0]]
+                    self._shapes[i] = (sh[0], sh[1], sh[2] * 2, sh[3] * 2)
+                else:
+                    src = outs[rsrcs[i][0]]
+                    outs[i] = capi.resize_nearest(src, src.shape[2] * 2, src.shape[3] * 2)
+                    self._shapes[i] = tuple(outs[i].shape)
             for j in rsrcs[i]:                                     # free activations nothing reads any more
                 if j >= 0 and last_use.get(j) == i and j not in heads:
                     outs[j] = None

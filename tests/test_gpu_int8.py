@@ -302,6 +302,48 @@ def test_conv2d_i8_staged_hand_over(tsx, port, cmid, a_strides):
         A(_dev(xq), dq=_dev(dqa), q_scales=_dev(qs), staged_out=small)
 
 
+@pytest.mark.parametrize("cmid", [64, 48])                # 32-channel fragments whole / the per-element path for the last 16
+@pytest.mark.parametrize("producer", ["1x1", "3x3", "3x3s2"])   # window-stationary 1x1 (flat pixel rows) / 3x3 / generic kernel
+def test_conv2d_i8_staged_hand_over_upsampled_into_a_channel_slice(tsx, port, cmid, producer):
+    """convolution -> nearest-neighbour resize x2 -> concatenation with a second convolution's output -> convolution,
+    without an fp32 tensor in between: the first producer writes every requantized pixel to the 2 x 2 staged pixels
+    it becomes (staged_upsample = 2) in its run of channels of the consumer's staged input, the second producer its own
+    run; the consumer's output equals the operator chain's (oracle) bit for bit."""
+    rng = np.random.default_rng(411)
+    n, cin, h, w = 2, 40, 7, 5
+    k, pads, strides = {"1x1": (1, (0,) * 4, (1, 1)), "3x3": (3, (1,) * 4, (1, 1)), "3x3s2": (3, (1,) * 4, (2, 2))}[producer]
+    hin, win = (h * 2 - 1, w * 2 - 1) if producer == "3x3s2" else (h, w)
+    xa = rng.integers(-128, 128, (n, cin, hin, win)).astype(np.int8)
+    xb = rng.integers(-128, 128, (n, cin, 2 * h, 2 * w)).astype(np.int8)
+    wa = rng.integers(-127, 128, (cmid, cin, k, k)).astype(np.int8)
+    wb = rng.integers(-127, 128, (32, cin, 1, 1)).astype(np.int8)
+    dqa = rng.uniform(1e-4, 3e-4, cmid).astype(np.float32)
+    dqb = rng.uniform(1e-4, 3e-4, 32).astype(np.float32)
+    ba = rng.standard_normal(cmid).astype(np.float32)
+    qs = np.full(n, 2.5, np.float32)
+    A = tsx.Conv2dI8(_dev(wa), pads, strides)
+    B = tsx.Conv2dI8(_dev(wb))
+    wc = rng.integers(-127, 128, (24, cmid + 32, 3, 3)).astype(np.int8)
+    dqc = rng.uniform(1e-4, 3e-4, 24).astype(np.float32)
+    C = tsx.Conv2dI8(_dev(wc), (1, 1, 1, 1))
+    whole = tsx.StagedInput(C, (n, cmid + 32, 2 * h, 2 * w))
+    A(_dev(xa), dq=_dev(dqa), bias=_dev(ba), act="leaky_relu", slope=0.1, q_scales=_dev(qs), want_f32=False,
+      staged_out=tsx.StagedSlice(whole, 0, cmid, upsample=2))
+    B(_dev(xb), dq=_dev(dqb), q_scales=_dev(qs), want_f32=False, staged_out=tsx.StagedSlice(whole, cmid, 32))
+    got = C.run_staged(whole, _dev(dqc))[0].cpu().numpy()
+    fa = port.leaky_relu(port.add_bias(port.conv2d_quantized(xa, wa, dqa, pads, strides), ba), 0.1)
+    assert fa.shape == (n, cmid, h, w)
+    cat = port.concat([port.resize_nearest(fa, 2 * h, 2 * w), port.conv2d_quantized(xb, wb, dqb)], 1)
+    exp = port.conv2d_quantized(port.quantize(cat, qs), wc, dqc, (1, 1, 1, 1))
+    assert np.array_equal(bits(got), bits(exp))
+    # the checker's view of the slice is the producer's own map
+    q = tsx.staged_interior(tsx.StagedSlice(whole, 0, cmid, upsample=2), range(n)).cpu().numpy()
+    assert np.array_equal(q, port.quantize(fa, qs))
+    with pytest.raises(tsx.TsxError):                # an upsampled map larger than the staged one
+        A(_dev(xa), dq=_dev(dqa), q_scales=_dev(qs), want_f32=False,
+          staged_out=tsx.StagedSlice(tsx.StagedInput(C, (n, cmid + 32, 2 * h - 2, 2 * w)), 0, cmid, upsample=2))
+
+
 @pytest.mark.parametrize("geom", [((3, 3), (2, 2), (0, 1, 0, 1)), ((2, 2), (2, 2), (0, 0, 0, 0)), ((3, 3), (1, 1), (1, 1, 1, 1)),
                                   ((5, 5), (1, 1), (2, 2, 2, 2))])
 @pytest.mark.parametrize("few_channels", [False, True])   # producer = window-stationary kernel / im2col-staged stem
