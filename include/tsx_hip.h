@@ -313,7 +313,10 @@ typedef struct tsx_staged_map {
  * quantized consumer, on the producer's requantized int8 output: quantize (src/kernels/cpu/quantize.cpp:70-125) is
  * monotone non-decreasing for a positive scale, so max-pooling the int8 values gives byte for byte what
  * pooling2d(fp32) -> quantize gives.  Window clipped to the map as in the reference; dst->h, dst->w are the
- * output size (tsx_pooling2d_out_size); dst's halo and channel padding beyond src->cp are left / zeroed. */
+ * output size (tsx_pooling2d_out_size); dst's halo is left as it is, its channels from c up to the next multiple of 64
+ * are zeroed (the channel padding of the map's last 64-channel block) and none beyond: `data` may point at a run of
+ * channels (a multiple of 64 of them, at a multiple of 16) inside a wider staged buffer whose pitch is cp -- an SPP
+ * block pools one run of a concatenation's channels into the next. */
 int tsx_max_pooling2d_i8_staged(const tsx_staged_map *src, const tsx_staged_map *dst, int32_t kh, int32_t kw, int32_t pad_top,
                                 int32_t pad_left, int32_t stride_h, int32_t stride_w, void *stream);
 

@@ -9,6 +9,8 @@
 // One lane per output element, adjacent lanes along W; one lane's sequential sum is the reference's.
 #include "tsx_common.hpp"
 
+#include <algorithm>
+
 namespace {
 
 struct PoolGeom {
@@ -116,11 +118,12 @@ struct PoolStagedGeom {
     int n, h, w, ho, wo, pad_top, pad_left, kh, kw, sh, sw;
     int s_hs, s_ws, s_cp, s_pt, s_pl;   // source buffer
     int d_hs, d_ws, d_cp, d_pt, d_pl;   // destination buffer
+    int cb;                             // channels handled: the map's, rounded up to whole 64-channel blocks
 };
 
 __global__ __launch_bounds__(256) void max_pooling2d_i8_staged_kernel(const int8_t *__restrict__ src, PoolStagedGeom g,
                                                                      int8_t *__restrict__ dst) {
-    const int chunks = g.d_cp / 16;
+    const int chunks = g.cb / 16;
     const int64_t total = int64_t(g.n) * g.ho * g.wo * chunks;
     const int64_t id = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
     if (id >= total) return;
@@ -140,7 +143,7 @@ __global__ __launch_bounds__(256) void max_pooling2d_i8_staged_kernel(const int8
         ni = int(rest / g.ho);
     }
     v4i r = {0, 0, 0, 0};   // channels the source does not have stay zero (channel padding)
-    if (chunk * 16 < g.s_cp) {
+    if (chunk * 16 < min(g.s_cp, g.cb)) {
         int hs = oh * g.sh - g.pad_top, ws = ow * g.sw - g.pad_left;
         const int he = min(hs + g.kh, g.h), we = min(ws + g.kw, g.w);
         hs = max(hs, 0);
@@ -219,8 +222,9 @@ int tsx_max_pooling2d_i8_staged(const tsx_staged_map *src, const tsx_staged_map 
                 "max_pooling2d_i8_staged: output %dx%d has windows outside the %dx%d map", dst->h, dst->w, src->h, src->w);
     PoolStagedGeom g{src->n, src->h, src->w, dst->h, dst->w, pad_top, pad_left, kh, kw, stride_h, stride_w,
                      src->hs, src->ws, src->cp, src->pad_top, src->pad_left,
-                     dst->hs, dst->ws, dst->cp, dst->pad_top, dst->pad_left};
-    const int64_t total = int64_t(dst->n) * dst->h * dst->w * (dst->cp / 16);
+                     dst->hs, dst->ws, dst->cp, dst->pad_top, dst->pad_left,
+                     int(std::min<int64_t>(dst->cp, tsx::round_up(dst->c, 64)))};
+    const int64_t total = int64_t(dst->n) * dst->h * dst->w * (g.cb / 16);
     TSX_REQUIRE(tsx::ceil_div(total, 256) < (int64_t(1) << 31), "max_pooling2d_i8_staged: tensor too large");
     hipLaunchKernelGGL(max_pooling2d_i8_staged_kernel, dim3(unsigned(tsx::ceil_div(total, 256))), dim3(256), 0,
                        tsx::as_stream(stream), static_cast<const int8_t *>(src->data), g, static_cast<int8_t *>(dst->data));

@@ -218,15 +218,39 @@ class YoloV4Int8:
         # writes its requantized output into its run of channels of that consumer's staged input (the CSP stages'
         # two-branch joins).  concat_of: source convolution -> (route, consumer, first channel, total channels).
         self._concat_of, self._concat_routes, self._concat_channels, self._folded_upsamples = {}, {}, {}, set()
+        self._spp_pools = {}   # max pooling layer -> (consumer, total channels, source run, own run, channels, window)
         for i, l in enumerate(L):
             if l["type"] != "route" or len(self.srcs[i]) < 2 or i in heads:
                 continue
             cons = consumers[i]
             if len(cons) != 1 or L[cons[0]]["type"] != "conv" or not self._stageable(cons[0]):
                 continue
+            s = rsrcs[i]
+            # An SPP block: one convolution and stride-1 "same" max poolings of its output, nothing else reading any
+            # of them.  quantize commutes with max, so the convolution writes its requantized output into its run of
+            # the consumer's staged channels and every pooling goes from one run of int8 channels into the next
+            # (cascaded: the k x k maximum is the (k - k' + 1)-maximum of the k' x k' maxima).
+            convs = [j for j in s if j >= 0 and L[j]["type"] == "conv"]
+            pools = [j for j in s if j >= 0 and L[j]["type"] == "maxpool"]
+            if len(convs) == 1 and pools and len(convs) + len(pools) == len(s) and len(set(s)) == len(s):
+                c = convs[0]
+                f = L[c]["filters"]
+                ok = (f % 64 == 0 and c not in heads and c not in folded.values() and sorted(consumers[c]) == sorted(pools + [i])
+                      and all(rsrcs[j] == [c] and consumers[j] == [i] and j not in heads and L[j]["size"] % 2 == 1 for j in pools)
+                      and len({L[j]["size"] for j in pools}) == len(pools))
+                if ok:
+                    total = f * len(s)
+                    self._concat_of[c] = (i, cons[0], s.index(c) * f, total, 1)
+                    self._concat_routes[i] = cons[0]
+                    self._concat_channels[i] = total
+                    prev_k, prev_off = 1, s.index(c) * f
+                    for j in sorted(pools, key=lambda j: L[j]["size"]):
+                        self._spp_pools[j] = (cons[0], total, prev_off, s.index(j) * f, f, L[j]["size"] - prev_k + 1)
+                        prev_k, prev_off = L[j]["size"], s.index(j) * f
+                    continue
             # a source is a convolution nothing else reads, or the 2x upsampling of one (the convolution then writes
             # every pixel to the 2 x 2 pixels it becomes: capi.StagedSlice(upsample=2))
-            s, prod = rsrcs[i], []
+            prod = []
             for j in s:
                 if j >= 0 and L[j]["type"] == "upsample" and consumers[j] == [i] and j not in heads:
                     c = rsrcs[j][0]
@@ -352,6 +376,14 @@ class YoloV4Int8:
                 else:
                     outs[i] = capi.concat_channels([outs[j] for j in s])
                     self._shapes[i] = tuple(outs[i].shape)
+            elif t == "maxpool" and i in self._spp_pools:
+                k1, total, src_off, dst_off, f, win = self._spp_pools[i]
+                sh = self._shapes[rsrcs[i][0]]
+                whole = staged_input(k1, (n, total, sh[2], sh[3]))
+                capi.max_pooling2d_staged(capi.StagedSlice(whole, src_off, f), capi.StagedSlice(whole, dst_off, f),
+                                          (win, win), (1, 1), (win // 2,) * 4)
+                outs[i] = None
+                self._shapes[i] = sh
             elif t == "maxpool":
                 k = l["size"]
                 # An SPP block pools one map with growing odd windows at stride 1: the k x k maximum is the

@@ -385,6 +385,33 @@ def test_max_pooling_on_staged_int8(tsx, port, geom, few_channels):
                                                         strides[0], strides[1], None))
 
 
+def test_max_pooling_on_a_channel_slice_of_staged_int8(tsx, port):
+    """An SPP block on int8: a convolution writes its requantized output into the last 64 channels of the consumer's
+    staged input, stride-1 max poolings go from one run of 64 channels into the next (5x5 of the convolution's run, then
+    5x5 of that = 9x9), and the consumer's output equals the operator chain conv -> pooling2d(fp32) x2 -> concat ->
+    quantize -> conv2d_quantized bit for bit."""
+    rng = np.random.default_rng(412)
+    n, cin, h, w, f = 2, 40, 11, 9, 64
+    xq = rng.integers(-128, 128, (n, cin, h, w)).astype(np.int8)
+    wa = rng.integers(-127, 128, (f, cin, 1, 1)).astype(np.int8)
+    dqa = rng.uniform(1e-3, 3e-3, f).astype(np.float32)
+    ba = rng.standard_normal(f).astype(np.float32)
+    qs = np.full(n, 4.0, np.float32)
+    A = tsx.Conv2dI8(_dev(wa))
+    wc = rng.integers(-127, 128, (24, 3 * f, 1, 1)).astype(np.int8)
+    dqc = rng.uniform(1e-4, 3e-4, 24).astype(np.float32)
+    C = tsx.Conv2dI8(_dev(wc))
+    whole = tsx.StagedInput(C, (n, 3 * f, h, w))
+    A(_dev(xq), dq=_dev(dqa), bias=_dev(ba), act="leaky_relu", slope=0.1, q_scales=_dev(qs), want_f32=False,
+      staged_out=tsx.StagedSlice(whole, 2 * f, f))
+    tsx.max_pooling2d_staged(tsx.StagedSlice(whole, 2 * f, f), tsx.StagedSlice(whole, f, f), (5, 5), (1, 1), (2, 2, 2, 2))
+    tsx.max_pooling2d_staged(tsx.StagedSlice(whole, f, f), tsx.StagedSlice(whole, 0, f), (5, 5), (1, 1), (2, 2, 2, 2))
+    got = C.run_staged(whole, _dev(dqc))[0].cpu().numpy()
+    fa = port.leaky_relu(port.add_bias(port.conv2d_quantized(xq, wa, dqa), ba), 0.1)
+    cat = port.concat([port.pooling2d(fa, "max", (9, 9), (1, 1), (4, 4, 4, 4)), port.pooling2d(fa, "max", (5, 5), (1, 1), (2, 2, 2, 2)), fa], 1)
+    assert np.array_equal(bits(got), bits(port.conv2d_quantized(port.quantize(cat, qs), wc, dqc)))
+
+
 def test_quantize_conv2d_fused_input(tsx, port):
     rng = np.random.default_rng(203)
     for n in (1, 4):
