@@ -127,6 +127,9 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
         });
     };
 
+    // the first window's loads leave before anything else is computed: their latency covers the rest of the set-up
+    window_load(0);
+
     // ---- B operand addresses: fragment j, lane l -> flat position P0 + (frag0 + j)*32 + l%32, K group l/32
     int b_base[NT];
     static_for<0, NT>([&](auto jc) {
@@ -169,7 +172,6 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
     // blocks' loads already in flight behind it; those are stored (and any further blocks fetched) when this
     // wavefront leaves block 0, behind the loop's only barrier.
     v4i wbat[3][FL_MAX_FILL];
-    window_load(0);
     if (RESIDENT) {
         static_for<0, 3>([&](auto bc) {
             constexpr int b = decltype(bc)::value;

@@ -161,6 +161,9 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
         });
     };
 
+    // the first window's loads leave before anything else is computed: their latency covers the rest of the set-up
+    window_load(0);
+
     // ---- B operand addresses: fragment j, lane l -> tile position j*32 + l%32, K group l/32
     int b_base[NT];
     static_for<0, NT>([&](auto jc) {
@@ -193,8 +196,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
         });
     });
 
-    // ---- prologue
-    window_load(0);
+    // ---- prologue (the first window is on its way)
     static_for<0, RING - 1>([&](auto sc) { a_load(sc, decltype(sc)::value); });
 
     // ---- epilogue operands, fetched while the first window is in flight: a wavefront that meets them only behind
