@@ -121,6 +121,10 @@ struct PoolStagedGeom {
     int cb;                             // channels handled: the map's, rounded up to whole 64-channel blocks
 };
 
+// KH, KW > 0: a window of that size with every load issued before the first comparison -- rows and columns outside the
+// map are clamped into it, which repeats elements the window holds anyway (max does not mind) -- where the
+// runtime-sized loop (KH = 0) waits for each 16-byte element in turn.
+template <int KH, int KW>
 __global__ __launch_bounds__(256) void max_pooling2d_i8_staged_kernel(const int8_t *__restrict__ src, PoolStagedGeom g,
                                                                      int8_t *__restrict__ dst) {
     const int chunks = g.cb / 16;
@@ -149,13 +153,28 @@ __global__ __launch_bounds__(256) void max_pooling2d_i8_staged_kernel(const int8
         hs = max(hs, 0);
         ws = max(ws, 0);
         const int8_t *base = src + ((int64_t(ni) * g.s_hs + g.s_pt) * g.s_ws + g.s_pl) * g.s_cp + chunk * 16;
-        r = *reinterpret_cast<const v4i *>(base + (int64_t(hs) * g.s_ws + ws) * g.s_cp);   // the first valid element
-        for (int ih = hs; ih < he; ++ih)
-            for (int iw = ws; iw < we; ++iw) {
-                const v4i v = *reinterpret_cast<const v4i *>(base + (int64_t(ih) * g.s_ws + iw) * g.s_cp);
+        if (KH > 0) {
+            v4i v[KH > 0 ? KH * KW : 1];
 #pragma unroll
-                for (int k = 0; k < 4; ++k) r[k] = int(max_i8x4(uint32_t(r[k]), uint32_t(v[k])));
-            }
+            for (int i = 0; i < KH; ++i)
+#pragma unroll
+                for (int j = 0; j < KW; ++j)
+                    v[i * KW + j] = *reinterpret_cast<const v4i *>(
+                        base + (int64_t(min(hs + i, he - 1)) * g.s_ws + min(ws + j, we - 1)) * g.s_cp);
+            r = v[0];
+#pragma unroll
+            for (int t = 1; t < KH * KW; ++t)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) r[k] = int(max_i8x4(uint32_t(r[k]), uint32_t(v[t][k])));
+        } else {
+            r = *reinterpret_cast<const v4i *>(base + (int64_t(hs) * g.s_ws + ws) * g.s_cp);   // the first valid element
+            for (int ih = hs; ih < he; ++ih)
+                for (int iw = ws; iw < we; ++iw) {
+                    const v4i v = *reinterpret_cast<const v4i *>(base + (int64_t(ih) * g.s_ws + iw) * g.s_cp);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) r[k] = int(max_i8x4(uint32_t(r[k]), uint32_t(v[k])));
+                }
+        }
     }
     *reinterpret_cast<v4i *>(dst + ((int64_t(ni) * g.d_hs + oh + g.d_pt) * g.d_ws + ow + g.d_pl) * g.d_cp + chunk * 16) = r;
 }
@@ -226,8 +245,15 @@ int tsx_max_pooling2d_i8_staged(const tsx_staged_map *src, const tsx_staged_map 
                      int(std::min<int64_t>(dst->cp, tsx::round_up(dst->c, 64)))};
     const int64_t total = int64_t(dst->n) * dst->h * dst->w * (g.cb / 16);
     TSX_REQUIRE(tsx::ceil_div(total, 256) < (int64_t(1) << 31), "max_pooling2d_i8_staged: tensor too large");
-    hipLaunchKernelGGL(max_pooling2d_i8_staged_kernel, dim3(unsigned(tsx::ceil_div(total, 256))), dim3(256), 0,
-                       tsx::as_stream(stream), static_cast<const int8_t *>(src->data), g, static_cast<int8_t *>(dst->data));
+    const dim3 grid(unsigned(tsx::ceil_div(total, 256)));
+    const int8_t *s8 = static_cast<const int8_t *>(src->data);
+    int8_t *d8 = static_cast<int8_t *>(dst->data);
+    if (kh == 3 && kw == 3)
+        hipLaunchKernelGGL((max_pooling2d_i8_staged_kernel<3, 3>), grid, dim3(256), 0, tsx::as_stream(stream), s8, g, d8);
+    else if (kh == 5 && kw == 5)
+        hipLaunchKernelGGL((max_pooling2d_i8_staged_kernel<5, 5>), grid, dim3(256), 0, tsx::as_stream(stream), s8, g, d8);
+    else
+        hipLaunchKernelGGL((max_pooling2d_i8_staged_kernel<0, 0>), grid, dim3(256), 0, tsx::as_stream(stream), s8, g, d8);
     TSX_LAUNCH_CHECK("max_pooling2d_i8_staged_kernel");
     return 0;
 }
