@@ -246,6 +246,22 @@ class StagedSlice:
         self.buf = staged.buf[c0:]          # the epilogue takes the address of channel c0 of the first pixel
 
 
+class StagedView:
+    """Another consumer's view of a StagedInput that holds the same tensor with at least as much halo: the buffer
+    entered `row0` rows and `col0` columns further in, with the owner's row and image pitch (what
+    tsx_conv2d_i8_staged_at reads: a buffer whose extents are larger than the convolution needs)."""
+
+    def __init__(self, owner, pad_top, pad_left):
+        if pad_top > owner.pad_top or pad_left > owner.pad_left:
+            raise TsxError("staged view: the owner's halo (%d, %d) is smaller than (%d, %d)" % (owner.pad_top, owner.pad_left, pad_top, pad_left))
+        self.row0, self.col0 = owner.pad_top - pad_top, owner.pad_left - pad_left
+        self.x_shape = owner.x_shape
+        self.hs, self.ws, self.cp = owner.hs, owner.ws, owner.cp
+        self.pad_top, self.pad_left = pad_top, pad_left
+        self.full_buf = owner.buf
+        self.buf = owner.buf[(self.row0 * owner.ws + self.col0) * owner.cp:]
+
+
 def staged_interior(staged, images):
     """The map inside a staged buffer (StagedInput / StagedPlain) as an int8 NCHW tensor of the given images:
     a copy, for checkers that compare a producer's requantized hand-over with the operator chain's values."""
@@ -253,7 +269,8 @@ def staged_interior(staged, images):
     c0 = getattr(staged, "c0", 0)
     buf = getattr(staged, "full_buf", staged.buf)
     t = buf[: n * staged.hs * staged.ws * staged.cp].view(n, staged.hs, staged.ws, staged.cp)
-    t = t[list(images), staged.pad_top:staged.pad_top + h, staged.pad_left:staged.pad_left + w, c0:c0 + c]
+    top, left = staged.pad_top + getattr(staged, "row0", 0), staged.pad_left + getattr(staged, "col0", 0)
+    t = t[list(images), top:top + h, left:left + w, c0:c0 + c]
     if getattr(staged, "upsample", 1) == 2:
         # the producer wrote every pixel four times: its own map is any of the four phases, and they must agree
         phases = [t[:, dy::2, dx::2] for dy in (0, 1) for dx in (0, 1)]

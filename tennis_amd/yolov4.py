@@ -317,17 +317,23 @@ class YoloV4Int8:
                 # consumers of the produced tensor
                 conv_cons = [k for k in consumers[out_id] if L[k]["type"] == "conv"]
                 others = [k for k in consumers[out_id] if L[k]["type"] != "conv"]
+                # one staged buffer -- the consumer's with the largest halo -- serves every consumer whose own staged
+                # input fits inside it (less halo, fewer rows: a 1x1 or a strided convolution beside a 3x3 one)
                 target, served = None, []
-                for k in conv_cons:
-                    if self._stageable(k):
-                        st = staged_input(k, shape)
-                        if target is None:
-                            target, served = st, [k]
-                        elif (st.hs, st.ws, st.cp, st.pad_top, st.pad_left) == (target.hs, target.ws, target.cp, target.pad_top, target.pad_left):
+                own = {k: staged_input(k, shape) for k in conv_cons if self._stageable(k)}
+                if own:
+                    owner = max(own, key=lambda k: (own[k].pad_top, own[k].pad_left, own[k].hs, own[k].ws))
+                    target = own[owner]
+                    for k, st in own.items():
+                        if k == owner or (st.hs, st.ws, st.cp, st.pad_top, st.pad_left) == (target.hs, target.ws, target.cp, target.pad_top, target.pad_left):
                             served.append(k)
+                            staged_for[k] = target
+                        elif (st.cp == target.cp and st.pad_top <= target.pad_top and st.pad_left <= target.pad_left
+                              and st.hs + target.pad_top - st.pad_top <= target.hs and st.ws + target.pad_left - st.pad_left <= target.ws):
+                            served.append(k)
+                            staged_for[k] = capi.StagedView(target, st.pad_top, st.pad_left)
                 for k in served:
                     assert self.scales[k] == self.scales[served[0]]   # calibrated on the same tensor
-                    staged_for[k] = target
                 want_f32 = bool(others) or out_id in heads or any(k not in served for k in conv_cons)
                 q_layer = served[0] if served else None
                 if i in self._concat_of and out_id == i:
