@@ -132,6 +132,46 @@ def test_conv2d_i8_accumulators_and_dequant(tsx, port, case):
     assert np.array_equal(bits(out.cpu().numpy()), bits(exp))
 
 
+def _random_conv_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        kh, kw = (int(v) for v in rng.choice([1, 2, 3, 5], 2))
+        st = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        dl = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        pads = tuple(int(rng.integers(0, k // 2 + 2)) for k in (kh, kh, kw, kw))
+        n, c, cout = int(rng.integers(1, 4)), int(rng.choice([3, 16, 40, 64, 70, 130])), int(rng.choice([8, 24, 32, 33, 64, 96, 130]))
+        h, w = int(rng.integers(5, 34)), int(rng.integers(5, 70))
+        if h + pads[0] + pads[1] < dl[0] * (kh - 1) + 1 or w + pads[2] + pads[3] < dl[1] * (kw - 1) + 1:
+            continue
+        cases.append((n, c, h, w, cout, kh, kw, pads, st, dl))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_conv_cases(24, 419))
+def test_conv2d_i8_random_geometries_with_every_output(tsx, port, case):
+    """Seeded random geometries (kernel 1..5, strides, dilations, asymmetric padding, ragged channel counts, maps wider
+    than a tile) through the full epilogue -- dequantize, bias, LeakyReLU, fp32 out, requantized int8 out, raw
+    accumulators -- against the oracle bit for bit: the tile / window / fragment arithmetic of whichever kernel the
+    planner picks."""
+    n, c, h, w, cout, kh, kw, pads, st, dl = case
+    rng = np.random.default_rng(hash(case) % (1 << 31))
+    x = rng.integers(-128, 128, (n, c, h, w)).astype(np.int8)
+    wt = rng.integers(-127, 128, (cout, c, kh, kw)).astype(np.int8)
+    dq = rng.uniform(1e-4, 1e-3, cout).astype(np.float32)
+    bias = rng.standard_normal(cout).astype(np.float32)
+    qs = np.full(n, 6.0, np.float32)
+    conv = tsx.Conv2dI8(_dev(wt), pads, st, dl)
+    out, q, acc = conv(_dev(x), dq=_dev(dq), bias=_dev(bias), act="leaky_relu", slope=0.1, q_scales=_dev(qs), want_acc=True)
+    exp, exp_q = port.conv2d_i8_fused(x, wt, dq, bias, "leaky_relu", 0.1, qs, pads, st, dl)
+    assert np.array_equal(acc.cpu().numpy(), port.conv2d_quantized(x, wt, dq, pads, st, dl, return_acc=True)[1])
+    assert np.array_equal(bits(out.cpu().numpy()), bits(exp))
+    assert np.array_equal(q.cpu().numpy(), exp_q)
+    # the same without the raw accumulators: the fragment-wise epilogue instead of the per-element one
+    out2, q2, _ = conv(_dev(x), dq=_dev(dq), bias=_dev(bias), act="leaky_relu", slope=0.1, q_scales=_dev(qs))
+    assert np.array_equal(bits(out2.cpu().numpy()), bits(exp)) and np.array_equal(q2.cpu().numpy(), exp_q)
+
+
 def test_conv2d_i8_padding_value(tsx, port):
     rng = np.random.default_rng(201)
     x = rng.integers(-128, 128, (2, 5, 6, 7)).astype(np.int8)
