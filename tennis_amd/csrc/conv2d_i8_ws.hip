@@ -230,7 +230,9 @@ int ws_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t 
     p.ow_magic = div_magic(ep.o_w, int64_t(p.ho) * p.wo);
     const int bm = 32 * WS_FM * pl.wm;
     const dim3 grid(unsigned(pl.tiles), unsigned((g.cout + bm - 1) / bm));
-    const size_t lds_bytes = size_t(2) * pl.wp * (64 * pl.cbs + 16);
+    // two window buffers (one channel block ahead); a layer whose channels fit one window never swaps and takes one:
+    // more workgroups per CU where the window is large (stride-2 3x3 layers on 32 or 64 channels)
+    const size_t lds_bytes = size_t(p.cblocks > 1 ? 2 : 1) * pl.wp * (64 * pl.cbs + 16);
     switch (pl.nt) {
         case 1: return ws_launch_nt<1>(p, grid, lds_bytes, stream);
         case 2: return ws_launch_nt<2>(p, grid, lds_bytes, stream);
