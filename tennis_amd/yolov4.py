@@ -248,15 +248,17 @@ class YoloV4Int8:
                         self._spp_pools[j] = (cons[0], total, prev_off, s.index(j) * f, f, L[j]["size"] - prev_k + 1)
                         prev_k, prev_off = L[j]["size"], s.index(j) * f
                     continue
-            # a source is a convolution nothing else reads, or the 2x upsampling of one (the convolution then writes
-            # every pixel to the 2 x 2 pixels it becomes: capi.StagedSlice(upsample=2))
+            # a source is a convolution, or the 2x upsampling of one that nothing else reads (the convolution then
+            # writes every pixel to the 2 x 2 pixels it becomes: capi.StagedSlice(upsample=2))
             prod = []
             for j in s:
                 if j >= 0 and L[j]["type"] == "upsample" and consumers[j] == [i] and j not in heads:
                     c = rsrcs[j][0]
                     prod.append((c, 2) if c >= 0 and L[c]["type"] == "conv" and consumers[c] == [j] else None)
                 else:
-                    prod.append((j, 1) if j >= 0 and L[j]["type"] == "conv" and consumers[j] == [i] else None)
+                    # read by this route once; further readers get the fp32 copy the convolution then also writes
+                    prod.append((j, 1) if j >= 0 and L[j]["type"] == "conv" and consumers[j].count(i) == 1
+                                and j not in self._concat_of else None)
             ok = all(pr is not None and pr[0] not in heads and pr[0] not in folded.values() for pr in prod) and \
                 len({pr[0] for pr in prod if pr}) == len(prod)
             if not ok:
@@ -320,7 +322,8 @@ class YoloV4Int8:
                 # one staged buffer -- the consumer's with the largest halo -- serves every consumer whose own staged
                 # input fits inside it (less halo, fewer rows: a 1x1 or a strided convolution beside a 3x3 one)
                 target, served = None, []
-                own = {k: staged_input(k, shape) for k in conv_cons if self._stageable(k)}
+                branch = i in self._concat_of and out_id == i
+                own = {} if branch else {k: staged_input(k, shape) for k in conv_cons if self._stageable(k)}
                 if own:
                     owner = max(own, key=lambda k: (own[k].pad_top, own[k].pad_left, own[k].hs, own[k].ws))
                     target = own[owner]
@@ -336,13 +339,16 @@ class YoloV4Int8:
                     assert self.scales[k] == self.scales[served[0]]   # calibrated on the same tensor
                 want_f32 = bool(others) or out_id in heads or any(k not in served for k in conv_cons)
                 q_layer = served[0] if served else None
-                if i in self._concat_of and out_id == i:
-                    # one branch of a channel concatenation: straight into its channels of the consumer's staged input
+                if branch:
+                    # one branch of a channel concatenation: straight into its channels of the consumer's staged input,
+                    # requantized with that consumer's scale; any other reader (a convolution with a scale of its own
+                    # included) takes the fp32 copy
                     route, k, c0, total, up = self._concat_of[i]
                     whole = staged_input(k, (n, total, ho * up, wo * up))
                     target = capi.StagedSlice(whole, c0, l["filters"], upsample=up)
                     staged_for[k] = whole
-                    want_f32, q_layer = False, k
+                    want_f32 = bool(conv_cons) or any(o != route for o in others) or out_id in heads
+                    q_layer = k
                 kw = dict(dq=self.dq[i], bias=self.bias[i], act=l["act"], slope=0.1, want_f32=want_f32)
                 if target is not None:
                     kw.update(q_scales=self.sx[q_layer], staged_out=target)
