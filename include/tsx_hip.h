@@ -101,7 +101,10 @@ typedef struct tsx_epilogue {
      * padded) input of the convolution that consumes it, [n][staged_hs][staged_ws][staged_cp] with output
      * pixel (oh, ow) at (oh + staged_pad_top, ow + staged_pad_left), instead of NCHW -- the consumer then
      * runs tsx_conv2d_i8_staged_at without a staging pass.  Needs q_scales_dev; the buffer's halo and
-     * channel padding are written once by tsx_conv2d_i8_stage_fill.  NULL = not used. */
+     * channel padding are written once by tsx_conv2d_i8_stage_fill.  staged_cp is a multiple of 32 (a
+     * consumer's own channel pitch is a multiple of 64; 32 describes a consumer that reads pairs of columns of
+     * a 32-channel tensor as one 64-channel pixel: staged_ws and staged_pad_left then count columns, not
+     * pairs).  NULL = not used. */
     int8_t *staged_out_dev;
     int32_t staged_hs, staged_ws, staged_cp, staged_pad_top, staged_pad_left;
     int32_t residual_after_act; /* 0: act(y + residual); 1: act(y) + residual */

@@ -262,6 +262,40 @@ class StagedView:
         self.buf = owner.buf[(self.row0 * owner.ws + self.col0) * owner.cp:]
 
 
+class StagedPairs:
+    """A StagedInput whose pixels are PAIRS of horizontally adjacent pixels of a tensor with half as many channels,
+    seen as that tensor: the bytes of [hs][ws][cp] are those of [hs][2 ws][cp / 2].  A tensor of 32 channels staged
+    by itself carries 32 bytes of padding per pixel; staged in pairs it carries none, and a 3 x 3 convolution of
+    stride 2 over it is a 3 x 2 convolution of stride (2, 1) over the pairs (pair_columns_weights), with 6 K-steps
+    instead of 9.  The producer's epilogue writes this view; the pair convolution reads `pairs`."""
+
+    def __init__(self, staged):
+        n, c2, h, w2 = staged.x_shape
+        if c2 != staged.cp or c2 % 64:
+            raise TsxError("staged pairs: %d channels per pair are not whole 64-channel blocks" % c2)
+        self.pairs = staged
+        self.x_shape = (n, c2 // 2, h, 2 * w2)
+        self.hs, self.ws, self.cp = staged.hs, 2 * staged.ws, staged.cp // 2
+        self.pad_top, self.pad_left = staged.pad_top, 2 * staged.pad_left
+        self.buf = staged.buf
+
+
+def pair_columns_weights(w):
+    """Weights [cout][c][kh][3] of a convolution with column stride 2 and one column of left padding, rewritten for
+    an input whose pixels are pairs of columns (channels [0, c): the even column, [c, 2c): the odd one):
+    [cout][2c][kh][2] for column stride 1, one PAIR of left padding and none on the right.  Output column ow reads
+    columns 2ow - 1 (odd half of pair ow - 1) and 2ow, 2ow + 1 (pair ow); the even half of pair ow - 1 gets zero
+    weights, which add nothing to an integer sum: the accumulators are those of the original convolution."""
+    cout, c, kh, kw = w.shape
+    if kw != 3:
+        raise TsxError("pair_columns_weights: kernel width %d, not 3" % kw)
+    wp = torch.zeros((cout, 2 * c, kh, 2), dtype=w.dtype, device=w.device)
+    wp[:, c:, :, 0] = w[:, :, :, 0]
+    wp[:, :c, :, 1] = w[:, :, :, 1]
+    wp[:, c:, :, 1] = w[:, :, :, 2]
+    return wp
+
+
 def staged_interior(staged, images):
     """The map inside a staged buffer (StagedInput / StagedPlain) as an int8 NCHW tensor of the given images:
     a copy, for checkers that compare a producer's requantized hand-over with the operator chain's values."""

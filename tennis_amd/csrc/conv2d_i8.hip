@@ -1001,7 +1001,7 @@ int check_epilogue(const tsx_epilogue *ep, const float *out_f32, const int8_t *o
                     "staged output needs dequantize scales and one consumer quantize scale per image");
         TSX_REQUIRE(ep->staged_upsample >= 0 && ep->staged_upsample <= 2, "staged output: upsample factor %d (1 or 2)", ep->staged_upsample);
         const int up = ep->staged_upsample == 2 ? 2 : 1;
-        TSX_REQUIRE(ep->staged_pad_top >= 0 && ep->staged_pad_left >= 0 && ep->staged_cp >= cout && ep->staged_cp % 64 == 0 &&
+        TSX_REQUIRE(ep->staged_pad_top >= 0 && ep->staged_pad_left >= 0 && ep->staged_cp >= cout && ep->staged_cp % 32 == 0 &&
                         up * ho + ep->staged_pad_top <= ep->staged_hs && up * wo + ep->staged_pad_left <= ep->staged_ws,
                     "staged output: %dx%dx%d does not fit [%d][%d][%d] at (%d,%d)", ho, wo, cout, ep->staged_hs,
                     ep->staged_ws, ep->staged_cp, ep->staged_pad_top, ep->staged_pad_left);
