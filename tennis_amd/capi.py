@@ -296,6 +296,19 @@ def pair_columns_weights(w):
     return wp
 
 
+def pair_outputs_weights(w):
+    """Weights [cout][c][kh][kw] of a convolution with column stride 1, rewritten to produce PAIRS of output columns as
+    one pixel of 2 cout channels: [2 cout][c][kh][kw + 1] for column stride 2 (same padding).  Channels [0, cout) are
+    the even output column (kernel columns 0..kw-1 of the wider window), [cout, 2 cout) the odd one (columns 1..kw); the
+    extra column carries zero weights.  Written as a staged hand-over this is byte for byte the StagedPairs layout; the
+    dequantize scales and the bias are the original ones twice."""
+    cout, c, kh, kw = w.shape
+    wp = torch.zeros((2 * cout, c, kh, kw + 1), dtype=w.dtype, device=w.device)
+    wp[:cout, :, :, :kw] = w
+    wp[cout:, :, :, 1:] = w
+    return wp
+
+
 def staged_interior(staged, images):
     """The map inside a staged buffer (StagedInput / StagedPlain) as an int8 NCHW tensor of the given images:
     a copy, for checkers that compare a producer's requantized hand-over with the operator chain's values."""

@@ -286,7 +286,7 @@ class YoloV4Int8:
         n = x.shape[0]
         if not hasattr(self, "_plan"):
             self._plan = self._chain_plan()
-            self._staged, self._pair_conv = {}, {}
+            self._staged, self._pair_conv, self._pair_prod = {}, {}, {}
         rsrcs, consumers, heads, folded = self._plan
         absorbed = {a: s for s, a in folded.items()}
         L = self.L
@@ -364,7 +364,19 @@ class YoloV4Int8:
                     kw.update(q_scales=self.sx[q_layer], staged_out=target)
                 if i in absorbed:
                     kw.update(residual=outs[rsrcs[absorbed[i]][1]], residual_after_act=True)
-                if i in staged_for and isinstance(staged_for[i], capi.StagedPairs):
+                cin = self.conv[i].w.shape[1]
+                if (isinstance(target, capi.StagedPairs) and not want_f32 and i not in absorbed and i not in staged_for
+                        and l["size"] == 3 and l["stride"] == 1 and cin * 12 <= 64):
+                    # the stem in front of a pair-staged layer: computed as pairs of output columns (a 3x4 window at column
+                    # stride 2, 2 x 32 output channels), so that its im2col rows are per pair -- half the staged bytes
+                    if i not in self._pair_prod:
+                        self._pair_prod[i] = (capi.Conv2dI8(capi.pair_outputs_weights(self.conv[i].w), (1, 1, 1, 1), (1, 2)),
+                                              torch.cat([self.dq[i], self.dq[i]]), torch.cat([self.bias[i], self.bias[i]]))
+                    pconv, dq2, bias2 = self._pair_prod[i]
+                    pconv(get(src), x_scales=self.sx[i], dq=dq2, bias=bias2, act=l["act"], slope=0.1, want_f32=False,
+                          q_scales=self.sx[q_layer], staged_out=target.pairs)
+                    y = None
+                elif i in staged_for and isinstance(staged_for[i], capi.StagedPairs):
                     y = self._pair_conv[i].run_staged(staged_for[i].pairs, **kw)[0]
                 elif i in staged_for:
                     y = conv.run_staged(staged_for[i], **kw)[0]

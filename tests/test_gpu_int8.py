@@ -384,7 +384,8 @@ def test_conv2d_i8_staged_hand_over_upsampled_into_a_channel_slice(tsx, port, cm
           staged_out=tsx.StagedSlice(tsx.StagedInput(C, (n, cmid + 32, 2 * h - 2, 2 * w)), 0, cmid, upsample=2))
 
 
-@pytest.mark.parametrize("producer", ["stem", "1x1", "3x3"])     # im2col-staged stem / window-stationary 1x1 / 3x3
+# im2col-staged stem / the same computed as pairs of output columns / window-stationary 1x1 / 3x3
+@pytest.mark.parametrize("producer", ["stem", "stem-pairs", "1x1", "3x3"])
 @pytest.mark.parametrize("size", [(9, 12), (32, 70)])
 def test_conv2d_i8_staged_hand_over_in_column_pairs(tsx, port, producer, size):
     """A 32-channel producer followed by a 3x3 convolution of stride 2: the producer writes pairs of columns as one
@@ -393,10 +394,10 @@ def test_conv2d_i8_staged_hand_over_in_column_pairs(tsx, port, producer, size):
     geometry) bit for bit."""
     rng = np.random.default_rng(431)
     n, (h, w) = 2, size
-    cin, k, pads = {"stem": (3, 3, (1,) * 4), "1x1": (48, 1, (0,) * 4), "3x3": (64, 3, (1,) * 4)}[producer]
+    cin, k, pads = {"stem": (3, 3, (1,) * 4), "stem-pairs": (3, 3, (1,) * 4), "1x1": (48, 1, (0,) * 4), "3x3": (64, 3, (1,) * 4)}[producer]
     xa = rng.integers(-128, 128, (n, cin, h, w)).astype(np.int8)
     wa = rng.integers(-127, 128, (32, cin, k, k)).astype(np.int8)
-    dqa = rng.uniform(1e-4, 3e-4, 32).astype(np.float32) * (20 if producer == "stem" else 1)
+    dqa = rng.uniform(1e-4, 3e-4, 32).astype(np.float32) * (20 if cin == 3 else 1)
     ba = rng.standard_normal(32).astype(np.float32)
     qs = np.full(n, 3.0, np.float32)
     wb = rng.integers(-127, 128, (40, 32, 3, 3)).astype(np.int8)
@@ -404,7 +405,13 @@ def test_conv2d_i8_staged_hand_over_in_column_pairs(tsx, port, producer, size):
     A = tsx.Conv2dI8(_dev(wa), pads)
     B = tsx.Conv2dI8(tsx.pair_columns_weights(_dev(wb)), (1, 1, 1, 0), (2, 1))
     st = tsx.StagedPairs(tsx.StagedInput(B, (n, 64, h, w // 2)))
-    A(_dev(xa), dq=_dev(dqa), bias=_dev(ba), act="leaky_relu", slope=0.1, q_scales=_dev(qs), want_f32=False, staged_out=st)
+    if producer == "stem-pairs":
+        # 2 x 32 output channels per pair of columns from a 3x4 window at column stride 2: the same bytes
+        A2 = tsx.Conv2dI8(tsx.pair_outputs_weights(_dev(wa)), pads, (1, 2))
+        A2(_dev(xa), dq=_dev(np.tile(dqa, 2)), bias=_dev(np.tile(ba, 2)), act="leaky_relu", slope=0.1, q_scales=_dev(qs),
+           want_f32=False, staged_out=st.pairs)
+    else:
+        A(_dev(xa), dq=_dev(dqa), bias=_dev(ba), act="leaky_relu", slope=0.1, q_scales=_dev(qs), want_f32=False, staged_out=st)
     got = B.run_staged(st.pairs, _dev(dqb))[0].cpu().numpy()
     fa = port.leaky_relu(port.add_bias(port.conv2d_quantized(xa, wa, dqa, pads), ba), 0.1)
     qa = port.quantize(fa, qs)
