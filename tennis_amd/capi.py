@@ -223,6 +223,19 @@ class StagedPlain:
         self.pad_top = self.pad_left = 0
         self.buf = torch.zeros(n * h * w * self.cp, dtype=torch.int8, device=device)
 
+    def column_pairs(self):
+        """The same buffer as a map of half the width whose pixels are pairs of columns with twice the channels (for a
+        producer that computes pairs of output columns: pair_outputs_weights)."""
+        n, c, h, w = self.x_shape
+        if c != self.cp or w % 2:
+            raise TsxError("column pairs: %d channels in a pitch of %d, width %d" % (c, self.cp, w))
+        v = object.__new__(StagedPlain)
+        v.x_shape = (n, 2 * c, h, w // 2)
+        v.hs, v.ws, v.cp = h, w // 2, 2 * self.cp
+        v.pad_top = v.pad_left = 0
+        v.buf = self.buf
+        return v
+
 
 class StagedSlice:
     """Channels [c0, c0 + channels) of a StagedInput, as the staged output of ONE producer of a channel concatenation:
@@ -296,16 +309,17 @@ def pair_columns_weights(w):
     return wp
 
 
-def pair_outputs_weights(w):
-    """Weights [cout][c][kh][kw] of a convolution with column stride 1, rewritten to produce PAIRS of output columns as
-    one pixel of 2 cout channels: [2 cout][c][kh][kw + 1] for column stride 2 (same padding).  Channels [0, cout) are
-    the even output column (kernel columns 0..kw-1 of the wider window), [cout, 2 cout) the odd one (columns 1..kw); the
-    extra column carries zero weights.  Written as a staged hand-over this is byte for byte the StagedPairs layout; the
-    dequantize scales and the bias are the original ones twice."""
+def pair_outputs_weights(w, stride_w=1):
+    """Weights [cout][c][kh][kw] of a convolution with column stride stride_w, rewritten to produce PAIRS of output
+    columns as one pixel of 2 cout channels: [2 cout][c][kh][kw + stride_w] for column stride 2 stride_w (same
+    padding; an even number of output columns).  Channels [0, cout) are the even output column (kernel columns
+    0..kw-1 of the wider window), [cout, 2 cout) the odd one (columns stride_w..stride_w+kw-1); the other columns carry
+    zero weights.  Written as a staged hand-over this is byte for byte the layout of the unpaired map with cout
+    channels per pixel; the dequantize scales and the bias are the original ones twice."""
     cout, c, kh, kw = w.shape
-    wp = torch.zeros((2 * cout, c, kh, kw + 1), dtype=w.dtype, device=w.device)
+    wp = torch.zeros((2 * cout, c, kh, kw + stride_w), dtype=w.dtype, device=w.device)
     wp[:cout, :, :, :kw] = w
-    wp[cout:, :, :, 1:] = w
+    wp[cout:, :, :, stride_w:] = w
     return wp
 
 

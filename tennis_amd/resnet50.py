@@ -201,8 +201,21 @@ class ResNet50Int8:
             if key not in self._staged:
                 self._staged[key] = capi.StagedPlain((n, stem.cout, h1, w1), self.dev)
             s_stem = self._staged[key]
-            self.conv[stem.name](x, dq=self._dq[stem.name], bias=self.bias[stem.name], act=relu(stem),
-                                 x_scales=sxs[stem.name], q_scales=sxs[c1.name], want_f32=False, staged_out=s_stem)
+            if w1 % 2 == 0 and stem.cout % 64 == 0 and stem.cin * stem.k * (stem.k + stem.stride) <= 512:
+                # the stem computed as pairs of output columns (a k x (k + stride) window at twice the column stride,
+                # 2 x cout channels): the same staged bytes from half as many im2col rows of the same padded length
+                dq1 = self._dq[stem.name]
+                if "stem_pairs" not in self._staged or self._staged["stem_pairs"][1] is not dq1:   # new scales: new dq
+                    pconv = (self._staged["stem_pairs"][0] if "stem_pairs" in self._staged else
+                             capi.Conv2dI8(capi.pair_outputs_weights(self.conv[stem.name].w, stem.stride), (stem.pad,) * 4,
+                                           (stem.stride, 2 * stem.stride)))
+                    self._staged["stem_pairs"] = (pconv, dq1, torch.cat([dq1] * 2), torch.cat([self.bias[stem.name]] * 2))
+                pconv, _, dq2, bias2 = self._staged["stem_pairs"]
+                pconv(x, dq=dq2, bias=bias2, act=relu(stem), x_scales=sxs[stem.name], q_scales=sxs[c1.name],
+                      want_f32=False, staged_out=s_stem.column_pairs())
+            else:
+                self.conv[stem.name](x, dq=self._dq[stem.name], bias=self.bias[stem.name], act=relu(stem),
+                                     x_scales=sxs[stem.name], q_scales=sxs[c1.name], want_f32=False, staged_out=s_stem)
             hp, wp = capi.pool_out_size(h1, w1, self.POOL[0], self.POOL[2], self.POOL[1])
             s_in = self._staged_input(c1, (n, stem.cout, hp, wp))
             capi.max_pooling2d_staged(s_stem, s_in, *self.POOL)

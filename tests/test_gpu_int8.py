@@ -384,6 +384,35 @@ def test_conv2d_i8_staged_hand_over_upsampled_into_a_channel_slice(tsx, port, cm
           staged_out=tsx.StagedSlice(tsx.StagedInput(C, (n, cmid + 32, 2 * h - 2, 2 * w)), 0, cmid, upsample=2))
 
 
+@pytest.mark.parametrize("k,stride,pad,size", [(7, 2, 3, (30, 44)), (3, 1, 1, (9, 12)), (5, 2, 2, (17, 40))])
+def test_conv2d_i8_stem_as_pairs_of_output_columns(tsx, port, k, stride, pad, size):
+    """A few-channel stem computed as pairs of output columns (a k x (k + stride) window at twice the column stride,
+    2 x cout channels, pair_outputs_weights) writes the very bytes the plain stem writes into a pixel-major int8
+    buffer: fused input quantize, bias, ReLU, requantize; values = the operator chain's (oracle)."""
+    import torch
+    rng = np.random.default_rng(433)
+    n, (h, w) = 2, size
+    x = rng.uniform(-1, 1, (n, 3, h, w)).astype(np.float32)
+    wa = rng.integers(-127, 128, (64, 3, k, k)).astype(np.int8)
+    sx = np.full(n, 127.0, np.float32)
+    dqa = (rng.uniform(0.5, 1.5, 64) / (127.0 * 127.0 * k)).astype(np.float32)
+    ba = (0.1 * rng.standard_normal(64)).astype(np.float32)
+    qs = np.full(n, 40.0, np.float32)
+    ho, wo = (h + 2 * pad - k) // stride + 1, (w + 2 * pad - k) // stride + 1
+    assert wo % 2 == 0
+    plain, paired = tsx.StagedPlain((n, 64, ho, wo), "cuda:0"), tsx.StagedPlain((n, 64, ho, wo), "cuda:0")
+    A = tsx.Conv2dI8(_dev(wa), (pad,) * 4, (stride, stride))
+    A(_dev(x), dq=_dev(dqa), bias=_dev(ba), act="relu", x_scales=_dev(sx), q_scales=_dev(qs), want_f32=False, staged_out=plain)
+    A2 = tsx.Conv2dI8(tsx.pair_outputs_weights(_dev(wa), stride), (pad,) * 4, (stride, 2 * stride))
+    A2(_dev(x), dq=_dev(np.tile(dqa, 2)), bias=_dev(np.tile(ba, 2)), act="relu", x_scales=_dev(sx), q_scales=_dev(qs),
+       want_f32=False, staged_out=paired.column_pairs())
+    assert torch.equal(plain.buf, paired.buf)
+    f = port.relu(port.add_bias(port.conv2d_quantized(port.quantize(x, sx), wa, dqa, (pad,) * 4, (stride, stride)), ba))
+    q = port.quantize(f, qs)
+    assert len(np.unique(q)) > 20
+    assert np.array_equal(tsx.staged_interior(paired, range(n)).cpu().numpy(), q)
+
+
 # im2col-staged stem / the same computed as pairs of output columns / window-stationary 1x1 / 3x3
 @pytest.mark.parametrize("producer", ["stem", "stem-pairs", "1x1", "3x3"])
 @pytest.mark.parametrize("size", [(9, 12), (32, 70)])
