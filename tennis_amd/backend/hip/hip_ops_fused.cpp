@@ -143,7 +143,8 @@ public:
         Tensor out_plain;
         if (m_dual) out_plain = stack.make(Tensor::Prototype(FLOAT32, conv_shape), device);
         void *stream = current_stream();
-        const void *packed = m_state.packed(g, w, device, stream, "conv2d_quantized_fused");
+        const bool pairs = pairs_apply(g, gn, out);
+        const void *packed = pairs ? nullptr : m_state.packed(g, w, device, stream, "conv2d_quantized_fused");
         tsx_epilogue ep{};
         ep.dq_dev = m_dq_dev.get(m_dq, device);
         ep.bias_dev = with_bias ? bias.data<float>() : nullptr;
@@ -176,6 +177,50 @@ public:
         if (m_staged_input) {
             check(tsx_conv2d_i8_staged_at(&g, x.data(), x.size(1), x.size(2), packed, &ep, out_f32, nullptr, nullptr, stream),
                   "tsx_conv2d_i8_staged_at");
+        } else if (pairs) {
+            // A few-channel stem whose only output is the staged int8 one: computed as PAIRS of output columns -- a
+            // kh x (kw + stride) window at twice the column stride with 2 x cout output channels (the even column's
+            // weights in window columns 0..kw-1, the odd one's in stride..stride+kw-1, zeros elsewhere, which add
+            // nothing to an integer sum).  A pair's 2 x cout channels are the two pixels' bytes in the staged layout,
+            // so the output is the same; the explicit im2col matrix has half the rows of the same padded length.
+            tsx_conv2d_geom g2 = g;
+            g2.kw = g.kw + g.stride_w;
+            g2.stride_w = 2 * g.stride_w;
+            g2.cout = 2 * g.cout;
+            if (m_pair_w.empty() || m_pair_source.data() != w.data() || m_pair_w.device() != device) {
+                const Tensor hw = w.view(MemoryDevice(CPU));
+                std::vector<int8_t> w2(size_t(g2.cout) * g.c * g.kh * g2.kw, 0);
+                const int8_t *src = hw.data<int8_t>();
+                for (int co = 0; co < g.cout; ++co)
+                    for (int r = 0; r < g.c * g.kh; ++r)
+                        for (int kx = 0; kx < g.kw; ++kx) {
+                            const int8_t v = src[(size_t(co) * g.c * g.kh + r) * g.kw + kx];
+                            w2[(size_t(co) * g.c * g.kh + r) * g2.kw + kx] = v;
+                            w2[(size_t(g.cout + co) * g.c * g.kh + r) * g2.kw + g.stride_w + kx] = v;
+                        }
+                m_pair_w = tensor::build(INT8, Shape({g2.cout, g.c, g.kh, g2.kw}), w2.data()).view(device);
+                m_pair_source = w;
+                m_pair_dq = m_dq;
+                m_pair_dq.insert(m_pair_dq.end(), m_dq.begin(), m_dq.end());
+            }
+            if (with_bias && (m_pair_bias.empty() || m_pair_bias_source.data() != bias.data() || m_pair_bias.device() != device)) {
+                const Tensor hb = bias.view(MemoryDevice(CPU));
+                std::vector<float> b2(hb.data<float>(), hb.data<float>() + g.cout);
+                b2.insert(b2.end(), hb.data<float>(), hb.data<float>() + g.cout);
+                m_pair_bias = tensor::build(FLOAT32, Shape({g2.cout}), b2.data()).view(device);
+                m_pair_bias_source = bias;
+            }
+            const void *packed2 = m_pair_state.packed(g2, m_pair_w, device, stream, "conv2d_quantized_fused");
+            ep.dq_dev = m_pair_dq_dev.get(m_pair_dq, device);
+            ep.bias_dev = with_bias ? m_pair_bias.data<float>() : nullptr;
+            ep.staged_ws = out.size(2) / 2;
+            ep.staged_cp = 2 * out.size(3);
+            ep.staged_pad_left = gn.pad_left / 2;
+            const size_t ws_bytes = tsx_conv2d_i8_workspace_bytes(&g2);
+            void *workspace = m_pair_state.workspace(ws_bytes, device);
+            check(tsx_quantize_conv2d_i8_nchw(&g2, x.data<float>(), m_q_dev.get(m_q, device), int32_t(m_q.size()), packed2,
+                                              m_padding_value, &ep, nullptr, nullptr, nullptr, workspace, ws_bytes, stream),
+                  "tsx_quantize_conv2d_i8_nchw");
         } else {
             const size_t ws_bytes = tsx_conv2d_i8_workspace_bytes(&g);
             void *workspace = m_state.workspace(ws_bytes, device);
@@ -204,6 +249,19 @@ private:
         const std::vector<int32_t> v = tensor::array::to_int(get(param));
         if (v.size() != count) TS_LOG_ERROR << "conv2d_quantized_fused: " << param << " must hold " << count << " integers" << eject;
         return v;
+    }
+
+    // the stem-as-pairs form applies: fp32 input of few channels, a kernel wider than one tap, only the staged int8
+    // output, an even number of output columns that pair up with whole staged pixels, and a window whose K pads to the
+    // same number of 64-byte steps
+    bool pairs_apply(const tsx_conv2d_geom &g, const tsx_conv2d_geom &gn, const Tensor &out) const {
+        if (!m_next || m_dual || m_residual || m_staged_input) return false;
+        if (g.c > 8 || g.kh * g.kw <= 1 || g.dilation_h != 1 || g.dilation_w != 1) return false;
+        if (m_wo % 2 || gn.pad_left % 2 || out.size(2) % 2 || out.size(3) != g.cout || g.cout % 32) return false;
+        const int k1 = g.c * g.kh * g.kw, k2 = g.c * g.kh * (g.kw + g.stride_w);
+        if ((k1 + 63) / 64 != (k2 + 63) / 64 || k2 > 512) return false;
+        const int wo2 = (g.w + g.pad_left + g.pad_right - (g.kw + g.stride_w)) / (2 * g.stride_w) + 1;
+        return wo2 == m_wo / 2;
     }
 
     // checks the inputs against the parameters; fills the geometry (and, with next_*, the consumer's); returns the
@@ -289,6 +347,11 @@ private:
     std::vector<float> m_dq, m_q;
     DeviceFloats m_dq_dev, m_q_dev;
     PackedConv m_state;
+    // the stem computed as pairs of output columns: rearranged weights, scales and bias, and their pack
+    PackedConv m_pair_state;
+    Tensor m_pair_w, m_pair_source, m_pair_bias, m_pair_bias_source;
+    std::vector<float> m_pair_dq;
+    DeviceFloats m_pair_dq_dev;
 };
 
 // max_pooling2d_staged: a MAX pooling2d node (src/kernels/cpu/pooling2d_core.cpp:48-93) between a fused producer and

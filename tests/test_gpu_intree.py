@@ -213,6 +213,26 @@ def test_resnet_shaped_module_in_tennis_workbench_on_hip(ts, tmp_path):
     assert np.array_equal(bits(fused), bits(own))
 
 
+def test_full_width_stem_as_column_pairs_in_tennis_workbench_on_hip(ts, tmp_path):
+    """The same at full width (one bottleneck per stage): with 64 output channels and an even number of output
+    columns the fused stem node runs as pairs of output columns (rearranged weights, half the im2col rows) into the
+    staged max pooling.  Bitwise equal to the operator-by-operator run of the same device operators, which has no
+    such form, and within the classifier's tolerance of TenniS's CPU device."""
+    from tennis_amd import module_file as mf, resnet50
+    desc, params = resnet50.make_parameters(seed=5, width=1.0, blocks=(1, 1, 1, 1), classes=10)
+    module = resnet50.to_module(desc, params, batch=2)
+    path = str(tmp_path / "resnet_full_width.tsm")
+    mf.write_module(path, module)
+    x = np.random.default_rng(2).random((2, 3, 64, 64), dtype=np.float32)
+    cpu = ts.run_module_intree("cpu", path, [x])
+    hand0, _ = ts.handover_counts_intree()
+    hip = ts.run_module_intree("hip", path, [x])
+    assert ts.handover_counts_intree()[0] > hand0
+    assert cpu.shape == (2, 10) and np.abs(cpu).max() > 0.1 and close(hip, cpu)
+    (own,) = mf.run_module(module, [x])
+    assert np.array_equal(bits(own), bits(hip))
+
+
 def test_zipper_option_leaky_relu_and_shared_convolution(ts, tmp_path):
     """The graph compiler's rewrite on the cases the fixtures do not hold: a chain that ends in leaky_relu behind an
     add_bias given by `dim`, and a convolution whose output has two readers (a relu and an add_bias), where only
