@@ -366,13 +366,15 @@ class YoloV4Int8:
                     kw.update(residual=outs[rsrcs[absorbed[i]][1]], residual_after_act=True)
                 cin = self.conv[i].w.shape[1]
                 if (isinstance(target, capi.StagedPairs) and not want_f32 and i not in absorbed and i not in staged_for
-                        and l["size"] == 3 and l["stride"] == 1 and cin * 12 <= 64):
+                        and l["size"] == 3 and l["stride"] == 1 and cin * 3 * 4 <= 64):
                     # the stem in front of a pair-staged layer: computed as pairs of output columns (a 3x4 window at column
-                    # stride 2, 2 x 32 output channels), so that its im2col rows are per pair -- half the staged bytes
-                    if i not in self._pair_prod:
-                        self._pair_prod[i] = (capi.Conv2dI8(capi.pair_outputs_weights(self.conv[i].w), (1, 1, 1, 1), (1, 2)),
-                                              torch.cat([self.dq[i], self.dq[i]]), torch.cat([self.bias[i], self.bias[i]]))
-                    pconv, dq2, bias2 = self._pair_prod[i]
+                    # stride 2, 2 x 32 output channels; its K still fits one 64-byte step), so that its im2col rows are
+                    # per pair -- half the staged bytes
+                    if i not in self._pair_prod or self._pair_prod[i][1] is not self.dq[i]:      # new scales: new dq
+                        pconv = (self._pair_prod[i][0] if i in self._pair_prod else
+                                 capi.Conv2dI8(capi.pair_outputs_weights(self.conv[i].w), (1, 1, 1, 1), (1, 2)))
+                        self._pair_prod[i] = (pconv, self.dq[i], torch.cat([self.dq[i]] * 2), torch.cat([self.bias[i]] * 2))
+                    pconv, _, dq2, bias2 = self._pair_prod[i]
                     pconv(get(src), x_scales=self.sx[i], dq=dq2, bias=bias2, act=l["act"], slope=0.1, want_f32=False,
                           q_scales=self.sx[q_layer], staged_out=target.pairs)
                     y = None
