@@ -143,22 +143,18 @@ __device__ __forceinline__ float mish_value(float x) {
 }
 
 // Mish for the epilogues of the int8 convolution kernels, where the activation's arithmetic, not memory or the MFMAs,
-// bounds a layer (the 608x608 and 304x304 layers of a YOLOv4-shaped backbone spend more issue slots on mish_value than
-// on everything else): one exponential and one division,
-//     tanh(softplus(x)) = w / (w + 2),  w = e (e + 2),  e = e^x,
-// with the quotient (correctly rounded but for rare ties) then brought onto the grid the host's tanh lives on:
-// 2 * (1 / (1 + u)) - 1 with 1 / (1 + u) in [0.5, 1] is a multiple of 2^-23, which (t + 1) - 1 reproduces -- including
-// the host's 0 (and so -0 for the product) once x is below about -17.  Three quarters of all results are the host's
-// bit for bit; the others are one grid step of tanh away (1.2e-7 |x|, at most 2e-6 where x is near -17), the same
-// distance the host's own rounding keeps from the exact function there.  NaN -> NaN, +-inf as the host's.
+// bounds a layer (the 608x608 and 304x304 layers of a YOLOv4-shaped backbone spend more issue slots on the epilogue
+// than the VALUs have in the time the layer's bytes take): one exponential and one reciprocal at the hardware's 1 ulp,
+//     tanh(softplus(x)) = w / (w + 2),  w = e (e + 2),  e = e^x = 2^(x log2 e),
+// 17 issue slots.  Relative error of the result about 2e-7 (the rounding of x log2 e reaches e as |x| 4e-8, which
+// matters only where tanh(softplus) follows e, i.e. for negative x where Mish itself is small), against a bar of
+// 1e-4 relative + 1e-5 absolute.  (t + 1) - 1 puts the quotient on the 2^-23 grid the host's tanh lives on
+// (2 * (1 / (1 + u)) - 1 with the reciprocal in [0.5, 1]) and so gives the host's 0 (-0 for the product) once x is
+// below about -17.  NaN -> NaN, +-inf as the host's.
 __device__ __forceinline__ float mish_short(float x) {
-    const float e = mish_exp(fminf(x, 30.f));              // beyond 30 (long before, in fact) the quotient is 1
+    const float e = __builtin_amdgcn_exp2f(__fmul_rn(fminf(x, 30.f), 1.4426950216293335f));   // beyond 30 the quotient is 1
     const float w = __fmul_rn(e, __fadd_rn(e, 2.f));
-    const float d = __fadd_rn(w, 2.f);
-    const float r0 = __builtin_amdgcn_rcpf(d);
-    const float r = __builtin_fmaf(r0, __builtin_fmaf(-d, r0, 1.f), r0);
-    const float q = __fmul_rn(w, r);
-    const float t = __builtin_fmaf(__builtin_fmaf(-d, q, w), r, q);   // remainder correction of the quotient
+    const float t = __fmul_rn(w, __builtin_amdgcn_rcpf(__fadd_rn(w, 2.f)));
     return __fmul_rn(x, __fsub_rn(__fadd_rn(t, 1.f), 1.f));
 }
 
