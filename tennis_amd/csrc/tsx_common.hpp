@@ -145,17 +145,17 @@ __device__ __forceinline__ float mish_value(float x) {
 // Mish for the epilogues of the int8 convolution kernels, where the activation's arithmetic, not memory or the MFMAs,
 // bounds a layer (the 608x608 and 304x304 layers of a YOLOv4-shaped backbone spend more issue slots on the epilogue
 // than the VALUs have in the time the layer's bytes take): one exponential and one reciprocal at the hardware's 1 ulp,
-//     tanh(softplus(x)) = w / (w + 2),  w = e (e + 2),  e = e^x = 2^(x log2 e),
-// 17 issue slots.  Relative error of the result about 2e-7 (the rounding of x log2 e reaches e as |x| 4e-8, which
-// matters only where tanh(softplus) follows e, i.e. for negative x where Mish itself is small), against a bar of
-// 1e-4 relative + 1e-5 absolute.  (t + 1) - 1 puts the quotient on the 2^-23 grid the host's tanh lives on
-// (2 * (1 / (1 + u)) - 1 with the reciprocal in [0.5, 1]) and so gives the host's 0 (-0 for the product) once x is
-// below about -17.  NaN -> NaN, +-inf as the host's.
+//     tanh(softplus(x)) = w / (w + 2) = 1 - 2 / (w + 2),  w = e (e + 2),  e = e^x = 2^(x log2 e),
+// 14 issue slots.  1 - 2r with r = 1 / (w + 2) in (0, 0.5] has the shape of the host's tanh, 2 * (1 / (1 + u)) - 1
+// (src/kernels/cpu/tanh.cpp:14-23): an absolute error of about 1e-7 in the quotient, so about 1e-7 |x| in the result
+// (relative 1e-7 for positive x; at most 2e-6 absolute for negative x, where Mish itself is small), against a bar of
+// 1e-4 relative + 1e-5 absolute -- and, like the host's, exactly 0 (-0 for the product) once x is below about -17,
+// where w + 2 rounds to 2.  NaN -> NaN, +-inf as the host's.
 __device__ __forceinline__ float mish_short(float x) {
     const float e = __builtin_amdgcn_exp2f(__fmul_rn(fminf(x, 30.f), 1.4426950216293335f));   // beyond 30 the quotient is 1
-    const float w = __fmul_rn(e, __fadd_rn(e, 2.f));
-    const float t = __fmul_rn(w, __builtin_amdgcn_rcpf(__fadd_rn(w, 2.f)));
-    return __fmul_rn(x, __fsub_rn(__fadd_rn(t, 1.f), 1.f));
+    const float d = __builtin_fmaf(e, __fadd_rn(e, 2.f), 2.f);
+    const float t = __builtin_fmaf(-2.f, __builtin_amdgcn_rcpf(d), 1.f);
+    return __fmul_rn(x, t);
 }
 
 // apply_act for the int8 convolution epilogues: Mish in its short form (every path of those kernels -- fragment-wise
