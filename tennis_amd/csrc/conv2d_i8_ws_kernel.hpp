@@ -492,19 +492,22 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
                         else *o = v[r];
                     });
                     if (!ROWM && want_q) {
-                        int qv[16];
+                        // the 16 requantized values as 4 dwords of 4 consecutive channels (quantize_pack: the value of
+                        // quantize_value, converted, clamped and packed by one instruction)
+                        uint32_t word[4] = {0u, 0u, 0u, 0u};
                         if (q_even) static_for<0, 16>([&](auto rc) {
                             constexpr int r = decltype(rc)::value;
-                            qv[r] = quantize_value(__fmul_rn(v[r], q_scale), true);
+                            word[r / 4] = quantize_pack<r % 4>(__fmul_rn(v[r], q_scale), true, word[r / 4]);
                         });
                         else static_for<0, 16>([&](auto rc) {
                             constexpr int r = decltype(rc)::value;
-                            qv[r] = quantize_value(__fmul_rn(v[r], q_scale), false);
+                            word[r / 4] = quantize_pack<r % 4>(__fmul_rn(v[r], q_scale), false, word[r / 4]);
                         });
+                        static_for<0, 4>([&](auto gc) { word[decltype(gc)::value] ^= 0x80808080u; });
                         if (p.out_i8) static_for<0, 16>([&](auto rc) {
                             constexpr int r = decltype(rc)::value;
                             constexpr int dco = 8 * (r / 4) + (r % 4);
-                            (p.out_i8 + tile_base + int64_t(dco) * howo)[lane_off] = int8_t(qv[r]);
+                            (p.out_i8 + tile_base + int64_t(dco) * howo)[lane_off] = int8_t(word[r / 4] >> (8 * (r % 4)));
                         });
                         if (EXTRA && p.st_out) {
                             // consumer's staged layout [pixel][channel].  Accumulator registers 4g..4g+3 of a lane are 4
@@ -512,12 +515,6 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
                             // fragment sit in lane +-32.  Two half-wave swaps leave every lane with 16 consecutive
                             // channels -- lower half cf..cf+15, upper half cf+16..cf+31 -- for one 16-byte store
                             // (4-byte stores at a pixel stride cost an L2 request each).
-                            uint32_t word[4];
-                            static_for<0, 4>([&](auto gc) {
-                                constexpr int g4 = decltype(gc)::value;
-                                word[g4] = uint32_t(qv[4 * g4] & 0xff) | (uint32_t(qv[4 * g4 + 1] & 0xff) << 8) |
-                                           (uint32_t(qv[4 * g4 + 2] & 0xff) << 16) | (uint32_t(qv[4 * g4 + 3] & 0xff) << 24);
-                            });
                             // swap(a, b): a's upper half-wave <-> b's lower half-wave
                             const auto s02 = __builtin_amdgcn_permlane32_swap(word[0], word[2], false, false);
                             const auto s13 = __builtin_amdgcn_permlane32_swap(word[1], word[3], false, false);

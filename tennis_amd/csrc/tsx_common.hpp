@@ -77,6 +77,18 @@ __device__ __forceinline__ int quantize_value(float v, bool half_even) {
     return in_range ? int(c) : -128;
 }
 
+// Byte SEL of `word` := quantize_value(v, half_even) + 128 (offset binary; the caller XORs the finished word with
+// 0x80808080): the conversion instruction saturates to [0, 255] and packs, so clamp, conversion and packing are one
+// instruction.  r + 128 is exact wherever the clamp does not apply anyway; NaN and |v| >= 2^31 give byte 0 = -128, the
+// reference's INT_MIN after its clamp, as in quantize_value.
+template <int SEL>
+__device__ __forceinline__ uint32_t quantize_pack(float v, bool half_even, uint32_t word) {
+    const float away = __builtin_truncf(v + __builtin_copysignf(0.49999997f, v));
+    const float r = half_even ? __builtin_rintf(v) : away;
+    const bool in_range = __builtin_fabsf(v) < 2147483648.0f;   // false for NaN as well
+    return __builtin_amdgcn_cvt_pk_u8_f32(in_range ? __fadd_rn(r, 128.f) : 0.f, SEL, word);
+}
+
 // relu / leaky_relu of element `in_body` (= linear index < 4*floor(count/4) of the whole
 // tensor): SIMD body vs scalar tail of src/kernels/cpu/relu.cpp:30-52 and
 // leaky_relu.cpp:41-66.  Body: max(x,0) returns +0 for -0 and NaN; the leaky form is one
