@@ -48,15 +48,22 @@ def sources():
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
-def build(verbose=True, jobs=8):
+def build(verbose=True, jobs=8, incremental=False):
+    """Compiles every kernel source and links the library.  incremental=True (development only) keeps an object
+    file that is newer than its source and every header."""
     os.makedirs(LIB_DIR, exist_ok=True)
     obj_dir = os.path.join(LIB_DIR, "obj")
     os.makedirs(obj_dir, exist_ok=True)
     procs = []
     objs = []
+    headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hpp", ".h"))]
+    headers.append(os.path.join(ROOT, "include", "tsx_hip.h"))
+    newest_header = max(os.path.getmtime(h) for h in headers)
     for src in sources():
         obj = os.path.join(obj_dir, os.path.basename(src)[:-4] + ".o")
         objs.append(obj)
+        if incremental and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(src), newest_header):
+            continue
         cmd = [HIPCC] + FLAGS + ["-c", src, "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
@@ -122,4 +129,4 @@ def build_backend(verbose=True):
 
 
 if __name__ == "__main__":
-    build()
+    build(incremental="--incremental" in sys.argv[1:])

@@ -116,9 +116,11 @@ def lib():
     """Load libtsx_hip.so (built in-tree by `python -m tennis_amd.build`); never falls back."""
     global _lib
     if _lib is None:
-        if not os.path.exists(LIB_PATH):
-            raise TsxError("libtsx_hip.so is not built: run `python -m tennis_amd.build` (no CPU fallback exists)")
-        L = ctypes.CDLL(LIB_PATH)
+        # TSX_HIP_LIBRARY: another build of the same library (the measurement build with phase stamps and probes)
+        path = os.environ.get("TSX_HIP_LIBRARY") or LIB_PATH
+        if not os.path.exists(path):
+            raise TsxError("%s is not built: run `python -m tennis_amd.build` (no CPU fallback exists)" % path)
+        L = ctypes.CDLL(path)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(L, name)
             fn.restype = res

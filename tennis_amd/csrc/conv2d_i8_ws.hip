@@ -166,6 +166,7 @@ WsPlan ws_plan(const WsGeom &g_in) {
     pl.packed_bytes = size_t(pl.ksteps_p) * pl.coutp * 64;
     pl.ok = true;
     fl_plan(g_in, &pl);   // layers the flat-tile kernel suits better (same packed weights)
+    rs_plan(g_in, &pl);   // ... and the weight-stationary one
     return pl;
 }
 
@@ -179,6 +180,7 @@ int ws_pack_weights(const WsGeom &g, const WsPlan &pl, const int8_t *w_oihw, int
 
 int ws_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t *packed, const EpiParams &ep,
               hipStream_t stream) {
+    if (rs_takes(pl, ep, int64_t(g.n) * g.cout * g.ho * g.wo)) return rs_launch(g, pl, xs, packed, ep, stream);
     if (pl.flat) return fl_launch(g, pl, xs, packed, ep, stream);
     WsParams p{};
     static_cast<EpiParams &>(p) = ep;

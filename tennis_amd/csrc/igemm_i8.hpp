@@ -170,6 +170,10 @@ struct WsPlan {
     bool flat, fl_resident;
     int fl_nta, fl_ntb, fl_wr, fl_wc, fl_wp, fl_rowp;
     int64_t fl_tiles;
+    // weight-stationary kernel (conv2d_i8_rs.hip) for the epilogues it writes: a tile is rs_frags consecutive
+    // fragments x 64 output channels; same packed weights
+    bool rs;
+    int rs_frags, rs_ptiles, rs_nr, rs_rowp, rs_wc, rs_lds;
 };
 
 struct WsGeom {
@@ -186,6 +190,12 @@ int ws_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t 
 // flat-tile kernel: fills the fl_* fields of a valid plan when the layer suits it; launch
 void fl_plan(const WsGeom &g, WsPlan *pl);
 int fl_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t *packed, const EpiParams &ep,
+              hipStream_t stream);
+// weight-stationary kernel: fills the rs_* fields of a valid plan when the layer suits it; whether it writes a
+// given epilogue; launch
+void rs_plan(const WsGeom &g, WsPlan *pl);
+bool rs_takes(const WsPlan &pl, const EpiParams &ep, int64_t count);
+int rs_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t *packed, const EpiParams &ep,
               hipStream_t stream);
 
 }  // namespace tsx
