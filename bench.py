@@ -108,45 +108,67 @@ def cpu_baseline_all_cores(x, x_scales, wq, dq, bias, pad):
                       "every loop" % (x.shape[0], dt), "host_cpus": os.cpu_count()}
 
 
-def config1_leg(reps=50):
-    """BASELINE config 1: fp32 conv2d 1x64x56x56 * 64x64x3x3, stride 1, pad 1, bias + ReLU -- the implicit im2col
-    GEMM on the fp32 MFMA, both Winograd modes in their bit-exact form and F(6,3) as one MFMA launch (all credited the
-    direct convolution's flops), time per launch from HIP events around back-to-back launches."""
+def _fp32_conv_rows(shape_x, shape_w, reps, seed):
+    """conv2d_f32 (implicit im2col GEMM on the fp32 MFMA), both Winograd modes in their bit-exact form and F(6,3) as
+    one MFMA launch on one 3x3 / stride 1 / pad 1 layer with bias + ReLU, all credited the direct convolution's
+    flops; seconds per launch = median of 5 batches of `reps` back-to-back launches between events."""
     import torch
     from tennis_amd import capi
     dev = torch.device("cuda:0")
-    g = torch.Generator(device="cuda").manual_seed(5)
-    x = torch.rand((1, 64, 56, 56), device=dev, generator=g) * 2 - 1
-    w = torch.randn((64, 64, 3, 3), device=dev, generator=g) * (2.0 / 576) ** 0.5
-    b = torch.randn(64, device=dev, generator=g) * 0.01
-    flops = 2.0 * 64 * 56 * 56 * 64 * 9
-    w63, w23 = capi.WinogradF63(w, (1, 1, 1, 1)), capi.WinogradF23(w, (1, 1, 1, 1))
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    n, c, h, w = shape_x
+    cout = shape_w[0]
+    x = torch.rand(shape_x, device=dev, generator=g) * 2 - 1
+    wt = torch.randn(shape_w, device=dev, generator=g) * (2.0 / (9 * c)) ** 0.5
+    b = torch.randn(cout, device=dev, generator=g) * 0.01
+    flops = 2.0 * n * cout * h * w * c * 9
+    w63, w23 = capi.WinogradF63(wt, (1, 1, 1, 1)), capi.WinogradF23(wt, (1, 1, 1, 1))
     rows = {}
-    for name, fn in (("im2col_gemm", lambda: capi.conv2d_f32(x, w, (1, 1, 1, 1), bias=b, act="relu")),
+    for name, fn in (("im2col_gemm", lambda: capi.conv2d_f32(x, wt, (1, 1, 1, 1), bias=b, act="relu")),
                      ("winograd_f63", lambda: w63(x, bias=b, act="relu")), ("winograd_f23", lambda: w23(x, bias=b, act="relu")),
                      ("winograd_f63_fast", lambda: w63(x, bias=b, act="relu", fast=True))):
         for _ in range(3):
             fn()
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(reps):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        t = e0.elapsed_time(e1) * 1e-3 / reps
+        per = []
+        for _ in range(5):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            per.append(e0.elapsed_time(e1) * 1e-3 / reps)
+        t = float(np.median(per))
         rows[name] = {"us": t * 1e6, "GFLOPS": flops / t / 1e9, "frac_of_fp32_mfma_peak": flops / t / 1e12 / PEAK_FP32_TFLOPS}
-    return {"workload": "BASELINE config 1: fp32 conv2d 1x64x56x56 * 64x64x3x3 s1 p1 + bias + ReLU; 231.2 MFLOP per launch "
-                        "(Winograd credited the same), 49 tiles of 64x64: a batch of one cannot fill 256 CUs", "reps": reps,
-            "peak_TFLOPS": PEAK_FP32_TFLOPS, **rows}
+    return flops, rows
 
 
-def ceiling_evidence(L, conv_launch, event_time, conv_ops, dev, stream):
-    """What bounds the config-2 MFMA kernel, measured: (1) the rate of a register-only MFMA loop against the number of
-    busy CUs and the operand data (the clock the part grants falls with both), (2) where one launch of the kernel
-    spends its time, per wavefront, from wall-clock and shader-clock stamps the kernel writes when asked
-    (tsx_debug_phase_stamps).  `python bench.py --ceiling`; under rocprofv3 --pmc GRBM_GUI_ACTIVE the same run gives
-    cycles / duration for the probe and the kernel from the counters' side."""
+def config1_leg(reps=50):
+    """BASELINE config 1: fp32 conv2d 1x64x56x56 * 64x64x3x3, stride 1, pad 1, bias + ReLU."""
+    flops, rows = _fp32_conv_rows((1, 64, 56, 56), (64, 64, 3, 3), reps, 5)
+    return {"workload": "BASELINE config 1: fp32 conv2d 1x64x56x56 * 64x64x3x3 s1 p1 + bias + ReLU; %.1f MFLOP per launch "
+                        "(Winograd credited the same), 49 tiles of 64x64: a batch of one cannot fill 256 CUs" % (flops / 1e6),
+            "reps": reps, "peak_TFLOPS": PEAK_FP32_TFLOPS, **rows}
+
+
+def winograd_shape_leg(reps=20):
+    """A layer the reference's own selector gives to Winograd F(6,3) (winograd_mode_select_on_arm,
+    src/kernels/common/function.cpp:154-173: Cin * Cout >= 65536 and a map larger than 16 x 16): 8x256x28x28 *
+    256x256x3x3, stride 1, pad 1, bias + ReLU -- the same four kernels as on config 1."""
+    flops, rows = _fp32_conv_rows((8, 256, 28, 28), (256, 256, 3, 3), reps, 6)
+    return {"workload": "fp32 conv2d 8x256x28x28 * 256x256x3x3 s1 p1 + bias + ReLU (a shape the reference routes to Winograd "
+                        "F(6,3)); %.2f GFLOP per launch by the direct convolution's count" % (flops / 1e9),
+            "reps": reps, "peak_TFLOPS": PEAK_FP32_TFLOPS, **rows}
+
+
+def ceiling_evidence(A, conv_launch, event_time, conv_ops, dev, stream, frags):
+    """What bounds the config-2 MFMA kernel, measured on the measurement build of the library (A; `python -m
+    tennis_amd.build --aids`): (1) the rate of a register-only MFMA loop against the number of busy CUs and the
+    operand data (the clock the part grants falls with both), (2) where one launch of the weight-stationary kernel
+    spends its time, per wavefront, from wall-clock and shader-clock stamps that build's kernel writes.
+    `python bench.py --ceiling`; under rocprofv3 --pmc GRBM_GUI_ACTIVE the same run gives cycles / duration for the
+    probe and the kernel from the counters' side."""
     import torch
     from tennis_amd import capi
     sink = torch.zeros(4, dtype=torch.int32, device=dev)
@@ -158,62 +180,63 @@ def ceiling_evidence(L, conv_launch, event_time, conv_ops, dev, stream):
         else:
             operands = torch.randint(-128, 128, (32768,), dtype=torch.int8, device=dev)
         for blocks in (64, 128, 224, 256, 512, 1024):
-            t = event_time(lambda: capi.check(L.tsx_probe_mfma_i8(capi._ptr(operands), iters, blocks, capi._ptr(sink), stream)), 3)
+            t = event_time(lambda: capi.check(A.tsx_probe_mfma_i8(capi._ptr(operands), iters, blocks, capi._ptr(sink), stream)), 3)
             rate = blocks * 4 * iters * 8 * 65536.0 / t
             simds = min(blocks * 4, 1024)      # a workgroup of 4 wavefronts fills one CU's SIMDs; beyond 256 they queue up
             probe.append({"operands": data, "workgroups": blocks, "POP_per_s": rate / 1e15,
                           "GHz_equivalent_per_busy_simd": rate / simds / 2048 / 1e9})
     t_conv = event_time(conv_launch, 50)
-    slots = 8192 * 8
+    slots = 256 * 8 * 24 * 2                         # [workgroup][wavefront][24 stamps][wall clock, shader clock]
     stamps = torch.zeros(slots, dtype=torch.int64, device=dev)
-    capi.check(L.tsx_debug_phase_stamps(capi._ptr(stamps), slots * 8))
+    capi.check(A.tsx_debug_phase_stamps(capi._ptr(stamps), slots * 8))
     try:
-        t_stamped = event_time(conv_launch, 20)      # the stamps of the last of 21 back-to-back launches remain
+        t_stamped = event_time(conv_launch, 20)      # the stamps of the last launch remain
     finally:
-        capi.check(L.tsx_debug_phase_stamps(None, 0))
-    st = stamps.cpu().numpy().reshape(-1, 8, 8)      # [workgroup][wavefront][4 x (wall, clock)]
-    st = st[st[:, 0, 0] != 0]                        # workgroups beyond the last tile leave at once
-    wall, clk = st[:, :, 0::2].astype(np.float64) * 10.0, st[:, :, 1::2].astype(np.float64)   # ns (100 MHz), cycles
+        capi.check(A.tsx_debug_phase_stamps(None, 0))
+    st = stamps.cpu().numpy().reshape(-1, 8, 24, 2)
+    st = st[st[:, 0, 0, 0] != 0]                     # workgroups beyond the last tile leave at once
+    wall, clk = st[..., 0].astype(np.float64) * 10.0, st[..., 1].astype(np.float64)   # ns (100 MHz), cycles
     t_first = wall[:, :, 0].min()
 
     def stats(v):
         return {"mean": float(v.mean()), "min": float(v.min()), "max": float(v.max())}
 
-    phases = {}
-    for name, waves in (("wavefronts 0-3 (4 fragments)", slice(0, 4)), ("wavefronts 4-7 (3 fragments)", slice(4, 8))):
-        w, c = wall[:, waves], clk[:, waves]
-        loop_ns = w[:, :, 2] - w[:, :, 1]
-        phases[name] = {
-            "entry_after_first_wavefront_ns": stats(w[:, :, 0] - t_first),
-            "prologue_ns": stats(w[:, :, 1] - w[:, :, 0]),
-            "k_loop_ns": stats(loop_ns),
-            "epilogue_until_stores_left_ns": stats(w[:, :, 3] - w[:, :, 2]),
-            "end_after_first_wavefront_ns": stats(w[:, :, 3] - t_first),
-            "k_loop_shader_cycles": stats(c[:, :, 2] - c[:, :, 1]),
-            "k_loop_clock_GHz": float(((c[:, :, 2] - c[:, :, 1]) / loop_ns).mean()),
-            "prologue_clock_GHz": float(((c[:, :, 1] - c[:, :, 0]) / (w[:, :, 1] - w[:, :, 0])).mean()),
-            "epilogue_clock_GHz": float(((c[:, :, 3] - c[:, :, 2]) / (w[:, :, 3] - w[:, :, 2])).mean()),
-        }
-    steps_per_simd = 36 * 2 * 7      # K-steps x halves x fragments of the two wavefronts of a SIMD
-    return {"workload": "BASELINE config 2 MFMA kernel (conv_i8_fl_kernel<4,3>): ceiling evidence",
+    mul, srv = wall[:, :4], wall[:, 4:]              # wavefronts 0-3 multiply, 4-7 serve (rows in, results out)
+    last_m, last_s = 1 + frags, 1 + frags + 2
+    per_fragment = np.diff(mul[:, :, 1:last_m + 1], axis=2)
+    phases = {
+        "entry_after_first_wavefront_ns": stats(wall[:, :, 0] - t_first),
+        "multiplying": {
+            "weights_to_registers_and_first_rows_ns": stats(mul[:, :, 1] - mul[:, :, 0]),
+            "fragment_ns": stats(per_fragment), "first_fragment_ns": stats(per_fragment[:, :, 0]),
+            "all_fragments_ns": stats(mul[:, :, last_m] - mul[:, :, 1]),
+            "shader_clock_GHz_in_the_loop": float(((clk[:, :4, last_m] - clk[:, :4, 1]) / (mul[:, :, last_m] - mul[:, :, 1])).mean())},
+        "serving": {
+            "ring_prologue_ns": stats(srv[:, :, 1] - srv[:, :, 0]),
+            "round_ns": stats(np.diff(srv[:, :, 1:1 + frags + 1], axis=2)),
+            "last_sums_to_stores_issued_ns": stats(srv[:, :, last_s - 1] - srv[:, :, last_s - 2]),
+            "stores_issued_to_stores_left_ns": stats(srv[:, :, last_s] - srv[:, :, last_s - 1])},
+        "end_after_first_wavefront_ns": stats(srv[:, :, last_s] - t_first),
+    }
+    return {"workload": "BASELINE config 2 MFMA kernel (conv_i8_rs_kernel, %d fragments per tile): ceiling evidence" % frags,
             "mfma_probe": probe,
             "kernel_us": t_conv * 1e6, "kernel_us_with_stamps": t_stamped * 1e6,
             "kernel_TOP_per_s": conv_ops / t_conv / 1e12,
             "workgroups_with_stamps": int(st.shape[0]),
             "phases": phases,
-            "k_loop_mfma_cycles_per_simd": steps_per_simd * 32,
-            "note": "wall clock = s_memrealtime (10 ns ticks), shader clock = s_memtime; k_loop_mfma_cycles_per_simd is "
-                    "what the loop's MFMAs alone occupy a SIMD's pipe for (504 v_mfma_i32_32x32x32_i8 x 32 cycles)"}
+            "fragment_mfma_cycles_per_simd": 36 * 32,
+            "note": "wall clock = s_memrealtime (10 ns ticks), shader clock = s_memtime; a stamp costs the wavefront "
+                    "150-300 cycles, so the stamped kernel runs longer than the plain one; fragment_mfma_cycles_per_simd "
+                    "is what one fragment's MFMAs alone occupy a SIMD's pipe for (36 v_mfma_i32_32x32x32_i8 x 32 cycles)"}
 
 
 def tennis_runtime_leg(reps=5):
     """The ResNet-50-shaped network (BASELINE config 4) as a `.tsm` module through TenniS's own loader, graph compiler
-    and Workbench on ComputingDevice("hip") -- the operator boundary as a TenniS user meets it (in-tree build of the
-    backend, oracle/ref.mk `intree`; absent where that library was not built)."""
+    and Workbench on ComputingDevice("hip") -- the operator boundary as a TenniS user meets it (TenniS built with this
+    repository's backend inside, tennis_amd/intree.py; absent where that library was not built)."""
     import tempfile
-    from oracle import ref
-    from tennis_amd import module_file as mf, resnet50
-    if not ref.intree_available():
+    from tennis_amd import intree, module_file as mf, resnet50
+    if not intree.available():
         return None
     n = 32
     desc, params = resnet50.make_parameters(seed=0)
@@ -222,18 +245,19 @@ def tennis_runtime_leg(reps=5):
     with tempfile.TemporaryDirectory() as tmp:
         path = os.path.join(tmp, "resnet50_int8_bs32.tsm")
         mf.write_module(path, module)
-        fused0 = ref.fused_chain_count_intree()
-        hand0 = ref.handover_counts_intree()
-        ms, logits = ref.time_module_intree("hip", path, [x], warmup=2, reps=reps, resident=True)
-        fused = ref.fused_chain_count_intree() - fused0
-        hand = tuple(a - b for a, b in zip(ref.handover_counts_intree(), hand0))
-        ms_upload, _ = ref.time_module_intree("hip", path, [x], warmup=2, reps=reps, resident=False)
+        fused0, hand0, host0 = intree.fused_chain_count(), intree.handover_counts(), intree.host_delegate_count()
+        ms, logits = intree.time_module("hip", path, [x], warmup=2, reps=reps, resident=True)
+        fused = intree.fused_chain_count() - fused0
+        hand = tuple(a - b for a, b in zip(intree.handover_counts(), hand0))
+        ms_upload, _ = intree.time_module("hip", path, [x], warmup=2, reps=reps, resident=False)
+        host_runs = intree.host_delegate_count() - host0
     return {"workload": "BASELINE config 4 network as a .tsm module (every activation quantized with one fixed multiplier) "
                         "in TenniS's Workbench on device hip: quantize+conv+bias+relu chains (and residual joins) fused by "
                         "the backend's zipper option, int8 hand-over between fused nodes, fp32 inner_prod classifier; input "
                         "bound from device memory, each run ends with the logits on the host",
             "img_per_s": n / (ms * 1e-3), "ms_per_batch": ms, "reps": reps, "chains_fused_by_the_graph_compiler": fused,
             "int8_hand_overs": hand[0], "dual_output_nodes": hand[1],
+            "operator_runs_handed_to_host_operators": host_runs,
             "ms_per_batch_input_uploaded_every_run": ms_upload,
             "logits_finite": bool(np.isfinite(logits).all())}
 
@@ -273,14 +297,15 @@ def resnet_leg(steps=20):
             "steps": steps, "logits_finite": bool(torch.isfinite(logits).all().item())}
 
 
-def yolo_leg(steps=5):
+def yolo_leg(steps=5, mish="exact"):
     """YOLOv4-shaped int8 network, batch 8 at 3x608x608 (BASELINE config 5): img/s of the whole forward pass
-    (three head tensors), replayed from a captured HIP graph."""
+    (three head tensors), replayed from a captured HIP graph.  mish = "exact": the Mish layers give the operator
+    chain's values bit for bit (the default of the library); "fast": the opt-in one-exponential form."""
     import torch
     from tennis_amd import yolov4
     n, size = 8, 608
     L, heads = yolov4.layers()
-    net = yolov4.YoloV4Int8(L, heads, yolov4.make_parameters(L, seed=0))
+    net = yolov4.YoloV4Int8(L, heads, yolov4.make_parameters(L, seed=0), mish=mish)
     x = torch.rand((n, 3, size, size), device="cuda")
     net.calibrate(x)
     side = torch.cuda.Stream()
@@ -301,7 +326,8 @@ def yolo_leg(steps=5):
     dt = (time.perf_counter() - t0) / steps
     macs = yolov4.total_macs(L, n, size)
     return {"workload": "BASELINE config 5: YOLOv4-shaped int8 network (CSPDarknet53 + SPP + PANet, Mish / LeakyReLU), "
-                        "batch 8, 3x608x608, random-init weights, per-channel int8 weights, per-tensor int8 activations",
+                        "batch 8, 3x608x608, random-init weights, per-channel int8 weights, per-tensor int8 activations; "
+                        "Mish in its %s form" % mish,
             "img_per_s": n / dt, "ms_per_batch": dt * 1e3, "TOPS": 2.0 * macs / dt / 1e12, "gmac_per_image": macs / n / 1e9,
             "steps": steps, "outputs_finite": bool(all(torch.isfinite(o).all().item() for o in outs))}
 
@@ -385,6 +411,14 @@ def kernels_leg(reps=20):
     w63, w23 = capi.WinogradF63(w1, (1, 1, 1, 1)), capi.WinogradF23(w1, (1, 1, 1, 1))
     timed("winograd F(6,3) config 1 (direct-conv flops)", "mfma_f32", flops1, lambda: w63(x1, bias=b1, act="relu"))
     timed("winograd F(2,3) config 1 (direct-conv flops)", "mfma_f32", flops1, lambda: w23(x1, bias=b1, act="relu"))
+    # fp32 on a shape the reference's selector routes to Winograd F(6,3): 8x256x28x28 * 256x256x3x3
+    x8, w8, b8 = torch.rand((8, 256, 28, 28), device=dev) * 2 - 1, rnd(256, 256, 3, 3) * 0.03, rnd(256) * 0.01
+    flops8 = 2.0 * 8 * 256 * 28 * 28 * 256 * 9
+    timed("conv2d_f32 8x256x28x28 (gemm_f32_kernel)", "mfma_f32", flops8, lambda: capi.conv2d_f32(x8, w8, (1, 1, 1, 1), bias=b8, act="relu"))
+    w63b = capi.WinogradF63(w8, (1, 1, 1, 1))
+    timed("winograd F(6,3) 8x256x28x28, bit-exact form (direct-conv flops)", "mfma_f32", flops8, lambda: w63b(x8, bias=b8, act="relu"))
+    timed("winograd F(6,3) 8x256x28x28, one MFMA launch (direct-conv flops)", "mfma_f32", flops8,
+          lambda: w63b(x8, bias=b8, act="relu", fast=True))
     # int8 GEMM: largest and a mid shape of BASELINE config 3, and the weight-streaming single row
     k = n = 4096
     gemm = capi.GemmI8(ri8(k, n))
@@ -438,7 +472,7 @@ def main():
                     help="for runs under a profiler: skip the int8-output variant (same kernel name as the roofline "
                          "kernel), the MFMA-rate probe and the CPU baseline, so per-kernel statistics cover the timed "
                          "kernels only")
-    ap.add_argument("--network", choices=("resnet", "yolo", "tennis"),
+    ap.add_argument("--network", choices=("resnet", "yolo", "yolo_fast_mish", "tennis"),
                     help="run only that network leg and print its figures (for per-kernel profiles of a network); "
                          "tennis = the ResNet-50-shaped module through TenniS's own runtime on device hip")
     ap.add_argument("--kernels", action="store_true",
@@ -459,7 +493,8 @@ def main():
     L = capi.lib()
     dev = torch.device("cuda:0")
     if args.network:
-        leg = {"resnet": resnet_leg, "yolo": yolo_leg, "tennis": tennis_runtime_leg}[args.network]
+        leg = {"resnet": resnet_leg, "yolo": yolo_leg, "yolo_fast_mish": lambda: yolo_leg(mish="fast"),
+               "tennis": tennis_runtime_leg}[args.network]
         print(json.dumps(leg()))
         return
     if args.kernels:
@@ -528,22 +563,39 @@ def main():
         ms_graph = (time.perf_counter() - t0) / args.steps * 1e3
 
     def event_time(fn, reps):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        """Seconds per launch: the median over 5 batches of `reps` back-to-back launches, each batch bracketed by
+        events on the launch stream."""
         fn()
         torch.cuda.synchronize()
-        e0.record()
-        for _ in range(reps):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / reps * 1e-3   # seconds per launch
+        per = []
+        for _ in range(5):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            per.append(e0.elapsed_time(e1) / reps * 1e-3)
+        return float(np.median(per))
 
     if args.ceiling:
+        A = capi.aids_lib()
+        if A is None:
+            print("bench.py --ceiling needs the measurement build: python -m tennis_amd.build --aids", file=sys.stderr)
+            sys.exit(4)
+        info = capi.conv2d_i8_plan_info(geom)
+        if info["fp32_kernel"] != "weight_stationary":
+            print("bench.py --ceiling reads the weight-stationary kernel's stamps; the plan is %r" % (info,), file=sys.stderr)
+            sys.exit(4)
+
+        def mfma_only_aids():
+            capi.check(A.tsx_conv2d_i8_staged(g, capi._ptr(ws), capi._ptr(packed), epp, capi._ptr(out), None, None, stream))
+
         conv_ops = 2.0 * cfg["n"] * cfg["cout"] * ho * wo * cfg["c"] * cfg["k"] * cfg["k"]
-        print(json.dumps(ceiling_evidence(L, mfma_only, event_time, conv_ops, dev, stream)))
+        print(json.dumps(ceiling_evidence(A, mfma_only_aids, event_time, conv_ops, dev, stream, int(info["fragments_per_tile"]))))
         return
 
-    reps = max(args.steps, 50)
+    reps = max(args.steps, 100)
     t_mfma = event_time(mfma_only, reps)
     t_stage = event_time(stage_only, reps)
 
@@ -565,11 +617,13 @@ def main():
     sink = torch.zeros(4, dtype=torch.int32, device=dev)
     probe_iters, probe_blocks = 20000, 512
 
-    def probe():
-        capi.check(L.tsx_probe_mfma_i8(capi._ptr(operands), probe_iters, probe_blocks, capi._ptr(sink), stream))
+    A = None if args.profile else capi.aids_lib()      # the measurement build holds the probe kernel
 
-    t_probe = None if args.profile else event_time(probe, 3)
-    sustained_tops = None if args.profile else probe_blocks * 4 * probe_iters * 8 * 65536.0 / t_probe / 1e12
+    def probe():
+        capi.check(A.tsx_probe_mfma_i8(capi._ptr(operands), probe_iters, probe_blocks, capi._ptr(sink), stream))
+
+    t_probe = event_time(probe, 3) if A is not None else None
+    sustained_tops = probe_blocks * 4 * probe_iters * 8 * 65536.0 / t_probe / 1e12 if A is not None else None
 
     # One device copy of known size: the dispatch the HBM counters of a profiler run are scaled by.
     calib_src = torch.empty(64 << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -589,6 +643,8 @@ def main():
 
     macs = cfg["n"] * cfg["cout"] * ho * wo * cfg["c"] * cfg["k"] * cfg["k"]
     ops = 2.0 * macs
+    mfma_kernel = {"weight_stationary": "conv_i8_rs_kernel", "flat_tile": "conv_i8_fl_kernel",
+                   "window_stationary": "conv_i8_ws_kernel", "igemm": "igemm_i8_kernel"}[capi.conv2d_i8_plan_info(geom)["fp32_kernel"]]
     tops = ops / (ms_per_step * 1e-3) / 1e12
     kernel_tops = ops / t_mfma / 1e12
 
@@ -609,14 +665,14 @@ def main():
                                "out; step = quantize+stage kernel + i8-MFMA implicit-GEMM kernel",
                    "algorithmic_ops_per_step": ops, "pct_of_int8_mfma_peak_whole_step": 100.0 * tops / PEAK_INT8_TOPS,
                    "launch": launch_mode, "ms_per_step_direct_calls": ms_direct, "ms_per_step_graph_replay": ms_graph},
-        "roofline": {"bound": "mfma", "kernel": "conv_i8_fl_kernel", "achieved": kernel_tops, "peak": PEAK_INT8_TOPS,
+        "roofline": {"bound": "mfma", "kernel": mfma_kernel, "achieved": kernel_tops, "peak": PEAK_INT8_TOPS,
                      "unit": "TOP/s", "frac": kernel_tops / PEAK_INT8_TOPS, "traffic": TRAFFIC_CONV_BYTES,
                      "traffic_unit": "HBM bytes per launch, a constant taken from rocprofv3 FETCH_SIZE / WRITE_SIZE of this "
                                      "kernel on this workload (profiles/conv2d_i8_config2_hbm_traffic.txt), not measured "
                                      "by this run; algorithmic 33.65e6",
                      "note": "int8 multiply-accumulate ops (TOP/s); 2*N*Cout*Ho*Wo*Cin*9 = %.4g ops per launch, "
-                             "avg launch %.2f us over %d back-to-back launches" % (ops, t_mfma * 1e6, reps)},
-        "sustained_mfma": None if args.profile else {
+                             "launch %.2f us = median of 5 batches of %d back-to-back launches" % (ops, t_mfma * 1e6, reps)},
+        "sustained_mfma": None if sustained_tops is None else {
             "value": sustained_tops, "unit": "TOPS", "frac_of_it": kernel_tops / sustained_tops,
             "note": "register-only v_mfma_i32_32x32x32_i8 loop on random int8 operands, measured in this "
                     "run: the rate the part sustains under load (clocks drop with operand activity)"},
@@ -634,11 +690,13 @@ def main():
     if not args.no_resnet and not args.profile:
         result["resnet50_int8_bs32"] = resnet_leg()
     if not args.no_yolo and not args.profile:
-        result["yolov4_int8_bs8"] = yolo_leg()
+        result["yolov4_int8_bs8"] = yolo_leg(mish="exact")
+        result["yolov4_int8_bs8_fast_mish"] = yolo_leg(mish="fast")
     if not args.no_gemm and not args.profile:
         result["gemm_i8_sweep"] = gemm_leg()
     if not args.profile:
         result["conv2d_f32_config1"] = config1_leg()
+        result["conv2d_f32_winograd_shape"] = winograd_shape_leg()
     if not args.no_resnet and not args.profile:
         result["resnet50_int8_bs32_tennis_runtime"] = tennis_runtime_leg()
     if args.cpu_images > 0 and not args.profile:

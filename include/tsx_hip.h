@@ -35,22 +35,6 @@ int tsx_version(void);
 /* Number of compute units of the current device (for launch heuristics and roofline peaks). */
 int tsx_device_cu_count(void);
 
-/* Diagnostic with no counterpart in the reference: launches `blocks` workgroups of 4 wavefronts, each
- * issuing iters * 8 register-only v_mfma_i32_32x32x32_i8 (65536 ops each) on operands read once from
- * operands_dev (32 KiB).  Timed by the caller, it gives the int8 MFMA rate this part sustains for the
- * given operand data -- the practical ceiling of the contraction kernels (clocks drop under the power
- * of random operands, so it is well below the nominal peak).  ops = blocks * 4 * iters * 8 * 65536. */
-int tsx_probe_mfma_i8(const void *operands_dev, int32_t iters, int32_t blocks, int32_t *sink_dev, void *stream);
-
-/* Measurement aid with no counterpart in the reference.  While a buffer is set (NULL switches it off; process-wide),
- * every wavefront of the flat-tile int8 convolution kernel (the kernel of large multi-tap layers such as BASELINE
- * config 2) writes four (wall clock at 100 MHz, shader clock) pairs to
- * buffer[(workgroup * 8 + wavefront) * 8 ...]: at kernel entry, at K-loop entry, at K-loop exit and after its last
- * store has left the wavefront -- where a launch's time goes, and the shader clock of each phase (shader cycles /
- * wall time).  Workgroup = blockIdx.y * gridDim.x + blockIdx.x; wavefronts whose slot lies beyond `bytes` write
- * nothing.  Costs a few scalar instructions per wavefront when set, one predictable branch when not. */
-int tsx_debug_phase_stamps(void *buffer_dev, size_t bytes);
-
 /* Geometry of one 2-D convolution, as base::Conv2D / base::Conv2DQuantized hand it to
  * their core: x [n,c,h,w], w [cout,c,kh,kw], Padding2D{top,bottom,left,right},
  * Stride2D, Dilation2D (include/backend/common_structure.h:10-62).  Output size follows
@@ -70,9 +54,12 @@ int tsx_conv2d_out_size(const tsx_conv2d_geom *g, int32_t *out_h, int32_t *out_w
 #define TSX_ACT_RELU       1  /* cpu::ReLU      src/kernels/cpu/relu.cpp:30-52 */
 #define TSX_ACT_LEAKY_RELU 2  /* cpu::LeakyReLU src/kernels/cpu/leaky_relu.cpp:41-66 */
 #define TSX_ACT_MISH       3  /* x * tanh(softplus(x)) as the operators softplus, tanh, mul compose it
-                                 (src/kernels/cpu/softplus.cpp:30-39, tanh.cpp:14-23, mul.cpp); the only
-                                 epilogue term that is not bit-exact: device expf/log differ from the host's
-                                 by a few ulp */
+                                 (src/kernels/cpu/softplus.cpp:30-39, tanh.cpp:14-23, mul.cpp): the host's chain of
+                                 rounded intermediates, its expf restated operation for operation -- bit for bit
+                                 the host's values */
+#define TSX_ACT_MISH_FAST  4  /* the same function from one hardware exponential and one reciprocal: 1e-7 relative,
+                                 a sixth of the arithmetic; for layers bound by the activation.  Opt-in: a
+                                 requantized int8 value differs from TSX_ACT_MISH's in about one of a million */
 
 /* Fused epilogue applied to the int32 accumulators.  It reproduces, rounding for
  * rounding, the reference's chain of separate operators on the fp32 tensor:
@@ -134,6 +121,12 @@ size_t tsx_conv2d_i8_packed_weight_bytes(const tsx_conv2d_geom *g);
 int tsx_conv2d_i8_pack_weights(const tsx_conv2d_geom *g, const int8_t *w_oihw_dev, void *packed_dev, void *stream);
 /* Scratch the conv needs (channel-blocked padded copy of the activations). */
 size_t tsx_conv2d_i8_workspace_bytes(const tsx_conv2d_geom *g);
+/* Which kernel the plan of this layer launches, as text ("kernel=flat_tile fp32_kernel=weight_stationary ..."):
+ * kernel = igemm | window_stationary | flat_tile, and fp32_kernel = the kernel that takes the layer when the
+ * epilogue is fp32 output with dequantize scales, bias and activation only.  No counterpart in the reference; for
+ * tests that must know a given kernel ran, and for logs.  The environment variables TSX_CONV_I8_FLAT and
+ * TSX_CONV_I8_RS ("0" = never, "force" = wherever the geometry allows) are read at every call that plans. */
+int tsx_conv2d_i8_plan_info(const tsx_conv2d_geom *g, char *text, size_t text_bytes);
 /* padding_value is the reference's float parameter; it is cast to int8 as the reference
  * does (conv2d_quantized_core.cpp:72).  Any of out_f32_dev / out_i8_dev / out_acc_dev may be
  * NULL; out_acc_dev receives the raw int32 accumulators (the reference's INT32 scratch). */

@@ -109,6 +109,48 @@ def build(verbose=True, jobs=8, incremental=False):
     return LIB_PATH
 
 
+AIDS_LIB_PATH = os.path.join(LIB_DIR, "libtsx_hip_aids.so")
+
+
+def build_aids(verbose=True, jobs=8):
+    """The measurement build: the sources that carry phase stamps or probes compiled again with
+    -DTSX_MEASUREMENT_AIDS, linked with the product's other objects into libtsx_hip_aids.so (bench.py --ceiling and
+    the sustained-MFMA probe load it; nothing else does).  Needs a finished product build."""
+    obj_dir = os.path.join(LIB_DIR, "obj")
+    aids_dir = os.path.join(LIB_DIR, "obj_aids")
+    os.makedirs(aids_dir, exist_ok=True)
+    def carries_aids(src):
+        text = open(src).read()
+        if "TSX_MEASUREMENT_AIDS" in text:
+            return True
+        return any("TSX_MEASUREMENT_AIDS" in open(os.path.join(CSRC, h)).read()
+                   for h in os.listdir(CSRC) if h.endswith(".hpp") and ('"%s"' % h) in text)
+    procs, objs = [], []
+    for src in sources():
+        name = os.path.basename(src)[:-4] + ".o"
+        if not carries_aids(src):
+            objs.append(os.path.join(obj_dir, name))
+            continue
+        obj = os.path.join(aids_dir, name)
+        objs.append(obj)
+        cmd = [HIPCC] + [f for f in FLAGS if not f.startswith("-Rpass")] + ["-DTSX_MEASUREMENT_AIDS", "-c", src, "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        while sum(p.poll() is None for _, p in procs) >= jobs:
+            procs[0][1].wait()
+    for src, p in procs:
+        out, _ = p.communicate()
+        if p.returncode != 0:
+            print(out, file=sys.stderr)
+            raise RuntimeError("hipcc failed: " + src)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", AIDS_LIB_PATH] + objs
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return AIDS_LIB_PATH
+
+
 BACKEND_DIR = os.path.join(HERE, "backend")
 BACKEND_LIB = os.path.join(LIB_DIR, "libtsx_backend.so")
 BACKEND_SOURCES = ["ts/ts_api.cpp", "ts/base_ops.cpp", "hip/hip_device.cpp", "hip/hip_ops_quantized.cpp", "hip/hip_ops_float.cpp", "hip/hip_ops_glue.cpp", "hip/hip_ops_v2.cpp", "hip/hip_ops_fused.cpp", "capi_ops.cpp"]
@@ -130,3 +172,5 @@ def build_backend(verbose=True):
 
 if __name__ == "__main__":
     build(incremental="--incremental" in sys.argv[1:])
+    if "--aids" in sys.argv[1:]:
+        build_aids()

@@ -20,7 +20,7 @@ _f32 = ctypes.c_float
 _sz = ctypes.c_size_t
 
 ACT_NONE, ACT_RELU, ACT_LEAKY_RELU = 0, 1, 2
-_ACT = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "leaky_relu": ACT_LEAKY_RELU, "mish": 3}
+_ACT = {None: ACT_NONE, "none": ACT_NONE, "relu": ACT_RELU, "leaky_relu": ACT_LEAKY_RELU, "mish": 3, "mish_fast": 4}
 
 
 class ConvGeom(ctypes.Structure):
@@ -48,7 +48,6 @@ SIGNATURES = {
     "tsx_last_error": (ctypes.c_char_p, []),
     "tsx_version": (ctypes.c_int, []),
     "tsx_device_cu_count": (ctypes.c_int, []),
-    "tsx_probe_mfma_i8": (ctypes.c_int, [_vp, _i32, _i32, _vp, _vp]),
     "tsx_conv2d_out_size": (ctypes.c_int, [ctypes.POINTER(ConvGeom), ctypes.POINTER(_i32), ctypes.POINTER(_i32)]),
     "tsx_quantize_f32_i8": (ctypes.c_int, [_vp, _i64, _vp, _i32, _vp, _vp]),
     "tsx_conv2d_i8_packed_weight_bytes": (_sz, [ctypes.POINTER(ConvGeom)]),
@@ -67,7 +66,6 @@ SIGNATURES = {
     "tsx_conv2d_i8_staged_dims": (ctypes.c_int, [ctypes.POINTER(ConvGeom), ctypes.POINTER(_i32), ctypes.POINTER(_i32),
                                                  ctypes.POINTER(_i32)]),
     "tsx_conv2d_i8_stage_fill": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _f32, _vp, _sz, _vp]),
-    "tsx_debug_phase_stamps": (ctypes.c_int, [_vp, _sz]),
     "tsx_conv2d_i8_stage_fill_halo": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _f32, _vp, _sz, _vp]),
     "tsx_conv2d_i8_staged_at": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _i32, _i32, _vp, ctypes.POINTER(Epilogue), _vp,
                                                _vp, _vp, _vp]),
@@ -87,6 +85,7 @@ SIGNATURES = {
     "tsx_add_f32": (ctypes.c_int, [_vp, _vp, _i64, _i32, _f32, _vp, _vp]),
     "tsx_add_broadcast_f32": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32, _vp, _vp]),
     "tsx_mish_f32": (ctypes.c_int, [_vp, _i64, _vp, _vp]),
+    "tsx_conv2d_i8_plan_info": (ctypes.c_int, [_vp, ctypes.c_char_p, _sz]),
     "tsx_softplus_f32": (ctypes.c_int, [_vp, _i64, _vp, _vp]),
     "tsx_tanh_f32": (ctypes.c_int, [_vp, _i64, _vp, _vp]),
     "tsx_mul_f32": (ctypes.c_int, [_vp, _vp, _i64, _vp, _vp]),
@@ -129,6 +128,27 @@ def lib():
     return _lib
 
 
+AIDS_LIB_PATH = os.path.join(os.path.dirname(LIB_PATH), "libtsx_hip_aids.so")
+_aids = None
+
+
+def aids_lib():
+    """The measurement build of the library (`python -m tennis_amd.build --aids`): the same entry points plus
+    tsx_probe_mfma_i8 and tsx_debug_phase_stamps (csrc/tsx_aids.h), its kernels carrying phase stamps.  None where
+    it is not built."""
+    global _aids
+    if _aids is None and os.path.exists(AIDS_LIB_PATH):
+        L = ctypes.CDLL(AIDS_LIB_PATH)
+        for name, (res, args) in list(SIGNATURES.items()) + [
+                ("tsx_probe_mfma_i8", (ctypes.c_int, [_vp, _i32, _i32, _vp, _vp])),
+                ("tsx_debug_phase_stamps", (ctypes.c_int, [_vp, _sz]))]:
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _aids = L
+    return _aids
+
+
 def check(rc):
     if rc != 0:
         raise TsxError("tsx error %d: %s" % (rc, lib().tsx_last_error().decode(errors="replace")))
@@ -163,6 +183,13 @@ def conv_out_size(geom):
     ho, wo = _i32(), _i32()
     check(lib().tsx_conv2d_out_size(ctypes.byref(geom), ctypes.byref(ho), ctypes.byref(wo)))
     return ho.value, wo.value
+
+
+def conv2d_i8_plan_info(geom):
+    """tsx_conv2d_i8_plan_info: the kernels the plan of this layer launches, as a dict of its key=value words."""
+    buf = ctypes.create_string_buffer(256)
+    check(lib().tsx_conv2d_i8_plan_info(ctypes.byref(geom), buf, len(buf)))
+    return dict(word.split("=", 1) for word in buf.value.decode().split())
 
 
 def quantize(x, scales):

@@ -1009,7 +1009,7 @@ int check_epilogue(const tsx_epilogue *ep, const float *out_f32, const int8_t *o
     }
     if (out_f32 || out_i8) {
         TSX_REQUIRE(ep && ep->dq_dev, "epilogue with dequantize scales required for fp32/int8 output");
-        TSX_REQUIRE(ep->act >= TSX_ACT_NONE && ep->act <= TSX_ACT_MISH, "unknown activation %d", ep->act);
+        TSX_REQUIRE(ep->act >= TSX_ACT_NONE && ep->act <= TSX_ACT_MISH_FAST, "unknown activation %d", ep->act);
     }
     if (out_i8) {
         TSX_REQUIRE(ep->q_scales_dev, "int8 output needs q_scales_dev");
@@ -1198,6 +1198,24 @@ size_t tsx_conv2d_i8_packed_weight_bytes(const tsx_conv2d_geom *g) {
 size_t tsx_conv2d_i8_workspace_bytes(const tsx_conv2d_geom *g) {
     Plan pl;
     return make_plan(g, &pl) ? 0 : pl.staged_bytes;
+}
+
+int tsx_conv2d_i8_plan_info(const tsx_conv2d_geom *g, char *text, size_t text_bytes) {
+    Plan pl;
+    int rc = make_plan(g, &pl);
+    if (rc) return rc;
+    TSX_REQUIRE(text && text_bytes > 0, "plan_info: no text buffer");
+    const char *base = !pl.use_ws ? "igemm" : pl.wsp.flat ? "flat_tile" : "window_stationary";
+    const bool rs = pl.use_ws && pl.wsp.rs;
+    if (rs)
+        std::snprintf(text, text_bytes, "kernel=%s fp32_kernel=weight_stationary fragments_per_tile=%d tiles=%d ring_rows=%d lds_bytes=%d",
+                      base, pl.wsp.rs_frags, pl.wsp.rs_ptiles * ((g->cout + 63) / 64), pl.wsp.rs_nr, pl.wsp.rs_lds);
+    else if (pl.use_ws && pl.wsp.flat)
+        std::snprintf(text, text_bytes, "kernel=%s fp32_kernel=%s fragments_per_tile=%d tiles=%lld resident=%d", base, base,
+                      pl.wsp.fl_nta + pl.wsp.fl_ntb, (long long)(pl.wsp.fl_tiles * (pl.wsp.coutp / 128)), int(pl.wsp.fl_resident));
+    else
+        std::snprintf(text, text_bytes, "kernel=%s fp32_kernel=%s", base, base);
+    return 0;
 }
 
 int tsx_conv2d_i8_pack_weights(const tsx_conv2d_geom *g, const int8_t *w_oihw_dev, void *packed_dev, void *stream) {

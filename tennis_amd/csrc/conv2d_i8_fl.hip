@@ -17,36 +17,23 @@
 #include "conv2d_i8_fl_kernel.hpp"
 
 #include <cstdlib>
+#include <cstring>
 
 #include <atomic>
 
-// phase-stamp buffer of tsx_debug_phase_stamps (null = off)
-static std::atomic<unsigned long long *> g_stamps{nullptr};
-static std::atomic<size_t> g_stamp_slots{0};
-
-extern "C" int tsx_debug_phase_stamps(void *buffer_dev, size_t bytes) {
-    if (buffer_dev && (bytes < 64 || reinterpret_cast<uintptr_t>(buffer_dev) % 8 != 0))
-        return tsx::fail(TSX_E_INVALID, "debug_phase_stamps: buffer must be 8-byte aligned and hold at least one wavefront's 64 bytes");
-    g_stamp_slots.store(buffer_dev ? bytes / 8 : 0);
-    g_stamps.store(static_cast<unsigned long long *>(buffer_dev));
-    return 0;
-}
 
 namespace tsx {
-
-void debug_phase_stamps(unsigned long long **buffer, int *slots) {
-    *buffer = g_stamps.load();
-    *slots = int(g_stamp_slots.load());
-}
 
 void fl_plan(const WsGeom &g, WsPlan *pl) {
     pl->flat = false;
     if (!pl->ok || g.gemm || g.kh * g.kw <= 1 || pl->wm != 4) return;
-    static const bool disabled = [] {
-        const char *e = std::getenv("TSX_CONV_I8_FLAT");   // "0": keep every layer on the window-stationary kernel
-        return e && e[0] == '0';
-    }();
-    if (disabled) return;
+    // TSX_CONV_I8_FLAT, read at every plan: "0" keeps every layer on the window-stationary kernel; "force" takes
+    // this kernel wherever the geometry allows, whatever the cost model says, with the largest tile that fits (tests
+    // of the kernel on small layers); "forceNM" the same with tiles of N + M fragments only
+    const char *e = std::getenv("TSX_CONV_I8_FLAT");
+    if (e && e[0] == '0') return;
+    const bool force = e && e[0] == 'f';
+    const int only = force && std::strlen(e) == 7 ? (e[5] - '0') * 10 + (e[6] - '0') : 0;
     const int64_t positions = int64_t(g.n) * g.ho * g.wo;
     if (positions >= (int64_t(1) << 31) - 256) return;
     if (pl->packed_bytes >= (size_t(1) << 31)) return;   // the kernel addresses the weights with 32-bit offsets
@@ -58,12 +45,15 @@ void fl_plan(const WsGeom &g, WsPlan *pl) {
     // layers of the YOLOv4-shaped network); small maps (ResNet's 14x14 and 7x7 layers, under 200 workgroups of
     // short tiles) run 1-20 % slower on it and stay where they were.  The smaller splits remain instantiated
     // for the planner to use once that changes.
-    static const int splits[3][2] = {{3, 3}, {4, 3}, {4, 4}};
+    // (the first three are the planner's; the smaller ones are instantiated for layers forced onto this kernel)
+    static const int splits[7][2] = {{3, 3}, {4, 3}, {4, 4}, {3, 2}, {2, 2}, {2, 1}, {1, 1}};
     // One workgroup per CU: the busiest CU's time, in units of one fragment x 32 channels on one SIMD, is
     //     rounds x (fixed + F)
     // -- the same form as the window-stationary plan's model, whose workgroups pair up on a CU.
     double best = -1;
-    for (const auto &s : splits) {
+    for (int si = 0; si < (force ? 7 : 3); ++si) {
+        const int *s = splits[si];
+        if (only && s[0] * 10 + s[1] != only) continue;
         const int f = s[0] + s[1];
         // rows between a tile's first and last position, and image ends in between (worst tile)
         const int dr = (f * 32) % g.wo == 0 ? f * 32 / g.wo - 1 : (f * 32 + g.wo - 2) / g.wo;
@@ -80,8 +70,9 @@ void fl_plan(const WsGeom &g, WsPlan *pl) {
         if (wp > FL_MAX_WP || size_t(2) * wr * rowp > size_t(FL_MAX_LDS)) continue;
         const int64_t tiles = (positions + f * 32 - 1) / (f * 32);
         const int64_t wgs = tiles * (pl->coutp / 128);
-        if (wgs < 160) continue;
-        const double cost = double((wgs + 255) / 256) * (0.75 + f);
+        if (wgs < 160 && !force) continue;
+        // forced: the largest tile that fits
+        const double cost = force ? double(16 - f) : double((wgs + 255) / 256) * (0.75 + f);
         if (best < 0 || cost < best) {
             best = cost;
             pl->fl_nta = s[0];
@@ -99,7 +90,7 @@ void fl_plan(const WsGeom &g, WsPlan *pl) {
     // the window-stationary plan's cost in the same units: its 4-wavefront workgroups sit two to a CU
     const int64_t ws_wgs = pl->tiles * (pl->coutp / 128);
     const double ws_cost = double((ws_wgs + 511) / 512) * 2 * (0.5 + pl->nt * (pl->nt > 4 ? 1.45 : 1.0));
-    if (best <= ws_cost) pl->flat = true;
+    if (best <= ws_cost || force) pl->flat = true;
 }
 
 int fl_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t *packed, const EpiParams &ep,
@@ -138,8 +129,6 @@ int fl_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t 
     p.wo_magic = div_magic(p.wo, p.positions);
     p.ho_magic = div_magic(p.ho, int64_t(g.n) * g.ho);
     p.howo_magic = div_magic(p.ho * p.wo, p.positions);
-    p.stamps = g_stamps.load();
-    p.stamp_slots = int(g_stamp_slots.load());
     // an output of L2 size or more that no fused consumer reads: stream it
     p.stream_out = (!ep.residual && !ep.st_out && ep.out_f32 && int64_t(g.n) * g.cout * g.ho * g.wo * 4 >= (int64_t(16) << 20)) ? 1 : 0;
     const dim3 grid(unsigned(p.tiles_per_xcd * 8), unsigned((g.cout + 127) / 128));

@@ -30,11 +30,6 @@ struct FlParams : EpiParams {
     int positions;          // n * ho * wo
     int stream_out;         // fp32 output written with streaming stores
     int resident;           // every channel block's window in LDS at once (cblocks buffers instead of 2)
-    // measurement aid (tsx_debug_phase_stamps): when set, every wavefront writes 8 values at
-    // stamps[(workgroup * 8 + wave) * 8]: wall clock (100 MHz) and shader clock at kernel entry, K-loop entry,
-    // K-loop exit and after its last store has left
-    unsigned long long *stamps;
-    int stamp_slots;
     // per-lane divisions by uniform divisors as one multiply-high (div_magic / udiv)
     unsigned wc_magic, wo_magic, ho_magic, howo_magic;
 };
@@ -72,14 +67,6 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
     const int m0 = (blockIdx.y * 4 + wave_m) * 32;   // first cout of this wavefront
     const int taps = p.kh * p.kw;
     const int win_bytes = p.wr * p.rowp;
-    const int stamp_slot = ((blockIdx.y * gridDim.x + blockIdx.x) * 8 + threadIdx.x / 64) * 8;
-    auto stamp = [&](int phase) __attribute__((always_inline)) {
-        if (p.stamps && lane == 0 && stamp_slot + 8 <= p.stamp_slots) {
-            p.stamps[stamp_slot + 2 * phase] = wall_clock64();
-            p.stamps[stamp_slot + 2 * phase + 1] = clock64();
-        }
-    };
-    stamp(0);
 
     // ---- window fill bookkeeping: chunk q = tid + i*512 -> pixel q / 4, 16-byte chunk q % 4
     // A uniform 64-bit base (the window's first staged row) plus one 32-bit byte offset per chunk: the loads take
@@ -195,7 +182,6 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
     };
     int toff = 0;   // buf * win_bytes + tap shift
     b_read(b0, toff);
-    stamp(1);
 
     // One K-step: both halves' MFMAs, the B reads one half-step ahead, the window change on a channel-block
     // boundary.  PREFETCH: also load the weights of the K-step FL_RING-1 ahead into the slot the previous step freed.
@@ -259,12 +245,6 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
         if (decltype(uc)::value < left) k_step(uc, std::false_type{});
     });
 
-    if (p.stamps) {
-        // the accumulators are written by the MFMAs still in flight: wait for them, so that the stamp marks the end
-        // of the multiplication rather than the issue of its last instruction
-        asm volatile("; accumulators complete" ::"v"(acc[0][15]), "v"(acc[NT - 1][15]) : "memory");
-        stamp(2);
-    }
 
     // ---- epilogue: accumulator register r of lane l = cout 8*(r/4) + 4*(l/32) + r%4, position l%32
     const int howo = p.ho * p.wo;
@@ -361,9 +341,11 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
                     v[r] = apply_act_conv_i8(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
                 });
             } else if (p.act == TSX_ACT_MISH) {
+                mish_fragment(v);
+            } else if (p.act == TSX_ACT_MISH_FAST) {
                 static_for<0, 16>([&](auto rc) {
                     constexpr int r = decltype(rc)::value;
-                    v[r] = apply_act_conv_i8(v[r], TSX_ACT_MISH, 0.f, true);
+                    v[r] = apply_act_conv_i8(v[r], TSX_ACT_MISH_FAST, 0.f, true);
                 });
             }
             if (EXTRA && p.residual && p.res_after) static_for<0, 16>([&](auto rc) {
@@ -432,10 +414,6 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
                 if (pok[j] && co0 + dco < p.cout) emit(p, acc[j][r], base + int64_t(dco) * howo, dq[r], bias[r], 0.f);
             });
         });
-    }
-    if (p.stamps) {
-        __builtin_amdgcn_s_waitcnt(0);   // every store of this wavefront has left
-        stamp(3);
     }
 }
 

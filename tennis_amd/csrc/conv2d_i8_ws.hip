@@ -226,7 +226,6 @@ int ws_launch(const WsGeom &g, const WsPlan &pl, const int8_t *xs, const int8_t 
     p.stream_out = (!ep.residual && !ep.st_out && ep.out_f32 && int64_t(g.n) * g.cout * g.ho * g.wo * 4 >= (int64_t(16) << 20)) ? 1 : 0;
     p.rowmajor = g.gemm ? 1 : 0;
     if (g.gemm) p.stream_out = 0;
-    debug_phase_stamps(&p.stamps, &p.stamp_slots);
     p.wc_magic = div_magic(p.wc, MAX_WP);
     p.tw_magic = div_magic(p.tw, 4 * 7 * 32);
     p.ow_magic = div_magic(ep.o_w, int64_t(p.ho) * p.wo);

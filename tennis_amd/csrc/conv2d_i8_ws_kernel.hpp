@@ -30,17 +30,10 @@ struct WsParams : EpiParams {
     int pix, chunk_shift, stage_bytes, tap_row, tap_col;
     int stream_out;   // fp32 output written with streaming stores
     int rowmajor;     // GEMM: output index position * cout + channel, row_scale[position] applied behind dq
-    // measurement aid (tsx_debug_phase_stamps): when set, every wavefront writes 8 values at
-    // stamps[(workgroup * 8 + wave) * 8]: wall clock (100 MHz) and shader clock at kernel entry, K-loop entry,
-    // K-loop exit and after its last store
-    unsigned long long *stamps;
-    int stamp_slots;
     // per-lane divisions by uniform divisors as one multiply-high (div_magic / udiv)
     unsigned wc_magic, tw_magic, ow_magic;
 };
 
-// buffer of tsx_debug_phase_stamps (null = off)
-void debug_phase_stamps(unsigned long long **buffer, int *slots);
 
 // One specialisation per fragment count, each defined by its own translation unit.
 template <int NT>
@@ -102,14 +95,6 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
     const int m0 = (blockIdx.y * p.wm + wave_m) * (32 * FM);         // first cout of this wavefront
     const int taps = p.kh * p.kw;
     const int win_bytes = p.wpix * p.pix;
-    const int stamp_slot = ((blockIdx.y * gridDim.x + blockIdx.x) * 8 + wave) * 8;
-    auto stamp = [&](int phase) __attribute__((always_inline)) {
-        if (p.stamps && lane == 0 && stamp_slot + 8 <= p.stamp_slots) {
-            p.stamps[stamp_slot + 2 * phase] = wall_clock64();
-            p.stamps[stamp_slot + 2 * phase + 1] = clock64();
-        }
-    };
-    stamp(0);
 
     // ---- window fill bookkeeping: chunk q = tid + i*256 -> pixel q / chunks-per-pixel, 16-byte chunk q % ...
     // A uniform 64-bit base (the window's first staged row and column) plus one 32-bit byte offset per chunk: the
@@ -275,7 +260,6 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
             }
         };
         static_for<0, RING - 1>([&](auto sc) { b_ahead(sc); });
-        stamp(1);
         auto k_step = [&](auto uc, auto prefetch) __attribute__((always_inline)) {
             constexpr int u = decltype(uc)::value;
             if (decltype(prefetch)::value) a_load(std::integral_constant<int, (u + RING - 1) % RING>{}, ks + RING - 1);
@@ -302,7 +286,6 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
         // SIMD: nothing else hides the LDS latency).
         v4i b0[NT], b1[NT];
         b_read(b0, toff);
-        stamp(1);
 
         // One K-step: both halves' MFMAs, the B reads one half-step ahead, the window swap on a channel-block boundary.
         // PREFETCH: also load the weights of the K-step RING-1 ahead into the ring slot the previous step freed.
@@ -357,11 +340,6 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
         });
     }
 
-    if (p.stamps) {
-        // wait for the MFMAs still in flight: the stamp marks the end of the multiplication, not its last issue
-        asm volatile("; accumulators complete" ::"v"(acc[0][0][15]), "v"(acc[FM - 1][NT - 1][15]) : "memory");
-        stamp(2);
-    }
 
     // ---- epilogue: accumulator register r of lane l = cout 8*(r/4) + 4*(l/32) + r%4, position l%32
     static_for<0, FM>([&](auto fc) {
@@ -464,9 +442,11 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
                             v[r] = apply_act_conv_i8(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
                         });
                     } else if (p.act == TSX_ACT_MISH) {
+                        mish_fragment(v);
+                    } else if (p.act == TSX_ACT_MISH_FAST) {
                         static_for<0, 16>([&](auto rc) {
                             constexpr int r = decltype(rc)::value;
-                            v[r] = apply_act_conv_i8(v[r], TSX_ACT_MISH, 0.f, true);
+                            v[r] = apply_act_conv_i8(v[r], TSX_ACT_MISH_FAST, 0.f, true);
                         });
                     }
                     if (EXTRA && p.residual && p.res_after) static_for<0, 16>([&](auto rc) {
@@ -558,10 +538,6 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
             });
         }
     });
-    if (p.stamps) {
-        __builtin_amdgcn_s_waitcnt(0);   // every store of this wavefront has left
-        stamp(3);
-    }
 }
 
 }  // namespace

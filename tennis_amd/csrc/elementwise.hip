@@ -61,7 +61,7 @@ __global__ __launch_bounds__(256) void elementwise_kernel(const float *__restric
             } else if (MODE == 5) {
                 v[j] = tsx::softplus_value(v[j]);
             } else if (MODE == 6) {
-                v[j] = __fsub_rn(__fmul_rn(2.f, __fdiv_rn(1.f, __fadd_rn(1.f, expf(-__fmul_rn(2.f, v[j]))))), 1.f);
+                v[j] = tsx::tanh_value(v[j]);
             } else if (MODE == 7) {
                 v[j] = __fmul_rn(v[j], u[j]);
             } else {
@@ -260,7 +260,7 @@ int tsx_leaky_relu_f32(const float *x_dev, int64_t count, float scale, float *ou
 int tsx_add_f32(const float *a_dev, const float *b_dev, int64_t count, int32_t act, float slope, float *out_dev,
                 void *stream) {
     TSX_REQUIRE(count >= 0 && (count == 0 || b_dev), "add: bad argument");
-    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_MISH, "add: unknown activation %d", act);
+    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_MISH_FAST, "add: unknown activation %d", act);
     return launch<3>(a_dev, count, b_dev, 1, 1, slope, out_dev, stream, act);
 }
 

@@ -111,8 +111,10 @@ __device__ __forceinline__ void epilogue_rows16(const EpiParams &p, const v16i &
 #pragma unroll
         for (int r = 0; r < 16; ++r) v[r] = apply_act_conv_i8(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
     } else if (p.act == TSX_ACT_MISH) {
+        mish_fragment(v);
+    } else if (p.act == TSX_ACT_MISH_FAST) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) v[r] = apply_act_conv_i8(v[r], TSX_ACT_MISH, 0.f, true);
+        for (int r = 0; r < 16; ++r) v[r] = apply_act_conv_i8(v[r], TSX_ACT_MISH_FAST, 0.f, true);
     }
     if (p.residual && p.res_after) {
 #pragma unroll

@@ -212,7 +212,7 @@ int tsx_depthwise_conv2d_f32(const tsx_conv2d_geom *g, const float *x_dev, const
     TSX_REQUIRE(g->cout == g->c, "depthwise_conv2d: one filter per channel (cout %d != c %d)", g->cout, g->c);
     TSX_REQUIRE(g->stride_h > 0 && g->stride_w > 0 && g->dilation_h > 0 && g->dilation_w > 0,
                 "depthwise_conv2d: stride and dilation must be positive");
-    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_MISH, "depthwise_conv2d: unknown activation %d", act);
+    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_MISH_FAST, "depthwise_conv2d: unknown activation %d", act);
     const int ho = tsx::conv_out(g->h, g->pad_top, g->pad_bottom, g->kh, g->stride_h, g->dilation_h);
     const int wo = tsx::conv_out(g->w, g->pad_left, g->pad_right, g->kw, g->stride_w, g->dilation_w);
     TSX_REQUIRE(ho > 0 && wo > 0, "depthwise_conv2d: empty output %dx%d", ho, wo);

@@ -232,6 +232,10 @@ int tsx_max_pooling2d_i8_staged(const tsx_staged_map *src, const tsx_staged_map 
                     "max_pooling2d_i8_staged: map %dx%dx%d does not fit [%d][%d][%d] at (%d,%d)", m->h, m->w, m->c, m->hs,
                     m->ws, m->cp, m->pad_top, m->pad_left);
         TSX_REQUIRE(reinterpret_cast<uintptr_t>(m->data) % 16 == 0, "max_pooling2d_i8_staged: buffers must be 16-byte aligned");
+        // whole 64-channel blocks are read and written: a map that is a run of channels inside a wider buffer must
+        // consist of whole blocks, or its last block would reach into the neighbouring run
+        TSX_REQUIRE(m->cp == tsx::round_up(m->c, 64) || m->c % 64 == 0,
+                    "max_pooling2d_i8_staged: %d channels inside a pitch of %d are not whole 64-channel blocks", m->c, m->cp);
     }
     TSX_REQUIRE(src->n == dst->n && src->c == dst->c, "max_pooling2d_i8_staged: batch / channels differ");
     // padding smaller than the window: together with the next check every window holds a valid element

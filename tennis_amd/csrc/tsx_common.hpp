@@ -7,6 +7,7 @@
 #include <type_traits>
 
 #include "tsx_hip.h"
+#include "tsx_mish.hpp"
 
 namespace tsx {
 
@@ -111,58 +112,16 @@ __device__ __forceinline__ float apply_act_basic(float v, int act, float slope, 
     return v;
 }
 
-// cpu::Softplus (src/kernels/cpu/softplus.cpp:30-39): float(log(double(expf(x)) + 1.0)).  The host goes through double
-// only to round log(1 + e) to float well; here log1pf does that in single precision (within an ulp or two of the
-// correctly rounded value) at a fraction of the cost -- a double-precision logarithm per element made the Mish
-// epilogue, not memory or the MFMAs, the bound of every Mish layer.  expf / log1pf are this device's library
-// routines in either form, so Mish values agree with the host's to a few ulp, not bit for bit.
-__device__ __forceinline__ float softplus_value(float x) { return log1pf(expf(x)); }
-
-// e^x for the Mish epilogue: the hardware's 2^a (v_exp_f32, 1 ulp) on a = x * log2(e) carried in two floats, so that
-// the product's rounding does not reach the result: 2^(ah + al) = 2^ah * (1 + al ln2 + ...).  About 1.5 ulp, no range
-// handling: arguments are below 89 in magnitude where the result matters (see mish_value).
-__device__ __forceinline__ float mish_exp(float x) {
-    const float ah = __fmul_rn(x, 1.4426950216293335f);
-    const float al = __builtin_fmaf(x, 1.925963033500011e-08f, __builtin_fmaf(x, 1.4426950216293335f, -ah));
-    const float e = __builtin_amdgcn_exp2f(ah);
-    return __builtin_fmaf(e, __fmul_rn(al, 0.6931471824645996f), e);
-}
-
-// Mish as TenniS graphs compose it, x * tanh(softplus(x)) with softplus = float(log(double(expf(x)) + 1.0))
-// (src/kernels/cpu/softplus.cpp:30-39) and tanh(y) = 2 * (1 / (1 + expf(-2y))) - 1 in float
-// (src/kernels/cpu/tanh.cpp:14-23): the same chain of rounded intermediates -- e, softplus, expf(-2 softplus), the
-// quotient, 2q - 1, the product -- each within an ulp or two of the host's, evaluated on the hardware's exp2 / log2 /
-// reciprocal instead of the library routines: ~45 issue slots against ~160 (two expf, a log1pf and an IEEE division
-// with all their range handling), which was what bounded every Mish layer.
-//   softplus: s = 1 + e with its rounding error c kept (two-sum), log(s) = log2(s) ln2 (constant in two floats) + c / s;
-//             for e below 2^-24 this is e itself, as log1p gives.
-//   quotient: reciprocal with one Newton step (correctly rounded but for rare ties).
-// Limits as the host's: x large -> x, x very negative -> -0 or 0, NaN -> NaN.
-__device__ __forceinline__ float mish_value(float x) {
-    const float e = mish_exp(fminf(x, 88.f));              // beyond 88 the host's expf overflows to inf and tanh gives 1: so does this
-    const float hi = fmaxf(e, 1.f), lo = fminf(e, 1.f);
-    const float s = __fadd_rn(hi, lo);
-    const float c = __fsub_rn(lo, __fsub_rn(s, hi));       // s + c = 1 + e exactly
-    const float l2 = __builtin_amdgcn_logf(s);             // log2(s), 1 ulp
-    const float rs = __builtin_amdgcn_rcpf(s);
-    const float sp = __builtin_fmaf(l2, 0.6931471824645996f, __builtin_fmaf(l2, -1.9046542121259336e-09f, __fmul_rn(c, rs)));
-    const float u = mish_exp(__fmul_rn(-2.f, sp));
-    const float d = __fadd_rn(1.f, u);
-    const float r0 = __builtin_amdgcn_rcpf(d);
-    const float q = __builtin_fmaf(r0, __builtin_fmaf(-d, r0, 1.f), r0);
-    const float t = __builtin_fmaf(2.f, q, -1.f);          // 2q is exact: one rounding, as fl(fl(2q) - 1)
-    return __fmul_rn(x, t);
-}
-
-// Mish for the epilogues of the int8 convolution kernels, where the activation's arithmetic, not memory or the MFMAs,
-// bounds a layer (the 608x608 and 304x304 layers of a YOLOv4-shaped backbone spend more issue slots on the epilogue
-// than the VALUs have in the time the layer's bytes take): one exponential and one reciprocal at the hardware's 1 ulp,
+// Mish, softplus and tanh in the host's arithmetic: tsx_mish.hpp (shared with the CPU build that pins them)
+// The fast form for layers bound by the activation's arithmetic (the 608x608 and 304x304 layers of a YOLOv4-shaped
+// backbone spend more issue slots on an exact Mish than the VALUs have in the time the layer's bytes take): one
+// exponential and one reciprocal at the hardware's 1 ulp,
 //     tanh(softplus(x)) = w / (w + 2) = 1 - 2 / (w + 2),  w = e (e + 2),  e = e^x = 2^(x log2 e),
-// 14 issue slots.  1 - 2r with r = 1 / (w + 2) in (0, 0.5] has the shape of the host's tanh, 2 * (1 / (1 + u)) - 1
-// (src/kernels/cpu/tanh.cpp:14-23): an absolute error of about 1e-7 in the quotient, so about 1e-7 |x| in the result
-// (relative 1e-7 for positive x; at most 2e-6 absolute for negative x, where Mish itself is small), against a bar of
-// 1e-4 relative + 1e-5 absolute -- and, like the host's, exactly 0 (-0 for the product) once x is below about -17,
-// where w + 2 rounds to 2.  NaN -> NaN, +-inf as the host's.
+// 14 issue slots.  1 - 2r with r = 1 / (w + 2) in (0, 0.5] has the shape of the host's tanh: an absolute error of about
+// 1e-7 in the quotient, so about 1e-7 |x| in the result (at most 2e-6 absolute for negative x, where Mish itself is
+// small) -- and, like the host's, exactly 0 (-0 for the product) once x is below about -17, where w + 2 rounds to 2.
+// NaN -> NaN, +-inf as the host's.  A requantized int8 value differs from the exact form's in about one of a million.
+// Opt-in (TSX_ACT_MISH_FAST); TSX_ACT_MISH is the exact form, mish_value.
 __device__ __forceinline__ float mish_short(float x) {
     const float e = __builtin_amdgcn_exp2f(__fmul_rn(fminf(x, 30.f), 1.4426950216293335f));   // beyond 30 the quotient is 1
     const float d = __builtin_fmaf(e, __fadd_rn(e, 2.f), 2.f);
@@ -170,16 +129,31 @@ __device__ __forceinline__ float mish_short(float x) {
     return __fmul_rn(x, t);
 }
 
-// apply_act for the int8 convolution epilogues: Mish in its short form (every path of those kernels -- fragment-wise
-// and per element -- goes through this one, so an element's value does not depend on the tile it falls into)
-__device__ __forceinline__ float apply_act_conv_i8(float v, int act, float slope, bool in_body) {
-    if (act != TSX_ACT_MISH) return apply_act_basic(v, act, slope, in_body);
-    return mish_short(v);
+// The activation of every epilogue: none / relu / leaky_relu / Mish (exact) / Mish (fast).  One function for all
+// kernels and all their paths, so an element's value never depends on the kernel or tile it falls into, and a fused
+// node gives what the separate operators give.
+__device__ __forceinline__ float apply_act(float v, int act, float slope, bool in_body) {
+    if (act == TSX_ACT_MISH) return mish_value(v);
+    if (act == TSX_ACT_MISH_FAST) return mish_short(v);
+    return apply_act_basic(v, act, slope, in_body);
+}
+// The exact Mish of the 16 values of an accumulator fragment, one value per turn of a loop that stays a loop: each
+// value's chain holds a dozen double-precision temporaries and twenty constants, and sixteen chains unrolled side by
+// side would push a kernel that keeps its accumulators and operands in registers into scratch memory.  The loop
+// counter is uniform: the values are reached by register indexing.
+__device__ __forceinline__ void mish_fragment(float (&v)[16]) {
+    typedef float v16f __attribute__((ext_vector_type(16)));
+    v16f t;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) t[r] = v[r];
+#pragma clang loop unroll(disable)
+    for (int r = 0; r < 16; ++r) t[r] = mish_value(t[r]);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) v[r] = t[r];
 }
 
-__device__ __forceinline__ float apply_act(float v, int act, float slope, bool in_body) {
-    if (act != TSX_ACT_MISH) return apply_act_basic(v, act, slope, in_body);
-    return mish_value(v);
+__device__ __forceinline__ float apply_act_conv_i8(float v, int act, float slope, bool in_body) {
+    return apply_act(v, act, slope, in_body);
 }
 
 #endif  // __HIPCC__

@@ -18,6 +18,33 @@ int fail(int code, const char *fmt, ...) {
 
 }  // namespace tsx
 
+extern "C" {
+
+
+const char *tsx_last_error(void) { return tsx::error_buffer(); }
+
+int tsx_version(void) { return 100; }
+
+int tsx_device_cu_count(void) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    return cus;
+}
+
+int tsx_conv2d_out_size(const tsx_conv2d_geom *g, int32_t *out_h, int32_t *out_w) {
+    TSX_REQUIRE(g && out_h && out_w, "null argument");
+    TSX_REQUIRE(g->stride_h > 0 && g->stride_w > 0 && g->dilation_h > 0 && g->dilation_w > 0 && g->kh > 0 && g->kw > 0,
+                "stride, dilation and kernel size must be positive");
+    *out_h = tsx::conv_out(g->h, g->pad_top, g->pad_bottom, g->kh, g->stride_h, g->dilation_h);
+    *out_w = tsx::conv_out(g->w, g->pad_left, g->pad_right, g->kw, g->stride_w, g->dilation_w);
+    return 0;
+}
+
+}  // extern "C"
+
+#ifdef TSX_MEASUREMENT_AIDS
+#include "tsx_aids.h"
 namespace {
 
 typedef int probe_v4i __attribute__((ext_vector_type(4)));
@@ -54,9 +81,7 @@ __global__ __launch_bounds__(256) void probe_mfma_i8_kernel(const probe_v4i *__r
 
 }  // namespace
 
-extern "C" {
-
-int tsx_probe_mfma_i8(const void *operands_dev, int32_t iters, int32_t blocks, int32_t *sink_dev, void *stream) {
+extern "C" int tsx_probe_mfma_i8(const void *operands_dev, int32_t iters, int32_t blocks, int32_t *sink_dev, void *stream) {
     TSX_REQUIRE(operands_dev && sink_dev && iters > 0 && blocks > 0, "probe_mfma_i8: bad argument");
     TSX_REQUIRE(reinterpret_cast<uintptr_t>(operands_dev) % 16 == 0, "probe_mfma_i8: operands must be 16-byte aligned");
     hipLaunchKernelGGL(probe_mfma_i8_kernel, dim3(unsigned(blocks)), dim3(256), 0, tsx::as_stream(stream),
@@ -64,25 +89,4 @@ int tsx_probe_mfma_i8(const void *operands_dev, int32_t iters, int32_t blocks, i
     TSX_LAUNCH_CHECK("probe_mfma_i8_kernel");
     return 0;
 }
-
-const char *tsx_last_error(void) { return tsx::error_buffer(); }
-
-int tsx_version(void) { return 100; }
-
-int tsx_device_cu_count(void) {
-    int dev = 0, cus = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return 0;
-    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-    return cus;
-}
-
-int tsx_conv2d_out_size(const tsx_conv2d_geom *g, int32_t *out_h, int32_t *out_w) {
-    TSX_REQUIRE(g && out_h && out_w, "null argument");
-    TSX_REQUIRE(g->stride_h > 0 && g->stride_w > 0 && g->dilation_h > 0 && g->dilation_w > 0 && g->kh > 0 && g->kw > 0,
-                "stride, dilation and kernel size must be positive");
-    *out_h = tsx::conv_out(g->h, g->pad_top, g->pad_bottom, g->kh, g->stride_h, g->dilation_h);
-    *out_w = tsx::conv_out(g->w, g->pad_left, g->pad_right, g->kw, g->stride_w, g->dilation_w);
-    return 0;
-}
-
-}  // extern "C"
+#endif  // TSX_MEASUREMENT_AIDS

@@ -660,7 +660,7 @@ int tsx_conv2d_winograd_f63_nchw(const tsx_conv2d_geom *q, const float *x_dev, c
     int rc = tsx::make_geom(q, padding_value, &g);
     if (rc) return rc;
     TSX_REQUIRE(x_dev && u_dev && out_dev, "winograd: null argument");
-    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_MISH, "winograd: unknown activation %d", act);
+    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_MISH_FAST, "winograd: unknown activation %d", act);
     const size_t need = tsx_winograd_f63_workspace_bytes(q);
     if (!workspace_dev || workspace_bytes < need)
         return tsx::fail(TSX_E_WORKSPACE, "winograd: workspace %zu < %zu bytes", workspace_bytes, need);
@@ -678,7 +678,7 @@ int tsx_conv2d_winograd_f63_nchw(const tsx_conv2d_geom *q, const float *x_dev, c
 
     const int64_t out_threads = int64_t(g.n) * g.cout * g.tiles;
     const int64_t count = int64_t(g.n) * g.cout * g.ho * g.wo;
-    if (act == TSX_ACT_MISH)
+    if (act >= TSX_ACT_MISH)
         hipLaunchKernelGGL(tsx::wino_output_transform_kernel<true>, dim3(unsigned(tsx::ceil_div(out_threads, 256))), dim3(256), 0,
                            stream, mm, g, bias_dev, act, slope, count / 4 * 4, out_dev);
     else
@@ -701,7 +701,7 @@ int tsx_conv2d_winograd_f63_fast_nchw(const tsx_conv2d_geom *q, const float *x_d
     int rc = tsx::make_geom(q, padding_value, &g);
     if (rc) return rc;
     TSX_REQUIRE(x_dev && u_dev && out_dev, "winograd: null argument");
-    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_MISH, "winograd: unknown activation %d", act);
+    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_MISH_FAST, "winograd: unknown activation %d", act);
     const size_t need = tsx_winograd_f63_fast_workspace_bytes(q);
     if (!workspace_dev || workspace_bytes < need)
         return tsx::fail(TSX_E_WORKSPACE, "winograd: workspace %zu < %zu bytes", workspace_bytes, need);
@@ -717,7 +717,7 @@ int tsx_conv2d_winograd_f63_fast_nchw(const tsx_conv2d_geom *q, const float *x_d
     const dim3 grid(unsigned(tsx::ceil_div(total_tiles, int64_t(tsx::WF_TILES))), unsigned(tsx::ceil_div(g.cout, tsx::WF_COUT)));
     const bool aligned = reinterpret_cast<uintptr_t>(u_dev) % 16 == 0;
     const int blocks = aligned && (g.c == 64 || g.c == 128 || g.c == 256) ? g.c / 16 : 0;
-    const bool mish = act == TSX_ACT_MISH;
+    const bool mish = act >= TSX_ACT_MISH;
 #define TSX_WF_LAUNCH(B, M)                                                                                         \
     hipLaunchKernelGGL((tsx::wino_f63_gemm_output_kernel<B, M>), grid, dim3(256), 0, stream, v, u_dev, g, bias_dev, act, \
                        slope, count / 4 * 4, out_dev)
@@ -757,7 +757,7 @@ int tsx_conv2d_winograd_f23_nchw(const tsx_conv2d_geom *q, const float *x_dev, c
     int rc = tsx::make_geom(q, padding_value, &g, 2);
     if (rc) return rc;
     TSX_REQUIRE(x_dev && u_dev && out_dev, "winograd_f23: null argument");
-    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_MISH, "winograd_f23: unknown activation %d", act);
+    TSX_REQUIRE(act >= TSX_ACT_NONE && act <= TSX_ACT_MISH_FAST, "winograd_f23: unknown activation %d", act);
     const size_t need = tsx_winograd_f23_workspace_bytes(q);
     if (!workspace_dev || workspace_bytes < need)
         return tsx::fail(TSX_E_WORKSPACE, "winograd_f23: workspace %zu < %zu bytes", workspace_bytes, need);
@@ -775,7 +775,7 @@ int tsx_conv2d_winograd_f23_nchw(const tsx_conv2d_geom *q, const float *x_dev, c
 
     const int64_t out_threads = int64_t(g.n) * g.cout * g.tiles;
     const int64_t count = int64_t(g.n) * g.cout * g.ho * g.wo;
-    if (act == TSX_ACT_MISH)
+    if (act >= TSX_ACT_MISH)
         hipLaunchKernelGGL(tsx::wino23_output_transform_kernel<true>, dim3(unsigned(tsx::ceil_div(out_threads, 256))), dim3(256), 0,
                            stream, mm, g, bias_dev, act, slope, count / 4 * 4, out_dev);
     else

@@ -154,9 +154,15 @@ def total_macs(L, batch, size):
 
 class YoloV4Int8:
     """The network on the device: calibrate(x) fixes one activation scale per convolution input, forward(x)
-    returns the three head tensors (fp32 NCHW)."""
+    returns the three head tensors (fp32 NCHW).  mish: "exact" -- the Mish layers give the values of the operator
+    chain softplus -> tanh -> mul bit for bit -- or "fast", the one-exponential form (1e-7 relative; about one
+    requantized int8 value in a million differs)."""
 
-    def __init__(self, L, heads, params, device="cuda:0"):
+    def __init__(self, L, heads, params, device="cuda:0", mish="exact"):
+        if mish not in ("exact", "fast"):
+            raise ValueError("mish: 'exact' or 'fast'")
+        if mish == "fast":
+            L = [dict(l, act="mish_fast") if l.get("act") == "mish" else l for l in L]
         self.L, self.heads, self.host = L, heads, params
         self.srcs, self.chans = resolve(L)
         self.dev = torch.device(device)

@@ -518,6 +518,9 @@ def test_max_pooling_on_a_channel_slice_of_staged_int8(tsx, port):
     fa = port.leaky_relu(port.add_bias(port.conv2d_quantized(xq, wa, dqa), ba), 0.1)
     cat = port.concat([port.pooling2d(fa, "max", (9, 9), (1, 1), (4, 4, 4, 4)), port.pooling2d(fa, "max", (5, 5), (1, 1), (2, 2, 2, 2)), fa], 1)
     assert np.array_equal(bits(got), bits(port.conv2d_quantized(port.quantize(cat, qs), wc, dqc)))
+    # a run that is no whole number of 64-channel blocks would pool into its neighbour's channels: refused
+    with pytest.raises(tsx.TsxError, match="whole 64-channel blocks"):
+        tsx.max_pooling2d_staged(tsx.StagedSlice(whole, 2 * f, 48), tsx.StagedSlice(whole, f, 48), (5, 5), (1, 1), (2, 2, 2, 2))
 
 
 def test_quantize_conv2d_fused_input(tsx, port):

@@ -1,9 +1,11 @@
 """YOLOv4-shaped int8 network: the device runner (tennis_amd/yolov4.py) against the CPU oracle interpreting
 the same layer list operator by operator.
 
-Every operator on the path is bit-exact except Mish (device expf/log), whose few-ulp differences can move a
-value across an int8 rounding boundary of the next quantize; the bar is therefore 2e-3 of the head's largest
-magnitude, with Mish-free (LeakyReLU-only) networks required to match bit for bit.
+Every operator on the path is bit-exact, Mish in its default (exact) form included: the heads of the small network
+match the oracle's bit for bit, and at full size every layer's fp32 output and int8 hand-over is the operator
+chain's -- the frozen bar allows 2 differing int8 values over the 190 M of the pass (none has been seen).  With the
+opt-in fast Mish (mish="fast": one hardware exponential and reciprocal, 1e-7 relative) a value now and then lands
+on the other side of a rounding boundary of the next quantize: at most 200 of the 190 M, each by one step.
 """
 import numpy as np
 import pytest
@@ -41,17 +43,17 @@ def oracle_forward(port, L, heads, srcs, params, scales, x):
     return [outs[h] for h in heads]
 
 
-@pytest.mark.parametrize("mish", [True, False])
+@pytest.mark.parametrize("mish", ["exact", "fast", None])
 def test_yolov4_shaped_network(port, mish):
     import torch
     from tennis_amd import yolov4
     L, heads = yolov4.layers(width=0.125, classes=3)
-    if not mish:
+    if mish is None:
         for l in L:
             if l["type"] == "conv" and l["act"] == "mish":
                 l["act"] = "leaky_relu"
     params = yolov4.make_parameters(L, seed=5)
-    net = yolov4.YoloV4Int8(L, heads, params)
+    net = yolov4.YoloV4Int8(L, heads, params, mish=mish or "exact")
     x = np.random.default_rng(6).uniform(0, 1, (2, 3, 64, 64)).astype(np.float32)
     xd = torch.from_numpy(x).cuda()
     scales = net.calibrate(xd)
@@ -64,25 +66,27 @@ def test_yolov4_shaped_network(port, mish):
     assert [g.shape for g in got] == [(2, 24, 8, 8), (2, 24, 4, 4), (2, 24, 2, 2)]
     for g, e in zip(got, exp):
         assert g.shape == e.shape and np.isfinite(e).all() and np.abs(e).max() > 0
-        if mish:
+        if mish == "fast":
             assert np.abs(g - e).max() <= 2e-3 * np.abs(e).max()
         else:
             assert np.array_equal(bits(g), bits(e))
 
 
-def test_full_size_network_every_layer(port, capsys):
+@pytest.mark.parametrize("mish", ["exact", "fast"])
+def test_full_size_network_every_layer(port, capsys, mish):
     """BASELINE config 5 at its real size (batch 8, 3x608x608, full width): every convolution of the chained
     pass checked by itself for the first and the last image -- the oracle runs the operator chain on the very
-    tensor the device kernel read, so one layer's result does not depend on another's.  Bar: bit-exact fp32
-    outputs and int8 hand-overs for LeakyReLU / linear layers.  Mish layers (device expf / log differ from the
-    host's by a few ulp): fp32 within 1e-4 relative + 1e-5 absolute, and int8 hand-over values that differ are
-    counted per layer, differ by one step only and stay below one in a thousand."""
+    tensor the device kernel read, so one layer's result does not depend on another's.  Bar for LeakyReLU / linear
+    layers: bit-exact fp32 outputs and int8 hand-overs.  Mish layers, exact form (the default): fp32 outputs bit for
+    bit, and at most 2 differing int8 hand-over values over the whole pass; fast form (only its Mish layers are
+    checked): fp32 within 1e-4 relative + 1e-5 absolute, int8 hand-over values that differ differ by one step and
+    number at most 200 over the whole pass."""
     import torch
     from tennis_amd import yolov4
     n = 8
     L, heads = yolov4.layers()
     params = yolov4.make_parameters(L, seed=0)
-    net = yolov4.YoloV4Int8(L, heads, params)
+    net = yolov4.YoloV4Int8(L, heads, params, mish=mish)
     x = torch.rand((n, 3, 608, 608), device="cuda", generator=torch.Generator(device="cuda").manual_seed(12))
     scales = net.calibrate(x)
     imgs = (0, n - 1)
@@ -91,43 +95,49 @@ def test_full_size_network_every_layer(port, capsys):
     torch.cuda.synchronize()
     rows, net.trace = net.trace[1], None
     assert all(torch.isfinite(o).all() for o in outs)
-    report, checked, worst_f32 = [], 0, 0.0
+    report, checked, worst_f32, f32_bits_off = [], 0, 0.0, 0
     for row in rows:
         i = row["layer"]
         l, p, s = L[i], params[i], np.float32(scales[i])
+        is_mish = l["act"] == "mish"
+        checked += 1
+        if mish == "fast" and not is_mish:
+            continue                                   # the other layers are the exact run's, checked there
         xq = row["in_q"] if row["in_q"] is not None else port.quantize(row["in_f32"], np.full(len(imgs), s, np.float32))
         dq = (np.float32(1.0) / (s * p["sw"])).astype(np.float32)
         pad = l["size"] // 2
         y = port.add_bias(port.conv2d_quantized(xq, p["wq"], dq, (pad,) * 4, (l["stride"],) * 2), p["bias"])
-        if l["act"] == "mish":
+        if is_mish:
             y = port.mish(y)
         elif l["act"] == "leaky_relu":
             y = port.leaky_relu(y, 0.1)
         if row["residual"] is not None:
             y = port.add(y, row["residual"])          # darknet's shortcut joins behind the activation
-        exact = l["act"] != "mish"
+        loose = is_mish and mish == "fast"
         if row["out_f32"] is not None:
-            if exact:
-                assert np.array_equal(bits(row["out_f32"]), bits(y)), "layer %d" % i
-            else:
+            if loose:
                 err = np.abs(row["out_f32"].astype(np.float64) - y)
-                assert (err <= 1e-4 * np.abs(y) + 1e-5).all(), "layer %d" % i      # the fp32 bar: 1e-4 rel + 1e-5 abs
+                assert (err <= 1e-4 * np.abs(y) + 1e-5).all(), "layer %d" % i
                 worst_f32 = max(worst_f32, float((err / (np.abs(y) + 1e-3)).max()))
+            else:
+                off = int(np.count_nonzero(bits(row["out_f32"]) != bits(y)))
+                assert off == 0, "layer %d: %d fp32 values differ" % (i, off)
         if row["out_q"] is not None:
             q = port.quantize(y, np.full(len(imgs), np.float32(scales[row["q_layer"]]), np.float32))
             diff = row["out_q"].astype(np.int32) - q.astype(np.int32)
             bad = int(np.count_nonzero(diff))
-            if exact:
+            if not is_mish:
                 assert bad == 0, "layer %d: %d int8 values differ" % (i, bad)
             else:
                 report.append((i, bad, diff.size))
-                assert np.abs(diff).max() <= 1 and bad <= 1e-3 * diff.size, "layer %d: %d of %d" % (i, bad, diff.size)
-        checked += 1
+                assert np.abs(diff).max() <= 1, "layer %d" % i
     assert checked == 110
+    total, values = sum(b for _, b, _ in report), sum(c for _, _, c in report)
     with capsys.disabled():
-        total = sum(b for _, b, _ in report)
-        print("\nMish layers, int8 hand-over values that differ from the host's (layer: differing / values): "
-              + ", ".join("%d: %d/%d" % r for r in report if r[1]) + "; total %d of %d; largest fp32 deviation %.2e of |value| + 1e-3" % (total, sum(c for _, _, c in report), worst_f32))
+        print("\nMish (%s) layers, int8 hand-over values that differ from the host's (layer: differing / values): " % mish
+              + (", ".join("%d: %d/%d" % r for r in report if r[1]) or "none")
+              + "; total %d of %d; largest fp32 deviation %.2e of |value| + 1e-3" % (total, values, worst_f32))
+    assert total <= (2 if mish == "exact" else 200), "%d int8 hand-over values of the Mish layers differ" % total
 
 
 def test_layer_list_matches_yolov4():
