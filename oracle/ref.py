@@ -54,96 +54,6 @@ def _check(rc):
         raise RuntimeError("reference raised: " + lib().ref_last_error().decode(errors="replace"))
 
 
-# ---- the reference built WITH this repository's "hip" device backend inside it (ref.mk `intree`):
-# TenniS's own Workbench / Stack / Tensor / operator factory running the backend's operators.
-_INTREE_PATH = os.path.join(_HERE, "_ref", "libref_driver_hip.so")
-_intree = None
-
-
-def intree_available():
-    return os.path.exists(_INTREE_PATH)
-
-
-def intree_lib():
-    global _intree
-    if _intree is None:
-        if not intree_available():
-            raise RuntimeError("in-tree build absent: run `make -C oracle -f ref.mk intree`")
-        _intree = ctypes.CDLL(_INTREE_PATH)   # RTLD_LOCAL: its TenniS copy stays apart from lib()'s
-        _intree.ref_last_error.restype = ctypes.c_char_p
-    return _intree
-
-
-def run_op_intree(device, op, params, inputs, out_bytes, threads=1, strict=True):
-    """Run operator ``op`` in a TenniS Workbench on ``device`` ("cpu" or "hip") of the in-tree build."""
-    L = intree_lib()
-    keep = []
-    p = (_Tensor * max(len(params), 1))(*[_pack(k, v, keep) for k, v in params.items()])
-    i = (_Tensor * max(len(inputs), 1))(*[_pack("", v, keep) for v in inputs])
-    buf = np.empty(out_bytes, dtype=np.uint8)
-    out = _Output()
-    out.data = buf.ctypes.data
-    out.capacity = out_bytes
-    rc = L.ref_run_op_on(device.encode(), int(strict), op.encode(), len(params), p, len(inputs), i, int(threads), ctypes.byref(out))
-    if rc != 0:
-        raise RuntimeError("TenniS raised: " + L.ref_last_error().decode(errors="replace"))
-    shape = tuple(out.shape[k] for k in range(out.ndim))
-    return buf[:out.bytes].view(_TS2NP[out.dtype]).reshape(shape).copy()
-
-
-def fused_chain_count_intree():
-    """Chains the "hip" device's zipper option has replaced so far in the in-tree library."""
-    L = intree_lib()
-    L.ref_hip_fused_chain_count.restype = ctypes.c_long
-    return int(L.ref_hip_fused_chain_count())
-
-
-def handover_counts_intree():
-    """(fused nodes that write a staged int8 output for the convolutions behind them, those of them that return
-    the fp32 form as well) so far in the in-tree library."""
-    L = intree_lib()
-    L.ref_hip_handover_count.restype = ctypes.c_long
-    L.ref_hip_dual_output_count.restype = ctypes.c_long
-    return int(L.ref_hip_handover_count()), int(L.ref_hip_dual_output_count())
-
-
-def run_module_intree(device, path, inputs, out_bytes=1 << 24, threads=1):
-    """Load a `.tsm` file into a TenniS Workbench on ``device`` ("cpu" or "hip") of the in-tree build: TenniS's own
-    module loader, graph compiler and runtime, with this repository's backend serving device "hip"."""
-    L = intree_lib()
-    keep = []
-    i = (_Tensor * max(len(inputs), 1))(*[_pack("", v, keep) for v in inputs])
-    buf = np.empty(out_bytes, dtype=np.uint8)
-    out = _Output()
-    out.data = buf.ctypes.data
-    out.capacity = out_bytes
-    rc = L.ref_run_module(str(path).encode(), device.encode(), len(inputs), i, int(threads), ctypes.byref(out))
-    if rc != 0:
-        raise RuntimeError("TenniS raised: " + L.ref_last_error().decode(errors="replace"))
-    shape = tuple(out.shape[k] for k in range(out.ndim))
-    return buf[:out.bytes].view(_TS2NP[out.dtype]).reshape(shape).copy()
-
-
-def time_module_intree(device, path, inputs, warmup=2, reps=10, out_bytes=1 << 24, threads=1, resident=False):
-    """ms per run of a `.tsm` module in a TenniS Workbench on ``device`` of the in-tree build (module loaded and
-    compiled once; each run ends with output 0 read back), and that output.  ``resident``: the inputs are moved to
-    the device before the timed loop instead of being uploaded by every run."""
-    L = intree_lib()
-    keep = []
-    i = (_Tensor * max(len(inputs), 1))(*[_pack("", v, keep) for v in inputs])
-    buf = np.empty(out_bytes, dtype=np.uint8)
-    out = _Output()
-    out.data = buf.ctypes.data
-    out.capacity = out_bytes
-    ms = ctypes.c_double(0.0)
-    rc = L.ref_time_module(str(path).encode(), device.encode(), len(inputs), i, int(threads), int(warmup), int(reps),
-                           int(bool(resident)), ctypes.byref(ms), ctypes.byref(out))
-    if rc != 0:
-        raise RuntimeError("TenniS raised: " + L.ref_last_error().decode(errors="replace"))
-    shape = tuple(out.shape[k] for k in range(out.ndim))
-    return ms.value, buf[:out.bytes].view(_TS2NP[out.dtype]).reshape(shape).copy()
-
-
 def _pack(name, value, keep):
     """Turn a python value into a _Tensor; ``keep`` holds the buffers alive."""
     if isinstance(value, str):

@@ -283,13 +283,4 @@ int ref_gemm_f32(int m, int n, int k, const float *a, const float *bm, float *c,
     });
 }
 
-// Chains replaced by the "hip" device's zipper option so far (in-tree build); -1 where the library holds no such option.
-long tsx_hip_fused_chain_count() __attribute__((weak));
-long ref_hip_fused_chain_count() { return tsx_hip_fused_chain_count ? tsx_hip_fused_chain_count() : -1; }
-// ... of which write a staged int8 output for the convolutions behind them / return the fp32 form as well
-long tsx_hip_handover_count() __attribute__((weak));
-long tsx_hip_dual_output_count() __attribute__((weak));
-long ref_hip_handover_count() { return tsx_hip_handover_count ? tsx_hip_handover_count() : -1; }
-long ref_hip_dual_output_count() { return tsx_hip_dual_output_count ? tsx_hip_dual_output_count() : -1; }
-
 }  // extern "C"

@@ -104,7 +104,7 @@ public:
         tsx_conv2d_geom g, gn;
         const Tensor::Prototype proto = out_proto(stack, g, gn);
         output.clear();
-        if (m_dual) output.push_back(Tensor::Prototype(FLOAT32, Shape({g.n, g.cout, m_ho, m_wo})));
+        if (m_dual) output.push_back(Tensor::Prototype(FLOAT32, m_out_shape));
         output.push_back(proto);
         return int(output.size());
     }
@@ -122,6 +122,11 @@ public:
         if (m_residual) residual = stack[int(stack.size()) - 1].view(device);
         const Shape conv_shape({g.n, g.cout, m_ho, m_wo});
         const bool same_shape = m_residual && residual.sizes() == conv_shape;
+        // A residual of another shape (it broadcasts into the convolution's output, or the output into it) joins in a
+        // pass of its own, as the separate `add` did: the epilogue writes fp32, the activation in front of the join
+        // (mode 2) stays in the epilogue, the one behind it (mode 1) follows the pass, and a staged int8 output is
+        // then quantized and staged from the sum by the staging kernel.
+        const bool split = m_residual && !same_shape;
         // The staged int8 output lives in a tensor this operator keeps from run to run: its halo and channel padding
         // are written once, when it is allocated, and every run's epilogue overwrites exactly the interior -- a
         // tensor from the stack is fresh memory each time and would need the halo filled again (one more launch per
@@ -141,25 +146,24 @@ public:
             out = *stack.push(proto, device);
         }
         Tensor out_plain;
-        if (m_dual) out_plain = stack.make(Tensor::Prototype(FLOAT32, conv_shape), device);
+        if (m_dual || (split && m_next)) out_plain = stack.make(Tensor::Prototype(FLOAT32, m_out_shape), device);
+        // the convolution's own result where it is not the node's fp32 output already
+        Tensor conv_out;
+        if (split && (m_next || !(m_out_shape == conv_shape))) conv_out = stack.make(Tensor::Prototype(FLOAT32, conv_shape), device);
         void *stream = current_stream();
         const bool pairs = pairs_apply(g, gn, out);
         const void *packed = pairs ? nullptr : m_state.packed(g, w, device, stream, "conv2d_quantized_fused");
         tsx_epilogue ep{};
         ep.dq_dev = m_dq_dev.get(m_dq, device);
         ep.bias_dev = with_bias ? bias.data<float>() : nullptr;
-        // a residual that needs broadcasting joins in a pass of its own: the activation in front of it (mode 2) stays
-        // in the epilogue, the one behind it (mode 1) follows that pass
-        const bool split = m_residual && !same_shape;
         ep.act = (split && m_residual == 1) ? TSX_ACT_NONE : m_act;
         ep.slope = m_slope;
         if (same_shape) {
             ep.residual_dev = residual.data<float>();
             ep.residual_after_act = m_residual == 2 ? 1 : 0;
         }
-        float *out_f32 = out.data<float>();
-        if (m_next) {
-            if (split) TS_LOG_ERROR << "conv2d_quantized_fused: a residual that broadcasts cannot be combined with next_*" << eject;
+        float *out_f32 = !conv_out.empty() ? conv_out.data<float>() : out.data<float>();
+        if (m_next && !split) {
             // the consumer's staged input: halo and channel padding (once), then the interior from the epilogue
             if (fill_halo)
                 check(tsx_conv2d_i8_stage_fill_halo(&gn, m_next_padding_value, out.data(), size_t(out.count()), stream),
@@ -229,16 +233,21 @@ public:
                   "tsx_quantize_conv2d_i8_nchw");
         }
         if (split) {
-            std::vector<int32_t> lhs(proto.sizes().begin(), proto.sizes().end()), rhs(lhs.size(), 1);
+            Tensor &sum = m_next ? out_plain : out;
+            std::vector<int32_t> lhs(conv_shape.begin(), conv_shape.end()), rhs(lhs.size(), 1);
             const Shape &rs = residual.sizes();
             for (size_t i = 0; i < rs.size(); ++i) rhs[lhs.size() - rs.size() + i] = rs[i];
-            check(tsx_add_broadcast_f32(out.data<float>(), lhs.data(), residual.data<float>(), rhs.data(), int32_t(lhs.size()),
-                                        out.data<float>(), stream),
+            check(tsx_add_broadcast_f32(out_f32, lhs.data(), residual.data<float>(), rhs.data(), int32_t(lhs.size()),
+                                        sum.data<float>(), stream),
                   "tsx_add_broadcast_f32");
             if (m_residual == 1 && m_act == TSX_ACT_RELU)
-                check(tsx_relu_f32(out.data<float>(), out.count(), out.data<float>(), stream), "tsx_relu_f32");
+                check(tsx_relu_f32(sum.data<float>(), sum.count(), sum.data<float>(), stream), "tsx_relu_f32");
             else if (m_residual == 1 && m_act == TSX_ACT_LEAKY_RELU)
-                check(tsx_leaky_relu_f32(out.data<float>(), out.count(), m_slope, out.data<float>(), stream), "tsx_leaky_relu_f32");
+                check(tsx_leaky_relu_f32(sum.data<float>(), sum.count(), m_slope, sum.data<float>(), stream), "tsx_leaky_relu_f32");
+            if (m_next)   // the whole staged tensor, halo included
+                check(tsx_conv2d_i8_stage(&gn, sum.data<float>(), 1, m_next_q_dev.get(m_next_q, device), int32_t(m_next_q.size()),
+                                          m_next_padding_value, out.data(), size_t(out.count()), stream),
+                      "tsx_conv2d_i8_stage");
         }
         if (m_dual) stack.push(Tensor::Pack({out_plain, out}));
         return 1;
@@ -309,24 +318,28 @@ private:
         if (ho <= 0 || wo <= 0) TS_LOG_ERROR << "conv2d_quantized_fused: empty output " << ho << "x" << wo << eject;
         m_ho = ho;
         m_wo = wo;
-        const Shape out({g.n, w.size(0), ho, wo});
+        Shape out({g.n, w.size(0), ho, wo});
         if (m_residual) {
-            // the other operand of the `add` this node absorbed: the output's shape, or one that broadcasts into it
+            // the other operand of the `add` this node absorbed: the two broadcast against each other as the operator's
+            // operands did (src/backend/base/element_wise_reduce.cpp:150-206), either one may be the one that repeats
             const Tensor &r = stack[int(stack.size()) - 1];
             bool fits = r.dtype() == FLOAT32 && r.dims() <= out.size();
             for (size_t i = 0; fits && i < r.dims(); ++i) {
-                const int32_t extent = r.size(i), target = out[out.size() - r.dims() + i];
-                fits = extent == target || extent == 1;
+                int32_t &target = out[out.size() - r.dims() + i];
+                const int32_t extent = r.size(i);
+                fits = extent == target || extent == 1 || target == 1;
+                if (target == 1) target = extent;
             }
             if (!fits)
-                TS_LOG_ERROR << "conv2d_quantized_fused: residual " << to_string(r.sizes()) << " does not broadcast into "
-                             << to_string(out) << eject;
+                TS_LOG_ERROR << "conv2d_quantized_fused: residual " << to_string(r.sizes()) << " and the convolution's output "
+                             << to_string(Shape({g.n, w.size(0), ho, wo})) << " do not broadcast" << eject;
         }
+        m_out_shape = out;
         if (!m_next) return Tensor::Prototype(FLOAT32, out);
         // the consumer's staged input
-        if (int32_t(m_next_q.size()) != g.n)
-            TS_LOG_ERROR << "conv2d_quantized_fused: " << m_next_q.size() << " next_quantize_scale values for a batch of " << g.n << eject;
-        gn = tsx_conv2d_geom{g.n, w.size(0), ho, wo, 1, m_next_ksize[0], m_next_ksize[1], m_next_pad[0], m_next_pad[1],
+        if (int32_t(m_next_q.size()) != out[0])
+            TS_LOG_ERROR << "conv2d_quantized_fused: " << m_next_q.size() << " next_quantize_scale values for a batch of " << out[0] << eject;
+        gn = tsx_conv2d_geom{out[0], out[1], out[2], out[3], 1, m_next_ksize[0], m_next_ksize[1], m_next_pad[0], m_next_pad[1],
                              m_next_pad[2], m_next_pad[3], m_next_stride[0], m_next_stride[1], m_next_dil[0], m_next_dil[1]};
         int32_t hs = 0, ws = 0, cp = 0;
         if (tsx_conv2d_i8_staged_dims(&gn, &hs, &ws, &cp) != 0) TS_LOG_ERROR << "[hip] conv2d_quantized_fused: " << tsx_last_error() << eject;
@@ -342,6 +355,7 @@ private:
     std::vector<int32_t> m_next_ksize, m_next_pad, m_next_stride, m_next_dil;
     float m_next_padding_value = 0.f;
     int m_ho = 0, m_wo = 0;
+    Shape m_out_shape;   // the node's output as NCHW: the convolution's, or its broadcast against the residual
     DeviceFloats m_next_q_dev;
     Tensor m_staged_out;
     std::vector<float> m_dq, m_q;

@@ -1,12 +1,17 @@
-"""The "hip" backend inside the real TenniS runtime: oracle/ref.mk's `intree` target compiles
-tennis_amd/backend/hip/*.cpp against TenniS's own headers and links them into the reference
-library, as TenniS does with its own device backends.  Each operator is then created and run by
-TenniS's Workbench on ComputingDevice("hip") and on ComputingDevice("cpu") -- same process, same
-operator factory, same Tensor/SyncMemory machinery -- and the two outputs compared.
+"""The "hip" backend inside the real TenniS runtime: tennis_amd/backend/intree/intree.mk compiles
+tennis_amd/backend/hip/*.cpp against TenniS's own headers and links them into the TenniS library, as TenniS does
+with its own device backends (tennis_amd/lib/intree/libtennis_hip.so, driven through tennis_amd/intree.py).  Each
+operator is then created and run by TenniS's Workbench on ComputingDevice("hip") and on ComputingDevice("cpu") --
+same process, same operator factory, same Tensor/SyncMemory machinery -- and the two outputs compared.
 
 Bar: bitwise for the int8 operators, the elementwise operators and Winograd F(6,3); 1e-4
 relative + 1e-5 absolute for the fp32 MFMA GEMM paths.  Skipped where the in-tree build is absent
-(it needs the reference tree at build time).
+(it needs the TenniS source tree at build time).
+
+A "hip" class hands inputs its kernel does not cover to the host operator of the same name.  So that a comparison
+of "hip" with "cpu" cannot quietly become one of "cpu" with "cpu", every test here runs under a check that the
+library's count of such hand-overs did not move -- except the tests marked `delegates`, which are about exactly
+those inputs and must see it rise.
 """
 import numpy as np
 import pytest
@@ -20,20 +25,41 @@ pytestmark = pytest.mark.gpu
 def ts():
     import torch
     assert torch.cuda.is_available(), "these tests need the MI355X"
-    from oracle import ref
-    if not ref.intree_available():
-        pytest.skip("oracle/_ref/libref_driver_hip.so not built in this tree")
-    ref.intree_lib()
-    return ref
+    from tennis_amd import intree
+    if not intree.available():
+        pytest.skip("tennis_amd/lib/intree/libtennis_hip_driver.so not built in this tree")
+    intree.lib()
+    return intree
 
 
-def conv_params(ref, pads, strides=(1, 1), dil=(1, 1), pv=0.0):
-    return ref._conv_params(pads, strides, dil, pv)
+@pytest.fixture(autouse=True)
+def host_delegate_watch(request, ts):
+    """Yields a dict; a test that hands some operator runs to the host on purpose sets watch["expected"] to their
+    number (tests marked `delegates` are about such inputs throughout and only need to see the count rise)."""
+    watch = {"expected": 0}
+    before = ts.host_delegate_count()
+    yield watch
+    moved = ts.host_delegate_count() - before
+    if request.node.get_closest_marker("delegates"):
+        assert moved > 0, "no operator run was handed to the host operator"
+    else:
+        assert moved == watch["expected"], "%d operator runs on \"hip\" were handed to the host operator, %d expected" % (
+            moved, watch["expected"])
+
+
+def conv_params(ts, pads, strides=(1, 1), dil=(1, 1), pv=0.0):
+    return {
+        "format": "NCHW",
+        "padding": np.array([[0, 0], [0, 0], [pads[0], pads[1]], [pads[2], pads[3]]], np.int32),
+        "padding_value": np.array([pv], np.float32),
+        "stride": np.array([1, 1, strides[0], strides[1]], np.int32),
+        "dilation": np.array([1, 1, dil[0], dil[1]], np.int32),
+    }
 
 
 def both(ts, op, params, inputs, out_bytes):
-    cpu = ts.run_op_intree("cpu", op, params, inputs, out_bytes)
-    hip = ts.run_op_intree("hip", op, params, inputs, out_bytes)
+    cpu = ts.run_op("cpu", op, params, inputs, out_bytes)
+    hip = ts.run_op("hip", op, params, inputs, out_bytes)
     assert cpu.shape == hip.shape and cpu.dtype == hip.dtype
     return cpu, hip
 
@@ -92,13 +118,14 @@ def test_fp32_operators_in_tennis_workbench(ts):
 
 def test_glue_operators_in_tennis_workbench(ts):
     """pooling2d / global_pooling2d / add / depthwise_conv2d run by TenniS's Workbench with strict device
-    lookup, so the "hip" classes (not the host fallback) produce the result; bitwise against the host operators."""
+    lookup, so the "hip" classes are the ones created, and (host_delegate_watch) none of them hands its inputs to the
+    host operator: the device produces the result; bitwise against the host operators."""
     rng = np.random.default_rng(902)
     x = rng.standard_normal((2, 6, 14, 12)).astype(np.float32)
 
     def strict_both(op, params, inputs, out_bytes):
-        cpu = ts.run_op_intree("cpu", op, params, inputs, out_bytes)
-        hip = ts.run_op_intree("hip", op, params, inputs, out_bytes, strict=True)
+        cpu = ts.run_op("cpu", op, params, inputs, out_bytes)
+        hip = ts.run_op("hip", op, params, inputs, out_bytes, strict=True)
         assert cpu.shape == hip.shape
         assert np.array_equal(bits(cpu), bits(hip)), (op, params)
 
@@ -126,9 +153,9 @@ def test_unregistered_operator_falls_back_to_cpu(ts):
     backend's converters."""
     x = np.linspace(-3, 3, 24, dtype=np.float32).reshape(2, 3, 4)
     with pytest.raises(RuntimeError):
-        ts.run_op_intree("hip", "sigmoid", {}, [x], x.nbytes, strict=True)
-    cpu = ts.run_op_intree("cpu", "sigmoid", {}, [x], x.nbytes)
-    hip = ts.run_op_intree("hip", "sigmoid", {}, [x], x.nbytes, strict=False)
+        ts.run_op("hip", "sigmoid", {}, [x], x.nbytes, strict=True)
+    cpu = ts.run_op("cpu", "sigmoid", {}, [x], x.nbytes)
+    hip = ts.run_op("hip", "sigmoid", {}, [x], x.nbytes, strict=False)
     assert np.array_equal(bits(cpu), bits(hip))
 
 
@@ -170,13 +197,13 @@ def test_module_file_in_tennis_workbench_on_hip(ts):
     path = os.path.join(root, "quantized_block.tsm")
     x = tensor_file.read_tensor(os.path.join(root, "quantized_block.input_0.t"))
     want = tensor_file.read_tensor(os.path.join(root, "quantized_block.output_0.t"))
-    fused0 = ts.fused_chain_count_intree()
-    cpu = ts.run_module_intree("cpu", path, [x])
-    assert ts.fused_chain_count_intree() == fused0        # the zipper option is for device "hip" only
-    hip = ts.run_module_intree("hip", path, [x])
+    fused0 = ts.fused_chain_count()
+    cpu = ts.run_module("cpu", path, [x])
+    assert ts.fused_chain_count() == fused0        # the zipper option is for device "hip" only
+    hip = ts.run_module("hip", path, [x])
     # TenniS's compiler, walking the graph with this backend's zipper option, has replaced both chains of the
     # module (quantize -> conv -> add_bias -> relu and quantize -> conv) by conv2d_quantized_fused nodes
-    assert ts.fused_chain_count_intree() == fused0 + 2
+    assert ts.fused_chain_count() == fused0 + 2
     assert np.array_equal(bits(cpu), bits(want))
     assert hip.shape == want.shape and np.array_equal(bits(hip), bits(want))
 
@@ -194,16 +221,16 @@ def test_resnet_shaped_module_in_tennis_workbench_on_hip(ts, tmp_path):
     path = str(tmp_path / "resnet_shaped.tsm")
     mf.write_module(path, module)
     x = np.random.default_rng(1).random((2, 3, 64, 64), dtype=np.float32)
-    cpu = ts.run_module_intree("cpu", path, [x])
-    fused0 = ts.fused_chain_count_intree()
-    hand0, dual0 = ts.handover_counts_intree()
-    hip = ts.run_module_intree("hip", path, [x])
-    assert ts.fused_chain_count_intree() == fused0 + 23   # every quantized convolution of the network, fused by TenniS's compiler
+    cpu = ts.run_module("cpu", path, [x])
+    fused0 = ts.fused_chain_count()
+    hand0, dual0 = ts.handover_counts()
+    hip = ts.run_module("hip", path, [x])
+    assert ts.fused_chain_count() == fused0 + 23   # every quantized convolution of the network, fused by TenniS's compiler
     # int8 hand-overs: c1 -> c2 -> c3 inside each of the 6 blocks (12), and each join that another block reads
     # (5: the last one feeds the pooling), plus the stem through its max pooling (2).  The joins in front of the two identity blocks are read by the next
     # block's first convolution AND its residual add, so they return both forms (dual output); the ones in front
     # of a projection block are read by two convolutions of different stride sharing one staged tensor.
-    hand, dual = ts.handover_counts_intree()
+    hand, dual = ts.handover_counts()
     assert (hand - hand0, dual - dual0) == (19, 2)
     assert cpu.shape == (2, 10) and hip.shape == (2, 10) and np.abs(cpu).max() > 0.1
     assert close(hip, cpu)
@@ -211,6 +238,30 @@ def test_resnet_shaped_module_in_tennis_workbench_on_hip(ts, tmp_path):
     (fused,) = mf.run_module(mf.fuse_quantized_chains(module), [x])
     assert np.array_equal(bits(own), bits(hip))          # the same device operators, with or without TenniS around them
     assert np.array_equal(bits(fused), bits(own))
+
+
+def test_cloned_workbenches_on_hip_one_per_host_thread(ts, tmp_path):
+    """TenniS's threading contract on "hip": one Workbench per thread, the further ones made by Workbench::clone
+    (src/runtime/workbench.cpp; every instruction's operator is re-created with the same parameters,
+    src/runtime/instruction.cpp:91-103; the thread-local contexts of include/utils/ctxmgr_lite_support.h:47-95 are
+    bound by each Workbench's own entry points).  The ResNet-50-shaped module -- fused nodes that keep their staged
+    int8 output from run to run, packed weights per operator instance, scratch per device context -- is loaded
+    once, cloned twice, and the three Workbenches run three times each on three different batches from three host
+    threads at once: every thread's logits must be, bit for bit, what a single Workbench gives for its batch."""
+    from tennis_amd import module_file as mf, resnet50
+    desc, params = resnet50.make_parameters(seed=3, width=0.25, blocks=(2, 1, 2, 1), classes=10)
+    path = str(tmp_path / "resnet_shaped.tsm")
+    mf.write_module(path, resnet50.to_module(desc, params, batch=2))
+    rng = np.random.default_rng(31)
+    batches = [rng.random((2, 3, 64, 64), dtype=np.float32) for _ in range(3)]
+    alone = [ts.run_module("hip", path, [x]) for x in batches]
+    assert not np.array_equal(alone[0], alone[1])
+    together = ts.run_module_cloned("hip", path, [[x] for x in batches], runs=3)
+    for t, (a, b) in enumerate(zip(alone, together)):
+        assert a.shape == b.shape == (2, 10) and np.array_equal(bits(a), bits(b)), "thread %d" % t
+    # a control of the driver entry by itself: one thread, the host device of the same library
+    (cpu,) = ts.run_module_cloned("cpu", path, [[batches[0]]], runs=1)
+    assert np.array_equal(bits(cpu), bits(ts.run_module("cpu", path, [batches[0]])))
 
 
 def test_full_width_stem_as_column_pairs_in_tennis_workbench_on_hip(ts, tmp_path):
@@ -224,10 +275,10 @@ def test_full_width_stem_as_column_pairs_in_tennis_workbench_on_hip(ts, tmp_path
     path = str(tmp_path / "resnet_full_width.tsm")
     mf.write_module(path, module)
     x = np.random.default_rng(2).random((2, 3, 64, 64), dtype=np.float32)
-    cpu = ts.run_module_intree("cpu", path, [x])
-    hand0, _ = ts.handover_counts_intree()
-    hip = ts.run_module_intree("hip", path, [x])
-    assert ts.handover_counts_intree()[0] > hand0
+    cpu = ts.run_module("cpu", path, [x])
+    hand0, _ = ts.handover_counts()
+    hip = ts.run_module("hip", path, [x])
+    assert ts.handover_counts()[0] > hand0
     assert cpu.shape == (2, 10) and np.abs(cpu).max() > 0.1 and close(hip, cpu)
     (own,) = mf.run_module(module, [x])
     assert np.array_equal(bits(own), bits(hip))
@@ -267,16 +318,17 @@ def test_zipper_option_leaky_relu_and_shared_convolution(ts, tmp_path):
     path = str(tmp_path / "zipper_cases.tsm")
     mf.write_module(path, module)
     x = (rng.standard_normal((n, c, h, w)) * 6).astype(np.float32)
-    cpu = ts.run_module_intree("cpu", path, [x])
-    fused0 = ts.fused_chain_count_intree()
-    hip = ts.run_module_intree("hip", path, [x])
-    assert ts.fused_chain_count_intree() == fused0 + 2
+    cpu = ts.run_module("cpu", path, [x])
+    fused0 = ts.fused_chain_count()
+    hip = ts.run_module("hip", path, [x])
+    assert ts.fused_chain_count() == fused0 + 2
     assert cpu.shape == (n, ca + 2 * cb, h, w)
     assert np.array_equal(bits(hip), bits(cpu))
     (own,) = mf.run_module(mf.fuse_quantized_chains(module), [x])     # the same rewrite outside TenniS
     assert np.array_equal(bits(own), bits(cpu))
 
 
+@pytest.mark.delegates
 def test_inputs_a_hip_class_does_not_cover_run_the_host_operator(ts):
     """A registered "hip" class that meets a data type or mode its kernel does not take hands the call to the
     host operator of the same name (TenniS itself falls back only for operators a device does not register):
@@ -285,8 +337,8 @@ def test_inputs_a_hip_class_does_not_cover_run_the_host_operator(ts):
     rng = np.random.default_rng(905)
 
     def same(op, params, inputs, out_bytes):
-        cpu = ts.run_op_intree("cpu", op, params, inputs, out_bytes)
-        hip = ts.run_op_intree("hip", op, params, inputs, out_bytes, strict=True)
+        cpu = ts.run_op("cpu", op, params, inputs, out_bytes)
+        hip = ts.run_op("hip", op, params, inputs, out_bytes, strict=True)
         assert cpu.shape == hip.shape and cpu.dtype == hip.dtype, (op, cpu.dtype, hip.dtype)
         assert np.array_equal(cpu.view(np.uint8), hip.view(np.uint8)), op
         return cpu
@@ -325,7 +377,7 @@ def test_inputs_a_hip_class_does_not_cover_run_the_host_operator(ts):
     errors = []
     for device in ("cpu", "hip"):
         with pytest.raises(RuntimeError) as e:
-            ts.run_op_intree(device, "pooling2d", p, [xn], xn.nbytes)
+            ts.run_op(device, "pooling2d", p, [xn], xn.nbytes)
         errors.append(str(e.value).split("only support")[-1])
     assert errors[0] == errors[1] and "NCHW" in errors[0]
 
@@ -353,10 +405,10 @@ def test_zipper_option_resolves_the_bias_axis_like_add_bias(ts, tmp_path):
     path = str(tmp_path / "bias_axis.tsm")
     mf.write_module(path, module)
     x = (rng.standard_normal((n, c, h, w)) * 6).astype(np.float32)
-    cpu = ts.run_module_intree("cpu", path, [x])
-    fused0 = ts.fused_chain_count_intree()
-    hip = ts.run_module_intree("hip", path, [x])
-    assert ts.fused_chain_count_intree() == fused0 + 1
+    cpu = ts.run_module("cpu", path, [x])
+    fused0 = ts.fused_chain_count()
+    hip = ts.run_module("hip", path, [x])
+    assert ts.fused_chain_count() == fused0 + 1
     assert np.array_equal(bits(hip), bits(cpu))
     fused = mf.fuse_quantized_chains(module)
     assert [m.op for m in fused.nodes].count("add_bias") == 1
@@ -364,7 +416,7 @@ def test_zipper_option_resolves_the_bias_axis_like_add_bias(ts, tmp_path):
     assert np.array_equal(bits(own), bits(cpu))
 
 
-def test_batch_norm_family_in_tennis_workbench(ts):
+def test_batch_norm_family_in_tennis_workbench(ts, host_delegate_watch):
     """batch_norm / batch_scale / fused_batch_norm created with strict device lookup, so the "hip" classes run:
     bitwise against TenniS's CPU operators; fp64 inputs go through the host delegate."""
     rng = np.random.default_rng(907)
@@ -377,14 +429,15 @@ def test_batch_norm_family_in_tennis_workbench(ts):
         e = dict(d, epsilon=np.array([1e-3], np.float32))
         for op, params, inputs in (("batch_norm", e, [x, mean, var]), ("batch_norm", d, [x, mean, var]),
                                    ("batch_scale", d, [x, scale, bias]), ("fused_batch_norm", e, [x, mean, var, scale, bias])):
-            cpu = ts.run_op_intree("cpu", op, params, inputs, x.nbytes)
-            hip = ts.run_op_intree("hip", op, params, inputs, x.nbytes, strict=True)
+            cpu = ts.run_op("cpu", op, params, inputs, x.nbytes)
+            hip = ts.run_op("hip", op, params, inputs, x.nbytes, strict=True)
             assert np.array_equal(bits(cpu), bits(hip)), (op, shape)
     xd = rng.standard_normal((2, 4, 3, 3))
     vd = rng.uniform(0.5, 2, 4)
     d = {"dim": np.array([1], np.int32)}
-    cpu = ts.run_op_intree("cpu", "batch_scale", d, [xd, vd, vd], xd.nbytes)
-    hip = ts.run_op_intree("hip", "batch_scale", d, [xd, vd, vd], xd.nbytes, strict=True)
+    cpu = ts.run_op("cpu", "batch_scale", d, [xd, vd, vd], xd.nbytes)
+    host_delegate_watch["expected"] = 1        # fp64: the one run of this test the device hands to the host operator
+    hip = ts.run_op("hip", "batch_scale", d, [xd, vd, vd], xd.nbytes, strict=True)
     assert hip.dtype == np.float64 and np.array_equal(cpu.view(np.uint8), hip.view(np.uint8))
 
 
@@ -431,13 +484,63 @@ def test_zipper_option_folds_residual_joins(ts, tmp_path):
     path = str(tmp_path / "residual_cases.tsm")
     mf.write_module(path, module)
     x = (rng.standard_normal((n, c, h, w)) * 6).astype(np.float32)
-    cpu = ts.run_module_intree("cpu", path, [x])
-    fused0 = ts.fused_chain_count_intree()
-    hip = ts.run_module_intree("hip", path, [x])
-    assert ts.fused_chain_count_intree() == fused0 + 4     # main (+ join), proj, dark (+ shortcut), scaled (+ offset)
+    cpu = ts.run_module("cpu", path, [x])
+    fused0 = ts.fused_chain_count()
+    hip = ts.run_module("hip", path, [x])
+    assert ts.fused_chain_count() == fused0 + 4     # main (+ join), proj, dark (+ shortcut), scaled (+ offset)
     assert cpu.shape == (n, 2 * co, h, w)
     assert np.array_equal(bits(hip), bits(cpu))
     fused = mf.fuse_quantized_chains(module)
     assert "add" not in [m.op for m in fused.nodes]
     (own,) = mf.run_module(fused, [x])
     assert np.array_equal(bits(own), bits(cpu))
+
+
+def test_zipper_option_residuals_that_broadcast_keep_running(ts, tmp_path):
+    """An `add` the zipper folds into a fused node whose operands do not have one shape: (a) the convolution's
+    [n, c, 1, 1] output added to an [n, c, h, w] tensor -- the convolution's result is the one that repeats -- and
+    (b) a per-channel [1, c, 1, 1] operand, each followed by another quantized chain, so the fused node also has to
+    hand its sum over as staged int8.  Both ran as separate operators before the rewrite and must keep running, with
+    the host device's values bit for bit."""
+    import sys, os
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"))
+    from make_modules import conv_params
+    from tennis_amd import module_file as mf
+    rng = np.random.default_rng(83)
+    n, c, h, w, co = 2, 16, 7, 9, 16
+    N = mf.Node
+    nodes = [N(mf.PARAMETER, "x")]
+
+    def chain(name, src, cin, kh, kw, pads, act=None):
+        wq = rng.integers(-127, 128, (co, cin, kh, kw)).astype(np.int8)
+        nodes.append(N("quantize", name + ".q", {"quantize_scale": np.array([7.5, 12.0], np.float32)}, [src]))
+        nodes.append(N(mf.CONST, name + ".w", {"value": wq}))
+        nodes.append(N("conv2d_quantized", name, dict(conv_params(pads),
+                                                      dequantize_scales=rng.uniform(1e-4, 1e-3, co).astype(np.float32)),
+                       [len(nodes) - 2, len(nodes) - 1]))
+        nodes.append(N(mf.CONST, name + ".b", {"value": rng.standard_normal(co).astype(np.float32)}))
+        nodes.append(N("add_bias", name + ".bias", {"format": "NCHW"}, [len(nodes) - 2, len(nodes) - 1]))
+        if act:
+            nodes.append(N(act, name + ".act", {}, [len(nodes) - 1]))
+        return len(nodes) - 1
+
+    g = chain("global", 0, c, h, w, (0, 0, 0, 0))                      # [n, co, 1, 1]
+    nodes.append(N(mf.CONST, "map", {"value": rng.standard_normal((n, co, h, w)).astype(np.float32)}))
+    nodes.append(N("add", "grown", {}, [g, len(nodes) - 1]))           # [n, co, h, w]
+    nodes.append(N("relu", "grown.relu", {}, [len(nodes) - 1]))
+    a = chain("behind_grown", len(nodes) - 1, co, 3, 3, (1, 1, 1, 1))
+    e = chain("scaled", 0, c, 1, 1, (0, 0, 0, 0), "relu")
+    nodes.append(N(mf.CONST, "offsets", {"value": rng.standard_normal((1, co, 1, 1)).astype(np.float32)}))
+    nodes.append(N("add", "offset", {}, [e, len(nodes) - 1]))
+    b = chain("behind_offset", len(nodes) - 1, co, 3, 3, (1, 1, 1, 1))
+    nodes.append(N("concat", "out", {"dim": np.array([1], np.int32)}, [a, b]))
+    module = mf.Module(nodes, [0], [len(nodes) - 1])
+    path = str(tmp_path / "broadcast_residuals.tsm")
+    mf.write_module(path, module)
+    x = (rng.standard_normal((n, c, h, w)) * 6).astype(np.float32)
+    cpu = ts.run_module("cpu", path, [x])
+    fused0 = ts.fused_chain_count()
+    hip = ts.run_module("hip", path, [x])
+    assert ts.fused_chain_count() == fused0 + 4
+    assert cpu.shape == (n, 2 * co, h, w)
+    assert np.array_equal(bits(hip), bits(cpu))
