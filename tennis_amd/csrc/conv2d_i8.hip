@@ -1481,7 +1481,7 @@ int tsx_gemm_i8(int32_t m, int32_t n, int32_t k, const int8_t *a_dev, const void
     }
     // Enough rows to fill MFMA fragments: the window-stationary kernel in its GEMM form (a 1x1 layer over m
     // one-pixel rows, row-major output).  Residual terms stay on the tiled kernel.
-    if (!p.residual && !p.st_out) {
+    if (!p.residual && !p.st_out && p.act != TSX_ACT_MISH) {   // (... and so does the exact Mish)
         const tsx::WsGeom wg{1, n, m, 1, m, 1, kp, kp / KSTEP, 1, 1, 1, 1, 1, 1, 1};
         const tsx::WsPlan wpl = tsx::ws_plan(wg);
         if (wpl.ok && wpl.ksteps_p == gemm_packed_ksteps(k) && wpl.coutp == p.coutp)

@@ -55,7 +55,7 @@ namespace {
 // LDS operand reads and the MFMAs -- and the wavefronts of a workgroup run through it independently.  The
 // wavefronts that finish first store their output while the others still multiply.  Otherwise the window
 // is double buffered, one channel block ahead, with one barrier per block.
-template <int NT, bool EXTRA, bool STREAM, bool RESIDENT>
+template <int NT, bool EXTRA, bool STREAM, bool RESIDENT, bool MISHX>
 __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile, int wave_m, int frag0) {
     const int tid = threadIdx.x, lane = tid % 64;
     const int P0 = tile * p.frags * 32;   // first flat position (n, oh, ow) of the tile
@@ -340,7 +340,7 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
                     constexpr int r = decltype(rc)::value;
                     v[r] = apply_act_conv_i8(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
                 });
-            } else if (p.act == TSX_ACT_MISH) {
+            } else if (MISHX && p.act == TSX_ACT_MISH) {
                 mish_fragment(v);
             } else if (p.act == TSX_ACT_MISH_FAST) {
                 static_for<0, 16>([&](auto rc) {
@@ -411,7 +411,7 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
             static_for<0, 16>([&](auto rc) {
                 constexpr int r = decltype(rc)::value;
                 constexpr int dco = 8 * (r / 4) + (r % 4);
-                if (pok[j] && co0 + dco < p.cout) emit(p, acc[j][r], base + int64_t(dco) * howo, dq[r], bias[r], 0.f);
+                if (pok[j] && co0 + dco < p.cout) emit<MISHX>(p, acc[j][r], base + int64_t(dco) * howo, dq[r], bias[r], 0.f);
             });
         });
     }
@@ -423,7 +423,7 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
 // long ones still multiply: part of the output leaves under the K loop.
 // EXTRA = false compiles the residual input and the staged-layout output out of the epilogue; STREAM selects
 // streaming fp32 stores.
-template <int NTA, int NTB, bool EXTRA, bool STREAM, bool RESIDENT>
+template <int NTA, int NTB, bool EXTRA, bool STREAM, bool RESIDENT, bool MISHX = false>
 __global__ __launch_bounds__(FL_THREADS) void conv_i8_fl_kernel(FlParams p_in) {
     FlParams p = p_in;
     if (!EXTRA) {
@@ -444,9 +444,9 @@ __global__ __launch_bounds__(FL_THREADS) void conv_i8_fl_kernel(FlParams p_in) {
     // the tile's output under the other group's K loop.
     if (wave < 4) {
         __builtin_amdgcn_s_setprio(3);
-        fl_wave<NTA, EXTRA, STREAM, RESIDENT>(p, lds, tile, wave, 0);
+        fl_wave<NTA, EXTRA, STREAM, RESIDENT, MISHX>(p, lds, tile, wave, 0);
     } else {
-        fl_wave<NTB, EXTRA, STREAM, RESIDENT>(p, lds, tile, wave - 4, NTA);
+        fl_wave<NTB, EXTRA, STREAM, RESIDENT, MISHX>(p, lds, tile, wave - 4, NTA);
     }
 }
 
@@ -456,12 +456,12 @@ template <>
 int fl_launch_nt<TSX_FL_NTA, TSX_FL_NTB>(const FlParams &p, dim3 grid, size_t lds_bytes, hipStream_t stream) {
     constexpr int NTA = TSX_FL_NTA, NTB = TSX_FL_NTB;
     // more than 64 KiB of dynamic LDS (up to the CU's 160 KiB) has to be granted per kernel and device
-    static std::atomic<bool> granted[2][3][64];
+    static std::atomic<bool> granted[2][4][64];
     int dev = 0;
     TSX_HIP(hipGetDevice(&dev));
 #define TSX_FL_LAUNCH(EXTRA, STREAM, RESIDENT, SLOT)                                                          \
     do {                                                                                                      \
-        auto kernel = conv_i8_fl_kernel<NTA, NTB, EXTRA, STREAM, RESIDENT>;                                   \
+        auto kernel = conv_i8_fl_kernel<NTA, NTB, EXTRA, STREAM, RESIDENT, SLOT == 3>;                        \
         if (lds_bytes > 65536 && dev < 64 && !granted[RESIDENT][SLOT][dev].load()) {                          \
             TSX_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),                               \
                                         hipFuncAttributeMaxDynamicSharedMemorySize, FL_MAX_LDS));             \
@@ -469,12 +469,15 @@ int fl_launch_nt<TSX_FL_NTA, TSX_FL_NTB>(const FlParams &p, dim3 grid, size_t ld
         }                                                                                                     \
         hipLaunchKernelGGL(kernel, grid, dim3(FL_THREADS), lds_bytes, stream, p);                             \
     } while (0)
+    // (slot 3: the instantiation with the exact Mish, which only its layers run)
     if (p.resident) {
-        if (p.residual || p.st_out) TSX_FL_LAUNCH(true, false, true, 0);
+        if (p.act == TSX_ACT_MISH) TSX_FL_LAUNCH(true, false, true, 3);
+        else if (p.residual || p.st_out) TSX_FL_LAUNCH(true, false, true, 0);
         else if (p.stream_out) TSX_FL_LAUNCH(false, true, true, 1);
         else TSX_FL_LAUNCH(false, false, true, 2);
     } else {
-        if (p.residual || p.st_out) TSX_FL_LAUNCH(true, false, false, 0);
+        if (p.act == TSX_ACT_MISH) TSX_FL_LAUNCH(true, false, false, 3);
+        else if (p.residual || p.st_out) TSX_FL_LAUNCH(true, false, false, 0);
         else if (p.stream_out) TSX_FL_LAUNCH(false, true, false, 1);
         else TSX_FL_LAUNCH(false, false, false, 2);
     }

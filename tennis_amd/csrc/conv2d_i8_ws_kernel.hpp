@@ -70,7 +70,7 @@ namespace {
 // MFMAs.  A wavefront with one fragment spends 2 MFMAs (64 cycles) on a K-step, half of an LDS read's latency: read
 // one half-step ahead (the other form), the small maps at the end of a network -- under one wavefront per SIMD,
 // nothing else to issue -- ran at one K-step per two LDS latencies.
-template <int NT, int FM, bool EXTRA, bool STREAM, bool ROWM, int FILL, bool LOOK>
+template <int NT, int FM, bool EXTRA, bool STREAM, bool ROWM, int FILL, bool LOOK, bool MISHX = false>
 __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <= 4 ? 2 : 1))) void conv_i8_ws_kernel(WsParams p_in) {
     WsParams p = p_in;
     if (!EXTRA) {
@@ -441,7 +441,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
                             constexpr int r = decltype(rc)::value;
                             v[r] = apply_act_conv_i8(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
                         });
-                    } else if (p.act == TSX_ACT_MISH) {
+                    } else if (MISHX && p.act == TSX_ACT_MISH) {
                         mish_fragment(v);
                     } else if (p.act == TSX_ACT_MISH_FAST) {
                         static_for<0, 16>([&](auto rc) {
@@ -533,7 +533,7 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
                     constexpr int r = decltype(rc)::value;
                     constexpr int dco = 8 * (r / 4) + (r % 4);
                     if (pos_ok && co0 + dco < p.cout)
-                        emit(p, acc[f][j][r], base + int64_t(dco) * co_stride, dq[r], bias[r], rs);
+                        emit<MISHX>(p, acc[f][j][r], base + int64_t(dco) * co_stride, dq[r], bias[r], rs);
                 });
             });
         }
@@ -552,23 +552,28 @@ int ws_launch_nt<TSX_WS_NT>(const WsParams &p, dim3 grid, size_t lds_bytes, hipS
     // one fragment per wavefront, a K of two rounds or more, and few enough workgroups that a SIMD holds one or
     // two wavefronts: the B ring (more registers: three workgroups per CU)
     const bool look = NT == 1 && small_fill && p.ksteps >= 2 * RING && int64_t(grid.x) * grid.y <= 1024;
-#define TSX_WS_LAUNCH(EXTRA, STREAM, ROWM)                                                                             \
+#define TSX_WS_LAUNCH(EXTRA, STREAM, ROWM, MISHX)                                                                      \
     do {                                                                                                               \
         constexpr int F = NT <= 2 ? SMALL_FILL : MAX_FILL;                                                             \
         if (NT == 1 && look)                                                                                           \
-            hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, EXTRA, STREAM, ROWM, F, NT == 1>), grid, dim3(WS_THREADS), \
-                               lds_bytes, stream, p);                                                                  \
+            hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, EXTRA, STREAM, ROWM, F, NT == 1, MISHX>), grid,           \
+                               dim3(WS_THREADS), lds_bytes, stream, p);                                                \
         else if (NT <= 2 && small_fill)                                                                                \
-            hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, EXTRA, STREAM, ROWM, F, false>), grid, dim3(WS_THREADS),  \
-                               lds_bytes, stream, p);                                                                  \
+            hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, EXTRA, STREAM, ROWM, F, false, MISHX>), grid,             \
+                               dim3(WS_THREADS), lds_bytes, stream, p);                                                \
         else                                                                                                           \
-            hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, EXTRA, STREAM, ROWM, MAX_FILL, false>), grid,             \
+            hipLaunchKernelGGL((conv_i8_ws_kernel<NT, WS_FM, EXTRA, STREAM, ROWM, MAX_FILL, false, MISHX>), grid,      \
                                dim3(WS_THREADS), lds_bytes, stream, p);                                                \
     } while (0)
-    if (p.rowmajor) TSX_WS_LAUNCH(false, false, true);
-    else if (p.residual || p.st_out) TSX_WS_LAUNCH(true, false, false);
-    else if (p.stream_out) TSX_WS_LAUNCH(false, true, false);
-    else TSX_WS_LAUNCH(false, false, false);
+    // the exact Mish: one instantiation (with every other epilogue term) that only its layers run
+    if (p.act == TSX_ACT_MISH) {
+        if (p.rowmajor) return fail(TSX_E_INVALID, "conv_i8_ws: the exact Mish is not compiled into the row-major form");
+        TSX_WS_LAUNCH(true, false, false, true);
+    }
+    else if (p.rowmajor) TSX_WS_LAUNCH(false, false, true, false);
+    else if (p.residual || p.st_out) TSX_WS_LAUNCH(true, false, false, false);
+    else if (p.stream_out) TSX_WS_LAUNCH(false, true, false, false);
+    else TSX_WS_LAUNCH(false, false, false, false);
 #undef TSX_WS_LAUNCH
     TSX_LAUNCH_CHECK("conv_i8_ws_kernel");
     return 0;

@@ -39,21 +39,26 @@ __device__ __forceinline__ int udiv(int n, int d, unsigned magic) { return magic
 
 // fp32 value of one accumulator after dequant -> row scale -> bias -> residual -> activation;
 // idx is the linear index in the output tensor.
+// MISHX: whether the exact Mish is compiled in.  Its double-precision chain costs a kernel some thirty registers at
+// the point of the epilogue; the convolution kernels carry it in instantiations of their own, which layers with
+// TSX_ACT_MISH are routed to, and every other layer runs code that never saw it.
+template <bool MISHX = true>
 __device__ __forceinline__ float epi_value(const EpiParams &p, int acc, int64_t idx, float dq, float bias, float row_scale) {
     float v = __fmul_rn(float(acc), dq);
     if (p.row_scale) v = __fmul_rn(v, row_scale);
     if (p.bias) v = __fadd_rn(v, bias);
     if (p.residual && !p.res_after) v = __fadd_rn(v, p.residual[idx]);
-    v = apply_act_conv_i8(v, p.act, p.slope, idx < p.act_body);
+    v = MISHX ? apply_act_conv_i8(v, p.act, p.slope, idx < p.act_body) : apply_act_without_exact_mish(v, p.act, p.slope, idx < p.act_body);
     if (p.residual && p.res_after) v = __fadd_rn(v, p.residual[idx]);
     return v;
 }
 
 // Epilogue of one accumulator: every requested output of element idx.
+template <bool MISHX = true>
 __device__ __forceinline__ void emit(const EpiParams &p, int acc, int64_t idx, float dq, float bias, float row_scale) {
     if (p.out_acc) p.out_acc[idx] = acc;
     if (!p.out_f32 && !p.out_i8 && !p.st_out) return;
-    const float v = epi_value(p, acc, idx, dq, bias, row_scale);
+    const float v = epi_value<MISHX>(p, acc, idx, dq, bias, row_scale);
     if (p.out_f32) p.out_f32[idx] = v;
     if (p.out_i8 || p.st_out) {
         const float s = p.n_qscales == 1 ? p.q_scales[0] : p.q_scales[idx / p.q_group_len];
@@ -86,6 +91,7 @@ __device__ __forceinline__ void emit(const EpiParams &p, int acc, int64_t idx, f
 // output, every element in the activation's SIMD-body range, one quantize scale for this lane's
 // image (q_scale, rounding half to even iff q_even).  st_dst = the lane's pixel in the consumer's
 // staged layout at its first channel row, or null.
+template <bool MISHX = true>
 __device__ __forceinline__ void epilogue_rows16(const EpiParams &p, const v16i &acc, const float (&dq)[16],
                                                 const float (&bias)[16], int64_t idx0, int64_t row_stride, float q_scale,
                                                 bool q_even, int8_t *st_dst) {
@@ -110,7 +116,7 @@ __device__ __forceinline__ void epilogue_rows16(const EpiParams &p, const v16i &
     } else if (p.act == TSX_ACT_LEAKY_RELU) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) v[r] = apply_act_conv_i8(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
-    } else if (p.act == TSX_ACT_MISH) {
+    } else if (MISHX && p.act == TSX_ACT_MISH) {
         mish_fragment(v);
     } else if (p.act == TSX_ACT_MISH_FAST) {
 #pragma unroll

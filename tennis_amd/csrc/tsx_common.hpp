@@ -137,23 +137,56 @@ __device__ __forceinline__ float apply_act(float v, int act, float slope, bool i
     if (act == TSX_ACT_MISH_FAST) return mish_short(v);
     return apply_act_basic(v, act, slope, in_body);
 }
-// The exact Mish of the 16 values of an accumulator fragment, one value per turn of a loop that stays a loop: each
+// The 2^(i/32) table of the host's expf held by the wavefront itself: lane l keeps entry l % 32 in two registers, and
+// a lane's look-up is two cross-lane reads (ds_bpermute) instead of a gather from memory -- twice per Mish value, in
+// the middle of its dependent chain.  Every lane must be active where it is used.
+struct Exp2fTableInLanes {
+    int lo, hi;
+    __device__ __forceinline__ explicit Exp2fTableInLanes(int lane) {
+        const uint64_t mine = exp2f_table[lane & 31];
+        lo = int(uint32_t(mine));
+        hi = int(uint32_t(mine >> 32));
+    }
+    __device__ __forceinline__ uint64_t operator()(uint64_t i) const {
+        const int addr = int(i) * 4;
+        return uint64_t(uint32_t(__builtin_amdgcn_ds_bpermute(addr, lo))) |
+               (uint64_t(uint32_t(__builtin_amdgcn_ds_bpermute(addr, hi))) << 32);
+    }
+};
+
+// The exact Mish of the 16 values of an accumulator fragment, two values per turn of a loop that stays a loop: each
 // value's chain holds a dozen double-precision temporaries and twenty constants, and sixteen chains unrolled side by
-// side would push a kernel that keeps its accumulators and operands in registers into scratch memory.  The loop
-// counter is uniform: the values are reached by register indexing.
+// side would push a kernel that keeps its accumulators and operands in registers into scratch memory; two give the
+// scheduler something to put into the other's latencies.  The loop counter is uniform: the values are reached by
+// register indexing.
 __device__ __forceinline__ void mish_fragment(float (&v)[16]) {
     typedef float v16f __attribute__((ext_vector_type(16)));
     v16f t;
 #pragma unroll
     for (int r = 0; r < 16; ++r) t[r] = v[r];
+    if (__builtin_amdgcn_ballot_w64(true) == ~0ull) {
+        const Exp2fTableInLanes table(int(threadIdx.x));
 #pragma clang loop unroll(disable)
-    for (int r = 0; r < 16; ++r) t[r] = mish_value(t[r]);
+        for (int r = 0; r < 16; r += 2) {
+            const float a = mish_value(t[r], table), b = mish_value(t[r + 1], table);
+            t[r] = a;
+            t[r + 1] = b;
+        }
+    } else {
+#pragma clang loop unroll(disable)
+        for (int r = 0; r < 16; ++r) t[r] = mish_value(t[r]);
+    }
 #pragma unroll
     for (int r = 0; r < 16; ++r) v[r] = t[r];
 }
 
 __device__ __forceinline__ float apply_act_conv_i8(float v, int act, float slope, bool in_body) {
     return apply_act(v, act, slope, in_body);
+}
+// ... for kernel instantiations that layers with the exact Mish are never routed to
+__device__ __forceinline__ float apply_act_without_exact_mish(float v, int act, float slope, bool in_body) {
+    if (act == TSX_ACT_MISH_FAST) return mish_short(v);
+    return apply_act_basic(v, act, slope, in_body);
 }
 
 #endif  // __HIPCC__

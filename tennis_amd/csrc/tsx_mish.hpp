@@ -14,9 +14,11 @@
 
 #ifdef __HIPCC__
 #define TSX_MISH_FN __device__ __forceinline__
+#define TSX_MISH_MEMBER __device__ __forceinline__
 #define TSX_MISH_TABLE static __device__ const
 #else
 #define TSX_MISH_FN static inline
+#define TSX_MISH_MEMBER inline
 #define TSX_MISH_TABLE static const
 #endif
 
@@ -39,6 +41,12 @@ TSX_MISH_FN float div_rn(float a, float b) { return __fdiv_rn(a, b); }   // IEEE
 #else
 TSX_MISH_FN float div_rn(float a, float b) { return a / b; }
 #endif
+// where expf_host finds 2^(i/32): this table in memory, or whatever holds a copy of it (on the device, the lanes of
+// the wavefront)
+struct Exp2fTableInMemory {
+    TSX_MISH_MEMBER uint64_t operator()(uint64_t i) const { return exp2f_table[i]; }
+};
+
 TSX_MISH_FN double f64_of_bits(uint64_t u) { double d; __builtin_memcpy(&d, &u, 8); return d; }
 TSX_MISH_FN uint64_t bits_of_f64(double d) { uint64_t u; __builtin_memcpy(&u, &d, 8); return u; }
 
@@ -47,14 +55,15 @@ TSX_MISH_FN uint64_t bits_of_f64(double d) { uint64_t u; __builtin_memcpy(&u, &d
 // early returns -- inf, 0, the largest and smallest finite results beyond |x| of 88 -- come out of the same
 // arithmetic on the clamped argument: the double result overflows or underflows the float conversion as the host's
 // special cases say.  NaN -> NaN.
-TSX_MISH_FN float expf_host(float x) {
+template <class Table = Exp2fTableInMemory>
+TSX_MISH_FN float expf_host(float x, const Table &table = Table()) {
     const double xd = double(__builtin_fminf(__builtin_fmaxf(x, -150.f), 89.f));
     const double z = 0x1.71547652b82fep+5 * xd;          // x * 32 / ln2
     double kd = z + 0x1.8p+52;                           // the integer nearest to z, in the low mantissa bits
     const uint64_t ki = bits_of_f64(kd);
     kd -= 0x1.8p+52;
     const double r = z - kd;
-    const double s = f64_of_bits(exp2f_table[ki & 31] + (ki << 47));
+    const double s = f64_of_bits(table(ki & 31) + (ki << 47));
     const double c = __builtin_fma(0x1.c6af84b912394p-5 / 32768.0, r, 0x1.ebfce50fac4f3p-3 / 1024.0);
     const double r2 = r * r;
     double y = __builtin_fma(0x1.62e42ff0c52d6p-1 / 32.0, r, 1.0);
@@ -91,18 +100,23 @@ TSX_MISH_FN double log_precise(double s) {
 }
 
 // cpu::Softplus (src/kernels/cpu/softplus.cpp:30-39): float(log(double(expf(x)) + 1.0))
-TSX_MISH_FN float softplus_value(float x) {
-    const double s = double(expf_host(x)) + 1.0;
+template <class Table = Exp2fTableInMemory>
+TSX_MISH_FN float softplus_value(float x, const Table &table = Table()) {
+    const double s = double(expf_host(x, table)) + 1.0;
     return s < __builtin_inf() ? float(log_precise(s)) : float(s);   // +inf and NaN pass through
 }
 
 // cpu::Tanh (src/kernels/cpu/tanh.cpp:14-23): T(2) * (T(1) / (T(1) + exp(-(T(2) * x)))) - T(1) in float
-TSX_MISH_FN float tanh_value(float y) {
-    const float u = expf_host(-(2.f * y));
+template <class Table = Exp2fTableInMemory>
+TSX_MISH_FN float tanh_value(float y, const Table &table = Table()) {
+    const float u = expf_host(-(2.f * y), table);
     const float q = div_rn(1.f, 1.f + u);
     return __builtin_fmaf(2.f, q, -1.f);   // 2q is exact: one rounding, fused or not
 }
 
-TSX_MISH_FN float mish_value(float x) { return x * tanh_value(softplus_value(x)); }
+template <class Table = Exp2fTableInMemory>
+TSX_MISH_FN float mish_value(float x, const Table &table = Table()) {
+    return x * tanh_value(softplus_value(x, table), table);
+}
 
 }  // namespace tsx
