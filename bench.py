@@ -34,8 +34,8 @@ CFG = dict(n=32, c=256, h=28, w=28, cout=256, k=3, pad=1)
 
 # HBM bytes per launch of the two kernels on this workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by a
 # known-size copy (profiles/conv2d_i8_config2_hbm_traffic.txt); a profiler figure, not measured by this script.
-TRAFFIC_CONV_BYTES = 43.97e6
-TRAFFIC_STAGE_BYTES = 33.15e6
+TRAFFIC_CONV_BYTES = 43.02e6
+TRAFFIC_STAGE_BYTES = 32.54e6
 
 
 def make_inputs(cfg, seed=1234):
@@ -201,22 +201,23 @@ def ceiling_evidence(A, conv_launch, event_time, conv_ops, dev, stream, frags):
     def stats(v):
         return {"mean": float(v.mean()), "min": float(v.min()), "max": float(v.max())}
 
-    mul, srv = wall[:, :4], wall[:, 4:]              # wavefronts 0-3 multiply, 4-7 serve (rows in, results out)
-    last_m, last_s = 1 + frags, 1 + frags + 2
-    per_fragment = np.diff(mul[:, :, 1:last_m + 1], axis=2)
+    # wavefronts 0-3 multiply: stamps = entry, weights in registers + first rows in LDS, last fragment done;
+    # wavefronts 4-7 serve (rows in, results out): entry, ring filled, last round done, stores issued, stores left
+    mul, srv = wall[:, :4], wall[:, 4:]
+    loop_ns = mul[:, :, 2] - mul[:, :, 1]
     phases = {
         "entry_after_first_wavefront_ns": stats(wall[:, :, 0] - t_first),
         "multiplying": {
             "weights_to_registers_and_first_rows_ns": stats(mul[:, :, 1] - mul[:, :, 0]),
-            "fragment_ns": stats(per_fragment), "first_fragment_ns": stats(per_fragment[:, :, 0]),
-            "all_fragments_ns": stats(mul[:, :, last_m] - mul[:, :, 1]),
-            "shader_clock_GHz_in_the_loop": float(((clk[:, :4, last_m] - clk[:, :4, 1]) / (mul[:, :, last_m] - mul[:, :, 1])).mean())},
+            "all_fragments_ns": stats(loop_ns),
+            "ns_per_fragment_full_tiles": float(np.median(loop_ns)) / frags,
+            "shader_clock_GHz_in_the_loop": float(((clk[:, :4, 2] - clk[:, :4, 1]) / loop_ns).mean())},
         "serving": {
             "ring_prologue_ns": stats(srv[:, :, 1] - srv[:, :, 0]),
-            "round_ns": stats(np.diff(srv[:, :, 1:1 + frags + 1], axis=2)),
-            "last_sums_to_stores_issued_ns": stats(srv[:, :, last_s - 1] - srv[:, :, last_s - 2]),
-            "stores_issued_to_stores_left_ns": stats(srv[:, :, last_s] - srv[:, :, last_s - 1])},
-        "end_after_first_wavefront_ns": stats(srv[:, :, last_s] - t_first),
+            "all_rounds_ns": stats(srv[:, :, 2] - srv[:, :, 1]),
+            "last_sums_to_stores_issued_ns": stats(srv[:, :, 3] - srv[:, :, 2]),
+            "stores_issued_to_stores_left_ns": stats(srv[:, :, 4] - srv[:, :, 3])},
+        "end_after_first_wavefront_ns": stats(srv[:, :, 4] - t_first),
     }
     return {"workload": "BASELINE config 2 MFMA kernel (conv_i8_rs_kernel, %d fragments per tile): ceiling evidence" % frags,
             "mfma_probe": probe,
@@ -225,9 +226,9 @@ def ceiling_evidence(A, conv_launch, event_time, conv_ops, dev, stream, frags):
             "workgroups_with_stamps": int(st.shape[0]),
             "phases": phases,
             "fragment_mfma_cycles_per_simd": 36 * 32,
-            "note": "wall clock = s_memrealtime (10 ns ticks), shader clock = s_memtime; a stamp costs the wavefront "
-                    "150-300 cycles, so the stamped kernel runs longer than the plain one; fragment_mfma_cycles_per_simd "
-                    "is what one fragment's MFMAs alone occupy a SIMD's pipe for (36 v_mfma_i32_32x32x32_i8 x 32 cycles)"}
+            "note": "wall clock = s_memrealtime (10 ns ticks), shader clock = s_memtime; the last position tile holds "
+                    "fewer fragments than the others (it sets the minima); fragment_mfma_cycles_per_simd is what one "
+                    "fragment's MFMAs alone occupy a SIMD's pipe for (36 v_mfma_i32_32x32x32_i8 x 32 cycles)"}
 
 
 def tennis_runtime_leg(reps=5):

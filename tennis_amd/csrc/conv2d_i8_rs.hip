@@ -129,8 +129,16 @@ __global__ __launch_bounds__(RS_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
         ++stamp_k;
     };
 #define RS_STAMP() stamp()
+// per fragment / round as well with -DTSX_MEASUREMENT_AIDS=2: the stamps inside the loops cost the kernel a quarter of
+// its speed, so the measurement build leaves them out and divides the loop's time by its fragments
+#if TSX_MEASUREMENT_AIDS >= 2
+#define RS_STAMP_FINE() stamp()
+#else
+#define RS_STAMP_FINE() ((void)0)
+#endif
 #else
 #define RS_STAMP() ((void)0)
+#define RS_STAMP_FINE() ((void)0)
 #endif
     RS_STAMP();
 
@@ -245,7 +253,7 @@ __global__ __launch_bounds__(RS_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
                 cur[kr] = nxt[kr];
                 nxt[kr] = nn4[kr];
             });
-            RS_STAMP();
+            RS_STAMP_FINE();
         };
         int f = f0;
         fragment(std::integral_constant<int, 0>{}, std::false_type{}, f);
@@ -262,6 +270,7 @@ __global__ __launch_bounds__(RS_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
         } else {
             static_for<0, 8>([&](auto ic) { xchg_write(std::integral_constant<int, 0>{}, ic); });
         }
+        RS_STAMP();
         lds_fence_barrier();
         return;
     }
@@ -471,13 +480,14 @@ __global__ __launch_bounds__(RS_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
         off_d = off_e;
         off_e = off_f;
         lds_fence_barrier();
-        RS_STAMP();
+        RS_STAMP_FINE();
     };
     fill_issue(std::integral_constant<int, 1>{}, f0 - 1);   // the set that round f0+1 stores
     for (int r = f0; r < f1; r += 2) {
         round(std::integral_constant<int, 0>{}, r);
         if (r + 1 < f1) round(std::integral_constant<int, 1>{}, r + 1);
     }
+    RS_STAMP();
     // off_a = fragment f1-2, off_b = fragment f1-1
     if (f1 - 2 >= f0) finish_fragment((f1 - f0) & 1, off_a);
     lds_fence_barrier();   // the last fragment's partial sums

@@ -22,10 +22,12 @@ extern "C" {
 int tsx_probe_mfma_i8(const void *operands_dev, int32_t iters, int32_t blocks, int32_t *sink_dev, void *stream);
 
 /* While a buffer is set (NULL switches it off; process-wide), every wavefront of the weight-stationary int8
- * convolution kernel writes (wall clock at 100 MHz, shader clock) pairs at its phase boundaries, up to 24 pairs at
- * buffer[((workgroup * 8 + wavefront) * 24 + k) * 2 ...]: kernel entry, first barrier, every fragment (multiplying
- * wavefronts 0-3) or round (serving wavefronts 4-7), and for the serving ones stores issued, stores left.
- * Wavefronts whose slot lies beyond `bytes` write nothing. */
+ * convolution kernel writes (wall clock at 100 MHz, shader clock) pairs at its phase boundaries, at
+ * buffer[((workgroup * 8 + wavefront) * 24 + k) * 2 ...]:
+ *   multiplying wavefronts 0-3: k = 0 kernel entry, 1 weights in registers and first rows in LDS, 2 last fragment done;
+ *   serving wavefronts 4-7:     k = 0 kernel entry, 1 ring filled, 2 last round done, 3 stores issued, 4 stores left.
+ * (Compiled with -DTSX_MEASUREMENT_AIDS=2 the kernel also stamps every fragment / round, between k = 1 and the
+ * phase behind it; those stamps slow the loop by a quarter.)  Wavefronts whose slot lies beyond `bytes` write nothing. */
 int tsx_debug_phase_stamps(void *buffer_dev, size_t bytes);
 
 #ifdef __cplusplus
