@@ -124,7 +124,8 @@ def _fp32_conv_rows(shape_x, shape_w, reps, seed):
     flops = 2.0 * n * cout * h * w * c * 9
     w63, w23 = capi.WinogradF63(wt, (1, 1, 1, 1)), capi.WinogradF23(wt, (1, 1, 1, 1))
     rows = {}
-    for name, fn in (("im2col_gemm", lambda: capi.conv2d_f32(x, wt, (1, 1, 1, 1), bias=b, act="relu")),
+    direct, _ = capi.conv2d_f32_prepared(x, wt, (1, 1, 1, 1), bias=b, act="relu")
+    for name, fn in (("im2col_gemm", direct),
                      ("winograd_f63", lambda: w63(x, bias=b, act="relu")), ("winograd_f23", lambda: w23(x, bias=b, act="relu")),
                      ("winograd_f63_fast", lambda: w63(x, bias=b, act="relu", fast=True))):
         for _ in range(3):

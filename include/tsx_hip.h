@@ -209,6 +209,12 @@ int tsx_gemm_i8(int32_t m, int32_t n, int32_t k, const int8_t *a_dev, const void
  * floating-point path: 1e-4 relative / 1e-5 absolute against the reference CPU kernels. */
 int tsx_conv2d_f32_nchw(const tsx_conv2d_geom *g, const float *x_dev, const float *w_oihw_dev, float padding_value,
                         const float *bias_dev, int32_t act, float slope, float *out_dev, void *stream);
+/* Which kernel tsx_conv2d_f32_nchw launches for this layer and these weights (their alignment counts), as text:
+ * "kernel=small_3x3 | register_fed | staged_64x64 | staged_32x32_ksplit tiles=<output tiles>".  No counterpart in
+ * the reference; for tests that must know a given kernel ran, and for logs.  The environment variables
+ * TSX_CONV_F32_SMALL and TSX_GEMM_F32_REGFED ("0" = never, "force" = wherever the operands allow) are read at every
+ * call. */
+int tsx_conv2d_f32_plan_info(const tsx_conv2d_geom *g, const float *w_oihw_dev, char *text, size_t text_bytes);
 
 /* cpu::InnerProd::inner_prod (src/kernels/cpu/inner_prod.cpp:54-69, interface
  * include/backend/base/base_inner_prod.h:32-48): out[m][n] = lhs[m][k] * rhs, rhs being [k][n], or

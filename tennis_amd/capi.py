@@ -74,6 +74,7 @@ SIGNATURES = {
     "tsx_gemm_i8_workspace_bytes": (_sz, [_i32, _i32]),
     "tsx_gemm_i8": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, ctypes.POINTER(Epilogue), _vp, _vp, _vp, _vp, _sz, _vp]),
     "tsx_conv2d_f32_nchw": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, _vp, _f32, _vp, _i32, _f32, _vp, _vp]),
+    "tsx_conv2d_f32_plan_info": (ctypes.c_int, [ctypes.POINTER(ConvGeom), _vp, ctypes.c_char_p, _sz]),
     "tsx_inner_prod_f32": (ctypes.c_int, [_i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp]),
     "tsx_add_bias_f32": (ctypes.c_int, [_vp, _i64, _i32, _i64, _vp, _vp, _vp]),
     "tsx_relu_f32": (ctypes.c_int, [_vp, _i64, _vp, _vp]),
@@ -505,6 +506,37 @@ def conv2d_f32(x, w, pads=(0, 0, 0, 0), strides=(1, 1), dilations=(1, 1), paddin
     check(lib().tsx_conv2d_f32_nchw(ctypes.byref(geom), _ptr(x), _ptr(w), float(padding_value), _ptr(bias), _ACT[act],
                                     float(slope), _ptr(out), _stream()))
     return out
+
+
+def conv2d_f32_plan_info(x_shape, w, pads=(0, 0, 0, 0), strides=(1, 1), dilations=(1, 1)):
+    """tsx_conv2d_f32_plan_info as a dict ({"kernel": ..., "tiles": ...}) for an input of x_shape and weights w."""
+    w = _dev(w, torch.float32)
+    geom = make_geom(tuple(x_shape), tuple(w.shape), pads, strides, dilations)
+    text = ctypes.create_string_buffer(256)
+    check(lib().tsx_conv2d_f32_plan_info(ctypes.byref(geom), _ptr(w), text, 256))
+    return dict(item.split("=", 1) for item in text.value.decode().split())
+
+
+def conv2d_f32_prepared(x, w, pads=(0, 0, 0, 0), strides=(1, 1), dilations=(1, 1), padding_value=0.0, bias=None,
+                        act=None, slope=0.0):
+    """(launch, out): tsx_conv2d_f32_nchw on fixed tensors with every argument marshalled once, for callers that issue
+    the same layer again and again (a layer of a few microseconds is otherwise bound by this module's per-call work:
+    geometry, output allocation, argument conversion).  `launch()` enqueues one convolution on the stream that was
+    current here and raises TsxError like conv2d_f32; `out` is the tensor it writes."""
+    x = _dev(x, torch.float32)
+    w = _dev(w, torch.float32)
+    bias = _dev(bias, torch.float32)
+    geom = make_geom(tuple(x.shape), tuple(w.shape), pads, strides, dilations)
+    ho, wo = conv_out_size(geom)
+    out = torch.empty((x.shape[0], w.shape[0], ho, wo), dtype=torch.float32, device=x.device)
+    fn = lib().tsx_conv2d_f32_nchw
+    args = (ctypes.byref(geom), _ptr(x), _ptr(w), float(padding_value), _ptr(bias), _ACT[act], float(slope), _ptr(out),
+            _stream())
+    keep = (x, w, bias, geom)
+
+    def launch(_keep=keep):
+        check(fn(*args))
+    return launch, out
 
 
 def inner_prod_f32(lhs, rhs, transpose=False):

@@ -19,6 +19,10 @@
 // accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32.
 #include "gemm_f32.hpp"
 
+#include <algorithm>
+#include <atomic>
+#include <cstdlib>
+
 namespace tsx {
 namespace {
 
@@ -27,7 +31,7 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 constexpr int KC = 32;          // K per staged chunk
 constexpr int THREADS = 256;
 
-constexpr int MAX_SLOTS = 8;    // B elements a thread fetches per chunk (KC * BN / THREADS at BN = 64)
+constexpr int MAX_SLOTS = 16;   // B elements a thread fetches per chunk (KC * BN / THREADS at BN = 64; 16 in the register-fed kernel)
 
 // B operand = implicit im2col of an NCHW tensor (src/kernels/cpu/im2col.cpp:37-111).
 struct ConvLoader {
@@ -76,6 +80,18 @@ struct ConvLoader {
         if (hh < 0 || hh >= h || ww < 0 || ww >= w) return padding_value;
         return img[(int64_t(slot_ci[i]) * h + hh) * w + ww];
     }
+    // The same in two steps, for loads that are issued unconditionally and resolved later: the address to read
+    // (any valid one when the element is padding or beyond the matrix), whether the loaded value is the element,
+    // and whether the element exists at all (else it is 0; an existing element outside the map is padding_value).
+    __device__ __forceinline__ const float *slot_address(int i, int kdim, bool &inside, bool &valid) const {
+        valid = col_ok && slot_k[i] < kdim;
+        const int inv_kw = (65536 + kw - 1) / kw;
+        const int r = (slot_tap[i] * inv_kw) >> 16, s = slot_tap[i] - r * kw;
+        const int hh = h0 + r * dil_h, ww = w0 + s * dil_w;
+        inside = valid && hh >= 0 && hh < h && ww >= 0 && ww < w;
+        return inside ? img + (int64_t(slot_ci[i]) * h + hh) * w + ww : x;
+    }
+    __device__ __forceinline__ float fill_value() const { return padding_value; }
 };
 
 // B operand = plain matrix: element (k, n) at b[k*ld_k + n*ld_n] (+ batch stride).
@@ -95,6 +111,11 @@ struct MatLoader {
         if (!col_ok || slot_k[i] >= kdim) return 0.f;
         return colp[int64_t(slot_k[i]) * ld_k];
     }
+    __device__ __forceinline__ const float *slot_address(int i, int kdim, bool &inside, bool &valid) const {
+        valid = inside = col_ok && slot_k[i] < kdim;
+        return inside ? colp + int64_t(slot_k[i]) * ld_k : b;
+    }
+    __device__ __forceinline__ float fill_value() const { return 0.f; }
 };
 
 struct GemmArgs {
@@ -109,6 +130,36 @@ struct GemmArgs {
     float slope;
     int64_t act_body;     // elements of the output inside the activation's SIMD body
 };
+
+// A 32 x 32 accumulator tile's bias values and its stores.  Lane l holds rows row0 + 8 (r / 4) + 4 (l / 32) + r % 4
+// (r = 0 .. 15) of column l % 32.  The sixteen bias values are requested in one go, well before they are added (a
+// load inside the store loop would cost a memory round trip per row); rows beyond m read the last row's.
+__device__ __forceinline__ void tile_bias_load(const GemmArgs &g, int row0, int lane, float (&bias)[16]) {
+    if (g.bias) {
+        static_for<0, 16>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            bias[r] = g.bias[min(row0 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4), g.m - 1)];
+        });
+    } else {
+        static_for<0, 16>([&](auto rc) { bias[decltype(rc)::value] = 0.f; });
+    }
+}
+
+__device__ __forceinline__ void tile_store(const GemmArgs &g, float *c, const v16f &acc, const float (&bias)[16], int row0,
+                                           int lane, int64_t col_base, int64_t row_stride) {
+    const bool with_bias = g.bias != nullptr;
+    static_for<0, 16>([&](auto rc) {
+        constexpr int r = decltype(rc)::value;
+        const int row = row0 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
+        if (row < g.m) {
+            const int64_t idx = col_base + int64_t(row) * row_stride;
+            float v = acc[r];
+            if (with_bias) v = __fadd_rn(v, bias[r]);
+            c[idx] = apply_act_basic(v, g.act, g.slope, idx < g.act_body);   // the entry points take none / relu / leaky_relu
+        }
+    });
+}
+
 
 template <class Loader, int WM, int WN, int WK>
 __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmArgs g, Loader ld) {
@@ -179,6 +230,9 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmArgs g, Loader ld
         });
     }
 
+    float bias[16];
+    if (wk == 0) tile_bias_load(g, m0 + wm * 32, lane, bias);
+
     // reduce the K split: wavefronts wk > 0 hand their partial tile to wk == 0
     if constexpr (WK > 1) {
         __syncthreads();
@@ -213,17 +267,297 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmArgs g, Loader ld
         col_base = col;
         row_stride = g.n;
     }
-    float *c = g.c + batch * g.c_batch;
-    static_for<0, 16>([&](auto rc) {
-        constexpr int r = decltype(rc)::value;
-        const int row = m0 + wm * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
-        if (row < g.m) {
-            const int64_t idx = col_base + int64_t(row) * row_stride;
-            float v = acc[r];
-            if (g.bias) v = __fadd_rn(v, g.bias[row]);
-            c[idx] = apply_act_basic(v, g.act, g.slope, idx < g.act_body);   // the entry points take none / relu / leaky_relu
-        }
+    tile_store(g, g.c + batch * g.c_batch, acc, bias, m0 + wm * 32, lane, col_base, row_stride);
+}
+
+// Small problems (a single 64-channel 56x56 layer: 196 tiles of 32 x 32): the staged kernel above walks K chunk by
+// chunk with one global round trip per chunk and nothing else on the CU to hide it.  Here the operands go from
+// global memory straight into the MFMA operand registers -- no LDS staging, no barrier in the loop -- and the eight
+// wavefronts of a workgroup take the 32-deep K chunks of one 32 x 32 tile in turn (chunk c goes to wavefront c % 8),
+// each with the next chunk's 20 loads in flight while it multiplies the current one; their partial tiles are summed
+// through LDS in a fixed order (results do not depend on timing).  Which k an MFMA step carries is free as long as
+// both operands agree: lane l (half hf = l / 32) takes k = hf * 16 + j of the chunk at step j, so its A operands are
+// four 16-byte loads of its row and its B operands 16 gathers that are contiguous across the 32 lanes of a half.
+// Needs 16-byte aligned rows of A (K a multiple of 4).
+constexpr int KS_WAVES = 8;
+
+template <class Loader>
+__global__ __launch_bounds__(64 * KS_WAVES) void gemm_f32_regfed_kernel(GemmArgs g, Loader ld) {
+    typedef float v4f_ __attribute__((ext_vector_type(4)));
+    __shared__ float red[KS_WAVES - 1][16][64];
+    const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int hf = lane / 32;
+    const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+    const int batch = blockIdx.z;
+    const float *a = g.a + batch * g.a_batch;
+    if constexpr (std::is_same<Loader, MatLoader>::value) ld.b += batch * g.b_batch;
+    ld.set_column(n0 + lane % 32, g.n);
+    const int arow = min(m0 + lane % 32, g.m - 1);          // rows beyond m are loaded from the last row and never stored
+    const float *arowp = a + int64_t(arow) * g.k + hf * 16;
+    static_for<0, 16>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        ld.init_slot(i, wave * KC + hf * 16 + i);
     });
+    const int chunks = (g.k + KC - 1) / KC;
+
+    v16f acc;
+    static_for<0, 16>([&](auto rc) { acc[decltype(rc)::value] = 0.f; });
+    constexpr int NBUF = 2;      // chunks in flight per wavefront
+    v4f_ a_reg[NBUF][4];
+    float b_reg[NBUF][16];
+    unsigned b_mask[NBUF];       // bit i: slot i's loaded value is the element; bit 16 + i: the element exists
+    const float fill = ld.fill_value();
+    auto load_chunk = [&](auto bufc, int c) __attribute__((always_inline)) {
+        constexpr int buf = decltype(bufc)::value;
+        const int k0 = c * KC + hf * 16;
+        static_for<0, 4>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            // K is a multiple of 4: a group of four k is inside K or wholly beyond it (then the row's first group)
+            a_reg[buf][i] = *reinterpret_cast<const v4f_ *>(k0 + 4 * i < g.k ? arowp + int64_t(c) * KC + 4 * i : arowp - hf * 16);
+        });
+        // every load issued without a branch around it; what a padding or out-of-range element reads is replaced
+        // when the chunk is multiplied
+        unsigned mask = 0;
+        static_for<0, 16>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            bool inside, valid;
+            const float *ptr = ld.slot_address(i, g.k, inside, valid);
+            b_reg[buf][i] = *ptr;
+            mask |= (inside ? 1u << i : 0u) | (valid ? 1u << (16 + i) : 0u);
+            ld.advance_slot(i, KC * KS_WAVES);
+        });
+        b_mask[buf] = mask;
+    };
+    auto multiply = [&](auto bufc, int c) __attribute__((always_inline)) {
+        constexpr int buf = decltype(bufc)::value;
+        const int k0 = c * KC + hf * 16;
+        const unsigned mask = b_mask[buf];
+        static_for<0, 16>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const float bv = (mask >> j) & 1u ? b_reg[buf][j] : ((mask >> (16 + j)) & 1u ? fill : 0.f);
+            const float av = k0 + j < g.k ? a_reg[buf][j / 4][j % 4] : 0.f;
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc, 0, 0, 0);
+        });
+    };
+    // chunk c of this wavefront's sequence lives in buffer (its ordinal % NBUF); NBUF - 1 chunks ahead are in flight
+    int c = wave;
+    static_for<0, NBUF - 1>([&](auto bc) {
+        if (c + decltype(bc)::value * KS_WAVES < chunks) load_chunk(bc, c + decltype(bc)::value * KS_WAVES);
+    });
+    while (c < chunks) {
+        bool done = false;
+        static_for<0, NBUF>([&](auto bc) {
+            constexpr int b_ = decltype(bc)::value;
+            if (!done) {
+                if (c + (NBUF - 1) * KS_WAVES < chunks)
+                    load_chunk(std::integral_constant<int, (b_ + NBUF - 1) % NBUF>{}, c + (NBUF - 1) * KS_WAVES);
+                multiply(bc, c);
+                c += KS_WAVES;
+                done = c >= chunks;
+            }
+        });
+    }
+
+    float bias[16];
+    if (wave > 0) {
+        static_for<0, 16>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            red[wave - 1][r][lane] = acc[r];
+        });
+    } else {
+        tile_bias_load(g, m0, lane, bias);
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    static_for<0, KS_WAVES - 1>([&](auto wc) {
+        constexpr int w = decltype(wc)::value;
+        static_for<0, 16>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            acc[r] += red[w][r][lane];
+        });
+    });
+
+    const int col = n0 + lane % 32;
+    if (col >= g.n) return;
+    int64_t col_base, row_stride;
+    if (g.howo > 0) {
+        const int n = col / g.howo;
+        col_base = int64_t(n) * g.m * g.howo + (col - n * g.howo);
+        row_stride = g.howo;
+    } else {
+        col_base = col;
+        row_stride = g.n;
+    }
+    tile_store(g, g.c + batch * g.c_batch, acc, bias, m0, lane, col_base, row_stride);
+}
+
+// A single small 3x3 layer (BASELINE config 1: 1 x 64 x 56 x 56, 64 output channels: 196 tiles of 32 x 32, under one
+// per CU) is bound by what the kernels above do per element of B: the im2col gather computes an address, two
+// bounds and a padding select per element per K chunk, and walks K in dependent round trips.  This kernel orders K
+// as the layer is laid out -- (input channel, tap) -- and gives every lane ONE input channel per MFMA step: lane l of
+// a wavefront supplies output position l % 32 and, at step (t, tap), channel 2 (wave + 8 t) + l / 32.  A lane's nine
+// taps of a channel are nine fixed byte offsets, and which of them fall into the padding depends on the lane's
+// position only: both are computed once, and every load of B is "uniform channel base + the lane's tap offset".
+// The eight wavefronts of a workgroup take the channel pairs of one 32 x 32 tile in turn and issue ALL their B loads
+// (T pairs x 9 taps, one register each) and all their 16-byte pieces of the tile's 32 rows of A before waiting for
+// any; A goes through LDS transposed ([k][row]: a lane reading its own row from global memory would touch 64 cache
+// lines per instruction).  One round trip to memory in all, then T x 9 MFMAs per wavefront with A read from LDS, and
+// the partial tiles summed through LDS in a fixed order.  T = channel pairs per wavefront: 4 (up to 64 input
+// channels) or 2 (up to 32).  Tensors under 4 GiB (32-bit byte offsets), channels a multiple of 4 (rows of A are
+// read in 16-byte pieces).
+constexpr int SMALL_PITCH = 33;      // floats between consecutive k of the A tile in LDS (32 rows + 1)
+
+template <int T>
+__global__ __launch_bounds__(64 * KS_WAVES) void conv3x3_f32_small_kernel(GemmArgs g, ConvLoader ld) {
+    typedef float v4f_ __attribute__((ext_vector_type(4)));
+    constexpr int TAPS = 9;
+    extern __shared__ __attribute__((aligned(16))) float lds_f[];   // A: K x SMALL_PITCH; then the partial tiles
+    const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int hf = lane / 32;
+    const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+    const int K = g.k;
+    // the loader's fields as scalars of their own (the struct also carries the other kernels' per-thread state)
+    const float *const x = ld.x;
+    const int C = ld.c, H = ld.h, W = ld.w, dil_h = ld.dil_h, dil_w = ld.dil_w, howo = ld.howo, wo_ = ld.wo;
+    const int stride_h = ld.stride_h, stride_w = ld.stride_w, pad_top = ld.pad_top, pad_left = ld.pad_left;
+    const float padding_value = ld.padding_value;
+    const float *const a_base = g.a;
+    const int M = g.m, N = g.n;
+
+    // ---- B: this lane's position, its base offset and which taps lie inside the map
+    const int col = n0 + lane % 32;
+    const bool col_ok = col < N;
+    const int cc = col_ok ? col : 0;
+    const int img_n = cc / howo, rpos = cc - img_n * howo;
+    const int oh = rpos / wo_, ow = rpos - oh * wo_;
+    const int h0 = oh * stride_h - pad_top, w0 = ow * stride_w - pad_left;
+    // Byte offsets of the lane's nine taps from the first channel of its pair (32 bits: the launcher admits tensors
+    // under 4 GiB only); a tap in the padding points at the channel's first pixel and its value is replaced below.
+    // With them every load below is "uniform base + the lane's offset", no address arithmetic per load.
+    const unsigned plane4 = unsigned(H * W) * 4u;
+    const unsigned lane_base = (unsigned(img_n) * unsigned(C) + unsigned(hf)) * plane4;
+    const int pos_off = h0 * W + w0;          // may be negative: only used where the tap is inside
+    unsigned inside = 0;                      // bit tap: the tap's pixel exists
+    unsigned b_off[TAPS];
+    static_for<0, TAPS>([&](auto jc) {
+        constexpr int j = decltype(jc)::value, r = j / 3, q = j % 3;
+        const int hh = h0 + r * dil_h, ww = w0 + q * dil_w;
+        const bool in = col_ok & (unsigned(hh) < unsigned(H)) & (unsigned(ww) < unsigned(W));
+        inside |= unsigned(in) << j;
+        b_off[j] = lane_base + (in ? unsigned(pos_off + r * dil_h * W + q * dil_w) * 4u : 0u);
+    });
+    float b_reg[T][TAPS];
+    static_for<0, T>([&](auto tc) {
+        constexpr int t = decltype(tc)::value;
+        const int pair = wave + KS_WAVES * t;                 // channels 2 pair, 2 pair + 1 (c is even)
+        const char *chan = reinterpret_cast<const char *>(x) + (2 * pair < C ? size_t(2 * pair) * plane4 : size_t(0));
+        static_for<0, TAPS>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            b_reg[t][j] = *reinterpret_cast<const float *>(chan + b_off[j]);     // resolved below
+        });
+    });
+
+    // ---- A: rows m0 .. m0 + 31, all of K, into LDS as [k][SMALL_PITCH] (rows beyond m: the last row, never stored).
+    // A wavefront's load covers 8 rows x 128 bytes (8 whole cache lines); its four stores then go to banks
+    // 4 (lane % 8) + lane / 8 (+ j): no two lanes of a half wavefront share one, and the MFMA loop's reads (32
+    // consecutive rows of one k) share none either.
+    // All of a wavefront's pieces are requested before the first is stored: one round trip, not one per piece.
+    {
+        constexpr int PIECES = (4 * ((T * 36 + 7) / 8) + KS_WAVES - 1) / KS_WAVES;   // per wavefront, at most (K <= 144 T)
+        const int k4s = K / 4, groups = (k4s + 7) / 8;  // 16-byte pieces per row; groups of 8 pieces
+        const int kk = lane % 8, rr = lane / 8;
+        v4f_ piece[PIECES];
+        static_for<0, PIECES>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            const int item = wave + KS_WAVES * i;
+            const int row = 8 * (item % 4) + rr, k4 = min(8 * (item / 4) + kk, k4s - 1);
+            const unsigned a_off = (unsigned(min(m0 + row, M - 1)) * unsigned(K) + 4u * unsigned(k4)) * 4u;
+            piece[i] = *reinterpret_cast<const v4f_ *>(reinterpret_cast<const char *>(a_base) + a_off);
+        });
+        static_for<0, PIECES>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            const int item = wave + KS_WAVES * i;
+            const int row = 8 * (item % 4) + rr, k4 = 8 * (item / 4) + kk;
+            if (item < 4 * groups && k4 < k4s) {
+                float *dst = lds_f + 4 * k4 * SMALL_PITCH + row;
+                dst[0] = piece[i][0];
+                dst[SMALL_PITCH] = piece[i][1];
+                dst[2 * SMALL_PITCH] = piece[i][2];
+                dst[3 * SMALL_PITCH] = piece[i][3];
+            }
+        });
+    }
+    __syncthreads();
+
+    v16f acc;
+    static_for<0, 16>([&](auto rc) { acc[decltype(rc)::value] = 0.f; });
+    const float *arow = lds_f + lane % 32;
+    static_for<0, T>([&](auto tc) {
+        constexpr int t = decltype(tc)::value;
+        const int ci = 2 * (wave + KS_WAVES * t) + hf;
+        const bool c_ok = 2 * (wave + KS_WAVES * t) < C;
+        const float *ak = arow + (c_ok ? ci : 0) * (TAPS * SMALL_PITCH);
+        static_for<0, TAPS>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const float av = c_ok ? ak[j * SMALL_PITCH] : 0.f;
+            // a tap in the padding reads padding_value; a column beyond n or a channel beyond c contributes nothing
+            const float bv = !(c_ok && col_ok) ? 0.f : ((inside >> j) & 1u) ? b_reg[t][j] : padding_value;
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc, 0, 0, 0);
+        });
+    });
+
+    float bias[16];
+    if (wave == 0) tile_bias_load(g, m0, lane, bias);
+    __syncthreads();                                    // every wavefront is done with A: its space takes the partial tiles
+    float (*red)[16][64] = reinterpret_cast<float (*)[16][64]>(lds_f);
+    if (wave > 0) {
+        static_for<0, 16>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            red[wave - 1][r][lane] = acc[r];
+        });
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    static_for<0, KS_WAVES - 1>([&](auto wc) {
+        constexpr int w = decltype(wc)::value;
+        static_for<0, 16>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            acc[r] += red[w][r][lane];
+        });
+    });
+    if (!col_ok) return;
+    tile_store(g, g.c, acc, bias, m0, lane, int64_t(img_n) * M * howo + rpos, howo);
+}
+
+// Whether the small-layer kernel takes a convolution, and its launch.  Dynamic LDS beyond 64 KiB has to be granted per
+// kernel and device.
+template <int T>
+int launch_conv3x3_small(const GemmArgs &g, const ConvLoader &ld, hipStream_t stream) {
+    const size_t lds_bytes = std::max(size_t(g.k) * SMALL_PITCH * 4, size_t(KS_WAVES - 1) * 16 * 64 * 4);
+    static std::atomic<bool> granted[64];
+    int dev = 0;
+    TSX_HIP(hipGetDevice(&dev));
+    auto kernel = conv3x3_f32_small_kernel<T>;
+    if (lds_bytes > 65536 && dev < 64 && !granted[dev].load()) {
+        TSX_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        granted[dev].store(true);
+    }
+    const dim3 grid(unsigned(ceil_div(g.n, 32)), unsigned(ceil_div(g.m, 32)));
+    hipLaunchKernelGGL(kernel, grid, dim3(64 * KS_WAVES), lds_bytes, stream, g, ld);
+    TSX_LAUNCH_CHECK("conv3x3_f32_small_kernel");
+    return 0;
+}
+
+inline bool conv3x3_small_takes(const GemmArgs &g, const ConvLoader &ld) {
+    const char *e = std::getenv("TSX_CONV_F32_SMALL");      // "0": never; "force": wherever the layer allows (tests)
+    if (e && e[0] == '0') return false;
+    if (ld.kh != 3 || ld.kw != 3 || ld.c > 64 || ld.c % 2 != 0 || g.k % 4 != 0 || reinterpret_cast<uintptr_t>(g.a) % 16 != 0)
+        return false;
+    // 32-bit byte offsets into the input and the weights
+    const int64_t images = ceil_div(int64_t(g.n), int64_t(ld.howo));
+    if (images * ld.c * ld.h * ld.w * 4 >= (int64_t(1) << 32) || int64_t(g.m) * g.k * 4 >= (int64_t(1) << 32)) return false;
+    const int64_t tiles32 = ceil_div(g.m, 32) * ceil_div(g.n, 32);
+    return (e && e[0] == 'f') || tiles32 <= 512;
 }
 
 // inner_prod with few rows (a classifier behind a batch of 32: M = 32, K = 2048, N = 1000).  The tiled kernel
@@ -318,12 +652,30 @@ __global__ __launch_bounds__(64 * SK_WAVES) void inner_prod_skinny_kernel(Skinny
     });
 }
 
-template <class Loader>
-int launch(const GemmArgs &g, const Loader &ld, int batches, hipStream_t stream) {
+enum GemmKernel { GEMM_REGISTER_FED, GEMM_STAGED_64, GEMM_STAGED_32_KSPLIT };
+
+inline GemmKernel choose_gemm(const GemmArgs &g, int batches) {
     // Big problems: 64x64 tiles, no K split.  Small ones (fewer tiles than SIMDs): 32x32 tiles
     // with the four wavefronts splitting K, so a single small layer still spreads over the chip.
     const int64_t tiles64 = ceil_div(g.m, 64) * ceil_div(g.n, 64) * batches;
-    if (tiles64 >= 512 || g.k < 4 * KC) {
+    // TSX_GEMM_F32_REGFED: "0" never, "force" wherever the operands allow (tests); otherwise small problems
+    const char *e = std::getenv("TSX_GEMM_F32_REGFED");
+    const bool regfed_ok = g.k % 4 == 0 && g.k >= KC && reinterpret_cast<uintptr_t>(g.a) % 16 == 0 && g.a_batch % 4 == 0;
+    const int64_t tiles32 = ceil_div(g.m, 32) * ceil_div(g.n, 32) * batches;
+    if (regfed_ok && !(e && e[0] == '0') && ((e && e[0] == 'f') || tiles32 <= 512)) return GEMM_REGISTER_FED;
+    return tiles64 >= 512 || g.k < 4 * KC ? GEMM_STAGED_64 : GEMM_STAGED_32_KSPLIT;
+}
+
+template <class Loader>
+int launch(const GemmArgs &g, const Loader &ld, int batches, hipStream_t stream) {
+    const GemmKernel kernel = choose_gemm(g, batches);
+    if (kernel == GEMM_REGISTER_FED) {
+        dim3 grid(unsigned(ceil_div(g.n, 32)), unsigned(ceil_div(g.m, 32)), unsigned(batches));
+        hipLaunchKernelGGL((gemm_f32_regfed_kernel<Loader>), grid, dim3(64 * KS_WAVES), 0, stream, g, ld);
+        TSX_LAUNCH_CHECK("gemm_f32_regfed_kernel");
+        return 0;
+    }
+    if (kernel == GEMM_STAGED_64) {
         dim3 grid(unsigned(ceil_div(g.n, 64)), unsigned(ceil_div(g.m, 64)), unsigned(batches));
         hipLaunchKernelGGL((gemm_f32_kernel<Loader, 2, 2, 1>), grid, dim3(THREADS), 0, stream, g, ld);
     } else {
@@ -360,9 +712,10 @@ int gemm_f32_batched(const float *a, int64_t a_batch, const float *b, int64_t ld
 
 extern "C" {
 
-int tsx_conv2d_f32_nchw(const tsx_conv2d_geom *geo, const float *x_dev, const float *w_oihw_dev, float padding_value,
-                        const float *bias_dev, int32_t act, float slope, float *out_dev, void *stream) {
-    TSX_REQUIRE(geo && x_dev && w_oihw_dev && out_dev, "conv2d_f32: null argument");
+// The GEMM view of a convolution: weights [cout][c kh kw] x implicit im2col [c kh kw][n ho wo].
+static int conv_f32_problem(const tsx_conv2d_geom *geo, const float *x_dev, const float *w_oihw_dev, float padding_value,
+                            const float *bias_dev, int32_t act, float slope, float *out_dev, tsx::GemmArgs &g,
+                            tsx::ConvLoader &ld) {
     TSX_REQUIRE(geo->n > 0 && geo->c > 0 && geo->h > 0 && geo->w > 0 && geo->cout > 0 && geo->kh > 0 && geo->kw > 0,
                 "conv2d_f32: non-positive extent");
     TSX_REQUIRE(geo->stride_h > 0 && geo->stride_w > 0 && geo->dilation_h > 0 && geo->dilation_w > 0,
@@ -373,7 +726,7 @@ int tsx_conv2d_f32_nchw(const tsx_conv2d_geom *geo, const float *x_dev, const fl
     TSX_REQUIRE(ho > 0 && wo > 0, "conv2d_f32: empty output %dx%d", ho, wo);
     const int64_t cols = int64_t(geo->n) * ho * wo;
     TSX_REQUIRE(cols < (int64_t(1) << 31), "conv2d_f32: too many output positions");
-    tsx::GemmArgs g{};
+    g = tsx::GemmArgs{};
     g.a = w_oihw_dev;
     g.c = out_dev;
     g.m = geo->cout;
@@ -384,7 +737,7 @@ int tsx_conv2d_f32_nchw(const tsx_conv2d_geom *geo, const float *x_dev, const fl
     g.act = act;
     g.slope = slope;
     g.act_body = (cols * geo->cout) / 4 * 4;
-    tsx::ConvLoader ld{};
+    ld = tsx::ConvLoader{};
     ld.x = x_dev;
     ld.c = geo->c;
     ld.h = geo->h;
@@ -400,7 +753,38 @@ int tsx_conv2d_f32_nchw(const tsx_conv2d_geom *geo, const float *x_dev, const fl
     ld.wo = wo;
     ld.howo = ho * wo;
     ld.padding_value = padding_value;
+    return 0;
+}
+
+int tsx_conv2d_f32_nchw(const tsx_conv2d_geom *geo, const float *x_dev, const float *w_oihw_dev, float padding_value,
+                        const float *bias_dev, int32_t act, float slope, float *out_dev, void *stream) {
+    TSX_REQUIRE(geo && x_dev && w_oihw_dev && out_dev, "conv2d_f32: null argument");
+    tsx::GemmArgs g;
+    tsx::ConvLoader ld;
+    const int rc = conv_f32_problem(geo, x_dev, w_oihw_dev, padding_value, bias_dev, act, slope, out_dev, g, ld);
+    if (rc) return rc;
+    if (tsx::conv3x3_small_takes(g, ld))
+        return geo->c <= 32 ? tsx::launch_conv3x3_small<2>(g, ld, tsx::as_stream(stream))
+                            : tsx::launch_conv3x3_small<4>(g, ld, tsx::as_stream(stream));
     return tsx::launch(g, ld, 1, tsx::as_stream(stream));
+}
+
+int tsx_conv2d_f32_plan_info(const tsx_conv2d_geom *geo, const float *w_oihw_dev, char *text, size_t text_bytes) {
+    TSX_REQUIRE(geo && w_oihw_dev && text && text_bytes > 0, "conv2d_f32_plan_info: null argument");
+    tsx::GemmArgs g;
+    tsx::ConvLoader ld;
+    const int rc = conv_f32_problem(geo, nullptr, w_oihw_dev, 0.f, nullptr, TSX_ACT_NONE, 0.f, nullptr, g, ld);
+    if (rc) return rc;
+    const char *name = "small_3x3";
+    int tile = 32;
+    if (!tsx::conv3x3_small_takes(g, ld)) {
+        const tsx::GemmKernel k = tsx::choose_gemm(g, 1);
+        name = k == tsx::GEMM_REGISTER_FED ? "register_fed" : k == tsx::GEMM_STAGED_64 ? "staged_64x64" : "staged_32x32_ksplit";
+        if (k == tsx::GEMM_STAGED_64) tile = 64;
+    }
+    std::snprintf(text, text_bytes, "kernel=%s tiles=%lld", name,
+                  (long long)(tsx::ceil_div(g.m, tile) * tsx::ceil_div(g.n, tile)));
+    return 0;
 }
 
 int tsx_inner_prod_f32(int32_t m, int32_t n, int32_t k, const float *lhs_dev, const float *rhs_dev, int32_t transpose,

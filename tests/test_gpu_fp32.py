@@ -68,6 +68,115 @@ def test_conv2d_f32_config1_bias_relu(tsx, port):
     assert (got >= 0).all()
 
 
+def small_layer_cases(count, seed):
+    """Seeded 3x3 layers of the kind the small-layer kernel admits (a multiple of 4 channels, up to 64): strides,
+    dilations, asymmetric padding, output channels and positions that end inside a 32 x 32 tile, several images."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        c = int(rng.choice([4, 8, 16, 28, 32, 36, 48, 60, 64]))
+        cout = int(rng.choice([1, 7, 32, 33, 64, 70, 100]))
+        n, h, w = int(rng.integers(1, 4)), int(rng.integers(3, 24)), int(rng.integers(3, 30))
+        st = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        dl = (int(rng.choice([1, 1, 2, 3])), int(rng.choice([1, 1, 2])))
+        pads = tuple(int(rng.integers(0, 4)) for _ in range(4))
+        if h + pads[0] + pads[1] < 2 * dl[0] + 1 or w + pads[2] + pads[3] < 2 * dl[1] + 1:
+            continue
+        cases.append((n, c, h, w, cout, 3, 3, pads, st, dl))
+    return cases
+
+
+SMALL_FIXED = [
+    (1, 64, 56, 56, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),      # BASELINE config 1
+    (2, 64, 28, 28, 128, 3, 3, (1, 0, 2, 1), (2, 1), (1, 1)),
+    (1, 60, 30, 30, 70, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),
+    (3, 32, 5, 5, 48, 3, 3, (3, 3, 3, 3), (1, 1), (2, 2)),        # more padding than map
+    (1, 4, 3, 3, 1, 3, 3, (0, 0, 0, 0), (1, 1), (1, 1)),          # one output value
+]
+
+
+@pytest.mark.parametrize("case", small_layer_cases(16, 411) + SMALL_FIXED)
+def test_conv2d_f32_small_layer_kernel(tsx, port, monkeypatch, case):
+    """The small-layer 3x3 kernel by itself (TSX_CONV_F32_SMALL=force puts layers of any size on it, and
+    tsx_conv2d_f32_plan_info confirms it), with a padding value, bias and LeakyReLU, and without any of them."""
+    n, c, h, w, cout, kh, kw, pads, st, dl = case
+    monkeypatch.setenv("TSX_CONV_F32_SMALL", "force")
+    rng = np.random.default_rng(hash(case) % (1 << 31))
+    x = rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)
+    wt = (rng.standard_normal((cout, c, kh, kw)) * np.sqrt(2.0 / (c * kh * kw))).astype(np.float32)
+    bias = (rng.standard_normal(cout) * 0.1).astype(np.float32)
+    wd = _dev(wt)
+    assert tsx.conv2d_f32_plan_info(x.shape, wd, pads, st, dl)["kernel"] == "small_3x3"
+    got = tsx.conv2d_f32(_dev(x), wd, pads, st, dl, padding_value=0.75, bias=_dev(bias), act="leaky_relu", slope=0.1).cpu().numpy()
+    exp = port.add_bias(port.conv2d_f32(x, wt, pads, st, dl, padding_value=0.75), bias)
+    exp = np.where(exp > 0, exp, np.float32(0.1) * exp)
+    assert got.shape == exp.shape
+    assert _close(got, exp), np.abs(got - exp).max()
+    got = tsx.conv2d_f32(_dev(x), wd, pads, st, dl).cpu().numpy()
+    assert _close(got, port.conv2d_f32(x, wt, pads, st, dl)), case
+
+
+def test_conv2d_f32_small_layer_kernel_exact_integers(tsx, port, monkeypatch):
+    """Small-integer data (every product and partial sum exact in fp32): equal bits whatever the summation order,
+    so a wrong tap, channel or padding element cannot hide inside the tolerance."""
+    monkeypatch.setenv("TSX_CONV_F32_SMALL", "force")
+    rng = np.random.default_rng(412)
+    for (n, c, h, w, cout, pads, st, dl) in ((2, 8, 9, 10, 5, (1, 2, 2, 1), (1, 1), (1, 1)), (1, 64, 20, 33, 40, (1, 1, 1, 1), (1, 1), (1, 1)),
+                                             (3, 36, 11, 7, 66, (2, 0, 1, 3), (2, 1), (1, 2))):
+        x = rng.integers(-8, 9, (n, c, h, w)).astype(np.float32)
+        wt = rng.integers(-4, 5, (cout, c, 3, 3)).astype(np.float32)
+        wd = _dev(wt)
+        assert tsx.conv2d_f32_plan_info(x.shape, wd, pads, st, dl)["kernel"] == "small_3x3"
+        got = tsx.conv2d_f32(_dev(x), wd, pads, st, dl, padding_value=3.0).cpu().numpy()
+        assert np.array_equal(bits(got), bits(port.conv2d_f32(x, wt, pads, st, dl, padding_value=3.0)))
+
+
+def test_conv2d_f32_kernel_choice(tsx, monkeypatch):
+    """What the planner picks by itself: the small-layer kernel for config 1, the register-fed kernel for a small
+    layer it does not admit (128 channels), staged tiles for large layers; "0" switches either off."""
+    import torch
+    w64 = torch.zeros((64, 64, 3, 3), device="cuda")
+    assert tsx.conv2d_f32_plan_info((1, 64, 56, 56), w64, (1, 1, 1, 1))["kernel"] == "small_3x3"
+    assert tsx.conv2d_f32_plan_info((32, 64, 56, 56), w64, (1, 1, 1, 1))["kernel"] == "staged_64x64"
+    assert tsx.conv2d_f32_plan_info((1, 128, 28, 28), torch.zeros((128, 128, 3, 3), device="cuda"), (1, 1, 1, 1))["kernel"] == "register_fed"
+    monkeypatch.setenv("TSX_CONV_F32_SMALL", "0")
+    assert tsx.conv2d_f32_plan_info((1, 64, 56, 56), w64, (1, 1, 1, 1))["kernel"] == "register_fed"
+    monkeypatch.setenv("TSX_GEMM_F32_REGFED", "0")
+    assert tsx.conv2d_f32_plan_info((1, 64, 56, 56), w64, (1, 1, 1, 1))["kernel"] == "staged_32x32_ksplit"
+
+
+@pytest.mark.parametrize("case", CONV_CASES + small_layer_cases(6, 413))
+def test_conv2d_f32_register_fed_kernel(tsx, port, monkeypatch, case):
+    """The register-fed kernel by itself (TSX_GEMM_F32_REGFED=force; it needs K a multiple of 4 and at least one
+    32-deep chunk, other cases are skipped), bias + ReLU and a padding value."""
+    n, c, h, w, cout, kh, kw, pads, st, dl = case
+    monkeypatch.setenv("TSX_CONV_F32_SMALL", "0")
+    monkeypatch.setenv("TSX_GEMM_F32_REGFED", "force")
+    rng = np.random.default_rng(hash(case) % (1 << 31))
+    x = rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)
+    wt = (rng.standard_normal((cout, c, kh, kw)) * np.sqrt(2.0 / (c * kh * kw))).astype(np.float32)
+    bias = (rng.standard_normal(cout) * 0.1).astype(np.float32)
+    wd = _dev(wt)
+    if tsx.conv2d_f32_plan_info(x.shape, wd, pads, st, dl)["kernel"] != "register_fed":
+        assert (c * kh * kw) % 4 != 0 or c * kh * kw < 32, case
+        pytest.skip("K = %d: the register-fed kernel takes multiples of 4 from 32 up" % (c * kh * kw))
+    got = tsx.conv2d_f32(_dev(x), wd, pads, st, dl, padding_value=-0.5, bias=_dev(bias), act="relu").cpu().numpy()
+    exp = port.relu(port.add_bias(port.conv2d_f32(x, wt, pads, st, dl, padding_value=-0.5), bias))
+    assert _close(got, exp), np.abs(got - exp).max()
+
+
+@pytest.mark.parametrize("transpose", [False, True])
+def test_inner_prod_f32_register_fed_kernel(tsx, port, monkeypatch, transpose):
+    monkeypatch.setenv("TSX_GEMM_F32_REGFED", "force")
+    rng = np.random.default_rng(414)
+    for m, k, n in ((130, 200, 260), (65, 64, 33), (200, 1024, 96)):
+        lhs = rng.standard_normal((m, k)).astype(np.float32)
+        rhs = (rng.standard_normal((k, n)) * 0.05).astype(np.float32)
+        arg = np.ascontiguousarray(rhs.T) if transpose else rhs
+        got = tsx.inner_prod_f32(_dev(lhs), _dev(arg), transpose).cpu().numpy()
+        assert _close(got, port.inner_prod_f32(lhs, arg, transpose)), (m, k, n)
+
+
 def test_conv2d_f32_padding_value_and_exact_integers(tsx, port):
     # small-integer data: every product and partial sum is exact in fp32, so any order gives equal bits
     rng = np.random.default_rng(401)
