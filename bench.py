@@ -409,7 +409,8 @@ def kernels_leg(reps=20):
     # fp32 BASELINE config 1 (1x64x56x56 * 64x64x3x3, bias + ReLU): implicit GEMM and both Winograd modes
     x1, w1, b1 = torch.rand((1, 64, 56, 56), device=dev) * 2 - 1, rnd(64, 64, 3, 3) * 0.06, rnd(64) * 0.01
     flops1 = 2.0 * 64 * 56 * 56 * 64 * 9
-    timed("conv2d_f32 config 1 (gemm_f32_kernel)", "mfma_f32", flops1, lambda: capi.conv2d_f32(x1, w1, (1, 1, 1, 1), bias=b1, act="relu"))
+    c1_launch, _ = capi.conv2d_f32_prepared(x1, w1, (1, 1, 1, 1), bias=b1, act="relu")
+    timed("conv2d_f32 config 1 (conv3x3_f32_small_kernel)", "mfma_f32", flops1, c1_launch)
     w63, w23 = capi.WinogradF63(w1, (1, 1, 1, 1)), capi.WinogradF23(w1, (1, 1, 1, 1))
     timed("winograd F(6,3) config 1 (direct-conv flops)", "mfma_f32", flops1, lambda: w63(x1, bias=b1, act="relu"))
     timed("winograd F(2,3) config 1 (direct-conv flops)", "mfma_f32", flops1, lambda: w23(x1, bias=b1, act="relu"))
@@ -428,7 +429,8 @@ def kernels_leg(reps=20):
     for m in (4096, 256, 1):
         a, rs = ri8(m, k), torch.rand(m, device=dev) * 1e-2
         if m > 32:
-            timed("gemm_i8 M=%d K=N=4096 (conv_i8_ws_kernel, row-major)" % m, "mfma_i8", 2.0 * m * n * k,
+            timed("gemm_i8 M=%d K=N=4096 (%s)" % (m, "gemm_i8_ksplit_kernel" if m <= 512 else "conv_i8_ws_kernel, row-major"),
+                  "mfma_i8", 2.0 * m * n * k,
                   lambda a=a, rs=rs: gemm(a, dq=dq, row_scale=rs, bias=bias))
         else:
             timed("gemm_i8 M=%d K=N=4096 (gemm_i8_skinny_kernel)" % m, "hbm", m * k + k * n + 4.0 * m * n + 4.0 * n,

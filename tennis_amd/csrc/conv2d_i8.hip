@@ -24,6 +24,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <mutex>
 
 namespace {
@@ -924,6 +925,133 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_i8_skinny_kernel(GemmParam
     });
 }
 
+// ------------------------------------------------------------------ K-split int8 GEMM (a few hundred rows)
+// A GEMM with a few hundred activation rows and a large weight matrix has too few output tiles to give every CU a
+// tile of a shape that reuses its operands: the tiled kernels would walk K serially on a fraction of the chip, or
+// read the weights once per 32 rows.  Here a workgroup owns FR x FC fragments (32 FR rows x
+// 32 FC output columns) and its 8 wavefronts SPLIT K (interleaved K-steps): each wavefront loads the operands of
+// BATCH K-steps straight from global memory into MFMA operand registers (no LDS on the way in: no two wavefronts
+// read the same bytes), multiplies them into its own FR x FC accumulators, and the eight partial tiles are added
+// through LDS -- int32, exact, so the order is free and results equal the tiled kernels' and the oracle's.  The
+// epilogue then runs on all eight wavefronts with lanes along 4 consecutive output columns (one 16-byte store per
+// lane for plain fp32 output).
+// acc register r of lane l: column (weight row) 8*(r/4) + 4*(l/32) + r%4 of the fragment, activation row l%32.
+constexpr int KS_WAVES = 8;
+
+template <int FR, int FC, int BATCH>
+__global__ __launch_bounds__(KS_WAVES * 64) void gemm_i8_ksplit_kernel(GemmParams p) {
+    constexpr int FRAGS = FR * FC;
+    __shared__ int red[4][FRAGS][16][64];
+    const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int frag0 = blockIdx.x * FC, row0 = blockIdx.y * FR * 32;
+    const int frags = p.coutp / 32;
+    const int ksteps = p.cblocks;
+    // B operands: activation rows row0 + 32 fr + lane % 32 (beyond m: the last row, never stored), the 16 K bytes
+    // of group lane / 32 of each half K-step.  Lanes of rows beyond m load nothing (a masked lane costs the
+    // memory pipeline nothing; with a single row the B loads all but vanish).
+    const int8_t *b_ptr[FR];
+    bool row_ok[FR];
+    tsx::static_for<0, FR>([&](auto fc_) {
+        constexpr int fr = decltype(fc_)::value;
+        b_ptr[fr] = p.xs + int64_t(min(row0 + fr * 32 + lane % 32, p.positions - 1)) * p.cp + (lane / 32) * 16;
+        row_ok[fr] = row0 + fr * 32 + lane % 32 < p.positions;
+    });
+    // A operands: packed[ks][frag][half][lane][16]; fragments beyond the packed columns: the last one, never stored
+    const int8_t *a_ptr[FC];
+    tsx::static_for<0, FC>([&](auto fc_) {
+        constexpr int fc = decltype(fc_)::value;
+        a_ptr[fc] = p.wp + (int64_t(min(frag0 + fc, frags - 1)) * 128 + lane) * 16;
+    });
+    const int64_t a_kstride = int64_t(frags) * 2048;
+    v16i acc[FR][FC];
+    tsx::static_for<0, FRAGS>([&](auto fc_) {
+        constexpr int f = decltype(fc_)::value;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[f / FC][f % FC][r] = 0;
+    });
+    const v4i zero = {0, 0, 0, 0};
+    for (int ks0 = wave; ks0 < ksteps; ks0 += KS_WAVES * BATCH) {
+        v4i a[BATCH][FC][2], b[BATCH][FR][2];
+        tsx::static_for<0, BATCH>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            const int ks = ks0 + u * KS_WAVES;
+            const bool on = ks < ksteps;        // uniform
+            const int kk = on ? ks : 0;
+            tsx::static_for<0, 2>([&](auto hc) {
+                constexpr int h = decltype(hc)::value;
+                tsx::static_for<0, FC>([&](auto fc_) {
+                    constexpr int fc = decltype(fc_)::value;
+                    a[u][fc][h] = on ? *reinterpret_cast<const v4i *>(a_ptr[fc] + kk * a_kstride + h * 1024) : zero;
+                });
+                tsx::static_for<0, FR>([&](auto fr_) {
+                    constexpr int fr = decltype(fr_)::value;
+                    b[u][fr][h] = (on && row_ok[fr]) ? *reinterpret_cast<const v4i *>(b_ptr[fr] + kk * 64 + h * 32) : zero;
+                });
+            });
+        });
+        tsx::static_for<0, BATCH>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            tsx::static_for<0, 2>([&](auto hc) {
+                constexpr int h = decltype(hc)::value;
+                tsx::static_for<0, FRAGS>([&](auto fc_) {
+                    constexpr int fr = decltype(fc_)::value / FC, fc = decltype(fc_)::value % FC;
+                    acc[fr][fc] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[u][fc][h], b[u][fr][h], acc[fr][fc], 0, 0, 0);
+                });
+            });
+        });
+    }
+    // eight partial tiles -> four (wavefronts 4..7 hand theirs to 0..3) -> LDS, where every wavefront picks up its
+    // share of the sums
+    if (wave >= 4) {
+        tsx::static_for<0, FRAGS>([&](auto fc_) {
+            constexpr int f = decltype(fc_)::value;
+            tsx::static_for<0, 16>([&](auto rc) { red[wave - 4][f][decltype(rc)::value][lane] = acc[f / FC][f % FC][decltype(rc)::value]; });
+        });
+    }
+    __syncthreads();
+    if (wave < 4) {
+        tsx::static_for<0, FRAGS>([&](auto fc_) {
+            constexpr int f = decltype(fc_)::value;
+            tsx::static_for<0, 16>([&](auto rc) { acc[f / FC][f % FC][decltype(rc)::value] += red[wave][f][decltype(rc)::value][lane]; });
+        });
+    }
+    __syncthreads();
+    if (wave < 4) {
+        tsx::static_for<0, FRAGS>([&](auto fc_) {
+            constexpr int f = decltype(fc_)::value;
+            tsx::static_for<0, 16>([&](auto rc) { red[wave][f][decltype(rc)::value][lane] = acc[f / FC][f % FC][decltype(rc)::value]; });
+        });
+    }
+    __syncthreads();
+    // (fragment f, register group g): registers 4g .. 4g+3 of a lane are 4 consecutive output columns of one row
+    const bool plain = p.out_f32 && !p.out_i8 && !p.st_out && !p.out_acc && !p.residual && p.act <= TSX_ACT_LEAKY_RELU &&
+                       p.cout % 4 == 0 && reinterpret_cast<uintptr_t>(p.out_f32) % 16 == 0 && reinterpret_cast<uintptr_t>(p.dq) % 16 == 0;
+    for (int item = wave; item < FRAGS * 4; item += KS_WAVES) {
+        const int f = item / 4, g4 = item % 4;
+        const int fr = f / FC, fc = f % FC;
+        int sum[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sum[j] = red[0][f][4 * g4 + j][lane] + red[1][f][4 * g4 + j][lane] + red[2][f][4 * g4 + j][lane] + red[3][f][4 * g4 + j][lane];
+        const int row = row0 + fr * 32 + lane % 32;
+        const int co = (frag0 + fc) * 32 + 8 * g4 + 4 * (lane / 32);
+        if (row >= p.positions || co >= p.cout) continue;
+        const float rs = p.row_scale ? p.row_scale[row] : 0.f;
+        const int64_t idx = int64_t(row) * p.cout + co;
+        if (plain) {
+            typedef float v4f __attribute__((ext_vector_type(4)));
+            const v4f dq = *reinterpret_cast<const v4f *>(p.dq + co);       // co % 4 == 0; dq is required with fp32 output
+            v4f v;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = tsx::epi_value<false>(p, sum[j], idx + j, dq[j], p.bias ? p.bias[co + j] : 0.f, rs);
+            *reinterpret_cast<v4f *>(p.out_f32 + idx) = v;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (co + j < p.cout) emit(p, sum[j], idx + j, p.dq ? p.dq[co + j] : 0.f, p.bias ? p.bias[co + j] : 0.f, rs);
+        }
+    }
+}
+
 // ------------------------------------------------------------------ host side
 
 constexpr int BM = 128, BN = 128;
@@ -1478,6 +1606,19 @@ int tsx_gemm_i8(int32_t m, int32_t n, int32_t k, const int8_t *a_dev, const void
         hipLaunchKernelGGL(gemm_i8_skinny_kernel, dim3(unsigned(tsx::ceil_div(n, 32))), dim3(SK_WAVES * 64), 0, stream, p);
         TSX_LAUNCH_CHECK("gemm_i8_skinny_kernel");
         return 0;
+    }
+    // TSX_GEMM_I8_KSPLIT: "0" never, "force" every GEMM of more than 32 rows (tests); otherwise up to 512 rows against
+    // 8 MiB of weights and more (measured, K = N = 4096: 256 rows 16.8 us against 23.1 on the window-stationary
+    // kernel; with K = N = 2048 that kernel is ahead, 9.6 us against 10.9)
+    {
+        const char *e = std::getenv("TSX_GEMM_I8_KSPLIT");
+        const int64_t tiles = tsx::ceil_div(m, 64) * tsx::ceil_div(n, 64);
+        if (!(e && e[0] == '0') && ((e && e[0] == 'f') || (m <= 512 && int64_t(kp) * n >= (int64_t(8) << 20)))) {
+            hipLaunchKernelGGL((gemm_i8_ksplit_kernel<2, 2, 4>), dim3(unsigned(tsx::ceil_div(n, 64)), unsigned(tsx::ceil_div(m, 64))),
+                               dim3(KS_WAVES * 64), 0, stream, p);
+            TSX_LAUNCH_CHECK("gemm_i8_ksplit_kernel");
+            return 0;
+        }
     }
     // Enough rows to fill MFMA fragments: the window-stationary kernel in its GEMM form (a 1x1 layer over m
     // one-pixel rows, row-major output).  Residual terms stay on the tiled kernel.

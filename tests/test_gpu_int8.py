@@ -611,6 +611,38 @@ def test_gemm_i8_f32_output_only(tsx, port, m, k, n, act):
         assert np.array_equal(bits(out.cpu().numpy()), bits(exp)), (m, k, n, act, row_scale is None)
 
 
+@pytest.mark.parametrize("m,k,n", [(33, 64, 128), (256, 1024, 1024), (130, 200, 260), (257, 320, 96), (100, 512, 30),
+                                   (64, 4096, 192), (500, 192, 1000), (65, 2048, 66)])
+def test_gemm_i8_k_split_kernel(tsx, port, monkeypatch, m, k, n):
+    """The K-split kernel by itself (TSX_GEMM_I8_KSPLIT=force gives it every GEMM of more than 32 rows; by itself
+    the planner takes it for up to 512 rows against 8 MiB of weights): its 16-byte fp32 epilogue with and without
+    row scale, bias and ReLU, and its per-element epilogue with the raw accumulators, requantized rows and
+    LeakyReLU; rows and columns that end inside a 64 x 64 tile, K-steps that do not divide by the 8 wavefronts."""
+    monkeypatch.setenv("TSX_GEMM_I8_KSPLIT", "force")
+    rng = np.random.default_rng(330 + m + n)
+    a = rng.integers(-128, 128, (m, k)).astype(np.int8)
+    b = rng.integers(-128, 128, (k, n)).astype(np.int8)
+    dqw = rng.uniform(1e-4, 1e-3, n).astype(np.float32)
+    dqa = rng.uniform(0.5, 2.0, m).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    qs = rng.uniform(5, 20, m).astype(np.float32)
+    g = tsx.GemmI8(_dev(b))
+    for row_scale, with_bias, act in ((dqa, True, "relu"), (None, True, None), (dqa, False, None)):
+        out, _, _ = g(_dev(a), dq=_dev(dqw), row_scale=None if row_scale is None else _dev(row_scale),
+                      bias=_dev(bias) if with_bias else None, act=act)
+        exp = port.gemm_i8_dequant(a, b, dqw, row_scale, bias if with_bias else None)
+        if act == "relu":
+            exp = port.relu(exp)
+        assert np.array_equal(bits(out.cpu().numpy()), bits(exp)), (m, k, n, act, row_scale is None, with_bias)
+    out, q, acc = g(_dev(a), dq=_dev(dqw), row_scale=_dev(dqa), bias=_dev(bias), act="leaky_relu", slope=0.1, q_scales=_dev(qs),
+                    want_acc=True)
+    exp, exp_acc = port.gemm_i8_dequant(a, b, dqw, dqa, bias, return_acc=True)
+    exp = port.leaky_relu(exp, 0.1)
+    assert np.array_equal(acc.cpu().numpy(), exp_acc)
+    assert np.array_equal(bits(out.cpu().numpy()), bits(exp))
+    assert np.array_equal(q.cpu().numpy(), port.quantize(exp, qs))
+
+
 def test_gemm_i8_requantized_rows(tsx, port):
     """int8 output with one consumer scale per row (base_quantize.cpp:26 groups by the first extent)."""
     rng = np.random.default_rng(320)
