@@ -1341,6 +1341,9 @@ int tsx_conv2d_i8_plan_info(const tsx_conv2d_geom *g, char *text, size_t text_by
     else if (pl.use_ws && pl.wsp.flat)
         std::snprintf(text, text_bytes, "kernel=%s fp32_kernel=%s fragments_per_tile=%d tiles=%lld resident=%d", base, base,
                       pl.wsp.fl_nta + pl.wsp.fl_ntb, (long long)(pl.wsp.fl_tiles * (pl.wsp.coutp / 128)), int(pl.wsp.fl_resident));
+    else if (pl.use_ws)
+        std::snprintf(text, text_bytes, "kernel=%s fp32_kernel=%s fragments_per_wavefront=%d wavefronts_along_cout=%d tiles=%lld blocks_per_window=%d",
+                      base, base, pl.wsp.nt, pl.wsp.wm, (long long)(pl.wsp.tiles * ((g->cout + 32 * pl.wsp.wm - 1) / (32 * pl.wsp.wm))), pl.wsp.cbs);
     else
         std::snprintf(text, text_bytes, "kernel=%s fp32_kernel=%s", base, base);
     return 0;

@@ -341,7 +341,10 @@ __device__ __forceinline__ void fl_wave(const FlParams &p, int8_t *lds, int tile
                     v[r] = apply_act_conv_i8(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
                 });
             } else if (MISHX && p.act == TSX_ACT_MISH) {
-                mish_fragment(v);
+                // nothing but the requantized values leaves: the exact form only where it decides a rounding
+                if (!p.out_f32 && want_q)
+                    mish_fragment_for_rounding(v, res[j], EXTRA && p.residual && p.res_after, p.q_scales[p.n_qscales == 1 ? 0 : pimg[j]]);
+                else mish_fragment(v);
             } else if (p.act == TSX_ACT_MISH_FAST) {
                 static_for<0, 16>([&](auto rc) {
                     constexpr int r = decltype(rc)::value;

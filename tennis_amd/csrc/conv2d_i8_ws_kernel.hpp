@@ -442,7 +442,10 @@ __global__ __launch_bounds__(WS_THREADS) __attribute__((amdgpu_waves_per_eu(NT <
                             v[r] = apply_act_conv_i8(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
                         });
                     } else if (MISHX && p.act == TSX_ACT_MISH) {
-                        mish_fragment(v);
+                        // nothing but the requantized values leaves: the exact form only where it decides a rounding (the
+                        // largest tile has no registers left for it)
+                        if (NT < 7 && !ROWM && !p.out_f32 && want_q) mish_fragment_for_rounding(v, res[j], EXTRA && p.residual && p.res_after, q_scale);
+                        else mish_fragment(v);
                     } else if (p.act == TSX_ACT_MISH_FAST) {
                         static_for<0, 16>([&](auto rc) {
                             constexpr int r = decltype(rc)::value;

@@ -117,7 +117,9 @@ __device__ __forceinline__ void epilogue_rows16(const EpiParams &p, const v16i &
 #pragma unroll
         for (int r = 0; r < 16; ++r) v[r] = apply_act_conv_i8(v[r], TSX_ACT_LEAKY_RELU, p.slope, true);
     } else if (MISHX && p.act == TSX_ACT_MISH) {
-        mish_fragment(v);
+        // nothing but the requantized values leaves: the exact form only where it decides a rounding
+        if (!p.out_f32 && (p.out_i8 || st_dst)) mish_fragment_for_rounding(v, res, p.residual && p.res_after, q_scale);
+        else mish_fragment(v);
     } else if (p.act == TSX_ACT_MISH_FAST) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) v[r] = apply_act_conv_i8(v[r], TSX_ACT_MISH_FAST, 0.f, true);

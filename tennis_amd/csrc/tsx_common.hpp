@@ -180,6 +180,36 @@ __device__ __forceinline__ void mish_fragment(float (&v)[16]) {
     for (int r = 0; r < 16; ++r) v[r] = t[r];
 }
 
+// The exact Mish where only a requantized int8 value leaves the kernel: round((mish(x) [+ add]) * scale) has to be
+// the exact form's, the float in between does not.  mish_short is within 5.21 * 2^-24 |x| of mish_value for every
+// float x (all 2^32 inputs compared on the device, tests/test_gpu_yolo.py), so wherever the short form's product
+// lies further from a rounding boundary k + 1/2 than that bound (taken as 8 * 2^-24 |x scale|, plus 2^-21 of the
+// product for the two float roundings behind the activation) both forms round to the same integer.  The few values
+// that lie closer -- about one in ten thousand -- are evaluated again by the exact chain, a wavefront at a time and
+// only where a lane asks.  Values in v: pre-activation in, mish out (exact where it matters).
+__device__ __forceinline__ void mish_fragment_for_rounding(float (&v)[16], const float (&add)[16], bool with_add, float scale) {
+    typedef float v16f __attribute__((ext_vector_type(16)));
+    v16f x, m;
+    unsigned near = 0;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        x[r] = v[r];
+        m[r] = mish_short(v[r]);
+        const float sum = with_add ? __fadd_rn(m[r], add[r]) : m[r];
+        const float a = __builtin_fabsf(__fmul_rn(sum, scale));
+        const float dist = __builtin_fabsf(__fsub_rn(__fsub_rn(a, __builtin_floorf(a)), 0.5f));
+        const float margin = __builtin_fmaf(__builtin_fabsf(__fmul_rn(v[r], scale)), 0x1p-21f, __builtin_fmaf(a, 0x1p-21f, 1e-30f));
+        near |= dist > margin ? 0u : 1u << r;      // NaN and infinity: near
+    }
+    if (__builtin_amdgcn_ballot_w64(near != 0) != 0) {
+#pragma clang loop unroll(disable)
+        for (int r = 0; r < 16; ++r)
+            if ((near >> r) & 1u) m[r] = mish_value(x[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) v[r] = m[r];
+}
+
 __device__ __forceinline__ float apply_act_conv_i8(float v, int act, float slope, bool in_body) {
     return apply_act(v, act, slope, in_body);
 }

@@ -186,6 +186,45 @@ def test_flat_tile_kernel_all_epilogue_terms(tsx, port, force, case, after, act)
     assert np.array_equal(bits(got), bits(port.conv2d_quantized(exp_q, wb, dqb, (ck // 2,) * 4)))
 
 
+@pytest.mark.parametrize("kernel", ["window_stationary", "flat_tile", "igemm"])
+@pytest.mark.parametrize("after", [None, False, True])
+def test_exact_mish_where_only_int8_leaves(tsx, port, force, kernel, after):
+    """A layer that hands over nothing but requantized int8 values (no fp32 output) evaluates the exact Mish only
+    where it decides a rounding and the one-exponential form elsewhere: the bytes must be those of the operator
+    chain all the same.  Checked through a consumer convolution on each kernel family, without a residual, with one
+    in front of the activation (the exact form throughout) and with one behind it; consumer scales of 20 to 60 put
+    some thousand of the 10^5..10^6 values within 10^-4 of a rounding boundary."""
+    n, cin, h, w, cout, s = (4, 70, 24, 26, 130, 1) if kernel != "igemm" else (4, 70, 24, 26, 130, 2)
+    k = 3 if kernel != "igemm" else 1
+    force(kernel)
+    rng = np.random.default_rng(977 + (0 if after is None else 1 + int(after)))
+    xq = rng.integers(-128, 128, (n, cin, h, w)).astype(np.int8)
+    wa = rng.integers(-127, 128, (cout, cin, k, k)).astype(np.int8)
+    dqa = rng.uniform(2e-5, 6e-5, cout).astype(np.float32)
+    ba = rng.standard_normal(cout).astype(np.float32)
+    qs = rng.uniform(20.0, 60.0, n).astype(np.float32)
+    A = tsx.Conv2dI8(_dev(wa), (k // 2,) * 4, (s, s))
+    assert _plan(tsx, A, xq.shape)["kernel"] == kernel
+    plain = port.conv2d_i8_fused(xq, wa, dqa, ba, None, pads=(k // 2,) * 4, strides=(s, s))[0]
+    res = None if after is None else (rng.standard_normal(plain.shape) * 0.5).astype(np.float32)
+    exp = port.mish(plain) if after is None else port.add(port.mish(plain), res) if after else port.mish(port.add(plain, res))
+    exp_q = port.quantize(exp, qs)
+    wb = rng.integers(-127, 128, (40, cout, 3, 3)).astype(np.int8)
+    dqb = rng.uniform(1e-4, 3e-4, 40).astype(np.float32)
+    B = tsx.Conv2dI8(_dev(wb), (1, 1, 1, 1))
+    sb = tsx.StagedInput(B, tuple(plain.shape))
+    sa = tsx.StagedInput(A, tuple(xq.shape))
+    A.stage(_dev(xq), sa)
+    A.run_staged(sa, _dev(dqa), _dev(ba), "mish", 0.0, q_scales=_dev(qs), staged_out=sb, want_f32=False,
+                 residual=None if res is None else _dev(res), residual_after_act=bool(after))
+    got = B.run_staged(sb, _dev(dqb))[0].cpu().numpy()
+    assert np.array_equal(bits(got), bits(port.conv2d_quantized(exp_q, wb, dqb, (1, 1, 1, 1))))
+    # the same layer's NCHW int8 output
+    q = A.run_staged(sa, _dev(dqa), _dev(ba), "mish", 0.0, q_scales=_dev(qs), want_f32=False,
+                     residual=None if res is None else _dev(res), residual_after_act=bool(after))[1]
+    assert np.array_equal(q.cpu().numpy(), exp_q)
+
+
 def test_flat_tile_kernel_reads_a_wider_staged_buffer(tsx, port, force):
     """A 3x3 convolution without padding reading the staged input of a padded one (tsx_conv2d_i8_staged_at: the
     buffer's row and image pitch are larger than the layer's own)."""

@@ -146,3 +146,27 @@ def test_layer_list_matches_yolov4():
     assert sum(1 for l in L if l["type"] == "conv") == 110          # the 110 convolutions of yolov4.cfg
     macs = yolov4.total_macs(L, 1, 608)
     assert 60e9 < macs < 68e9                                        # ~64 GMAC per 608x608 image
+
+
+def test_fast_mish_error_bound_every_float():
+    """|mish_short(x) - mish_value(x)| <= 5.21 * 2^-24 |x| for every float x (measured maximum, at x = 0.768): the
+    bound the int8-only epilogues rely on (with 8 * 2^-24 |x|) when they evaluate the exact form only next to a
+    rounding boundary.  All 2^32 bit patterns, both forms through the C ABI (tsx_add_f32 with the fast activation
+    on x + 0, tsx_mish_f32), compared in float64 on the device; non-finite results must coincide."""
+    import torch
+    from tennis_amd import capi
+    dev = torch.device("cuda:0")
+    chunk = 1 << 26
+    zeros = torch.zeros(chunk, device=dev)
+    worst = 0.0
+    for first in range(0, 1 << 32, chunk):
+        b = torch.arange(first, first + chunk, device=dev, dtype=torch.int64)
+        x = torch.where(b >= (1 << 31), b - (1 << 32), b).to(torch.int32).view(torch.float32)
+        fast = capi.add(x, zeros, act="mish_fast")
+        exact = capi.mish(x)
+        finite = torch.isfinite(x) & (x != 0)
+        assert bool((torch.isfinite(fast) == torch.isfinite(exact))[finite].all()), first
+        both = finite & torch.isfinite(exact)
+        ratio = (fast.double() - exact.double()).abs() / (x.double().abs() * 2.0 ** -24)
+        worst = max(worst, float(torch.where(both, ratio, torch.zeros_like(ratio)).max()))
+    assert worst <= 6.0, worst
