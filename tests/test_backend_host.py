@@ -43,6 +43,41 @@ def test_argument_errors_need_no_device():
     assert (ho, wo) == (28, 28)
 
 
+def test_kernel_choices_need_no_device(monkeypatch):
+    """Which kernel a layer takes is decided on the host from the geometry (and the weights' alignment) alone, and the
+    plan-info entry points report it: config 2 on the weight-stationary int8 kernel, config 1 on the small-layer fp32
+    kernel, and the environment switches that tests use to put small layers on a given kernel."""
+    from tennis_amd import capi
+    L = capi.lib()
+    for name in ("TSX_CONV_I8_FLAT", "TSX_CONV_I8_RS", "TSX_CONV_F32_SMALL", "TSX_GEMM_F32_REGFED"):
+        monkeypatch.delenv(name, raising=False)
+
+    def i8(geom):
+        buf = ctypes.create_string_buffer(256)
+        assert L.tsx_conv2d_i8_plan_info(ctypes.byref(geom), buf, len(buf)) == 0
+        return dict(word.split("=", 1) for word in buf.value.decode().split())
+
+    def f32(geom, weights_address=4096):
+        buf = ctypes.create_string_buffer(256)
+        assert L.tsx_conv2d_f32_plan_info(ctypes.byref(geom), ctypes.c_void_p(weights_address), buf, len(buf)) == 0
+        return dict(word.split("=", 1) for word in buf.value.decode().split())
+
+    c2 = capi.ConvGeom(32, 256, 28, 28, 256, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1)
+    assert i8(c2)["fp32_kernel"] == "weight_stationary"
+    monkeypatch.setenv("TSX_CONV_I8_RS", "0")
+    assert i8(c2)["fp32_kernel"] != "weight_stationary"
+    c1 = capi.ConvGeom(1, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1)
+    assert f32(c1) == {"kernel": "small_3x3", "tiles": "196"}
+    assert f32(c1, weights_address=4100)["kernel"] == "staged_32x32_ksplit"       # rows of A not 16-byte aligned
+    big = capi.ConvGeom(32, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1)
+    assert f32(big)["kernel"] == "staged_64x64"
+    monkeypatch.setenv("TSX_CONV_F32_SMALL", "force")
+    assert f32(big)["kernel"] == "small_3x3"
+    monkeypatch.setenv("TSX_CONV_F32_SMALL", "0")
+    assert f32(c1)["kernel"] == "register_fed"
+    assert L.tsx_conv2d_f32_plan_info(ctypes.byref(c1), None, None, 0) == -1
+
+
 def test_hot_path_operators_are_registered_for_hip():
     from tennis_amd import operators as ops
     for name in ops.SYMBOLS:
