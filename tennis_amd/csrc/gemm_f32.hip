@@ -230,9 +230,6 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmArgs g, Loader ld
         });
     }
 
-    float bias[16];
-    if (wk == 0) tile_bias_load(g, m0 + wm * 32, lane, bias);
-
     // reduce the K split: wavefronts wk > 0 hand their partial tile to wk == 0
     if constexpr (WK > 1) {
         __syncthreads();
@@ -267,7 +264,19 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmArgs g, Loader ld
         col_base = col;
         row_stride = g.n;
     }
-    tile_store(g, g.c + batch * g.c_batch, acc, bias, m0 + wm * 32, lane, col_base, row_stride);
+    // bias values row by row: requesting the sixteen at once (as the small-problem kernels below do) costs this
+    // kernel, whose register budget is the K loop's, a wavefront of occupancy, and its layers are large
+    float *c = g.c + batch * g.c_batch;
+    static_for<0, 16>([&](auto rc) {
+        constexpr int r = decltype(rc)::value;
+        const int row = m0 + wm * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
+        if (row < g.m) {
+            const int64_t idx = col_base + int64_t(row) * row_stride;
+            float v = acc[r];
+            if (g.bias) v = __fadd_rn(v, g.bias[row]);
+            c[idx] = apply_act_basic(v, g.act, g.slope, idx < g.act_body);   // the entry points take none / relu / leaky_relu
+        }
+    });
 }
 
 // Small problems (a single 64-channel 56x56 layer: 196 tiles of 32 x 32): the staged kernel above walks K chunk by
