@@ -429,7 +429,7 @@ def kernels_leg(reps=20):
     for m in (4096, 256, 1):
         a, rs = ri8(m, k), torch.rand(m, device=dev) * 1e-2
         if m > 32:
-            timed("gemm_i8 M=%d K=N=4096 (%s)" % (m, "gemm_i8_ksplit_kernel" if m <= 512 else "conv_i8_ws_kernel, row-major"),
+            timed("gemm_i8 M=%d K=N=4096 (%s)" % (m, "gemm_i8_ksplit_lds_kernel" if m <= 512 else "conv_i8_ws_kernel, row-major"),
                   "mfma_i8", 2.0 * m * n * k,
                   lambda a=a, rs=rs: gemm(a, dq=dq, row_scale=rs, bias=bias))
         else:

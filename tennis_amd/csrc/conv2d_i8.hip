@@ -23,6 +23,7 @@
 #include "igemm_i8.hpp"
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstdlib>
 #include <mutex>
@@ -938,6 +939,62 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_i8_skinny_kernel(GemmParam
 // acc register r of lane l: column (weight row) 8*(r/4) + 4*(l/32) + r%4 of the fragment, activation row l%32.
 constexpr int KS_WAVES = 8;
 
+// The end of a K-split tile: the eight wavefronts' partial accumulators -> four (wavefronts 4..7 hand theirs to 0..3)
+// -> LDS, where every wavefront picks up its share of the sums and runs the epilogue on it.  red: 4 x FR FC x 16 x 64 ints.
+template <int FR, int FC>
+__device__ __forceinline__ void ksplit_finish(const GemmParams &p, v16i (&acc)[FR][FC], int (*red)[FR * FC][16][64], int frag0,
+                                              int row0, int lane, int wave) {
+    constexpr int FRAGS = FR * FC;
+    if (wave >= 4) {
+        tsx::static_for<0, FRAGS>([&](auto fc_) {
+            constexpr int f = decltype(fc_)::value;
+            tsx::static_for<0, 16>([&](auto rc) { red[wave - 4][f][decltype(rc)::value][lane] = acc[f / FC][f % FC][decltype(rc)::value]; });
+        });
+    }
+    __syncthreads();
+    if (wave < 4) {
+        tsx::static_for<0, FRAGS>([&](auto fc_) {
+            constexpr int f = decltype(fc_)::value;
+            tsx::static_for<0, 16>([&](auto rc) { acc[f / FC][f % FC][decltype(rc)::value] += red[wave][f][decltype(rc)::value][lane]; });
+        });
+    }
+    __syncthreads();
+    if (wave < 4) {
+        tsx::static_for<0, FRAGS>([&](auto fc_) {
+            constexpr int f = decltype(fc_)::value;
+            tsx::static_for<0, 16>([&](auto rc) { red[wave][f][decltype(rc)::value][lane] = acc[f / FC][f % FC][decltype(rc)::value]; });
+        });
+    }
+    __syncthreads();
+    // (fragment f, register group g): registers 4g .. 4g+3 of a lane are 4 consecutive output columns of one row
+    const bool plain = p.out_f32 && !p.out_i8 && !p.st_out && !p.out_acc && !p.residual && p.act <= TSX_ACT_LEAKY_RELU &&
+                       p.cout % 4 == 0 && reinterpret_cast<uintptr_t>(p.out_f32) % 16 == 0 && reinterpret_cast<uintptr_t>(p.dq) % 16 == 0;
+    for (int item = wave; item < FRAGS * 4; item += KS_WAVES) {
+        const int f = item / 4, g4 = item % 4;
+        const int fr = f / FC, fc = f % FC;
+        int sum[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sum[j] = red[0][f][4 * g4 + j][lane] + red[1][f][4 * g4 + j][lane] + red[2][f][4 * g4 + j][lane] + red[3][f][4 * g4 + j][lane];
+        const int row = row0 + fr * 32 + lane % 32;
+        const int co = (frag0 + fc) * 32 + 8 * g4 + 4 * (lane / 32);
+        if (row >= p.positions || co >= p.cout) continue;
+        const float rs = p.row_scale ? p.row_scale[row] : 0.f;
+        const int64_t idx = int64_t(row) * p.cout + co;
+        if (plain) {
+            typedef float v4f __attribute__((ext_vector_type(4)));
+            const v4f dq = *reinterpret_cast<const v4f *>(p.dq + co);       // co % 4 == 0; dq is required with fp32 output
+            v4f v;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = tsx::epi_value<false>(p, sum[j], idx + j, dq[j], p.bias ? p.bias[co + j] : 0.f, rs);
+            *reinterpret_cast<v4f *>(p.out_f32 + idx) = v;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (co + j < p.cout) emit(p, sum[j], idx + j, p.dq ? p.dq[co + j] : 0.f, p.bias ? p.bias[co + j] : 0.f, rs);
+        }
+    }
+}
+
 template <int FR, int FC, int BATCH>
 __global__ __launch_bounds__(KS_WAVES * 64) void gemm_i8_ksplit_kernel(GemmParams p) {
     constexpr int FRAGS = FR * FC;
@@ -1000,56 +1057,117 @@ __global__ __launch_bounds__(KS_WAVES * 64) void gemm_i8_ksplit_kernel(GemmParam
             });
         });
     }
-    // eight partial tiles -> four (wavefronts 4..7 hand theirs to 0..3) -> LDS, where every wavefront picks up its
-    // share of the sums
-    if (wave >= 4) {
-        tsx::static_for<0, FRAGS>([&](auto fc_) {
-            constexpr int f = decltype(fc_)::value;
-            tsx::static_for<0, 16>([&](auto rc) { red[wave - 4][f][decltype(rc)::value][lane] = acc[f / FC][f % FC][decltype(rc)::value]; });
+    ksplit_finish<FR, FC>(p, acc, red, frag0, row0, lane, wave);
+}
+
+// The same tile with the activations through LDS.  Read straight into MFMA operand registers, the activation
+// operand of a K-step is 32 rows x 32 bytes per load instruction, which the CU's vector memory path serves at half
+// the rate of whole cache lines.  Here the workgroup copies its 64 rows in chunks of 16 K-steps (1 KiB per row, one
+// row per load instruction, double-buffered: chunk c + 1 is on its way while chunk c is multiplied, one barrier per
+// chunk) and every wavefront reads the operands of its own two K-steps of the chunk from LDS; the weights still go
+// from global memory straight into registers (1 KiB contiguous per operand).  For K of 2048 and more.
+constexpr int KL_CHUNK = 16;                      // K-steps per chunk
+constexpr int KL_PITCH = KL_CHUNK * KSTEP + 16;   // bytes per row and chunk in LDS (the 16: rows 8 apart share banks, not all)
+constexpr int KL_LDS = 2 * 64 * KL_PITCH;         // two chunk buffers; the partial sums reuse them (65 536 bytes)
+
+__global__ __launch_bounds__(KS_WAVES * 64) void gemm_i8_ksplit_lds_kernel(GemmParams p) {
+    extern __shared__ __attribute__((aligned(16))) int8_t kl_lds[];
+    static_assert(KL_LDS >= 4 * 4 * 16 * 64 * 4, "the chunk buffers hold the partial sums");
+    const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const int frag0 = blockIdx.x * 2, row0 = blockIdx.y * 64;
+    const int frags = p.coutp / 32;
+    const int ksteps = p.cblocks;
+    const int chunks = (ksteps + KL_CHUNK - 1) / KL_CHUNK;
+    const v4i zero = {0, 0, 0, 0};
+    // chunk copy: wavefront w moves rows w, w + 8, ... (beyond m: the last row, never stored), lane l bytes 16 l ..
+    const int8_t *src[8];
+    tsx::static_for<0, 8>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        src[i] = p.xs + int64_t(min(row0 + wave + 8 * i, p.positions - 1)) * p.cp + lane * 16;
+    });
+    v4i stage[8];
+    auto load_chunk = [&](int c) __attribute__((always_inline)) {
+        const int koff = c * (KL_CHUNK * KSTEP);
+        const bool inside = koff + lane * 16 < p.cp;             // K-steps beyond K: zeros
+        tsx::static_for<0, 8>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            stage[i] = inside ? *reinterpret_cast<const v4i *>(src[i] + koff) : zero;
         });
-    }
-    __syncthreads();
-    if (wave < 4) {
-        tsx::static_for<0, FRAGS>([&](auto fc_) {
-            constexpr int f = decltype(fc_)::value;
-            tsx::static_for<0, 16>([&](auto rc) { acc[f / FC][f % FC][decltype(rc)::value] += red[wave][f][decltype(rc)::value][lane]; });
+    };
+    auto store_chunk = [&](int buf) __attribute__((always_inline)) {
+        tsx::static_for<0, 8>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            *reinterpret_cast<v4i *>(kl_lds + (buf * 64 + wave + 8 * i) * KL_PITCH + lane * 16) = stage[i];
         });
-    }
-    __syncthreads();
-    if (wave < 4) {
-        tsx::static_for<0, FRAGS>([&](auto fc_) {
-            constexpr int f = decltype(fc_)::value;
-            tsx::static_for<0, 16>([&](auto rc) { red[wave][f][decltype(rc)::value][lane] = acc[f / FC][f % FC][decltype(rc)::value]; });
+    };
+    const int8_t *a_ptr[2];
+    tsx::static_for<0, 2>([&](auto fc_) {
+        constexpr int fc = decltype(fc_)::value;
+        a_ptr[fc] = p.wp + (int64_t(min(frag0 + fc, frags - 1)) * 128 + lane) * 16;
+    });
+    const int64_t a_kstride = int64_t(frags) * 2048;
+    v16i acc[2][2];
+    tsx::static_for<0, 4>([&](auto fc_) {
+        constexpr int f = decltype(fc_)::value;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[f / 2][f % 2][r] = 0;
+    });
+    // this wavefront's K-steps of a chunk: wave and wave + 8; their weights are requested a chunk ahead
+    v4i a_next[2][2][2];
+    auto load_weights = [&](int c) __attribute__((always_inline)) {
+        tsx::static_for<0, 2>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            const int ks = c * KL_CHUNK + wave + 8 * u;
+            const bool on = ks < ksteps;        // uniform
+            const int kk = on ? ks : 0;
+            tsx::static_for<0, 2>([&](auto hc) {
+                constexpr int h = decltype(hc)::value;
+                tsx::static_for<0, 2>([&](auto fc_) {
+                    constexpr int fc = decltype(fc_)::value;
+                    a_next[u][fc][h] = on ? *reinterpret_cast<const v4i *>(a_ptr[fc] + kk * a_kstride + h * 1024) : zero;
+                });
+            });
         });
-    }
+    };
+    load_chunk(0);
+    load_weights(0);
+    store_chunk(0);
     __syncthreads();
-    // (fragment f, register group g): registers 4g .. 4g+3 of a lane are 4 consecutive output columns of one row
-    const bool plain = p.out_f32 && !p.out_i8 && !p.st_out && !p.out_acc && !p.residual && p.act <= TSX_ACT_LEAKY_RELU &&
-                       p.cout % 4 == 0 && reinterpret_cast<uintptr_t>(p.out_f32) % 16 == 0 && reinterpret_cast<uintptr_t>(p.dq) % 16 == 0;
-    for (int item = wave; item < FRAGS * 4; item += KS_WAVES) {
-        const int f = item / 4, g4 = item % 4;
-        const int fr = f / FC, fc = f % FC;
-        int sum[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) sum[j] = red[0][f][4 * g4 + j][lane] + red[1][f][4 * g4 + j][lane] + red[2][f][4 * g4 + j][lane] + red[3][f][4 * g4 + j][lane];
-        const int row = row0 + fr * 32 + lane % 32;
-        const int co = (frag0 + fc) * 32 + 8 * g4 + 4 * (lane / 32);
-        if (row >= p.positions || co >= p.cout) continue;
-        const float rs = p.row_scale ? p.row_scale[row] : 0.f;
-        const int64_t idx = int64_t(row) * p.cout + co;
-        if (plain) {
-            typedef float v4f __attribute__((ext_vector_type(4)));
-            const v4f dq = *reinterpret_cast<const v4f *>(p.dq + co);       // co % 4 == 0; dq is required with fp32 output
-            v4f v;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) v[j] = tsx::epi_value<false>(p, sum[j], idx + j, dq[j], p.bias ? p.bias[co + j] : 0.f, rs);
-            *reinterpret_cast<v4f *>(p.out_f32 + idx) = v;
-        } else {
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                if (co + j < p.cout) emit(p, sum[j], idx + j, p.dq ? p.dq[co + j] : 0.f, p.bias ? p.bias[co + j] : 0.f, rs);
+    for (int c = 0; c < chunks; ++c) {
+        v4i a[2][2][2], b[2][2][2];
+        tsx::static_for<0, 8>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            a[i / 4][(i / 2) % 2][i % 2] = a_next[i / 4][(i / 2) % 2][i % 2];
+        });
+        if (c + 1 < chunks) {
+            load_chunk(c + 1);
+            load_weights(c + 1);
         }
+        tsx::static_for<0, 2>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            tsx::static_for<0, 2>([&](auto hc) {
+                constexpr int h = decltype(hc)::value;
+                tsx::static_for<0, 2>([&](auto fr_) {
+                    constexpr int fr = decltype(fr_)::value;
+                    b[u][fr][h] = *reinterpret_cast<const v4i *>(kl_lds + ((c & 1) * 64 + fr * 32 + lane % 32) * KL_PITCH +
+                                                                 (wave + 8 * u) * KSTEP + h * 32 + (lane / 32) * 16);
+                });
+            });
+        });
+        tsx::static_for<0, 2>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            tsx::static_for<0, 2>([&](auto hc) {
+                constexpr int h = decltype(hc)::value;
+                tsx::static_for<0, 4>([&](auto fc_) {
+                    constexpr int fr = decltype(fc_)::value / 2, fc = decltype(fc_)::value % 2;
+                    acc[fr][fc] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[u][fc][h], b[u][fr][h], acc[fr][fc], 0, 0, 0);
+                });
+            });
+        });
+        if (c + 1 < chunks) store_chunk((c + 1) & 1);
+        __syncthreads();
     }
+    ksplit_finish<2, 2>(p, acc, reinterpret_cast<int (*)[4][16][64]>(kl_lds), frag0, row0, lane, wave);
 }
 
 // ------------------------------------------------------------------ host side
@@ -1617,8 +1735,22 @@ int tsx_gemm_i8(int32_t m, int32_t n, int32_t k, const int8_t *a_dev, const void
         const char *e = std::getenv("TSX_GEMM_I8_KSPLIT");
         const int64_t tiles = tsx::ceil_div(m, 64) * tsx::ceil_div(n, 64);
         if (!(e && e[0] == '0') && ((e && e[0] == 'f') || (m <= 512 && int64_t(kp) * n >= (int64_t(8) << 20)))) {
-            hipLaunchKernelGGL((gemm_i8_ksplit_kernel<2, 2, 4>), dim3(unsigned(tsx::ceil_div(n, 64)), unsigned(tsx::ceil_div(m, 64))),
-                               dim3(KS_WAVES * 64), 0, stream, p);
+            const dim3 grid(unsigned(tsx::ceil_div(n, 64)), unsigned(tsx::ceil_div(m, 64)));
+            // activations through LDS where K gives the double buffer something to overlap ("forcereg": never)
+            if (kp >= 2048 && !(e && e[0] == 'f' && e[5] == 'r')) {
+                static std::atomic<bool> granted[64];
+                int dev = 0;
+                TSX_HIP(hipGetDevice(&dev));
+                if (dev < 64 && !granted[dev].load()) {     // dynamic LDS beyond 64 KiB: granted per kernel and device
+                    TSX_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_i8_ksplit_lds_kernel),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+                    granted[dev].store(true);
+                }
+                hipLaunchKernelGGL(gemm_i8_ksplit_lds_kernel, grid, dim3(KS_WAVES * 64), KL_LDS, stream, p);
+                TSX_LAUNCH_CHECK("gemm_i8_ksplit_lds_kernel");
+                return 0;
+            }
+            hipLaunchKernelGGL((gemm_i8_ksplit_kernel<2, 2, 4>), grid, dim3(KS_WAVES * 64), 0, stream, p);
             TSX_LAUNCH_CHECK("gemm_i8_ksplit_kernel");
             return 0;
         }

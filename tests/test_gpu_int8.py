@@ -612,13 +612,18 @@ def test_gemm_i8_f32_output_only(tsx, port, m, k, n, act):
 
 
 @pytest.mark.parametrize("m,k,n", [(33, 64, 128), (256, 1024, 1024), (130, 200, 260), (257, 320, 96), (100, 512, 30),
-                                   (64, 4096, 192), (500, 192, 1000), (65, 2048, 66)])
-def test_gemm_i8_k_split_kernel(tsx, port, monkeypatch, m, k, n):
-    """The K-split kernel by itself (TSX_GEMM_I8_KSPLIT=force gives it every GEMM of more than 32 rows; by itself
-    the planner takes it for up to 512 rows against 8 MiB of weights): its 16-byte fp32 epilogue with and without
-    row scale, bias and ReLU, and its per-element epilogue with the raw accumulators, requantized rows and
-    LeakyReLU; rows and columns that end inside a 64 x 64 tile, K-steps that do not divide by the 8 wavefronts."""
-    monkeypatch.setenv("TSX_GEMM_I8_KSPLIT", "force")
+                                   (64, 4096, 192), (500, 192, 1000), (65, 2048, 66), (100, 2500, 72)])
+@pytest.mark.parametrize("mode", ["force", "forcereg"])
+def test_gemm_i8_k_split_kernel(tsx, port, monkeypatch, m, k, n, mode):
+    """The K-split kernels by themselves (TSX_GEMM_I8_KSPLIT=force gives them every GEMM of more than 32 rows; by
+    itself the planner takes them for up to 512 rows against 8 MiB of weights): activations through LDS for K of
+    2048 and more, straight into registers below (and everywhere with "forcereg").  The 16-byte fp32 epilogue with
+    and without row scale, bias and ReLU, and the per-element epilogue with the raw accumulators, requantized rows
+    and LeakyReLU; rows and columns that end inside a 64 x 64 tile, K-steps that do not divide by the 8 wavefronts
+    or fill the last chunk of 16."""
+    if mode == "forcereg" and k < 2048:
+        pytest.skip("below K = 2048 both modes run the same kernel")
+    monkeypatch.setenv("TSX_GEMM_I8_KSPLIT", mode)
     rng = np.random.default_rng(330 + m + n)
     a = rng.integers(-128, 128, (m, k)).astype(np.int8)
     b = rng.integers(-128, 128, (k, n)).astype(np.int8)
