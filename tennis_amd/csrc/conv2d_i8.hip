@@ -939,60 +939,92 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_i8_skinny_kernel(GemmParam
 // acc register r of lane l: column (weight row) 8*(r/4) + 4*(l/32) + r%4 of the fragment, activation row l%32.
 constexpr int KS_WAVES = 8;
 
-// The end of a K-split tile: the eight wavefronts' partial accumulators -> four (wavefronts 4..7 hand theirs to 0..3)
-// -> LDS, where every wavefront picks up its share of the sums and runs the epilogue on it.  red: 4 x FR FC x 16 x 64 ints.
-template <int FR, int FC>
+// The end of a K-split tile: the eight wavefronts' partial accumulators go to LDS (SLOTS = 8: all eight and one
+// barrier; SLOTS = 4, for a kernel with 64 KiB of LDS: wavefronts 4..7 hand theirs to 0..3 first), where every
+// wavefront picks up its share of the sums and runs the epilogue on it: (fragment f, register group g) -- registers
+// 4g .. 4g+3 of a lane are 4 consecutive output columns of one row.  The scales and biases of a wavefront's share are
+// requested before the reduction and arrive under it.  red: SLOTS x FR FC x 16 x 64 ints.
+template <int FR, int FC, int SLOTS>
 __device__ __forceinline__ void ksplit_finish(const GemmParams &p, v16i (&acc)[FR][FC], int (*red)[FR * FC][16][64], int frag0,
                                               int row0, int lane, int wave) {
+    typedef float v4f __attribute__((ext_vector_type(4)));
     constexpr int FRAGS = FR * FC;
-    if (wave >= 4) {
-        tsx::static_for<0, FRAGS>([&](auto fc_) {
-            constexpr int f = decltype(fc_)::value;
-            tsx::static_for<0, 16>([&](auto rc) { red[wave - 4][f][decltype(rc)::value][lane] = acc[f / FC][f % FC][decltype(rc)::value]; });
-        });
-    }
-    __syncthreads();
-    if (wave < 4) {
-        tsx::static_for<0, FRAGS>([&](auto fc_) {
-            constexpr int f = decltype(fc_)::value;
-            tsx::static_for<0, 16>([&](auto rc) { acc[f / FC][f % FC][decltype(rc)::value] += red[wave][f][decltype(rc)::value][lane]; });
-        });
-    }
-    __syncthreads();
-    if (wave < 4) {
+    constexpr int ITEMS = (FRAGS * 4 + KS_WAVES - 1) / KS_WAVES;
+    const bool plain = p.out_f32 && !p.out_i8 && !p.st_out && !p.out_acc && !p.residual && p.act <= TSX_ACT_LEAKY_RELU &&
+                       p.cout % 4 == 0 && reinterpret_cast<uintptr_t>(p.out_f32) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(p.dq) % 16 == 0 && reinterpret_cast<uintptr_t>(p.bias) % 16 == 0;
+    int row[ITEMS], co[ITEMS];
+    bool ok[ITEMS];
+    float rs[ITEMS];
+    v4f dq[ITEMS], bias[ITEMS];
+    tsx::static_for<0, ITEMS>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        const int item = wave + KS_WAVES * i;
+        const int f = item / 4, g4 = item % 4;
+        row[i] = row0 + (f / FC) * 32 + lane % 32;
+        co[i] = (frag0 + f % FC) * 32 + 8 * g4 + 4 * (lane / 32);
+        ok[i] = item < FRAGS * 4 && row[i] < p.positions && co[i] < p.cout;
+        rs[i] = (ok[i] && p.row_scale) ? p.row_scale[row[i]] : 0.f;
+        const v4f z = {0.f, 0.f, 0.f, 0.f};
+        dq[i] = (plain && ok[i]) ? *reinterpret_cast<const v4f *>(p.dq + co[i]) : z;      // co % 4 == 0
+        bias[i] = (plain && ok[i] && p.bias) ? *reinterpret_cast<const v4f *>(p.bias + co[i]) : z;
+    });
+    if (SLOTS == 8) {
         tsx::static_for<0, FRAGS>([&](auto fc_) {
             constexpr int f = decltype(fc_)::value;
             tsx::static_for<0, 16>([&](auto rc) { red[wave][f][decltype(rc)::value][lane] = acc[f / FC][f % FC][decltype(rc)::value]; });
         });
-    }
-    __syncthreads();
-    // (fragment f, register group g): registers 4g .. 4g+3 of a lane are 4 consecutive output columns of one row
-    const bool plain = p.out_f32 && !p.out_i8 && !p.st_out && !p.out_acc && !p.residual && p.act <= TSX_ACT_LEAKY_RELU &&
-                       p.cout % 4 == 0 && reinterpret_cast<uintptr_t>(p.out_f32) % 16 == 0 && reinterpret_cast<uintptr_t>(p.dq) % 16 == 0;
-    for (int item = wave; item < FRAGS * 4; item += KS_WAVES) {
-        const int f = item / 4, g4 = item % 4;
-        const int fr = f / FC, fc = f % FC;
-        int sum[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) sum[j] = red[0][f][4 * g4 + j][lane] + red[1][f][4 * g4 + j][lane] + red[2][f][4 * g4 + j][lane] + red[3][f][4 * g4 + j][lane];
-        const int row = row0 + fr * 32 + lane % 32;
-        const int co = (frag0 + fc) * 32 + 8 * g4 + 4 * (lane / 32);
-        if (row >= p.positions || co >= p.cout) continue;
-        const float rs = p.row_scale ? p.row_scale[row] : 0.f;
-        const int64_t idx = int64_t(row) * p.cout + co;
-        if (plain) {
-            typedef float v4f __attribute__((ext_vector_type(4)));
-            const v4f dq = *reinterpret_cast<const v4f *>(p.dq + co);       // co % 4 == 0; dq is required with fp32 output
-            v4f v;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) v[j] = tsx::epi_value<false>(p, sum[j], idx + j, dq[j], p.bias ? p.bias[co + j] : 0.f, rs);
-            *reinterpret_cast<v4f *>(p.out_f32 + idx) = v;
-        } else {
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                if (co + j < p.cout) emit(p, sum[j], idx + j, p.dq ? p.dq[co + j] : 0.f, p.bias ? p.bias[co + j] : 0.f, rs);
+        __syncthreads();
+    } else {
+        if (wave >= 4) {
+            tsx::static_for<0, FRAGS>([&](auto fc_) {
+                constexpr int f = decltype(fc_)::value;
+                tsx::static_for<0, 16>([&](auto rc) { red[wave - 4][f][decltype(rc)::value][lane] = acc[f / FC][f % FC][decltype(rc)::value]; });
+            });
         }
+        __syncthreads();
+        if (wave < 4) {
+            tsx::static_for<0, FRAGS>([&](auto fc_) {
+                constexpr int f = decltype(fc_)::value;
+                tsx::static_for<0, 16>([&](auto rc) { acc[f / FC][f % FC][decltype(rc)::value] += red[wave][f][decltype(rc)::value][lane]; });
+            });
+        }
+        __syncthreads();
+        if (wave < 4) {
+            tsx::static_for<0, FRAGS>([&](auto fc_) {
+                constexpr int f = decltype(fc_)::value;
+                tsx::static_for<0, 16>([&](auto rc) { red[wave][f][decltype(rc)::value][lane] = acc[f / FC][f % FC][decltype(rc)::value]; });
+            });
+        }
+        __syncthreads();
     }
+    tsx::static_for<0, ITEMS>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        const int item = wave + KS_WAVES * i;
+        if (item < FRAGS * 4) {         // uniform
+            const int f = item / 4, g4 = item % 4;
+            int sum[4] = {0, 0, 0, 0};
+            tsx::static_for<0, SLOTS>([&](auto sc) {
+                constexpr int sl = decltype(sc)::value;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) sum[j] += red[sl][f][4 * g4 + j][lane];
+            });
+            if (ok[i]) {
+                const int64_t idx = int64_t(row[i]) * p.cout + co[i];
+                if (plain) {
+                    v4f v;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) v[j] = tsx::epi_value<false>(p, sum[j], idx + j, dq[i][j], bias[i][j], rs[i]);
+                    *reinterpret_cast<v4f *>(p.out_f32 + idx) = v;
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (co[i] + j < p.cout)
+                            emit(p, sum[j], idx + j, p.dq ? p.dq[co[i] + j] : 0.f, p.bias ? p.bias[co[i] + j] : 0.f, rs[i]);
+                }
+            }
+        }
+    });
 }
 
 template <int FR, int FC, int BATCH>
@@ -1057,7 +1089,7 @@ __global__ __launch_bounds__(KS_WAVES * 64) void gemm_i8_ksplit_kernel(GemmParam
             });
         });
     }
-    ksplit_finish<FR, FC>(p, acc, red, frag0, row0, lane, wave);
+    ksplit_finish<FR, FC, 4>(p, acc, red, frag0, row0, lane, wave);
 }
 
 // The same tile with the activations through LDS.  Read straight into MFMA operand registers, the activation
@@ -1068,11 +1100,11 @@ __global__ __launch_bounds__(KS_WAVES * 64) void gemm_i8_ksplit_kernel(GemmParam
 // from global memory straight into registers (1 KiB contiguous per operand).  For K of 2048 and more.
 constexpr int KL_CHUNK = 16;                      // K-steps per chunk
 constexpr int KL_PITCH = KL_CHUNK * KSTEP + 16;   // bytes per row and chunk in LDS (the 16: rows 8 apart share banks, not all)
-constexpr int KL_LDS = 2 * 64 * KL_PITCH;         // two chunk buffers; the partial sums reuse them (65 536 bytes)
+constexpr int KL_LDS = 2 * 64 * KL_PITCH;         // two chunk buffers; the partial tiles reuse them (131 072 bytes)
 
 __global__ __launch_bounds__(KS_WAVES * 64) void gemm_i8_ksplit_lds_kernel(GemmParams p) {
     extern __shared__ __attribute__((aligned(16))) int8_t kl_lds[];
-    static_assert(KL_LDS >= 4 * 4 * 16 * 64 * 4, "the chunk buffers hold the partial sums");
+    static_assert(KL_LDS >= 8 * 4 * 16 * 64 * 4, "the chunk buffers hold the eight partial tiles");
     const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const int frag0 = blockIdx.x * 2, row0 = blockIdx.y * 64;
     const int frags = p.coutp / 32;
@@ -1167,7 +1199,7 @@ __global__ __launch_bounds__(KS_WAVES * 64) void gemm_i8_ksplit_lds_kernel(GemmP
         if (c + 1 < chunks) store_chunk((c + 1) & 1);
         __syncthreads();
     }
-    ksplit_finish<2, 2>(p, acc, reinterpret_cast<int (*)[4][16][64]>(kl_lds), frag0, row0, lane, wave);
+    ksplit_finish<2, 2, 8>(p, acc, reinterpret_cast<int (*)[4][16][64]>(kl_lds), frag0, row0, lane, wave);
 }
 
 // ------------------------------------------------------------------ host side
@@ -1728,13 +1760,20 @@ int tsx_gemm_i8(int32_t m, int32_t n, int32_t k, const int8_t *a_dev, const void
         TSX_LAUNCH_CHECK("gemm_i8_skinny_kernel");
         return 0;
     }
-    // TSX_GEMM_I8_KSPLIT: "0" never, "force" every GEMM of more than 32 rows (tests); otherwise up to 512 rows against
-    // 8 MiB of weights and more (measured, K = N = 4096: 256 rows 16.8 us against 23.1 on the window-stationary
-    // kernel; with K = N = 2048 that kernel is ahead, 9.6 us against 10.9)
+    // TSX_GEMM_I8_KSPLIT: "0" never, "force" every GEMM of more than 32 rows (tests); otherwise GEMMs with a K long
+    // enough to split (2048 and more: the LDS form) whose 64 x 64 tiles run in one round (at most 256: that form holds
+    // one workgroup per CU).  Measured against the window-stationary kernel: K = N = 4096 with 48 / 256 rows 10.9 /
+    // 12.4 us against 14.1 / 23.0; K = N = 2048 with 64 / 256 / 512 rows 7.5 / 7.9 / 8.6 us against 8.0 / 9.5 / 10.3;
+    // K = 4096, N = 1024 with 256 / 1024 rows 10.9 / 14.2 us against 14.2 / 15.4; K = 8192, N = 2048 with 512 rows
+    // 20.7 us against 26.8.  Beyond one round it wins or loses by the shape (N = 4096, K = 4096, 512 rows: 23.6 us
+    // against 24.0; N = 2048, K = 8192, 768 rows: 37.4 against 29.8), and with K = 1024 (the register form) it loses:
+    // 7.9 us against 6.2 at 256 rows.  (Chunks of 8 K-steps kept four deep in flight through rotating register sets
+    // measured slower by 0.9 us.)
     {
         const char *e = std::getenv("TSX_GEMM_I8_KSPLIT");
         const int64_t tiles = tsx::ceil_div(m, 64) * tsx::ceil_div(n, 64);
-        if (!(e && e[0] == '0') && ((e && e[0] == 'f') || (m <= 512 && int64_t(kp) * n >= (int64_t(8) << 20)))) {
+        const bool pays = tiles <= 256 && kp >= 2048;
+        if (!(e && e[0] == '0') && ((e && e[0] == 'f') || pays)) {
             const dim3 grid(unsigned(tsx::ceil_div(n, 64)), unsigned(tsx::ceil_div(m, 64)));
             // activations through LDS where K gives the double buffer something to overlap ("forcereg": never)
             if (kp >= 2048 && !(e && e[0] == 'f' && e[5] == 'r')) {
