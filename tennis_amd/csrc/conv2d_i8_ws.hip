@@ -34,7 +34,6 @@
 #include "conv2d_i8_ws_kernel.hpp"
 
 #include <algorithm>
-#include <cstdlib>
 
 namespace tsx {
 namespace {
